@@ -1,0 +1,250 @@
+"""cuasr_amd: semiring GEMM for AMD Instinct MI355X (gfx950).
+
+The product is ``lib/libcuasr_amd.so`` (hand-written HIP kernels behind the C
+ABI of ``include/cuasr_amd.h``) and the C++ operator templates in
+``include/cuasr/`` that mirror cuASR's ``device::Srgemm`` /
+``device::SrgemmSplitKParallel``.  This module is a thin ctypes binding of the
+same C ABI for Python callers (tests, the benchmark); torch tensors are used
+only as handles to device memory.  There is no CPU fallback: if the library
+has not been built, loading raises.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libcuasr_amd.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "cuasr_amd.h")
+
+# enums of include/cuasr_amd.h
+OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
+       "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
+DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3}
+COLUMN_MAJOR, ROW_MAJOR = 0, 1
+KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3}
+STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
+                "kErrorInvalidLayout", "kErrorInvalidProblem", "kErrorNotSupported",
+                "kErrorWorkspaceNull", "kErrorInternal", "kErrorArchMismatch",
+                "kErrorInsufficientDriver", "kErrorMemoryAllocation", "kInvalid"]
+SUCCESS = 0
+
+_NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}
+
+
+class Scalar(ctypes.Union):
+    _fields_ = [("f32", ctypes.c_float), ("f64", ctypes.c_double), ("i32", ctypes.c_int32),
+                ("u32", ctypes.c_uint32), ("bits", ctypes.c_uint64)]
+
+
+class SrgemmDesc(ctypes.Structure):
+    """cuasr_amd_srgemm_desc"""
+    _fields_ = [
+        ("add_op", ctypes.c_int32), ("mult_op", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("layout_a", ctypes.c_int32), ("layout_b", ctypes.c_int32), ("layout_c", ctypes.c_int32),
+        ("m", ctypes.c_int32), ("n", ctypes.c_int32), ("k", ctypes.c_int32),
+        ("split_k_slices", ctypes.c_int32),
+        ("A", ctypes.c_void_p), ("lda", ctypes.c_int64),
+        ("B", ctypes.c_void_p), ("ldb", ctypes.c_int64),
+        ("C", ctypes.c_void_p), ("ldc", ctypes.c_int64),
+        ("D", ctypes.c_void_p), ("ldd", ctypes.c_int64),
+        ("alpha", Scalar), ("beta", Scalar), ("add_identity", Scalar), ("mult_identity", Scalar),
+        ("alpha_ptr", ctypes.c_void_p), ("beta_ptr", ctypes.c_void_p),
+        ("kernel", ctypes.c_int32), ("reserved", ctypes.c_int32),
+    ]
+
+
+class CuasrError(RuntimeError):
+    def __init__(self, status, what):
+        self.status = int(status)
+        name = STATUS_NAMES[self.status] if 0 <= self.status < len(STATUS_NAMES) else "?"
+        super().__init__(f"{what}: status {self.status} ({name})")
+
+
+_lib = None
+
+
+def load():
+    """Load the built library; raises if it is missing (no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is not built; run `python -m cuasr_amd.build` (needs hipcc). "
+                "cuasr_amd has no CPU fallback.")
+        lib = ctypes.CDLL(LIB_PATH)
+        lib.cuasr_amd_abi_version.restype = ctypes.c_int
+        lib.cuasr_amd_status_string.restype = ctypes.c_char_p
+        lib.cuasr_amd_status_string.argtypes = [ctypes.c_int]
+        lib.cuasr_amd_srgemm_can_implement.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm_can_implement.argtypes = [ctypes.POINTER(SrgemmDesc)]
+        lib.cuasr_amd_srgemm.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p]
+        lib.cuasr_amd_splitk_workspace_bytes.restype = ctypes.c_size_t
+        lib.cuasr_amd_splitk_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
+        lib.cuasr_amd_srgemm_splitk.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm_splitk.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_selected_kernel.restype = ctypes.c_char_p
+        lib.cuasr_amd_selected_kernel.argtypes = [ctypes.POINTER(SrgemmDesc)]
+        _lib = lib
+    return _lib
+
+
+# --------------------------------------------------------------------------
+# Semiring constants, as the reference functors define them
+# (include/cuasr/functional.h:28-36, :41-42, :84-85, :127-128, :167-168,
+#  :207-208, :247-248; binary_xor: examples/01_userdefined_semiring/
+#  userdefined_semiring.cu:57).  "Infinity" there is numeric_limits::max() and
+# "-infinity" numeric_limits::min() (the smallest positive normal for floating
+# point).  With infinities=True the floating-point values become true +/-inf.
+# --------------------------------------------------------------------------
+def _limits(dtype, infinities):
+    npd = np.dtype(_NP_OF[dtype])
+    if npd.kind == "f":
+        if infinities:
+            return npd.type(np.inf), npd.type(-np.inf)
+        fi = np.finfo(npd)
+        return fi.max, fi.tiny
+    ii = np.iinfo(npd)
+    return npd.type(ii.max), npd.type(ii.min)
+
+
+def op_identity(op, dtype, infinities=False):
+    hi, lo = _limits(dtype, infinities)
+    npd = _NP_OF[dtype]
+    return {"plus": npd(0), "multiplies": npd(1), "minimum": hi, "maximum": lo,
+            "logical_and": npd(1), "logical_or": npd(0),
+            "bit_and": npd(np.iinfo(npd).max if np.dtype(npd).kind == "u" else -1)
+            if np.dtype(npd).kind in "iu" else npd(1),
+            "bit_or": npd(0), "bit_xor": npd(0)}[op]
+
+
+def op_annihilator(op, dtype, infinities=False):
+    hi, lo = _limits(dtype, infinities)
+    npd = _NP_OF[dtype]
+    return {"plus": hi, "multiplies": npd(0), "minimum": lo, "maximum": hi,
+            "logical_and": npd(0), "logical_or": npd(1), "bit_and": npd(0),
+            "bit_or": npd(np.iinfo(npd).max if np.dtype(npd).kind == "u" else -1)
+            if np.dtype(npd).kind in "iu" else npd(1),
+            "bit_xor": npd(0)}[op]
+
+
+def _set_scalar(s, value, dtype):
+    s.bits = 0
+    if dtype == "f32":
+        s.f32 = float(value)
+    elif dtype == "f64":
+        s.f64 = float(value)
+    elif dtype == "i32":
+        s.i32 = int(value)
+    else:
+        s.u32 = int(value) & 0xFFFFFFFF
+
+
+class MatRef:
+    """A matrix in device memory: pointer, leading dimension (elements), layout."""
+
+    def __init__(self, ptr, ld, layout, rows, cols):
+        self.ptr, self.ld, self.layout, self.rows, self.cols = int(ptr or 0), int(ld), int(layout), int(rows), int(cols)
+
+    @staticmethod
+    def of(t):
+        """From a 2-D torch tensor whose rows or columns are contiguous."""
+        if isinstance(t, MatRef):
+            return t
+        rows, cols = t.shape
+        s0, s1 = t.stride()
+        if s0 == 1 and (cols <= 1 or s1 >= rows):
+            return MatRef(t.data_ptr(), s1 if cols > 1 else max(rows, 1), COLUMN_MAJOR, rows, cols)
+        if s1 == 1 and (rows <= 1 or s0 >= cols):
+            return MatRef(t.data_ptr(), s0 if rows > 1 else max(cols, 1), ROW_MAJOR, rows, cols)
+        raise ValueError("matrix must have unit stride along rows or columns")
+
+
+def _torch_dtype_name(t):
+    import torch
+    return {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32",
+            getattr(torch, "uint32", None): "u32"}[t.dtype]
+
+
+def make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,
+              split_k_slices=1, kernel="auto", alpha_ptr=None, beta_ptr=None):
+    a, b, d = MatRef.of(A), MatRef.of(B), MatRef.of(D)
+    c = MatRef.of(C) if C is not None else MatRef(0, d.ld, d.layout, d.rows, d.cols)
+    desc = SrgemmDesc()
+    desc.add_op, desc.mult_op, desc.dtype = OPS[add_op], OPS[mult_op], DTYPES[dtype]
+    desc.layout_a, desc.layout_b, desc.layout_c = a.layout, b.layout, d.layout
+    if c.ptr and c.layout != d.layout and min(d.rows, d.cols) > 1:
+        raise ValueError("C and D must share a layout")
+    if a.cols != b.rows or (a.rows, b.cols) != (d.rows, d.cols):
+        raise ValueError("shape mismatch")
+    desc.m, desc.n, desc.k = d.rows, d.cols, a.cols
+    desc.split_k_slices = split_k_slices
+    desc.A, desc.lda = a.ptr or None, a.ld
+    desc.B, desc.ldb = b.ptr or None, b.ld
+    desc.C, desc.ldc = c.ptr or None, c.ld
+    desc.D, desc.ldd = d.ptr or None, d.ld
+    _set_scalar(desc.alpha, alpha, dtype)
+    _set_scalar(desc.beta, beta, dtype)
+    _set_scalar(desc.add_identity, add_identity, dtype)
+    _set_scalar(desc.mult_identity, mult_identity, dtype)
+    desc.alpha_ptr = alpha_ptr
+    desc.beta_ptr = beta_ptr
+    desc.kernel = KERNELS[kernel]
+    desc.reserved = 0
+    return desc
+
+
+def _stream_handle(stream):
+    if stream is None:
+        import torch
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return ctypes.c_void_p(int(getattr(stream, "cuda_stream", stream)))
+
+
+def srgemm(add_op, mult_op, A, B, C, D, alpha=None, beta=None, add_identity=None,
+           mult_identity=None, dtype=None, kernel="auto", stream=None,
+           alpha_ptr=None, beta_ptr=None, infinities=False):
+    """D = add(mult(alpha, A (x) B), mult(beta, C)) on the GPU, asynchronously.
+
+    Defaults follow the reference epilogue (semiring_linear_combination.h:67-71):
+    alpha = MultOp::Identity, beta = MultOp::Annihilator; the identities default
+    to the reference functor constants (or +/-inf with ``infinities=True``).
+    """
+    dtype = dtype or _torch_dtype_name(D)
+    alpha = op_identity(mult_op, dtype, infinities) if alpha is None else alpha
+    beta = op_annihilator(mult_op, dtype, infinities) if beta is None else beta
+    add_identity = op_identity(add_op, dtype, infinities) if add_identity is None else add_identity
+    mult_identity = op_identity(mult_op, dtype, infinities) if mult_identity is None else mult_identity
+    desc = make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,
+                     1, kernel, alpha_ptr, beta_ptr)
+    st = load().cuasr_amd_srgemm(ctypes.byref(desc), _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_srgemm")
+    return D
+
+
+def splitk_workspace_bytes(m, n, slices, dtype):
+    desc = SrgemmDesc()
+    desc.m, desc.n, desc.split_k_slices, desc.dtype = m, n, slices, DTYPES[dtype]
+    return int(load().cuasr_amd_splitk_workspace_bytes(ctypes.byref(desc)))
+
+
+def srgemm_splitk(add_op, mult_op, A, B, C, D, slices, workspace, alpha=None, beta=None,
+                  add_identity=None, mult_identity=None, dtype=None, kernel="auto",
+                  stream=None, alpha_ptr=None, beta_ptr=None, infinities=False):
+    """Parallel split-K SRGEMM: partial products of ``slices`` K-slices into
+    ``workspace`` (device memory, >= splitk_workspace_bytes), then a reduction
+    with the semiring's add and the epilogue."""
+    dtype = dtype or _torch_dtype_name(D)
+    alpha = op_identity(mult_op, dtype, infinities) if alpha is None else alpha
+    beta = op_annihilator(mult_op, dtype, infinities) if beta is None else beta
+    add_identity = op_identity(add_op, dtype, infinities) if add_identity is None else add_identity
+    mult_identity = op_identity(mult_op, dtype, infinities) if mult_identity is None else mult_identity
+    desc = make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,
+                     slices, kernel, alpha_ptr, beta_ptr)
+    ws = workspace.data_ptr() if hasattr(workspace, "data_ptr") else workspace
+    st = load().cuasr_amd_srgemm_splitk(ctypes.byref(desc), ctypes.c_void_p(ws or None), _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_srgemm_splitk")
+    return D

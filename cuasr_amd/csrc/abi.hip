@@ -1,0 +1,192 @@
+// C ABI of libcuasr_amd: validation, transposition of column-major outputs,
+// kernel-family selection and launch.  Host-side counterpart of
+// include/cuasr/gemm/device/srgemm.h:196-356 and
+// include/cuasr/gemm/device/srgemm_splitk_parallel.h:220-357.
+#include "semiring.h"
+
+namespace cuasr_amd {
+
+launch_fn find_valu_f32(int, int);
+launch_fn find_valu_f64(int, int);
+launch_fn find_valu_i32(int, int);
+launch_fn find_valu_u32(int, int);
+launch_fn find_mfma_f32(int, int);
+
+launch_fn find_valu(int dtype, int add_op, int mult_op) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return find_valu_f32(add_op, mult_op);
+    case CUASR_AMD_F64: return find_valu_f64(add_op, mult_op);
+    case CUASR_AMD_I32: return find_valu_i32(add_op, mult_op);
+    case CUASR_AMD_U32: return find_valu_u32(add_op, mult_op);
+    default: return nullptr;
+  }
+}
+
+launch_fn find_mfma(int dtype, int add_op, int mult_op) {
+  if (dtype == CUASR_AMD_F32) return find_mfma_f32(add_op, mult_op);
+  return nullptr;
+}
+
+static size_t elem_size(int dtype) { return dtype == CUASR_AMD_F64 ? 8 : 4; }
+
+static bool is_bitwise(int op) { return op == kBitAnd || op == kBitOr || op == kBitXor; }
+
+// add must be associative and commutative with an identity; mult is any of the
+// "times-like" operators.  Both lists mirror what the reference can spell.
+static bool valid_add(int op) {
+  return op == kPlus || op == kMinimum || op == kMaximum || op == kLogicalOr || op == kBitOr || op == kBitXor ||
+         op == kMultiplies || op == kLogicalAnd || op == kBitAnd;
+}
+static bool valid_mult(int op) { return op >= kPlus && op <= kBitXor; }
+
+static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
+  if (!d) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_U32) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
+  const int layouts[3] = {d->layout_a, d->layout_b, d->layout_c};
+  for (int l : layouts)
+    if (l != CUASR_AMD_COLUMN_MAJOR && l != CUASR_AMD_ROW_MAJOR) return CUASR_AMD_ERROR_INVALID_LAYOUT;
+  if (!valid_add(d->add_op) || !valid_mult(d->mult_op)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  const bool fp = d->dtype == CUASR_AMD_F32 || d->dtype == CUASR_AMD_F64;
+  if (fp && (is_bitwise(d->add_op) || is_bitwise(d->mult_op))) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->m < 0 || d->n < 0 || d->k < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (d->reserved != 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (splitk ? d->split_k_slices < 1 : d->split_k_slices != 1) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (d->kernel < CUASR_AMD_KERNEL_AUTO || d->kernel > CUASR_AMD_KERNEL_MFMA) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  auto min_ld = [](int layout, int rows, int cols) { return (long long)(layout == CUASR_AMD_COLUMN_MAJOR ? rows : cols); };
+  if (d->m > 0 && d->k > 0 && d->lda < min_ld(d->layout_a, d->m, d->k)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (d->n > 0 && d->k > 0 && d->ldb < min_ld(d->layout_b, d->k, d->n)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (d->m > 0 && d->n > 0) {
+    if (d->ldd < min_ld(d->layout_c, d->m, d->n)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+    if (d->C && d->ldc < min_ld(d->layout_c, d->m, d->n)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+    if (!d->D) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+    if (d->k > 0 && (!d->A || !d->B)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  }
+  const size_t es = elem_size(d->dtype);
+  const void *ptrs[6] = {d->A, d->B, d->C, d->D, d->alpha_ptr, d->beta_ptr};
+  for (const void *q : ptrs)
+    if (reinterpret_cast<uintptr_t>(q) % es) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+  if (d->kernel == CUASR_AMD_KERNEL_VALU && !find_valu(d->dtype, d->add_op, d->mult_op))
+    return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->kernel == CUASR_AMD_KERNEL_MFMA && !find_mfma(d->dtype, d->add_op, d->mult_op))
+    return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  return CUASR_AMD_SUCCESS;
+}
+
+static Problem canonical(const cuasr_amd_srgemm_desc *d) {
+  Problem p{};
+  const long long sa_m = d->layout_a == CUASR_AMD_COLUMN_MAJOR ? 1 : d->lda;
+  const long long sa_k = d->layout_a == CUASR_AMD_COLUMN_MAJOR ? d->lda : 1;
+  const long long sb_k = d->layout_b == CUASR_AMD_COLUMN_MAJOR ? 1 : d->ldb;
+  const long long sb_n = d->layout_b == CUASR_AMD_COLUMN_MAJOR ? d->ldb : 1;
+  if (d->layout_c == CUASR_AMD_ROW_MAJOR) {
+    p.m = d->m; p.n = d->n;
+    p.A = d->A; p.sa_m = sa_m; p.sa_k = sa_k;
+    p.B = d->B; p.sb_k = sb_k; p.sb_n = sb_n;
+  } else {
+    // column-major C: run the transposed problem, C^T = B^T (x) A^T
+    p.m = d->n; p.n = d->m;
+    p.A = d->B; p.sa_m = sb_n; p.sa_k = sb_k;
+    p.B = d->A; p.sb_k = sa_k; p.sb_n = sa_m;
+  }
+  p.k = d->k;
+  p.C = d->C; p.ldc = d->ldc;
+  p.D = d->D; p.ldd = d->ldd;
+  p.alpha = d->alpha; p.beta = d->beta;
+  p.add_identity = d->add_identity; p.mult_identity = d->mult_identity;
+  p.alpha_ptr = d->alpha_ptr; p.beta_ptr = d->beta_ptr;
+  p.add_op = d->add_op; p.mult_op = d->mult_op;
+  p.slices = 1; p.k_per_slice = d->k; p.workspace = nullptr;
+  return p;
+}
+
+enum Family { kNaive = 1, kValu = 2, kMfma = 3 };
+
+static int pick_family(const cuasr_amd_srgemm_desc *d) {
+  if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
+  if (find_mfma(d->dtype, d->add_op, d->mult_op)) return kMfma;
+  if (find_valu(d->dtype, d->add_op, d->mult_op)) return kValu;
+  return kNaive;
+}
+
+static launch_fn family_fn(int family, const cuasr_amd_srgemm_desc *d) {
+  switch (family) {
+    case kMfma: return find_mfma(d->dtype, d->add_op, d->mult_op);
+    case kValu: return find_valu(d->dtype, d->add_op, d->mult_op);
+    default: return find_naive(d->dtype);
+  }
+}
+
+}  // namespace cuasr_amd
+
+using namespace cuasr_amd;
+
+extern "C" {
+
+int cuasr_amd_abi_version(void) { return CUASR_AMD_ABI_VERSION; }
+
+const char *cuasr_amd_status_string(int status) {
+  switch (status) {
+    case CUASR_AMD_SUCCESS: return "success";
+    case CUASR_AMD_ERROR_MISALIGNED_OPERAND: return "misaligned operand";
+    case CUASR_AMD_ERROR_INVALID_DATA_TYPE: return "invalid data type";
+    case CUASR_AMD_ERROR_INVALID_LAYOUT: return "invalid layout";
+    case CUASR_AMD_ERROR_INVALID_PROBLEM: return "invalid problem";
+    case CUASR_AMD_ERROR_NOT_SUPPORTED: return "not supported";
+    case CUASR_AMD_ERROR_WORKSPACE_NULL: return "workspace is null";
+    case CUASR_AMD_ERROR_INTERNAL: return "internal error";
+    case CUASR_AMD_ERROR_ARCH_MISMATCH: return "architecture mismatch";
+    case CUASR_AMD_ERROR_INSUFFICIENT_DRIVER: return "insufficient driver";
+    case CUASR_AMD_ERROR_MEMORY_ALLOCATION: return "memory allocation failed";
+    default: return "invalid status";
+  }
+}
+
+int cuasr_amd_srgemm_can_implement(const cuasr_amd_srgemm_desc *desc) { return validate(desc, false); }
+
+const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc) {
+  if (validate(desc, true) != CUASR_AMD_SUCCESS) return nullptr;
+  switch (pick_family(desc)) {
+    case kMfma: return "mfma";
+    case kValu: return "valu";
+    default: return "naive";
+  }
+}
+
+int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
+  const int st = validate(desc, false);
+  if (st != CUASR_AMD_SUCCESS) return st;
+  const Problem p = canonical(desc);
+  const launch_fn fn = family_fn(pick_family(desc), desc);
+  if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+}
+
+size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
+  if (!desc || desc->m < 0 || desc->n < 0 || desc->split_k_slices < 1) return 0;
+  if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_U32) return 0;
+  return elem_size(desc->dtype) * size_t(desc->m) * size_t(desc->n) * size_t(desc->split_k_slices);
+}
+
+int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
+  const int st = validate(desc, true);
+  if (st != CUASR_AMD_SUCCESS) return st;
+  if (!workspace) return CUASR_AMD_ERROR_WORKSPACE_NULL;
+  if (reinterpret_cast<uintptr_t>(workspace) % elem_size(desc->dtype)) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+  Problem p = canonical(desc);
+  p.slices = desc->split_k_slices;
+  // slice extent: whole k-tiles of 16, spread evenly; trailing slices may be
+  // empty and then hold the additive identity
+  const int tile = 16;
+  const long long tiles = (p.k + tile - 1) / tile;
+  const long long per = (tiles + p.slices - 1) / p.slices;
+  p.k_per_slice = int(per * tile > 0 ? per * tile : tile);
+  p.workspace = workspace;
+  const launch_fn fn = family_fn(pick_family(desc), desc);
+  const launch_fn red = find_reduce(desc->dtype);
+  if (!fn || !red) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+  return red(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+}
+
+}  // extern "C"

@@ -1,0 +1,124 @@
+// Two small kernel families with run-time operators:
+//   * the naive SRGEMM (one thread per output element) -- runs any operator
+//     pair the element type defines, and serves as an on-device cross-check;
+//   * the split-K reduction: D = epilogue(add over slices of workspace, C),
+//     the second kernel of the parallel split-K
+//     (include/cuasr/reduction/kernel/reduce_split_k.h:146-237).
+#include "semiring.h"
+
+namespace cuasr_amd {
+
+// ---------------------------------------------------------------- naive SRGEMM
+template <typename T>
+__global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
+  const int j = blockIdx.x * 16 + (threadIdx.x & 15);
+  const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
+  const int z = blockIdx.z;
+  if (i >= p.m || j >= p.n) return;
+  const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
+  const T *A = reinterpret_cast<const T *>(p.A) + (long long)i * p.sa_m;
+  const T *B = reinterpret_cast<const T *>(p.B) + (long long)j * p.sb_n;
+  int k0 = 0, k1 = p.k;
+  if (p.workspace) {
+    k0 = z * p.k_per_slice;
+    k1 = min(p.k, k0 + p.k_per_slice);
+  }
+  T acc = e.ident;
+  for (int kk = k0; kk < k1; ++kk) {
+    const T prod = apply_op<T>(p.mult_op, A[(long long)kk * p.sa_k], B[(long long)kk * p.sb_k]);
+    acc = apply_op<T>(p.add_op, acc, prod);
+  }
+  if (p.workspace) {
+    reinterpret_cast<T *>(p.workspace)[((long long)z * p.m + i) * p.n + j] = acc;
+    return;
+  }
+  T out = apply_op<T>(p.mult_op, e.alpha, acc);
+  if (e.source_needed) {
+    const T c = reinterpret_cast<const T *>(p.C)[(long long)i * p.ldc + j];
+    out = apply_op<T>(p.add_op, out, apply_op<T>(p.mult_op, e.beta, c));
+  }
+  reinterpret_cast<T *>(p.D)[(long long)i * p.ldd + j] = out;
+}
+
+template <typename T> static hipError_t launch_naive(const Problem &p, hipStream_t s) {
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  dim3 grid((p.n + 15) / 16, (p.m + 15) / 16, p.workspace ? p.slices : 1);
+  hipLaunchKernelGGL(naive_srgemm_kernel<T>, grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+launch_fn find_naive(int dtype) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return launch_naive<float>;
+    case CUASR_AMD_F64: return launch_naive<double>;
+    case CUASR_AMD_I32: return launch_naive<int32_t>;
+    case CUASR_AMD_U32: return launch_naive<uint32_t>;
+    default: return nullptr;
+  }
+}
+
+// ------------------------------------------------------------ split-K reduction
+// Each thread owns V consecutive elements of one row.  acc starts at the
+// additive identity and folds the slices in ascending order; when the source
+// is not needed it is replaced by the identity and the two-operand epilogue is
+// still applied (reduce_split_k.h:212-227).
+template <typename T, int V>
+__global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
+  const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
+  const long long per_row = (p.n + V - 1) / V;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= per_row * p.m) return;
+  const int i = int(idx / per_row);
+  const int j = int(idx % per_row) * V;
+  const long long slice = (long long)p.m * p.n;
+  const T *ws = reinterpret_cast<const T *>(p.workspace) + (long long)i * p.n + j;
+  T acc[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) acc[v] = e.ident;
+  if (V > 1) {
+    typedef T vec_t __attribute__((ext_vector_type(V)));
+    for (int s = 0; s < p.slices; ++s) {
+      const vec_t w = *reinterpret_cast<const vec_t *>(ws + s * slice);
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[v]);
+    }
+  } else {
+    for (int s = 0; s < p.slices; ++s) acc[0] = apply_op<T>(p.add_op, acc[0], ws[s * slice]);
+  }
+  const T *C = reinterpret_cast<const T *>(p.C);
+  T *D = reinterpret_cast<T *>(p.D);
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    if (j + v < p.n) {
+      const T src = e.source_needed ? C[(long long)i * p.ldc + j + v] : e.ident;
+      const T lhs = apply_op<T>(p.mult_op, e.alpha, acc[v]);
+      D[(long long)i * p.ldd + j + v] = apply_op<T>(p.add_op, lhs, apply_op<T>(p.mult_op, e.beta, src));
+    }
+  }
+}
+
+template <typename T> static hipError_t launch_reduce(const Problem &p, hipStream_t s) {
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  constexpr int V = 16 / sizeof(T);
+  const bool vec = (p.n % V == 0) && (reinterpret_cast<uintptr_t>(p.workspace) % 16 == 0);
+  if (vec) {
+    const long long work = (long long)p.m * (p.n / V);
+    hipLaunchKernelGGL((reduce_splitk_kernel<T, V>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
+  } else {
+    const long long work = (long long)p.m * p.n;
+    hipLaunchKernelGGL((reduce_splitk_kernel<T, 1>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
+  }
+  return hipGetLastError();
+}
+
+launch_fn find_reduce(int dtype) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return launch_reduce<float>;
+    case CUASR_AMD_F64: return launch_reduce<double>;
+    case CUASR_AMD_I32: return launch_reduce<int32_t>;
+    case CUASR_AMD_U32: return launch_reduce<uint32_t>;
+    default: return nullptr;
+  }
+}
+
+}  // namespace cuasr_amd

@@ -1,0 +1,116 @@
+// Device-side scalar operators of the semirings and the shared problem record.
+//
+// Operator semantics are those of the reference functors
+// (include/cuasr/functional.h:46-49, :89-92, :132, :172, :212, :252 and
+// examples/01_userdefined_semiring/userdefined_semiring.cu:56-66): minimum and
+// maximum return one of their operands, logical and/or return 0 or 1, the
+// bitwise forms exist for integer element types only.  For floating point the
+// min/max forms map to the hardware min/max instructions, which agree with the
+// reference's comparisons for every input that is not a NaN and not a tie
+// between +0 and -0.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <type_traits>
+
+#include "../../include/cuasr_amd.h"
+
+namespace cuasr_amd {
+
+enum : int { kPlus = 0, kMultiplies = 1, kMinimum = 2, kMaximum = 3, kLogicalAnd = 4,
+             kLogicalOr = 5, kBitAnd = 6, kBitOr = 7, kBitXor = 8 };
+
+template <typename T> struct is_fp : std::integral_constant<bool, std::is_floating_point<T>::value> {};
+
+template <typename T> __device__ __forceinline__ T hw_min(T l, T r) { return r < l ? r : l; }
+template <typename T> __device__ __forceinline__ T hw_max(T l, T r) { return l < r ? r : l; }
+template <> __device__ __forceinline__ float hw_min<float>(float l, float r) { return __builtin_fminf(l, r); }
+template <> __device__ __forceinline__ float hw_max<float>(float l, float r) { return __builtin_fmaxf(l, r); }
+template <> __device__ __forceinline__ double hw_min<double>(double l, double r) { return __builtin_fmin(l, r); }
+template <> __device__ __forceinline__ double hw_max<double>(double l, double r) { return __builtin_fmax(l, r); }
+
+// Compile-time operator: Op<kMinimum>::apply(l, r)
+template <int OP> struct Op {
+  template <typename T> static __device__ __forceinline__ T apply(T l, T r) {
+    if constexpr (OP == kPlus) return l + r;
+    else if constexpr (OP == kMultiplies) return l * r;
+    else if constexpr (OP == kMinimum) return hw_min<T>(l, r);
+    else if constexpr (OP == kMaximum) return hw_max<T>(l, r);
+    else if constexpr (OP == kLogicalAnd) return T((l != T(0)) && (r != T(0)));
+    else if constexpr (OP == kLogicalOr) return T((l != T(0)) || (r != T(0)));
+    else if constexpr (!is_fp<T>::value) {
+      if constexpr (OP == kBitAnd) return l & r;
+      else if constexpr (OP == kBitOr) return l | r;
+      else return l ^ r;
+    } else {
+      return l;  // bitwise on floating point is rejected on the host
+    }
+  }
+};
+
+// Run-time operator (naive kernel, reduction epilogue)
+template <typename T> __device__ __forceinline__ T apply_op(int op, T l, T r) {
+  switch (op) {
+    case kPlus: return Op<kPlus>::apply(l, r);
+    case kMultiplies: return Op<kMultiplies>::apply(l, r);
+    case kMinimum: return Op<kMinimum>::apply(l, r);
+    case kMaximum: return Op<kMaximum>::apply(l, r);
+    case kLogicalAnd: return Op<kLogicalAnd>::apply(l, r);
+    case kLogicalOr: return Op<kLogicalOr>::apply(l, r);
+    case kBitAnd: return Op<kBitAnd>::apply(l, r);
+    case kBitOr: return Op<kBitOr>::apply(l, r);
+    default: return Op<kBitXor>::apply(l, r);
+  }
+}
+
+template <typename T> __host__ __device__ __forceinline__ T scalar_as(const cuasr_amd_scalar &s);
+template <> __host__ __device__ __forceinline__ float scalar_as<float>(const cuasr_amd_scalar &s) { return s.f32; }
+template <> __host__ __device__ __forceinline__ double scalar_as<double>(const cuasr_amd_scalar &s) { return s.f64; }
+template <> __host__ __device__ __forceinline__ int32_t scalar_as<int32_t>(const cuasr_amd_scalar &s) { return s.i32; }
+template <> __host__ __device__ __forceinline__ uint32_t scalar_as<uint32_t>(const cuasr_amd_scalar &s) { return s.u32; }
+
+// The problem in kernel form.  The host has already turned a column-major C
+// into the transposed problem (C^T = B^T (x) A^T, as the reference does in
+// include/cuasr/gemm/device/srgemm.h:432-453, :513-523), so C and D are always
+// row-major here and A, B are addressed by element strides.
+struct Problem {
+  int m, n, k;
+  const void *A; long long sa_m, sa_k;   // A[i][kk] at A + i*sa_m + kk*sa_k
+  const void *B; long long sb_k, sb_n;   // B[kk][j] at B + kk*sb_k + j*sb_n
+  const void *C; long long ldc;          // C[i][j] at C + i*ldc + j
+  void *D;       long long ldd;
+  cuasr_amd_scalar alpha, beta, add_identity, mult_identity;
+  const void *alpha_ptr, *beta_ptr;
+  int add_op, mult_op;
+  // split-K: slice z covers k in [z*k_per_slice, min(k, (z+1)*k_per_slice));
+  // partial accumulators go to workspace[z][m][n] (row-major, ld = n)
+  int slices, k_per_slice;
+  void *workspace;
+};
+
+// Epilogue scalars resolved on the device (alpha/beta may live in device memory).
+template <typename T> struct EpilogueScalars {
+  T alpha, beta, ident;
+  bool source_needed;
+};
+
+template <typename T> __device__ __forceinline__ EpilogueScalars<T> resolve_scalars(const Problem &p, int mult_op) {
+  EpilogueScalars<T> e;
+  e.alpha = p.alpha_ptr ? *reinterpret_cast<const T *>(p.alpha_ptr) : scalar_as<T>(p.alpha);
+  e.beta = p.beta_ptr ? *reinterpret_cast<const T *>(p.beta_ptr) : scalar_as<T>(p.beta);
+  e.ident = scalar_as<T>(p.add_identity);
+  // source needed <=> add_identity != mult(beta, mult_identity)
+  // (epilogue/thread/semiring_linear_combination.h:118-125)
+  e.source_needed = e.ident != apply_op<T>(mult_op, e.beta, scalar_as<T>(p.mult_identity));
+  return e;
+}
+
+typedef hipError_t (*launch_fn)(const Problem &, hipStream_t);
+
+// kernel-family lookups, one definition per translation unit that owns them
+launch_fn find_naive(int dtype);
+launch_fn find_valu(int dtype, int add_op, int mult_op);
+launch_fn find_mfma(int dtype, int add_op, int mult_op);
+launch_fn find_reduce(int dtype);
+
+}  // namespace cuasr_amd

@@ -1,0 +1,299 @@
+// LDS-staged, register-blocked vector-ALU SRGEMM tile kernel for gfx950.
+//
+// Plays the role of the reference's threadblock/warp/thread hierarchy
+// (include/cuasr/gemm/threadblock/srmma_pipelined.h:153-288,
+//  include/cuasr/gemm/warp/srmma_simt.h:190-199,
+//  include/cuasr/gemm/thread/srmma_sm50.h:118-146, include/cuasr/arch/srmma.h:84-91)
+// and of the kernel body include/cuasr/gemm/kernel/srgemm.h:156-321, with a
+// design of its own:
+//   * one workgroup = 256 threads = 4 wave64, output tile (16*TM) x (16*TN);
+//   * thread (ty, tx) of a 16x16 arrangement owns TM x TN accumulators in
+//     16-byte groups, so every LDS fragment read is one ds_read_b128 and every
+//     D access one 16-byte global access;
+//   * A and B panels live in LDS k-major ([kk][m] and [kk][n]), double
+//     buffered, one barrier per k-tile; the next tile's global loads are in
+//     flight while the current tile is computed;
+//   * A ragged last k-tile is handled by shortening the loop, never by padding
+//     (a padded identity is not neutral for every semiring), so the result is
+//     the host reference's for any K.
+// blockIdx.x walks output tiles through an XCD-aware, row-grouped order;
+// blockIdx.y is the split-K slice.
+#pragma once
+#include "semiring.h"
+
+namespace cuasr_amd {
+
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
+struct ValuTile {
+  static constexpr int KU = 2;  // k-steps unrolled together (lets two sums meet in one 3-input min/max)
+  static constexpr int VW = 16 / sizeof(T);
+  static constexpr int BM = 16 * TM, BN = 16 * TN;
+  static constexpr int LDA = BM + VW, LDB = BN + VW;
+  static constexpr int A_ELEMS = BM * BK / 256, B_ELEMS = BN * BK / 256;
+  static constexpr int HM = TM / VW, GN = TN / VW;
+  static_assert(A_ELEMS >= VW && B_ELEMS >= VW && HM >= 1 && GN >= 1, "tile too small");
+  static_assert(BK % VW == 0 && BK % KU == 0, "BK must hold whole vectors");
+  typedef T vec_t __attribute__((ext_vector_type(VW)));
+
+  struct Smem {
+    T a[2][BK][LDA];
+    T b[2][BK][LDB];
+  };
+
+  // ---- global -> registers.  ROWS is the panel extent (BM or BN), s_x the
+  // element stride along the panel's m/n index, s_k along k.  Indices that
+  // fall outside the matrix are clamped to its last row/column/k: what is
+  // fetched there is never used (rows and columns past the edge are not
+  // stored, k past the end is not iterated), so no branch and no fill value.
+  //   VEC:  a thread owns ELEMS/VW groups of VW elements consecutive along the
+  //         panel's contiguous direction, one 16-byte load each; the host
+  //         guarantees alignment and that extents along that direction are
+  //         multiples of VW, so a clamped group never straddles the edge.
+  //   !VEC: a thread owns ELEMS single elements.
+  template <int ROWS, int ELEMS>
+  static __device__ __forceinline__ void load_panel(T (&r)[ELEMS], const T *base, long long s_x, long long s_k,
+                                                    int x0, int x_end, int k0, int k_end, bool x_contig) {
+    const int tid = threadIdx.x;
+    if constexpr (VEC) {
+      constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
+#pragma unroll
+      for (int p = 0; p < VECS; ++p) {
+        const int v = tid + 256 * p;
+        const int xx = min(x0 + (x_contig ? (v % XV) * VW : v / KV), x_end - (x_contig ? VW : 1));
+        const int kk = min(k0 + (x_contig ? v / XV : (v % KV) * VW), k_end - (x_contig ? 1 : VW));
+        const vec_t t = *reinterpret_cast<const vec_t *>(base + (long long)xx * s_x + (long long)kk * s_k);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) r[p * VW + e] = t[e];
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < ELEMS; ++p) {
+        const int el = tid + 256 * p;
+        const int xx = min(x0 + (x_contig ? el % ROWS : el / BK), x_end - 1);
+        const int kk = min(k0 + (x_contig ? el / ROWS : el % BK), k_end - 1);
+        r[p] = base[(long long)xx * s_x + (long long)kk * s_k];
+      }
+    }
+  }
+
+  // ---- registers -> LDS ([kk][x], k-major), same ownership as load_panel
+  template <int ROWS, int LD, int ELEMS>
+  static __device__ __forceinline__ void store_panel(const T (&r)[ELEMS], T (*dst)[LD], bool x_contig) {
+    const int tid = threadIdx.x;
+    if constexpr (VEC) {
+      constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
+      if (x_contig) {
+#pragma unroll
+        for (int p = 0; p < VECS; ++p) {
+          const int v = tid + 256 * p;
+          vec_t t;
+#pragma unroll
+          for (int e = 0; e < VW; ++e) t[e] = r[p * VW + e];
+          *reinterpret_cast<vec_t *>(&dst[v / XV][(v % XV) * VW]) = t;
+        }
+      } else {
+#pragma unroll
+        for (int p = 0; p < VECS; ++p) {
+          const int v = tid + 256 * p;
+#pragma unroll
+          for (int e = 0; e < VW; ++e) dst[(v % KV) * VW + e][v / KV] = r[p * VW + e];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < ELEMS; ++p) {
+        const int el = tid + 256 * p;
+        dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = r[p];
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void step(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int kk,
+                                              int ty, int tx) {
+    T a[TM], b[TN];
+#pragma unroll
+    for (int h = 0; h < HM; ++h) {
+      const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk][ty * VW + h * 16 * VW]);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) a[h * VW + e] = t[e];
+    }
+#pragma unroll
+    for (int g = 0; g < GN; ++g) {
+      const vec_t t = *reinterpret_cast<const vec_t *>(&bs[kk][tx * VW + g * 16 * VW]);
+#pragma unroll
+      for (int e = 0; e < VW; ++e) b[g * VW + e] = t[e];
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = Op<ADD>::apply(acc[i][j], Op<MUL>::apply(a[i], b[j]));
+  }
+
+  static __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int &bm, int &bn) {
+    const int total = tiles_m * tiles_n;
+    // consecutive workgroup ids land on consecutive XCDs (8 of them, one L2
+    // each): give every XCD one contiguous run of the tile order
+    if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
+    constexpr int GROUP = 8;
+    const int width = GROUP * tiles_n;
+    const int group = id / width, first = group * GROUP;
+    const int gsz = min(tiles_m - first, GROUP);
+    bm = first + (id % width) % gsz;
+    bn = (id % width) / gsz;
+  }
+
+  static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
+    int bm, bn;
+    tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
+    const int m0 = bm * BM, n0 = bn * BN;
+    const T *A = reinterpret_cast<const T *>(p.A);
+    const T *B = reinterpret_cast<const T *>(p.B);
+    const T ident = scalar_as<T>(p.add_identity);
+
+    int kb = 0, ke = p.k;
+    if (p.workspace) {
+      kb = blockIdx.y * p.k_per_slice;
+      ke = min(p.k, kb + p.k_per_slice);
+    }
+    const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
+
+    T acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) acc[i][j] = ident;
+
+    const int ntiles = (ke - kb + BK - 1) / BK;
+    T ra[A_ELEMS], rb[B_ELEMS];
+    if (ntiles > 0) {
+      load_panel<BM, A_ELEMS>(ra, A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_xc);
+      load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_xc);
+      store_panel<BM, LDA, A_ELEMS>(ra, sm.a[0], a_xc);
+      store_panel<BN, LDB, B_ELEMS>(rb, sm.b[0], b_xc);
+    }
+    __syncthreads();
+    int buf = 0;
+    for (int t = 0; t < ntiles; ++t) {
+      const int k0 = kb + t * BK;
+      const bool more = t + 1 < ntiles;
+      if (more) {
+        load_panel<BM, A_ELEMS>(ra, A, p.sa_m, p.sa_k, m0, p.m, k0 + BK, ke, a_xc);
+        load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, k0 + BK, ke, b_xc);
+      }
+      const int kcount = min(BK, ke - k0);
+      if (kcount == BK) {
+#pragma unroll KU
+        for (int kk = 0; kk < BK; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
+      } else {
+#pragma unroll 1
+        for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
+      }
+      if (more) {
+        store_panel<BM, LDA, A_ELEMS>(ra, sm.a[buf ^ 1], a_xc);
+        store_panel<BN, LDB, B_ELEMS>(rb, sm.b[buf ^ 1], b_xc);
+      }
+      __syncthreads();
+      buf ^= 1;
+    }
+
+    // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or raw partials
+    T *out;
+    long long ld_out;
+    const bool partial = p.workspace != nullptr;
+    EpilogueScalars<T> e;
+    if (partial) {
+      out = reinterpret_cast<T *>(p.workspace) + (long long)blockIdx.y * p.m * p.n;
+      ld_out = p.n;
+      e.alpha = e.beta = e.ident = ident;
+      e.source_needed = false;
+    } else {
+      out = reinterpret_cast<T *>(p.D);
+      ld_out = p.ldd;
+      e = resolve_scalars<T>(p, MUL);
+    }
+    const T *C = reinterpret_cast<const T *>(p.C);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = m0 + ty * VW + (i / VW) * 16 * VW + (i % VW);
+      if (row >= p.m) continue;
+#pragma unroll
+      for (int g = 0; g < GN; ++g) {
+        const int col = n0 + tx * VW + g * 16 * VW;
+        if (col >= p.n) continue;
+        T v[VW];
+#pragma unroll
+        for (int c = 0; c < VW; ++c) v[c] = acc[i][g * VW + c];
+        if (!partial) {
+#pragma unroll
+          for (int c = 0; c < VW; ++c) v[c] = Op<MUL>::apply(e.alpha, v[c]);
+          if (e.source_needed) {
+            T src[VW];
+            if constexpr (VEC) {
+              const vec_t t = *reinterpret_cast<const vec_t *>(C + (long long)row * p.ldc + col);
+#pragma unroll
+              for (int c = 0; c < VW; ++c) src[c] = t[c];
+            } else {
+#pragma unroll
+              for (int c = 0; c < VW; ++c) src[c] = C[(long long)row * p.ldc + min(col + c, p.n - 1)];
+            }
+#pragma unroll
+            for (int c = 0; c < VW; ++c) v[c] = Op<ADD>::apply(v[c], Op<MUL>::apply(e.beta, src[c]));
+          }
+        }
+        if constexpr (VEC) {
+          vec_t t;
+#pragma unroll
+          for (int c = 0; c < VW; ++c) t[c] = v[c];
+          *reinterpret_cast<vec_t *>(out + (long long)row * ld_out + col) = t;
+        } else {
+#pragma unroll
+          for (int c = 0; c < VW; ++c)
+            if (col + c < p.n) out[(long long)row * ld_out + col + c] = v[c];
+        }
+      }
+    }
+  }
+};
+
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
+__global__ __launch_bounds__(256) void valu_srgemm_kernel(Problem p) {
+  using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC>;
+  __shared__ typename Tile::Smem sm;
+  Tile::run(p, sm);
+}
+
+// 16-byte access is legal for the whole problem: aligned bases, leading
+// dimensions and contiguous extents that are multiples of the vector width
+template <typename T> static bool vector_friendly(const Problem &p) {
+  constexpr int VW = 16 / sizeof(T);
+  auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
+  if (!al(p.A) || !al(p.B)) return false;
+  if (a_xc ? (p.m % VW || p.sa_k % VW) : (p.sa_k != 1 || p.k % VW || p.sa_m % VW)) return false;
+  if (b_xc ? (p.n % VW || p.sb_k % VW) : (p.sb_k != 1 || p.k % VW || p.sb_n % VW)) return false;
+  if (p.n % VW) return false;
+  if (p.workspace) return al(p.workspace);
+  // C is only dereferenced when the source is needed, but whether it is can
+  // depend on a device-side beta; require alignment whenever a pointer is given
+  if (!al(p.D) || p.ldd % VW) return false;
+  if (p.C && (!al(p.C) || p.ldc % VW)) return false;
+  return true;
+}
+
+template <typename T, int ADD, int MUL, int TM, int TN, int BK>
+static hipError_t launch_valu(const Problem &p, hipStream_t s) {
+  constexpr int BM = 16 * TM, BN = 16 * TN;
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  if (vector_friendly<T>(p))
+    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true>), grid, dim3(256), 0, s, p);
+  else
+    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, false>), grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
+}  // namespace cuasr_amd

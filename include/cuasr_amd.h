@@ -1,0 +1,170 @@
+/*
+ * cuasr_amd C ABI: semiring GEMM (SRGEMM) on AMD Instinct MI355X (gfx950).
+ *
+ *     D = add( mult(alpha, A (x) B), mult(beta, C) )
+ *     (A (x) B)[i][j] = add over k of mult(A[i][k], B[k][j]), starting from add_identity
+ *
+ * This is the boundary the C++ operator templates in include/cuasr/ call, and
+ * the one a foreign-function binding would bind.  Plain C types only; all
+ * matrix pointers are device pointers owned by the caller; nothing here
+ * allocates, frees or synchronises.  Every call is asynchronous on `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream).
+ *
+ * Reference interfaces replaced (paths relative to the cuASR tree):
+ *   cuasr_amd_srgemm                  device::Srgemm::operator()/run
+ *                                     include/cuasr/gemm/device/srgemm.h:303-356
+ *   cuasr_amd_srgemm_can_implement    device::Srgemm::can_implement  :196-215
+ *                                     kernel::Srgemm::can_implement
+ *                                     include/cuasr/gemm/kernel/srgemm.h:118-153
+ *   cuasr_amd_splitk_workspace_bytes  device::SrgemmSplitKParallel::get_workspace_size
+ *                                     include/cuasr/gemm/device/srgemm_splitk_parallel.h:226-235
+ *   cuasr_amd_srgemm_splitk           device::SrgemmSplitKParallel::initialize/run
+ *                                     include/cuasr/gemm/device/srgemm_splitk_parallel.h:238-357
+ *   status codes                      cutlass::Status as used by the reference
+ *                                     test/device/testbed.h:24-46
+ */
+#ifndef CUASR_AMD_H
+#define CUASR_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CUASR_AMD_ABI_VERSION 1
+
+/* Same names and order as cutlass::Status, so static_cast<int>(status) agrees. */
+typedef enum cuasr_amd_status {
+  CUASR_AMD_SUCCESS = 0,
+  CUASR_AMD_ERROR_MISALIGNED_OPERAND = 1,
+  CUASR_AMD_ERROR_INVALID_DATA_TYPE = 2,
+  CUASR_AMD_ERROR_INVALID_LAYOUT = 3,
+  CUASR_AMD_ERROR_INVALID_PROBLEM = 4,
+  CUASR_AMD_ERROR_NOT_SUPPORTED = 5,
+  CUASR_AMD_ERROR_WORKSPACE_NULL = 6,
+  CUASR_AMD_ERROR_INTERNAL = 7,
+  CUASR_AMD_ERROR_ARCH_MISMATCH = 8,
+  CUASR_AMD_ERROR_INSUFFICIENT_DRIVER = 9,
+  CUASR_AMD_ERROR_MEMORY_ALLOCATION = 10,
+  CUASR_AMD_INVALID = 11
+} cuasr_amd_status;
+
+/* Scalar operators.  (lhs, rhs) semantics follow include/cuasr/functional.h:
+ * minimum = rhs < lhs ? rhs : lhs, maximum = lhs < rhs ? rhs : lhs,
+ * logical_and/or produce 0 or 1 (functional.h:212, :252); bit_* are bitwise
+ * and only defined for the integer element types. */
+typedef enum cuasr_amd_op {
+  CUASR_AMD_OP_PLUS = 0,
+  CUASR_AMD_OP_MULTIPLIES = 1,
+  CUASR_AMD_OP_MINIMUM = 2,
+  CUASR_AMD_OP_MAXIMUM = 3,
+  CUASR_AMD_OP_LOGICAL_AND = 4,
+  CUASR_AMD_OP_LOGICAL_OR = 5,
+  CUASR_AMD_OP_BIT_AND = 6,
+  CUASR_AMD_OP_BIT_OR = 7,
+  CUASR_AMD_OP_BIT_XOR = 8
+} cuasr_amd_op;
+
+typedef enum cuasr_amd_dtype {
+  CUASR_AMD_F32 = 0,
+  CUASR_AMD_F64 = 1,
+  CUASR_AMD_I32 = 2,
+  CUASR_AMD_U32 = 3
+} cuasr_amd_dtype;
+
+typedef enum cuasr_amd_layout {
+  CUASR_AMD_COLUMN_MAJOR = 0, /* element (r, c) at r + c * ld */
+  CUASR_AMD_ROW_MAJOR = 1     /* element (r, c) at r * ld + c */
+} cuasr_amd_layout;
+
+/* Which kernel family runs.  AUTO picks the fastest one that is valid for the
+ * problem; the others exist so tests can pin every family against the oracle. */
+typedef enum cuasr_amd_kernel {
+  CUASR_AMD_KERNEL_AUTO = 0,
+  CUASR_AMD_KERNEL_NAIVE = 1, /* one thread per output element               */
+  CUASR_AMD_KERNEL_VALU = 2,  /* LDS-staged, register-blocked vector-ALU tile */
+  CUASR_AMD_KERNEL_MFMA = 3   /* matrix-core assisted tile                    */
+} cuasr_amd_kernel;
+
+/* One element of the problem's type; read through the member `dtype` names. */
+typedef union cuasr_amd_scalar {
+  float f32;
+  double f64;
+  int32_t i32;
+  uint32_t u32;
+  uint64_t bits;
+} cuasr_amd_scalar;
+
+/*
+ * Problem descriptor (device::Srgemm::Arguments, device/srgemm.h:139-183, plus
+ * what the reference fixes at compile time through its template parameters).
+ * A is m x k, B is k x n, C and D are m x n and share layout_c.  ld* are in
+ * elements.  D may alias C.  C is not dereferenced when the source is not
+ * needed, i.e. when add_identity == mult(beta, mult_identity)
+ * (epilogue/thread/semiring_linear_combination.h:118-125).
+ * alpha_ptr / beta_ptr, when non-NULL, are device pointers to one element
+ * that override alpha / beta (same file, :88-99, :112-115).
+ */
+typedef struct cuasr_amd_srgemm_desc {
+  int32_t add_op;          /* cuasr_amd_op */
+  int32_t mult_op;         /* cuasr_amd_op */
+  int32_t dtype;           /* cuasr_amd_dtype: A, B, C, D and accumulator */
+  int32_t layout_a;        /* cuasr_amd_layout */
+  int32_t layout_b;
+  int32_t layout_c;
+  int32_t m, n, k;
+  int32_t split_k_slices;  /* 1 for cuasr_amd_srgemm; >= 1 for the split-K call */
+  const void *A; int64_t lda;
+  const void *B; int64_t ldb;
+  const void *C; int64_t ldc;
+  void *D;       int64_t ldd;
+  cuasr_amd_scalar alpha;
+  cuasr_amd_scalar beta;
+  cuasr_amd_scalar add_identity;   /* AdditionOp::Identity        */
+  cuasr_amd_scalar mult_identity;  /* MultiplicationOp::Identity  */
+  const void *alpha_ptr;
+  const void *beta_ptr;
+  int32_t kernel;          /* cuasr_amd_kernel */
+  int32_t reserved;        /* must be 0 */
+} cuasr_amd_srgemm_desc;
+
+/* ABI version the library was built with. */
+int cuasr_amd_abi_version(void);
+
+/* Static text for a status code. */
+const char *cuasr_amd_status_string(int status);
+
+/* Validate a descriptor without touching the device.  Returns
+ * CUASR_AMD_ERROR_INVALID_PROBLEM for negative extents, ld smaller than the
+ * extent, or split_k_slices != 1; CUASR_AMD_ERROR_MISALIGNED_OPERAND for
+ * pointers not aligned to the element size; CUASR_AMD_ERROR_INVALID_DATA_TYPE /
+ * _INVALID_LAYOUT for unknown enums; CUASR_AMD_ERROR_NOT_SUPPORTED for an
+ * operator pair the element type does not define (bitwise on floating point)
+ * or a kernel family that cannot run the problem. */
+int cuasr_amd_srgemm_can_implement(const cuasr_amd_srgemm_desc *desc);
+
+/* Launch one SRGEMM.  Fails with CUASR_AMD_ERROR_INVALID_PROBLEM when
+ * split_k_slices > 1 (device/srgemm.h:198-200). */
+int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream);
+
+/* Bytes of device workspace the split-K call needs:
+ * sizeof(element) * m * n * split_k_slices. */
+size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
+
+/* Two launches on `stream`: partial products of `split_k_slices` K-slices into
+ * `workspace`, then a reduction with the semiring's add and the epilogue.
+ * CUASR_AMD_ERROR_WORKSPACE_NULL when workspace is NULL
+ * (device/srgemm_splitk_parallel.h:247-249). */
+int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
+                            void *stream);
+
+/* Name of the kernel family AUTO would choose for this descriptor
+ * ("naive", "valu", "mfma"), or NULL if the descriptor is invalid. */
+const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CUASR_AMD_H */

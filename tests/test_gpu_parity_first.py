@@ -1,0 +1,65 @@
+"""First GPU parity checks: every kernel family against the CPU oracle,
+bit-exact, through the C ABI."""
+import numpy as np
+import pytest
+
+from helpers import assert_same_bits, order_of, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+
+def run(oracle, add, mult, dtype, m, n, k, la, lb, lc, kernel, beta_one, seed=1, inf=True, splitk=0):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}[dtype]
+    if dtype in ("f32", "f64"):
+        A = inputs.integers(seed, m, k, -8, 8, npd, order_of(la))
+        B = inputs.integers(seed + 1, k, n, -8, 8, npd, order_of(lb))
+        C = inputs.integers(seed + 2, m, n, -8, 8, npd, order_of(lc))
+    else:
+        A = inputs.words32(seed, m, k, order_of(la)).astype(npd)
+        B = inputs.words32(seed + 1, k, n, order_of(lb)).astype(npd)
+        C = inputs.words32(seed + 2, m, n, order_of(lc)).astype(npd)
+    ident = cuasr_amd.op_identity(add, dtype, inf)
+    one = cuasr_amd.op_identity(mult, dtype, inf)
+    zero = cuasr_amd.op_annihilator(mult, dtype, inf)
+    if add == "maximum" and mult == "plus":
+        zero = ident  # the max-semiring zero, not plus::Annihilator
+    alpha, beta = one, (one if beta_one else zero)
+    want = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident)
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    dD = to_device(np.zeros_like(C))
+    if splitk:
+        ws = torch.empty(cuasr_amd.splitk_workspace_bytes(m, n, splitk, dtype) // 4 + 4, dtype=torch.int32, device="cuda")
+        cuasr_amd.srgemm_splitk(add, mult, dA, dB, dC, dD, splitk, ws, alpha, beta, ident, one, dtype=dtype, kernel=kernel)
+    else:
+        cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, alpha, beta, ident, one, dtype=dtype, kernel=kernel)
+    torch.cuda.synchronize()
+    assert_same_bits(to_host(dD, dtype), want, f"{add}-{mult} {dtype} {m}x{n}x{k} {la}{lb}{lc} {kernel}")
+
+
+@pytest.mark.parametrize("kernel", ["naive", "valu"])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (17, 27, 17), (128, 128, 64), (256, 384, 100), (509, 510, 23)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_minplus_f32(oracle, lib, kernel, shape, layouts):
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (False, True):
+        run(oracle, "minimum", "plus", "f32", *shape, la, lb, lc, kernel, beta_one)
+
+
+@pytest.mark.parametrize("kernel", ["naive", "valu"])
+@pytest.mark.parametrize("sr", [("maximum", "plus", "f64"), ("maximum", "minimum", "f64"), ("plus", "multiplies", "f32"),
+                                ("bit_xor", "bit_and", "u32"), ("logical_or", "logical_and", "i32")])
+def test_other_semirings(oracle, lib, kernel, sr):
+    for shape in [(128, 64, 32), (130, 70, 37), (256, 256, 256)]:
+        for layouts in ("ccc", "rcr"):
+            la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+            run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, kernel, True)
+
+
+@pytest.mark.parametrize("kernel", ["naive", "valu"])
+@pytest.mark.parametrize("slices", [1, 3, 8])
+def test_splitk_minplus(oracle, lib, kernel, slices):
+    run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", kernel, False, splitk=slices)
+    run(oracle, "minimum", "plus", "f32", 100, 60, 333, "col", "col", "col", kernel, True, splitk=slices)
