@@ -21,6 +21,9 @@
 #pragma once
 #include "semiring.h"
 
+#ifndef WAVES_ATTR
+#define WAVES_ATTR
+#endif
 namespace cuasr_amd {
 
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
@@ -124,9 +127,44 @@ struct ValuTile {
       for (int e = 0; e < VW; ++e) b[g * VW + e] = t[e];
     }
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = Op<ADD>::apply(acc[i][j], Op<MUL>::apply(a[i], b[j]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // Two k-steps at once, row by row: per accumulator two products and two
+  // adds, which the min/max semirings fold into one 3-input instruction.  The
+  // scheduling barrier after each row keeps the products of one row (2*TN
+  // registers) from piling up across rows.
+  static __device__ __forceinline__ void step2(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int kk,
+                                               int ty, int tx) {
+    T a[2][TM], b[2][TN];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+#pragma unroll
+      for (int h = 0; h < HM; ++h) {
+        const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk + s][ty * VW + h * 16 * VW]);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) a[s][h * VW + e] = t[e];
+      }
+#pragma unroll
+      for (int g = 0; g < GN; ++g) {
+        const vec_t t = *reinterpret_cast<const vec_t *>(&bs[kk + s][tx * VW + g * 16 * VW]);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) b[s][g * VW + e] = t[e];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const T t0 = Op<MUL>::apply(a[0][i], b[0][j]), t1 = Op<MUL>::apply(a[1][i], b[1][j]);
+        acc[i][j] = Op<ADD>::apply(Op<ADD>::apply(acc[i][j], t0), t1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 
   static __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int &bm, int &bn) {
@@ -184,8 +222,8 @@ struct ValuTile {
       }
       const int kcount = min(BK, ke - k0);
       if (kcount == BK) {
-#pragma unroll KU
-        for (int kk = 0; kk < BK; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
+#pragma unroll 1
+        for (int kk = 0; kk < BK; kk += 2) step2(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
       } else {
 #pragma unroll 1
         for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
@@ -253,12 +291,13 @@ struct ValuTile {
             if (col + c < p.n) out[(long long)row * ld_out + col + c] = v[c];
         }
       }
+      __builtin_amdgcn_sched_barrier(0);  // one row of C in flight at a time
     }
   }
 };
 
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
-__global__ __launch_bounds__(256) void valu_srgemm_kernel(Problem p) {
+__global__ __launch_bounds__(256) WAVES_ATTR void valu_srgemm_kernel(Problem p) {
   using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC>;
   __shared__ typename Tile::Smem sm;
   Tile::run(p, sm);

@@ -63,3 +63,36 @@ def test_other_semirings(oracle, lib, kernel, sr):
 def test_splitk_minplus(oracle, lib, kernel, slices):
     run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", kernel, False, splitk=slices)
     run(oracle, "minimum", "plus", "f32", 100, 60, 333, "col", "col", "col", kernel, True, splitk=slices)
+
+
+@pytest.mark.parametrize("add", ["minimum", "maximum"])
+@pytest.mark.parametrize("shape", [(128, 128, 16), (128, 128, 64), (256, 384, 100), (64, 4, 8), (4, 4, 4),
+                                   (516, 260, 52), (1024, 1024, 1024)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_tropical_mfma(oracle, lib, add, shape, layouts):
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (False, True):
+        run(oracle, add, "plus", "f32", *shape, la, lb, lc, "mfma", beta_one)
+
+
+@pytest.mark.parametrize("slices", [1, 3, 8])
+def test_splitk_mfma(oracle, lib, slices):
+    run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", "mfma", False, splitk=slices)
+    run(oracle, "minimum", "plus", "f32", 100, 60, 332, "col", "col", "col", "mfma", True, splitk=slices)
+
+
+def test_minplus_uniform_1024(oracle, lib):
+    """min-plus f32 1024^3, all column-major, uniform [0,1), identity +inf."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    n = 1024
+    A = inputs.uniform(11, n, n)
+    B = inputs.uniform(12, n, n)
+    C = np.full((n, n), np.inf, dtype=np.float32, order="F")
+    want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, np.inf, np.inf)
+    for kernel in ("auto", "valu", "naive"):
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, 0.0, np.inf, np.inf, 0.0, kernel=kernel)
+        torch.cuda.synchronize()
+        assert_same_bits(to_host(dD, "f32"), want, kernel)
