@@ -1,0 +1,115 @@
+"""Host-side checks of the C ABI that need no GPU: the library loads, exports
+every function include/cuasr_amd.h declares, and validates descriptors like the
+reference's can_implement / initialize do."""
+import ctypes
+import re
+
+import numpy as np
+import pytest
+
+import cuasr_amd
+from cuasr_amd import COLUMN_MAJOR, ROW_MAJOR, MatRef
+
+
+def declared_functions():
+    text = open(cuasr_amd.HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cuasr_amd_[a-z_]+)\s*\(", text)))
+
+
+def test_exports_match_header(lib):
+    names = declared_functions()
+    assert {"cuasr_amd_srgemm", "cuasr_amd_srgemm_splitk", "cuasr_amd_splitk_workspace_bytes",
+            "cuasr_amd_srgemm_can_implement"} <= set(names)
+    for name in names:
+        assert hasattr(lib, name), name
+    assert lib.cuasr_amd_abi_version() == 1
+
+
+def test_status_strings(lib):
+    assert lib.cuasr_amd_status_string(0) == b"success"
+    assert lib.cuasr_amd_status_string(6) == b"workspace is null"
+    assert len(cuasr_amd.STATUS_NAMES) == 12 and cuasr_amd.STATUS_NAMES[4] == "kErrorInvalidProblem"
+
+
+def desc(m=64, n=64, k=64, dtype="f32", add="minimum", mult="plus", la=COLUMN_MAJOR, lb=COLUMN_MAJOR, lc=COLUMN_MAJOR,
+         ptr=0x10000, **kw):
+    A = MatRef(ptr, kw.pop("lda", m if la == COLUMN_MAJOR else k), la, m, k)
+    B = MatRef(ptr, kw.pop("ldb", k if lb == COLUMN_MAJOR else n), lb, k, n)
+    ldc = kw.pop("ldc", m if lc == COLUMN_MAJOR else n)
+    C = MatRef(ptr, ldc, lc, m, n)
+    D = MatRef(kw.pop("dptr", ptr), kw.pop("ldd", ldc), lc, m, n)
+    return cuasr_amd.make_desc(add, mult, dtype, A, B, C, D, 0, 0, 0, 0, kw.pop("slices", 1), kw.pop("kernel", "auto"))
+
+
+def test_can_implement(lib):
+    ok = lambda d: lib.cuasr_amd_srgemm_can_implement(ctypes.byref(d))
+    assert ok(desc()) == 0
+    assert ok(desc(slices=2)) == 4            # kErrorInvalidProblem: split-K on the plain operator (device/srgemm.h:198-200)
+    assert ok(desc(lda=10)) == 4              # leading dimension smaller than the extent
+    assert ok(desc(ptr=0x10002)) == 1         # kErrorMisalignedOperand (kernel/srgemm.h:129-150)
+    assert ok(desc(dtype="f64", ptr=0x10004)) == 1
+    assert ok(desc(add="bit_xor", mult="bit_and")) == 5            # bitwise on floating point
+    assert ok(desc(dtype="u32", add="bit_xor", mult="bit_and")) == 0
+    assert ok(desc(dtype="f64", kernel="mfma")) == 5               # no matrix-core tile for this type
+    assert ok(desc(kernel="mfma")) == 0
+    assert ok(desc(m=63, kernel="mfma")) == 5                      # needs vector-sized contiguous extents
+    assert ok(desc(add="plus", mult="bit_or", dtype="i32", kernel="valu")) == 5
+    assert ok(desc(add="plus", mult="bit_or", dtype="i32", kernel="naive")) == 0
+    d = desc()
+    d.dtype = 9
+    assert ok(d) == 2
+    d = desc()
+    d.layout_b = 7
+    assert ok(d) == 3
+    d = desc()
+    d.m = -1
+    assert ok(d) == 4
+    d = desc(dptr=0)
+    assert ok(d) == 4
+
+
+def test_kernel_selection(lib):
+    sel = lambda d: lib.cuasr_amd_selected_kernel(ctypes.byref(d))
+    assert sel(desc()) == b"valu"
+    assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
+    assert sel(desc(kernel="mfma")) == b"mfma"
+
+
+def test_splitk_host_errors(lib):
+    d = desc(m=256, n=256, k=4096, slices=8)
+    assert cuasr_amd.splitk_workspace_bytes(256, 256, 8, "f32") == 4 * 256 * 256 * 8
+    assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "f64") == 8 * 100 * 7 * 3
+    # null workspace is rejected before anything touches the device
+    assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d), None, None) == 6
+    d0 = desc(slices=0)
+    assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
+    # the plain entry point refuses split-K descriptors without launching
+    assert lib.cuasr_amd_srgemm(ctypes.byref(d), None) == 4
+
+
+def test_semiring_constants():
+    # include/cuasr/functional.h:28-36, :41-42, :84-85, :127-128, :167-168, :207-208, :247-248
+    f32max, f32tiny = np.finfo(np.float32).max, np.finfo(np.float32).tiny
+    assert cuasr_amd.op_identity("minimum", "f32") == f32max
+    assert cuasr_amd.op_identity("maximum", "f32") == f32tiny          # numeric_limits::min(), not -max
+    assert cuasr_amd.op_identity("maximum", "f64") == np.finfo(np.float64).tiny
+    assert cuasr_amd.op_annihilator("plus", "f32") == f32max
+    assert cuasr_amd.op_identity("maximum", "i32") == np.iinfo(np.int32).min
+    assert cuasr_amd.op_identity("plus", "f64") == 0 and cuasr_amd.op_identity("multiplies", "i32") == 1
+    assert cuasr_amd.op_identity("logical_and", "i32") == 1 and cuasr_amd.op_annihilator("logical_or", "i32") == 1
+    assert cuasr_amd.op_identity("bit_and", "u32") == 0xFFFFFFFF and cuasr_amd.op_identity("bit_xor", "u32") == 0
+    assert cuasr_amd.op_identity("minimum", "f32", infinities=True) == np.inf
+    assert cuasr_amd.op_identity("maximum", "f64", infinities=True) == -np.inf
+
+
+def test_inputs_are_reproducible():
+    from cuasr_amd import inputs
+    a = inputs.uniform(7, 5, 3)
+    assert np.array_equal(a, np.asarray(inputs.uniform(7, 5, 3, order="C")))      # same entries in either layout
+    assert a.flags["F_CONTIGUOUS"] and a.min() >= 0 and a.max() < 1
+    assert inputs.splitmix64(1, 3).tolist() == inputs.splitmix64(1, 5)[:3].tolist()
+    g = inputs.graph_distances(1, 64)
+    assert np.all(np.diag(g) == 0) and np.isinf(g).mean() > 0.8
+    w = inputs.words32(3, 64, 64)
+    assert w.dtype == np.uint32 and 0.4 < np.unpackbits(np.ascontiguousarray(w).view(np.uint8)).mean() < 0.6

@@ -1,0 +1,214 @@
+"""Pins the CPU oracle (oracle/host_srgemm.c) without running any reference code:
+the reference's own known-answer vector, a literal pure-Python triple loop on
+ragged shapes / all layouts / every operator pair, and closed forms the
+mathematics fixes (GEMM, GF(2) bit planes, boolean reachability, Floyd-Warshall
+shortest paths, widest paths)."""
+import itertools
+import json
+import os
+
+import numpy as np
+import pytest
+
+from cuasr_amd import inputs
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+PY_OPS = {
+    "plus": lambda l, r: l + r,
+    "multiplies": lambda l, r: l * r,
+    "minimum": lambda l, r: r if r < l else l,
+    "maximum": lambda l, r: r if l < r else l,
+    "logical_and": lambda l, r: type(l)(bool(l) and bool(r)),
+    "logical_or": lambda l, r: type(l)(bool(l) or bool(r)),
+    "bit_and": lambda l, r: l & r,
+    "bit_or": lambda l, r: l | r,
+    "bit_xor": lambda l, r: l ^ r,
+}
+
+
+def literal_srgemm(add, mult, A, B, C, alpha, beta, ident):
+    """The reference host loop, literally (host_srgemm.h:75-109), in Python scalars
+    of the matrix dtype: accum = add(mult(a, b), accum), then
+    D = add(mult(alpha, accum), mult(beta, c))."""
+    f_add, f_mul = PY_OPS[add], PY_OPS[mult]
+    t = A.dtype.type
+    m, k = A.shape
+    n = B.shape[1]
+    D = np.empty((m, n), dtype=A.dtype)
+    with np.errstate(over="ignore"):
+        for i in range(m):
+            for j in range(n):
+                acc = t(ident)
+                for kk in range(k):
+                    acc = t(f_add(t(f_mul(A[i, kk], B[kk, j])), acc))
+                D[i, j] = t(f_add(t(f_mul(t(alpha), acc)), t(f_mul(t(beta), C[i, j]))))
+    return D
+
+
+def bits(x):
+    return np.ascontiguousarray(x).tobytes()
+
+
+def test_reference_known_answer_vector(oracle):
+    g = json.load(open(os.path.join(HERE, "golden", "regress_minplus_4x4x2.json")))
+    f = lambda key, r, c: np.array(g[key], dtype=np.float32).reshape(c, r).T
+    A, B, C = f("a_colmajor", 4, 2), f("b_colmajor", 2, 4), f("c_colmajor", 4, 4)
+    want = f("expected_colmajor", 4, 4)
+    for naive in (False, True):
+        for order in ("F", "C"):
+            got = oracle.srgemm("minimum", "plus", np.asarray(A, order=order), np.asarray(B, order=order),
+                                np.asarray(C, order=order), 0.0, 0.0, np.finfo(np.float32).max, naive=naive)
+            # the reference compares with EXPECT_FLOAT_EQ (4 ulp); the literals round-trip exactly
+            assert np.array_equal(got, want)
+    # only linear index 11 (column-major) differs from C, as in the reference test
+    diff = np.flatnonzero(want.T.ravel() != C.T.ravel())
+    assert diff.tolist() == [11]
+
+
+FLOAT_PAIRS = [("plus", "multiplies"), ("minimum", "plus"), ("maximum", "plus"), ("minimum", "multiplies"),
+               ("maximum", "multiplies"), ("minimum", "maximum"), ("maximum", "minimum"), ("logical_or", "logical_and")]
+INT_PAIRS = FLOAT_PAIRS + [("bit_xor", "bit_and"), ("bit_xor", "logical_and"), ("bit_or", "bit_and")]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.uint32])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (7, 6, 5), (17, 27, 17), (33, 34, 3)])
+def test_against_literal_loop(oracle, dtype, shape):
+    m, n, k = shape
+    pairs = FLOAT_PAIRS if np.dtype(dtype).kind == "f" else INT_PAIRS
+    lo = 0 if np.dtype(dtype).kind == "u" else -8
+    for (add, mult), (la, lb, lc) in zip(pairs, itertools.cycle(itertools.product("FC", repeat=3))):
+        A = inputs.integers(5, m, k, lo, 8, dtype, la)
+        B = inputs.integers(6, k, n, lo, 8, dtype, lb)
+        C = inputs.integers(7, m, n, lo, 8, dtype, lc)
+        for alpha, beta, ident in [(1, 0, 0), (1, 1, 3), (2, 1, 5)]:
+            want = literal_srgemm(add, mult, A, B, C, alpha, beta, ident)
+            for naive in (False, True):
+                got = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident, naive=naive)
+                assert bits(got) == bits(np.asarray(want, order=lc)), (add, mult, la, lb, lc, naive)
+
+
+def test_blocked_equals_naive_on_ragged_and_submatrix(oracle):
+    big_a = inputs.uniform(1, 140, 90)
+    big_b = inputs.uniform(2, 90, 150)
+    big_c = inputs.uniform(3, 140, 150)
+    for (r0, c0, m, n, k) in [(0, 0, 125, 125, 80), (15, 21, 70, 65, 33), (3, 2, 97, 130, 90)]:
+        A, B, C = big_a[r0:r0 + m, :k], big_b[:k, c0:c0 + n], big_c[r0:r0 + m, c0:c0 + n]  # ld > extent
+        for add, mult, ident in [("minimum", "plus", np.inf), ("maximum", "minimum", -np.inf), ("plus", "multiplies", 0.0)]:
+            one = {"plus": 0.0, "minimum": np.inf, "multiplies": 1.0}[mult]
+            x = oracle.srgemm(add, mult, A, B, C, one, one, ident, naive=False, nthreads=3)
+            y = oracle.srgemm(add, mult, A, B, C, one, one, ident, naive=True)
+            assert bits(x) == bits(y)
+
+
+def test_plus_times_is_gemm(oracle):
+    A = inputs.integers(1, 40, 50, -8, 8, np.float32)
+    B = inputs.integers(2, 50, 30, -8, 8, np.float32)
+    C = inputs.integers(3, 40, 30, -8, 8, np.float32)
+    got = oracle.srgemm("plus", "multiplies", A, B, C, 2.0, 3.0, 0.0)
+    want = 2.0 * (A.astype(np.float64) @ B.astype(np.float64)) + 3.0 * C
+    assert np.array_equal(got.astype(np.float64), want)  # small integers: exact in fp32
+    An, Bn = inputs.normal(4, 64, 300, np.float64), inputs.normal(5, 300, 48, np.float64)
+    got = oracle.srgemm("plus", "multiplies", An, Bn, np.zeros((64, 48), order="F"), 1.0, 0.0, 0.0)
+    bound = 1e-12 * (np.abs(An) @ np.abs(Bn))
+    assert np.all(np.abs(got - An @ Bn) <= bound)
+
+
+def test_gf2_and_boolean_closed_forms(oracle):
+    A = inputs.bernoulli(1, 45, 60, 0.3)
+    B = inputs.bernoulli(2, 60, 38, 0.3)
+    Z = np.zeros((45, 38), dtype=np.int32, order="F")
+    prod = A.astype(np.int64) @ B.astype(np.int64)
+    got = oracle.srgemm("bit_xor", "logical_and", A, B, Z, 1, 0, 0)
+    assert np.array_equal(got, (prod % 2).astype(np.int32))
+    got = oracle.srgemm("logical_or", "logical_and", A, B, Z, 1, 0, 0)
+    assert np.array_equal(got, (prod > 0).astype(np.int32))
+    # logical_and is not bitwise: 6 && 9 = 1, 6 & 9 = 0  (functional.h:212)
+    six, nine = np.full((1, 1), 6, np.int32), np.full((1, 1), 9, np.int32)
+    z1 = np.zeros((1, 1), np.int32)
+    assert oracle.srgemm("bit_xor", "logical_and", six, nine, z1, 1, 0, 0)[0, 0] == 1
+    assert oracle.srgemm("bit_xor", "bit_and", six, nine, z1, -1, 0, 0)[0, 0] == 0
+    # bit-packed GF(2): 32 independent products, one per bit plane
+    Aw, Bw = inputs.words32(3, 20, 37), inputs.words32(4, 37, 25)
+    Zw = np.zeros((20, 25), dtype=np.uint32, order="F")
+    got = oracle.srgemm("bit_xor", "bit_and", Aw, Bw, Zw, 0xFFFFFFFF, 0, 0)
+    for b in (0, 7, 31):
+        pa, pb = ((Aw >> np.uint32(b)) & 1).astype(np.int64), ((Bw >> np.uint32(b)) & 1).astype(np.int64)
+        assert np.array_equal((got >> np.uint32(b)) & 1, ((pa @ pb) % 2).astype(np.uint32))
+
+
+def floyd_warshall(D):
+    D = D.astype(np.float64).copy()
+    for kk in range(D.shape[0]):
+        D = np.minimum(D, D[:, kk:kk + 1] + D[kk:kk + 1, :])
+    return D
+
+
+def test_minplus_closure_is_floyd_warshall(oracle):
+    n = 48
+    D = inputs.graph_distances(9, n, density=0.15, integer_weights=True)  # sums < 2^24: exact in fp32
+    cur = D
+    for _ in range(6):  # 2^6 >= n - 1
+        cur = oracle.srgemm("minimum", "plus", cur, cur, cur, 0.0, 0.0, np.inf)
+    assert np.array_equal(cur.astype(np.float64), floyd_warshall(D))
+    again = oracle.srgemm("minimum", "plus", cur, cur, cur, 0.0, 0.0, np.inf)
+    assert bits(again) == bits(cur)  # closed: idempotent
+
+
+def test_maxmin_closure_is_widest_path(oracle):
+    n = 24
+    W = inputs.uniform(3, n, n, 0.0, 1.0, np.float64)
+    np.fill_diagonal(W, np.inf)
+    cur = W
+    for _ in range(5):
+        cur = oracle.srgemm("maximum", "minimum", cur, cur, cur, np.inf, np.inf, -np.inf)
+    ref = W.copy()
+    for kk in range(n):
+        ref = np.maximum(ref, np.minimum(ref[:, kk:kk + 1], ref[kk:kk + 1, :]))
+    assert np.array_equal(cur, ref)
+
+
+def test_invariants(oracle):
+    m, n, k = 37, 29, 41
+    A, B, C = inputs.uniform(1, m, k), inputs.uniform(2, k, n), inputs.uniform(3, m, n)
+    inf = np.float32(np.inf)
+    base = oracle.srgemm("minimum", "plus", A, B, C, 0.0, inf, inf)
+    # beta = semiring zero: D does not depend on C
+    other = oracle.srgemm("minimum", "plus", A, B, inputs.uniform(4, m, n), 0.0, inf, inf)
+    assert bits(base) == bits(other)
+    # beta = semiring one: D = min(A (x) B, C)
+    withc = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, inf)
+    assert np.array_equal(withc, np.minimum(base, C))
+    # A (x) I = A, I = semiring one on the diagonal, zero elsewhere
+    eye = np.full((k, k), inf, dtype=np.float32, order="F")
+    np.fill_diagonal(eye, 0.0)
+    assert np.array_equal(oracle.srgemm("minimum", "plus", A, eye, np.zeros((m, k), np.float32, order="F"), 0.0, inf, inf), A)
+    # order-freeness: permuting k changes nothing (the basis of bit-exact parity)
+    perm = np.argsort(inputs.uniform(8, k, 1)[:, 0])
+    assert bits(oracle.srgemm("minimum", "plus", np.asfortranarray(A[:, perm]), np.asfortranarray(B[perm, :]), C, 0.0, inf, inf)) == bits(base)
+    # transposition: (A (x) B)^T = B^T (x) A^T
+    tr = oracle.srgemm("minimum", "plus", np.asfortranarray(B.T), np.asfortranarray(A.T), np.asfortranarray(C.T), 0.0, inf, inf)
+    assert np.array_equal(tr.T, base)
+    # every layout combination gives the same values
+    for la, lb, lc in itertools.product("FC", repeat=3):
+        got = oracle.srgemm("minimum", "plus", np.asarray(A, order=la), np.asarray(B, order=lb), np.asarray(C, order=lc), 0.0, 0.0, inf)
+        assert np.array_equal(got, withc)
+    # reference-valued identity (numeric_limits::max) behaves like +inf on this data
+    fmax = np.finfo(np.float32).max
+    assert np.array_equal(oracle.srgemm("minimum", "plus", A, B, C, 0.0, fmax, fmax), base)
+
+
+@pytest.mark.parametrize("slices", [1, 2, 3, 8, 16])
+def test_splitk_model(oracle, slices):
+    m, n, k = 40, 24, 200
+    A, B, C = inputs.uniform(1, m, k, 0, 10), inputs.uniform(2, k, n, 0, 10), inputs.uniform(3, m, n, 0, 10)
+    inf = np.float32(np.inf)
+    for beta in (inf, np.float32(0.0)):  # zero (no source) and one
+        want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, beta, inf)
+        got = oracle.srgemm_splitk("minimum", "plus", A, B, C, 0.0, beta, inf, 0.0, slices)
+        assert bits(got) == bits(want)  # the reference example's own check (splitk_srgemm.cu:270-287)
+    # plus-times: slicing changes the summation order, not the value on small integers
+    Ai, Bi = inputs.integers(4, m, k, -8, 8), inputs.integers(5, k, n, -8, 8)
+    want = oracle.srgemm("plus", "multiplies", Ai, Bi, C, 1.0, 0.0, 0.0)
+    got = oracle.srgemm_splitk("plus", "multiplies", Ai, Bi, C, 1.0, 0.0, 0.0, 1.0, slices)
+    assert bits(got) == bits(want)
