@@ -53,6 +53,22 @@ def build(jobs=None, verbose=True):
     return LIB
 
 
+def build_cpp_tests():
+    """The C++ operator-API test program (tests/cpp), linked against the library."""
+    root = os.path.dirname(HERE)
+    src = os.path.join(root, "tests", "cpp", "test_device_api.cpp")
+    out = os.path.join(root, "tests", "cpp", "test_device_api")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    # plain host C++: the operator templates need only the HIP runtime API header
+    subprocess.check_call([os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-D__HIP_PLATFORM_AMD__",
+                           "-I", os.path.join(rocm, "include"),
+                           "-I", os.path.join(root, "include"), "-I", os.path.join(root, "oracle", "include"),
+                           src, "-L", LIB_DIR, "-lcuasr_amd", "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
+                           "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,$ORIGIN/../../cuasr_amd/lib", "-o", out])
+    return out
+
+
 if __name__ == "__main__":
     j = int(sys.argv[sys.argv.index("-j") + 1]) if "-j" in sys.argv else None
     print(build(j))
+    print(build_cpp_tests())

@@ -26,7 +26,7 @@ __global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
   T acc = e.ident;
   for (int kk = k0; kk < k1; ++kk) {
     const T prod = apply_op<T>(p.mult_op, A[(long long)kk * p.sa_k], B[(long long)kk * p.sb_k]);
-    acc = apply_op<T>(p.add_op, acc, prod);
+    acc = apply_op<T>(p.add_op, prod, acc);  // host reference order: add(prod, acc)
   }
   if (p.workspace) {
     reinterpret_cast<T *>(p.workspace)[((long long)z * p.m + i) * p.n + j] = acc;

@@ -29,8 +29,20 @@ template <> __device__ __forceinline__ float hw_max<float>(float l, float r) { r
 template <> __device__ __forceinline__ double hw_min<double>(double l, double r) { return __builtin_fmin(l, r); }
 template <> __device__ __forceinline__ double hw_max<double>(double l, double r) { return __builtin_fmax(l, r); }
 
-// Compile-time operator: Op<kMinimum>::apply(l, r)
+// Compile-time operator.
+//   Op<OP>::apply(l, r)   fast form: floating-point min/max are the hardware
+//                         instructions (order-free, one instruction)
+//   Op<OP>::strict(l, r)  the reference's comparison, operand order included:
+//                         minimum = rhs < lhs ? rhs : lhs, maximum = lhs < rhs ? rhs : lhs
+// The two differ only when the operands are +0 and -0 (or NaN).  Sums, minima
+// and maxima of data free of -0 never produce -0; products do (0 * negative),
+// so kernels use the strict form wherever `multiplies` feeds a min or max.
 template <int OP> struct Op {
+  template <typename T> static __device__ __forceinline__ T strict(T l, T r) {
+    if constexpr (OP == kMinimum) return r < l ? r : l;
+    else if constexpr (OP == kMaximum) return l < r ? r : l;
+    else return apply(l, r);
+  }
   template <typename T> static __device__ __forceinline__ T apply(T l, T r) {
     if constexpr (OP == kPlus) return l + r;
     else if constexpr (OP == kMultiplies) return l * r;
@@ -48,19 +60,33 @@ template <int OP> struct Op {
   }
 };
 
-// Run-time operator (naive kernel, reduction epilogue)
+// Run-time operator with the strict semantics (naive kernel, reduction, scalars)
 template <typename T> __device__ __forceinline__ T apply_op(int op, T l, T r) {
   switch (op) {
-    case kPlus: return Op<kPlus>::apply(l, r);
-    case kMultiplies: return Op<kMultiplies>::apply(l, r);
-    case kMinimum: return Op<kMinimum>::apply(l, r);
-    case kMaximum: return Op<kMaximum>::apply(l, r);
-    case kLogicalAnd: return Op<kLogicalAnd>::apply(l, r);
-    case kLogicalOr: return Op<kLogicalOr>::apply(l, r);
-    case kBitAnd: return Op<kBitAnd>::apply(l, r);
-    case kBitOr: return Op<kBitOr>::apply(l, r);
-    default: return Op<kBitXor>::apply(l, r);
+    case kPlus: return Op<kPlus>::strict(l, r);
+    case kMultiplies: return Op<kMultiplies>::strict(l, r);
+    case kMinimum: return Op<kMinimum>::strict(l, r);
+    case kMaximum: return Op<kMaximum>::strict(l, r);
+    case kLogicalAnd: return Op<kLogicalAnd>::strict(l, r);
+    case kLogicalOr: return Op<kLogicalOr>::strict(l, r);
+    case kBitAnd: return Op<kBitAnd>::strict(l, r);
+    case kBitOr: return Op<kBitOr>::strict(l, r);
+    default: return Op<kBitXor>::strict(l, r);
   }
+}
+
+// add(prod, acc) in the host reference's operand order
+// (tools/include/cuasr/reference/srgemm/host_srgemm.h:87), strict when a
+// product can be -0 and the add is a comparison
+template <int ADD, int MUL, typename T> __device__ __forceinline__ T fold(T prod, T acc) {
+  if constexpr ((ADD == kMinimum || ADD == kMaximum) && MUL == kMultiplies && is_fp<T>::value) return Op<ADD>::strict(prod, acc);
+  else return Op<ADD>::apply(acc, prod);
+}
+
+// add(lhs, rhs) of the epilogue, D = add(mult(alpha, acc), mult(beta, C)), same rule
+template <int ADD, int MUL, typename T> __device__ __forceinline__ T fold_epilogue(T lhs, T rhs) {
+  if constexpr ((ADD == kMinimum || ADD == kMaximum) && MUL == kMultiplies && is_fp<T>::value) return Op<ADD>::strict(lhs, rhs);
+  else return Op<ADD>::apply(lhs, rhs);
 }
 
 template <typename T> __host__ __device__ __forceinline__ T scalar_as(const cuasr_amd_scalar &s);

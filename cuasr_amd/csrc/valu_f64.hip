@@ -9,12 +9,12 @@ namespace cuasr_amd {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return launch_valu<double, ADD, MUL, 8, 4, 8>;
 
+launch_fn find_valu_strict(int dtype, int add_op, int mult_op);
+
 launch_fn find_valu_f64(int add_op, int mult_op) {
   PAIR(kPlus, kMultiplies)
   PAIR(kMinimum, kPlus)
   PAIR(kMaximum, kPlus)
-  PAIR(kMinimum, kMultiplies)
-  PAIR(kMaximum, kMultiplies)
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
   PAIR(kLogicalOr, kLogicalAnd)
@@ -23,7 +23,7 @@ launch_fn find_valu_f64(int add_op, int mult_op) {
   PAIR(kBitXor, kLogicalAnd)
   PAIR(kBitOr, kBitAnd)
 #endif
-  return nullptr;
+  return find_valu_strict(CUASR_AMD_F64, add_op, mult_op);
 }
 
 }  // namespace cuasr_amd

@@ -129,7 +129,7 @@ struct ValuTile {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = Op<ADD>::apply(acc[i][j], Op<MUL>::apply(a[i], b[j]));
+      for (int j = 0; j < TN; ++j) acc[i][j] = fold<ADD, MUL>(Op<MUL>::apply(a[i], b[j]), acc[i][j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -161,7 +161,7 @@ struct ValuTile {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const T t0 = Op<MUL>::apply(a[0][i], b[0][j]), t1 = Op<MUL>::apply(a[1][i], b[1][j]);
-        acc[i][j] = Op<ADD>::apply(Op<ADD>::apply(acc[i][j], t0), t1);
+        acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -277,7 +277,7 @@ struct ValuTile {
               for (int c = 0; c < VW; ++c) src[c] = C[(long long)row * p.ldc + min(col + c, p.n - 1)];
             }
 #pragma unroll
-            for (int c = 0; c < VW; ++c) v[c] = Op<ADD>::apply(v[c], Op<MUL>::apply(e.beta, src[c]));
+            for (int c = 0; c < VW; ++c) v[c] = fold_epilogue<ADD, MUL>(v[c], Op<MUL>::apply(e.beta, src[c]));
           }
         }
         if constexpr (VEC) {

@@ -1,0 +1,87 @@
+// Semiring operator functors of the cuASR API.
+//
+// Each functor has the reference's scalar semantics and constants
+// (include/cuasr/functional.h:28-36, :39-283 of the reference):
+//   plus        l + r           Identity 0,      Annihilator max()
+//   multiplies  l * r           Identity 1,      Annihilator 0
+//   minimum     r < l ? r : l   Identity max(),  Annihilator min()
+//   maximum     l < r ? r : l   Identity min(),  Annihilator max()
+//   binary_and  l && r (0/1)    Identity 1,      Annihilator 0
+//   binary_or   l || r (0/1)    Identity 0,      Annihilator 1
+// where max()/min() are std::numeric_limits<T>::max()/min() -- for floating
+// point min() is the smallest positive normal, exactly as in the reference.
+// Added here: binary_xor (the reference's user-defined example,
+// examples/01_userdefined_semiring/userdefined_semiring.cu:56-66), bitwise
+// and/or for bit-packed words, and cuasr::inf::minimum / maximum / plus whose
+// constants are true infinities (what shortest-path data with unreachable
+// pairs needs).
+//
+// The device kernels are not instantiated from these functors; a functor type
+// maps to an operator tag of the C ABI through cuasr::op_tag<Functor>, which
+// user code specialises for its own functor types (see binary_xor below).
+#pragma once
+#include <limits>
+
+#include "types.h"
+
+namespace cuasr {
+
+template <typename F> struct op_tag;  // { static int const value = CUASR_AMD_OP_...; }
+
+namespace detail {
+template <typename T> constexpr T highest() { return std::numeric_limits<T>::max(); }
+template <typename T> constexpr T lowest_ref() { return std::numeric_limits<T>::min(); }  // sic: the reference's "-inf"
+template <typename T> constexpr T pos_inf() {
+  return std::numeric_limits<T>::has_infinity ? std::numeric_limits<T>::infinity() : std::numeric_limits<T>::max();
+}
+template <typename T> constexpr T neg_inf() {
+  return std::numeric_limits<T>::has_infinity ? -std::numeric_limits<T>::infinity() : std::numeric_limits<T>::lowest();
+}
+}  // namespace detail
+
+#define CUASR_AMD_FUNCTOR(NAME, IDENT, ANNIH, EXPR)                               \
+  template <typename T, int N = 1> struct NAME {                                  \
+    static constexpr T Identity = IDENT;                                          \
+    static constexpr T Annihilator = ANNIH;                                       \
+    constexpr T operator()(T lhs, T const &rhs) const { return EXPR; }            \
+  };                                                                              \
+  template <typename T, int N> constexpr T NAME<T, N>::Identity;                  \
+  template <typename T, int N> constexpr T NAME<T, N>::Annihilator;
+#define CUASR_AMD_OP_TAG(NAME, TAG) \
+  template <typename T, int N> struct op_tag<NAME<T, N>> { static int const value = TAG; };
+
+CUASR_AMD_FUNCTOR(plus, static_cast<T>(0), detail::highest<T>(), static_cast<T>(lhs + rhs))
+CUASR_AMD_FUNCTOR(multiplies, static_cast<T>(1), static_cast<T>(0), static_cast<T>(lhs * rhs))
+CUASR_AMD_FUNCTOR(minimum, detail::highest<T>(), detail::lowest_ref<T>(), (rhs < lhs ? rhs : lhs))
+CUASR_AMD_FUNCTOR(maximum, detail::lowest_ref<T>(), detail::highest<T>(), (lhs < rhs ? rhs : lhs))
+CUASR_AMD_FUNCTOR(binary_and, static_cast<T>(true), static_cast<T>(false), static_cast<T>(lhs && rhs))
+CUASR_AMD_FUNCTOR(binary_or, static_cast<T>(false), static_cast<T>(true), static_cast<T>(lhs || rhs))
+CUASR_AMD_FUNCTOR(binary_xor, static_cast<T>(0), static_cast<T>(0), static_cast<T>(lhs ^ rhs))
+CUASR_AMD_FUNCTOR(bitwise_and, static_cast<T>(~static_cast<T>(0)), static_cast<T>(0), static_cast<T>(lhs & rhs))
+CUASR_AMD_FUNCTOR(bitwise_or, static_cast<T>(0), static_cast<T>(~static_cast<T>(0)), static_cast<T>(lhs | rhs))
+
+CUASR_AMD_OP_TAG(plus, CUASR_AMD_OP_PLUS)
+CUASR_AMD_OP_TAG(multiplies, CUASR_AMD_OP_MULTIPLIES)
+CUASR_AMD_OP_TAG(minimum, CUASR_AMD_OP_MINIMUM)
+CUASR_AMD_OP_TAG(maximum, CUASR_AMD_OP_MAXIMUM)
+CUASR_AMD_OP_TAG(binary_and, CUASR_AMD_OP_LOGICAL_AND)
+CUASR_AMD_OP_TAG(binary_or, CUASR_AMD_OP_LOGICAL_OR)
+CUASR_AMD_OP_TAG(binary_xor, CUASR_AMD_OP_BIT_XOR)
+CUASR_AMD_OP_TAG(bitwise_and, CUASR_AMD_OP_BIT_AND)
+CUASR_AMD_OP_TAG(bitwise_or, CUASR_AMD_OP_BIT_OR)
+
+/// The same operators with true infinities as their constants.
+namespace inf {
+CUASR_AMD_FUNCTOR(plus, static_cast<T>(0), detail::pos_inf<T>(), static_cast<T>(lhs + rhs))
+CUASR_AMD_FUNCTOR(minimum, detail::pos_inf<T>(), detail::neg_inf<T>(), (rhs < lhs ? rhs : lhs))
+CUASR_AMD_FUNCTOR(maximum, detail::neg_inf<T>(), detail::pos_inf<T>(), (lhs < rhs ? rhs : lhs))
+/// plus as the multiplication of a max-semiring: its zero is -inf
+CUASR_AMD_FUNCTOR(plus_for_max, static_cast<T>(0), detail::neg_inf<T>(), static_cast<T>(lhs + rhs))
+}  // namespace inf
+
+CUASR_AMD_OP_TAG(inf::plus, CUASR_AMD_OP_PLUS)
+CUASR_AMD_OP_TAG(inf::minimum, CUASR_AMD_OP_MINIMUM)
+CUASR_AMD_OP_TAG(inf::maximum, CUASR_AMD_OP_MAXIMUM)
+CUASR_AMD_OP_TAG(inf::plus_for_max, CUASR_AMD_OP_PLUS)
+
+}  // namespace cuasr

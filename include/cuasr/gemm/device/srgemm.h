@@ -1,0 +1,182 @@
+// cuasr::gemm::device::Srgemm -- the cuASR device-level SRGEMM operator,
+// implemented on libcuasr_amd (hand-written gfx950 kernels behind a C ABI).
+//
+// Same template head, member aliases, Arguments and methods as the reference
+// operator (include/cuasr/gemm/device/srgemm.h:28-357 and the column-major
+// specialisation :398-567); `cudaStream_t` becomes `hipStream_t`.  The tile
+// shape / swizzle / stage parameters are accepted and ignored: tiling is the
+// library's business.  Column-major C needs no specialisation here -- the
+// library runs the transposed problem itself.
+//
+// Ownership and threading follow the reference: the caller owns A, B, C, D and
+// the workspace (device memory); the operator object holds a by-value copy of
+// the arguments; nothing allocates or synchronises; launches are asynchronous
+// on the given stream; D may alias C.
+#pragma once
+#include <hip/hip_runtime_api.h>
+
+#include <type_traits>
+
+#include "default_srgemm_configuration.h"
+
+namespace cuasr {
+namespace gemm {
+namespace device {
+
+namespace detail {
+/// Fill the C-ABI descriptor from typed arguments.
+template <typename Op, typename Args>
+inline cuasr_amd_srgemm_desc make_desc(Args const &a, int kernel) {
+  using Element = typename Op::ElementC;
+  cuasr_amd_srgemm_desc d{};
+  d.add_op = op_tag<typename Op::AdditionOp>::value;
+  d.mult_op = op_tag<typename Op::MultiplicationOp>::value;
+  d.dtype = dtype_tag<Element>::value;
+  d.layout_a = Op::LayoutA::kAbiTag;
+  d.layout_b = Op::LayoutB::kAbiTag;
+  d.layout_c = Op::LayoutC::kAbiTag;
+  d.m = a.problem_size.m();
+  d.n = a.problem_size.n();
+  d.k = a.problem_size.k();
+  d.split_k_slices = a.split_k_slices;
+  d.A = a.ref_A.data(); d.lda = a.ref_A.stride(0);
+  d.B = a.ref_B.data(); d.ldb = a.ref_B.stride(0);
+  d.C = a.ref_C.data(); d.ldc = a.ref_C.stride(0);
+  d.D = a.ref_D.data(); d.ldd = a.ref_D.stride(0);
+  d.alpha = make_scalar<Element>(a.epilogue.alpha);
+  d.beta = make_scalar<Element>(a.epilogue.beta);
+  d.add_identity = make_scalar<Element>(Op::AdditionOp::Identity);
+  d.mult_identity = make_scalar<Element>(Op::MultiplicationOp::Identity);
+  d.alpha_ptr = a.epilogue.alpha_ptr;
+  d.beta_ptr = a.epilogue.beta_ptr;
+  d.kernel = kernel;
+  d.reserved = 0;
+  return d;
+}
+template <typename OperatorClass> struct kernel_of { static int const value = CUASR_AMD_KERNEL_AUTO; };
+template <> struct kernel_of<arch::OpClassMatrixCore> { static int const value = CUASR_AMD_KERNEL_MFMA; };
+}  // namespace detail
+
+template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, typename LayoutA_, typename ElementB_,
+          typename LayoutB_, typename ElementC_, typename LayoutC_, typename ElementAccumulator_ = ElementC_,
+          typename OperatorClass_ = arch::OpClassSimt, typename ArchTag_ = arch::Gfx950,
+          typename ThreadblockShape_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::ThreadblockShape,
+          typename WarpShape_ = typename DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_,
+                                                                     OperatorClass_, AdditionOp_, MultiplicationOp_,
+                                                                     ArchTag_>::WarpShape,
+          typename InstructionShape_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::InstructionShape,
+          typename EpilogueOutputOp_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::EpilogueOutputOp,
+          typename ThreadblockSwizzle_ = threadblock::GemmIdentityThreadblockSwizzle<>,
+          int Stages = DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_,
+                                                    AdditionOp_, MultiplicationOp_, ArchTag_>::kStages,
+          int AlignmentA = 1, int AlignmentB = 1, bool SplitKSerial = false>
+class Srgemm {
+ public:
+  using ElementA = ElementA_;
+  using LayoutA = LayoutA_;
+  using TensorRefA = TensorRef<ElementA const, LayoutA>;
+  using ElementB = ElementB_;
+  using LayoutB = LayoutB_;
+  using TensorRefB = TensorRef<ElementB const, LayoutB>;
+  using ElementC = ElementC_;
+  using LayoutC = LayoutC_;
+  using TensorRefC = TensorRef<ElementC const, LayoutC>;
+  using TensorRefD = TensorRef<ElementC, LayoutC>;
+  using ElementAccumulator = ElementAccumulator_;
+  using OperatorClass = OperatorClass_;
+  using ArchTag = ArchTag_;
+  using ThreadblockShape = ThreadblockShape_;
+  using WarpShape = WarpShape_;
+  using InstructionShape = InstructionShape_;
+  using EpilogueOutputOp = EpilogueOutputOp_;
+  using ThreadblockSwizzle = ThreadblockSwizzle_;
+  using AdditionOp = AdditionOp_;
+  using MultiplicationOp = MultiplicationOp_;
+  static int const kStages = Stages;
+  static int const kAlignmentA = AlignmentA;
+  static int const kAlignmentB = AlignmentB;
+  static int const kAlignmentC = EpilogueOutputOp::kCount;
+  static bool const kSplitKSerial = SplitKSerial;
+
+  static_assert(std::is_same<ElementA, ElementC>::value && std::is_same<ElementB, ElementC>::value &&
+                    std::is_same<ElementAccumulator, ElementC>::value,
+                "A, B, C and the accumulator share one element type (as in every reference configuration)");
+
+  struct Arguments {
+    GemmCoord problem_size;
+    TensorRef<ElementA const, LayoutA> ref_A;
+    TensorRef<ElementB const, LayoutB> ref_B;
+    TensorRef<ElementC const, LayoutC> ref_C;
+    TensorRef<ElementC, LayoutC> ref_D;
+    typename EpilogueOutputOp::Params epilogue;
+    int split_k_slices;
+
+    Arguments() : problem_size(0, 0, 0), split_k_slices(1) {}
+    Arguments(GemmCoord problem_size_, TensorRef<ElementA const, LayoutA> ref_A_, TensorRef<ElementB const, LayoutB> ref_B_,
+              TensorRef<ElementC const, LayoutC> ref_C_, TensorRef<ElementC, LayoutC> ref_D_,
+              typename EpilogueOutputOp::Params epilogue_ = typename EpilogueOutputOp::Params(), int split_k_slices_ = 1)
+        : problem_size(problem_size_), ref_A(ref_A_), ref_B(ref_B_), ref_C(ref_C_), ref_D(ref_D_), epilogue(epilogue_),
+          split_k_slices(split_k_slices_) {}
+  };
+
+  Srgemm() : ready_(false) {}
+
+  /// kErrorInvalidProblem when split_k_slices > 1: serial split-K (a
+  /// semaphore-ordered in-place reduction in the reference) is not offered;
+  /// use SrgemmSplitKParallel.
+  static Status can_implement(Arguments const &args) {
+    if (args.split_k_slices > 1) return kSplitKSerial ? Status::kErrorNotSupported : Status::kErrorInvalidProblem;
+    cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    return static_cast<Status>(cuasr_amd_srgemm_can_implement(&d));
+  }
+
+  static size_t get_workspace_size(Arguments const &) { return 0; }
+
+  Status initialize(Arguments const &args, void * /*workspace*/ = nullptr, hipStream_t /*stream*/ = nullptr) {
+    Status s = can_implement(args);
+    if (s != Status::kSuccess) return s;
+    desc_ = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    ready_ = true;
+    return Status::kSuccess;
+  }
+
+  /// Lightweight refresh of the operand pointers (reference: srgemm.h:285-300).
+  Status update(Arguments const &args, void * /*workspace*/ = nullptr) {
+    if (!ready_) return Status::kErrorInternal;
+    desc_.A = args.ref_A.data();
+    desc_.B = args.ref_B.data();
+    desc_.C = args.ref_C.data();
+    desc_.D = args.ref_D.data();
+    desc_.alpha = make_scalar<ElementC>(args.epilogue.alpha);
+    desc_.beta = make_scalar<ElementC>(args.epilogue.beta);
+    desc_.alpha_ptr = args.epilogue.alpha_ptr;
+    desc_.beta_ptr = args.epilogue.beta_ptr;
+    return Status::kSuccess;
+  }
+
+  Status run(hipStream_t stream = nullptr) {
+    if (!ready_) return Status::kErrorInternal;
+    return static_cast<Status>(cuasr_amd_srgemm(&desc_, stream));
+  }
+
+  Status operator()(hipStream_t stream = nullptr) { return run(stream); }
+
+  Status operator()(Arguments const &args, void *workspace = nullptr, hipStream_t stream = nullptr) {
+    Status s = initialize(args, workspace, stream);
+    return s == Status::kSuccess ? run(stream) : s;
+  }
+
+ private:
+  cuasr_amd_srgemm_desc desc_;
+  bool ready_;
+};
+
+}  // namespace device
+}  // namespace gemm
+}  // namespace cuasr

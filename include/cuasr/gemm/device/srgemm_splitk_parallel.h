@@ -1,0 +1,157 @@
+// cuasr::gemm::device::SrgemmSplitKParallel -- two-kernel parallel split-K:
+// partial products of `split_k_slices` K-slices go to a caller-provided
+// workspace, a second kernel folds them with the semiring's add and applies
+// the epilogue.  Mirrors include/cuasr/gemm/device/srgemm_splitk_parallel.h
+// :36-378 (and :424-607) of the reference: same template head, Arguments,
+// get_workspace_size = sizeof(accumulator) * M * N * slices, initialize(args,
+// workspace) returning kErrorWorkspaceNull for a null workspace, run(stream).
+#pragma once
+#include "srgemm.h"
+
+namespace cuasr {
+namespace reduction {
+namespace thread {
+/// Named by the reference's template head; carries no state here.
+template <typename AdditionOp, typename ElementAccumulator, typename Element, int Count = 1> struct SemiringReduce {
+  struct Params {};
+};
+}  // namespace thread
+}  // namespace reduction
+namespace epilogue {
+namespace thread {
+template <typename Element, int Count = 1, typename ElementOut = Element> struct Convert {
+  struct Params {};
+};
+}  // namespace thread
+}  // namespace epilogue
+
+namespace gemm {
+namespace device {
+
+template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, typename LayoutA_, typename ElementB_,
+          typename LayoutB_, typename ElementC_, typename LayoutC_, typename ElementAccumulator_ = ElementC_,
+          typename OperatorClass_ = arch::OpClassSimt, typename ArchTag_ = arch::Gfx950,
+          typename ThreadblockShape_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::ThreadblockShape,
+          typename WarpShape_ = typename DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_,
+                                                                     OperatorClass_, AdditionOp_, MultiplicationOp_,
+                                                                     ArchTag_>::WarpShape,
+          typename InstructionShape_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::InstructionShape,
+          typename EpilogueOutputOp_ = typename DefaultSemiRingConfiguration<
+              ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_, AdditionOp_, MultiplicationOp_,
+              ArchTag_>::EpilogueOutputOp,
+          typename ConvertScaledOp_ = epilogue::thread::Convert<ElementAccumulator_, 1, ElementAccumulator_>,
+          typename ReductionOp_ = reduction::thread::SemiringReduce<AdditionOp_, ElementAccumulator_, ElementAccumulator_, 1>,
+          typename ThreadblockSwizzle_ = threadblock::GemmSplitKHorizontalThreadblockSwizzle,
+          int Stages = DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_,
+                                                    AdditionOp_, MultiplicationOp_, ArchTag_>::kStages,
+          int kAlignmentA = 1, int kAlignmentB = 1>
+class SrgemmSplitKParallel {
+ public:
+  using ElementA = ElementA_;
+  using LayoutA = LayoutA_;
+  using ElementB = ElementB_;
+  using LayoutB = LayoutB_;
+  using ElementC = ElementC_;
+  using LayoutC = LayoutC_;
+  using ElementAccumulator = ElementAccumulator_;
+  using OperatorClass = OperatorClass_;
+  using ArchTag = ArchTag_;
+  using ThreadblockShape = ThreadblockShape_;
+  using WarpShape = WarpShape_;
+  using InstructionShape = InstructionShape_;
+  using EpilogueOutputOp = EpilogueOutputOp_;
+  using ConvertScaledOp = ConvertScaledOp_;
+  using ReductionOp = ReductionOp_;
+  using ThreadblockSwizzle = ThreadblockSwizzle_;
+  using AdditionOp = AdditionOp_;
+  using MultiplicationOp = MultiplicationOp_;
+  static int const kStages = Stages;
+
+  static_assert(std::is_same<ElementA, ElementC>::value && std::is_same<ElementB, ElementC>::value &&
+                    std::is_same<ElementAccumulator, ElementC>::value,
+                "A, B, C and the accumulator share one element type");
+
+  struct Arguments {
+    GemmCoord problem_size;
+    TensorRef<ElementA const, LayoutA> ref_A;
+    TensorRef<ElementB const, LayoutB> ref_B;
+    TensorRef<ElementC const, LayoutC> ref_C;
+    TensorRef<ElementC, LayoutC> ref_D;
+    typename EpilogueOutputOp::Params epilogue;
+    int split_k_slices;
+    typename ConvertScaledOp::Params convert;
+    typename ReductionOp::Params reduction;
+
+    Arguments() : problem_size(0, 0, 0), split_k_slices(1) {}
+    Arguments(GemmCoord problem_size_, TensorRef<ElementA const, LayoutA> ref_A_, TensorRef<ElementB const, LayoutB> ref_B_,
+              TensorRef<ElementC const, LayoutC> ref_C_, TensorRef<ElementC, LayoutC> ref_D_,
+              typename EpilogueOutputOp::Params epilogue_ = typename EpilogueOutputOp::Params(), int split_k_slices_ = 1,
+              typename ConvertScaledOp::Params convert_ = typename ConvertScaledOp::Params(),
+              typename ReductionOp::Params reduction_ = typename ReductionOp::Params())
+        : problem_size(problem_size_), ref_A(ref_A_), ref_B(ref_B_), ref_C(ref_C_), ref_D(ref_D_), epilogue(epilogue_),
+          split_k_slices(split_k_slices_), convert(convert_), reduction(reduction_) {}
+  };
+
+  SrgemmSplitKParallel() : workspace_(nullptr), ready_(false) {}
+
+  /// Stricter than the reference's stub (which always succeeds): the
+  /// descriptor is validated, slices must be >= 1.
+  static Status can_implement(Arguments const &args) {
+    if (args.split_k_slices < 1) return Status::kErrorInvalidProblem;
+    Arguments one = args;
+    one.split_k_slices = 1;
+    cuasr_amd_srgemm_desc d = detail::make_desc<SrgemmSplitKParallel>(one, detail::kernel_of<OperatorClass>::value);
+    return static_cast<Status>(cuasr_amd_srgemm_can_implement(&d));
+  }
+
+  static size_t get_workspace_size(Arguments const &args) {
+    cuasr_amd_srgemm_desc d = detail::make_desc<SrgemmSplitKParallel>(args, CUASR_AMD_KERNEL_AUTO);
+    return cuasr_amd_splitk_workspace_bytes(&d);
+  }
+
+  Status initialize(Arguments const &args, void *workspace) {
+    if (!workspace) return Status::kErrorWorkspaceNull;
+    Status s = can_implement(args);
+    if (s != Status::kSuccess) return s;
+    desc_ = detail::make_desc<SrgemmSplitKParallel>(args, detail::kernel_of<OperatorClass>::value);
+    workspace_ = workspace;
+    ready_ = true;
+    return Status::kSuccess;
+  }
+
+  Status update(Arguments const &args, void *workspace = nullptr) {
+    if (!workspace) return Status::kErrorWorkspaceNull;
+    if (!ready_) return Status::kErrorInternal;
+    desc_.A = args.ref_A.data();
+    desc_.B = args.ref_B.data();
+    desc_.C = args.ref_C.data();
+    desc_.D = args.ref_D.data();
+    workspace_ = workspace;
+    return Status::kSuccess;
+  }
+
+  Status run(hipStream_t stream = nullptr) {
+    if (!ready_) return Status::kErrorInternal;
+    return static_cast<Status>(cuasr_amd_srgemm_splitk(&desc_, workspace_, stream));
+  }
+
+  Status operator()(hipStream_t stream = nullptr) { return run(stream); }
+
+  Status operator()(Arguments const &args, void *workspace = nullptr, hipStream_t stream = nullptr) {
+    Status s = initialize(args, workspace);
+    return s == Status::kSuccess ? run(stream) : s;
+  }
+
+ private:
+  cuasr_amd_srgemm_desc desc_;
+  void *workspace_;
+  bool ready_;
+};
+
+}  // namespace device
+}  // namespace gemm
+}  // namespace cuasr

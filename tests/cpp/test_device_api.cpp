@@ -1,0 +1,260 @@
+// GPU test of the C++ operator API (cuasr::gemm::device::Srgemm and
+// SrgemmSplitKParallel) written the way the reference's own tests and examples
+// use it: the testbed sweep (test/device/testbed.h:268-361: m in {1,509},
+// n in {1,510}, k in {1,23}, integer-valued inputs in [-8,8], (0,0) forced to
+// 1, alpha = Mult::Identity, beta = Mult::Annihilator, bit-exact against the
+// host reference), example 00 (min-plus), example 01 (user-defined xor-and),
+// example 02 (split-K equals non-split), and the regress known-answer vector.
+// Prints one line per check; exit status is the number of failures.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include "cuasr/gemm/device/srgemm.h"
+#include "cuasr/gemm/device/srgemm_splitk_parallel.h"
+#include "cuasr/reference/srgemm/host_srgemm.h"
+
+using cuasr::Status;
+using cuasr::layout::ColumnMajor;
+using cuasr::layout::RowMajor;
+
+static int g_fail = 0, g_run = 0;
+#define HIP_OK(x)                                                                \
+  do {                                                                           \
+    hipError_t e_ = (x);                                                         \
+    if (e_ != hipSuccess) {                                                      \
+      std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+      std::exit(99);                                                             \
+    }                                                                            \
+  } while (0)
+
+static void report(bool ok, const char *what) {
+  ++g_run;
+  if (!ok) ++g_fail;
+  std::printf("%s %s\n", ok ? "PASS" : "FAIL", what);
+  std::fflush(stdout);
+}
+
+// splitmix64: the same generator the Python tests use
+static uint64_t mix(uint64_t z) {
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+template <typename T> static void fill_int(std::vector<T> &v, uint64_t seed, int lo, int hi) {
+  for (size_t i = 0; i < v.size(); ++i) v[i] = static_cast<T>(lo + int(mix(seed * 0x9E3779B97F4A7C15ull + i + 1) % uint64_t(hi - lo + 1)));
+}
+template <typename T> static void fill_unit(std::vector<T> &v, uint64_t seed, double lo, double hi) {
+  for (size_t i = 0; i < v.size(); ++i)
+    v[i] = static_cast<T>(lo + (hi - lo) * double(mix(seed * 0x9E3779B97F4A7C15ull + i + 1) >> 40) / 16777216.0);
+}
+
+template <typename T> struct DeviceBuf {
+  T *p = nullptr;
+  size_t n = 0;
+  explicit DeviceBuf(size_t count) : n(count) { HIP_OK(hipMalloc(reinterpret_cast<void **>(&p), (count ? count : 1) * sizeof(T))); }
+  DeviceBuf(std::vector<T> const &h) : DeviceBuf(h.size()) { upload(h); }
+  ~DeviceBuf() { (void)hipFree(p); }
+  void upload(std::vector<T> const &h) { HIP_OK(hipMemcpy(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice)); }
+  std::vector<T> download() const {
+    std::vector<T> h(n);
+    HIP_OK(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost));
+    return h;
+  }
+};
+
+template <typename L> static long long ld_of(int rows, int cols) { return std::is_same<L, ColumnMajor>::value ? rows : cols; }
+
+// one testbed case: device operator vs host reference, bit-exact
+template <typename Add, typename Mul, typename T, typename LA, typename LB, typename LC>
+static bool testbed_case(int m, int n, int k, T alpha, T beta) {
+  using Op = cuasr::gemm::device::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T>;
+  const long long lda = ld_of<LA>(m, k), ldb = ld_of<LB>(k, n), ldc = ld_of<LC>(m, n);
+  std::vector<T> A(size_t(m) * k), B(size_t(k) * n), C(size_t(m) * n), D(size_t(m) * n, T(0)), R(size_t(m) * n, T(0));
+  fill_int(A, 2019, -8, 8);
+  fill_int(B, 2018, -8, 8);
+  fill_int(C, 2017, -8, 8);
+  A[0] = B[0] = C[0] = T(1);  // as the reference testbed does (testbed.h:142-144)
+  DeviceBuf<T> dA(A), dB(B), dC(C), dD(D);
+  typename Op::Arguments args({m, n, k}, {dA.p, lda}, {dB.p, ldb}, {dC.p, ldc}, {dD.p, ldc}, {alpha, beta});
+  Op op;
+  if (Op::can_implement(args) != Status::kSuccess) return false;
+  if (op(args) != Status::kSuccess) return false;
+  HIP_OK(hipDeviceSynchronize());
+  cuasr::reference::host::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T, T> ref;
+  ref({m, n, k}, alpha, {A.data(), lda}, {B.data(), ldb}, beta, {C.data(), ldc}, {R.data(), ldc}, Add::Identity);
+  D = dD.download();
+  return std::memcmp(D.data(), R.data(), D.size() * sizeof(T)) == 0;
+}
+
+template <typename Add, typename Mul, typename T> static void testbed_sweep(const char *name) {
+  bool ok = true;
+  const int ms[2] = {1, 509}, ns[2] = {1, 510}, ks[2] = {1, 23};
+  for (int m : ms)
+    for (int n : ns)
+      for (int k : ks) {
+        const T alpha = Mul::Identity, beta = Mul::Annihilator;  // testbed.h:324-325
+        ok = ok && testbed_case<Add, Mul, T, ColumnMajor, ColumnMajor, ColumnMajor>(m, n, k, alpha, beta);
+        ok = ok && testbed_case<Add, Mul, T, RowMajor, ColumnMajor, RowMajor>(m, n, k, alpha, beta);
+        ok = ok && testbed_case<Add, Mul, T, ColumnMajor, RowMajor, RowMajor>(m, n, k, alpha, Mul::Identity);
+        ok = ok && testbed_case<Add, Mul, T, RowMajor, RowMajor, ColumnMajor>(m, n, k, alpha, Mul::Identity);
+      }
+  report(ok, name);
+}
+
+// ---- a user-defined functor, as in examples/01_userdefined_semiring: defined
+// by the user, made known to the library by specialising cuasr::op_tag
+namespace {
+template <typename T, int N = 1> struct my_xor {
+  static T constexpr Identity = static_cast<T>(false);
+  T operator()(T lhs, T const &rhs) const { lhs ^= rhs; return lhs; }
+};
+}  // namespace
+namespace cuasr {
+template <typename T, int N> struct op_tag<my_xor<T, N>> { static int const value = CUASR_AMD_OP_BIT_XOR; };
+}
+
+static void example_userdefined_xor_and() {
+  using Add = my_xor<int>;
+  using Mul = cuasr::binary_and<int>;
+  using Op = cuasr::gemm::device::Srgemm<Add, Mul, int, ColumnMajor, int, ColumnMajor, int, ColumnMajor, int>;
+  const int M = 256, N = 256, K = 256;
+  std::vector<int> A(M * K), B(K * N), C(M * N), R(M * N);
+  for (size_t i = 0; i < A.size(); ++i) A[i] = (mix(3090 * 77 + i) % 1000) < 25;  // Bernoulli(0.025), 0/1
+  for (size_t i = 0; i < B.size(); ++i) B[i] = (mix(3091 * 77 + i) % 1000) < 25;
+  for (size_t i = 0; i < C.size(); ++i) C[i] = (mix(3092 * 77 + i) % 1000) < 25;
+  for (int with_c = 0; with_c < 2; ++with_c) {
+    DeviceBuf<int> dA(A), dB(B), dC(C);
+    const int alpha = Mul::Identity, beta = with_c ? Mul::Identity : Mul::Annihilator;
+    typename Op::Arguments args({M, N, K}, {dA.p, M}, {dB.p, K}, {dC.p, M}, {dC.p, M}, {alpha, beta});  // D aliases C
+    Op op;
+    Status st = op(args, nullptr, nullptr);
+    HIP_OK(hipDeviceSynchronize());
+    cuasr::reference::host::Srgemm<Add, Mul, int, ColumnMajor, int, ColumnMajor, int, ColumnMajor, int, int> ref;
+    ref({M, N, K}, alpha, {A.data(), M}, {B.data(), K}, beta, {C.data(), M}, {R.data(), M}, Add::Identity);
+    std::vector<int> D = dC.download();
+    report(st == Status::kSuccess && D == R, with_c ? "example01 xor-and (user functor), D = C ^ A.B in place" : "example01 xor-and (user functor)");
+  }
+}
+
+static void example_minplus_and_known_answer() {
+  using Add = cuasr::minimum<float>;
+  using Mul = cuasr::plus<float>;
+  // the regress vector (test/regress/Srgemm_test.cu:15-62): column-major, D = min(C, A (x) B) in place
+  std::vector<float> A = {0.840187728f, 0.911647379f, 0.277774721f, 0.364784479f, 0.394382924f, 0.19755137f, 0.553969979f, 0.513400912f};
+  std::vector<float> B = {0.840187728f, 0.911647379f, 0.394382924f, 0.19755137f, 0.729605675f, 0.335222751f, 0.798440039f, 0.768229604f};
+  std::vector<float> C = {0.840187728f, 0.911647379f, 0.277774721f, 0.364784479f, 0.394382924f, 0.197551370f, 0.553969979f, 0.513400912f,
+                          0.729605675f, 0.335222751f, 0.477397054f, 0.952229738f, 0.798440039f, 0.768229604f, 0.628870904f, 0.916195095f};
+  std::vector<float> want = C;
+  want[11] = 0.848623633f;
+  using OpNN = cuasr::gemm::device::Srgemm<Add, Mul, float, ColumnMajor, float, ColumnMajor, float, ColumnMajor, float>;
+  DeviceBuf<float> dA(A), dB(B), dC(C);
+  OpNN::Arguments args({4, 4, 2}, {dA.p, 4}, {dB.p, 2}, {dC.p, 4}, {dC.p, 4}, {Mul::Identity, Mul::Identity});
+  OpNN op;
+  Status st = op(args);
+  HIP_OK(hipDeviceSynchronize());
+  report(st == Status::kSuccess && dC.download() == want, "regress known-answer 4x4x2 min-plus");
+
+  // example 00: A column-major, B row-major, C/D row-major, 512 cubed, uniform data
+  using OpNT = cuasr::gemm::device::Srgemm<Add, Mul, float, ColumnMajor, float, RowMajor, float, RowMajor, float>;
+  const int M = 512, N = 512, K = 512;
+  std::vector<float> a(M * K), b(K * N), c(M * N), r(M * N);
+  fill_unit(a, 1, 0.0, 1.0);
+  fill_unit(b, 2, 0.0, 1.0);
+  fill_unit(c, 3, 0.0, 1.0);
+  DeviceBuf<float> da(a), db(b), dc(c), dd(std::vector<float>(M * N, 0.f));
+  const float alpha = Mul::Identity;
+  bool ok = true;
+  for (float beta : {Mul::Annihilator, Mul::Identity}) {
+    OpNT::Arguments g({M, N, K}, {da.p, M}, {db.p, N}, {dc.p, N}, {dd.p, N}, {alpha, beta});
+    OpNT o;
+    ok = ok && o.initialize(g) == Status::kSuccess && o.run() == Status::kSuccess;
+    HIP_OK(hipDeviceSynchronize());
+    cuasr::reference::host::Srgemm<Add, Mul, float, ColumnMajor, float, RowMajor, float, RowMajor, float, float> ref;
+    ref({M, N, K}, alpha, {a.data(), M}, {b.data(), N}, beta, {c.data(), N}, {r.data(), N}, Add::Identity);
+    ok = ok && dd.download() == r;
+  }
+  report(ok, "example00 min-plus 512^3 (A col, B row, C row), beta = zero and one");
+
+  // update(): same operator object, new output pointer; alpha/beta from device memory
+  DeviceBuf<float> dd2(std::vector<float>(M * N, 0.f));
+  std::vector<float> ab = {Mul::Identity, Mul::Identity};
+  DeviceBuf<float> dab(ab);
+  OpNT o;
+  OpNT::Arguments g1({M, N, K}, {da.p, M}, {db.p, N}, {dc.p, N}, {dd.p, N}, {alpha, Mul::Identity});
+  bool ok2 = o.initialize(g1) == Status::kSuccess;
+  OpNT::Arguments g2({M, N, K}, {da.p, M}, {db.p, N}, {dc.p, N}, {dd2.p, N}, {dab.p, dab.p + 1});
+  ok2 = ok2 && o.update(g2) == Status::kSuccess && o() == Status::kSuccess;
+  HIP_OK(hipDeviceSynchronize());
+  report(ok2 && dd2.download() == r, "update() + alpha/beta by device pointer");
+}
+
+static void example_splitk() {
+  using Add = cuasr::minimum<float>;
+  using Mul = cuasr::plus<float>;
+  using SplitK = cuasr::gemm::device::SrgemmSplitKParallel<Add, Mul, float, RowMajor, float, ColumnMajor, float, RowMajor, float>;
+  using Plain = cuasr::gemm::device::Srgemm<Add, Mul, float, RowMajor, float, ColumnMajor, float, RowMajor, float>;
+  const int M = 128, N = 128, K = 4096;  // examples/02_splitk_srgemm/splitk_srgemm.cu:192-199
+  std::vector<float> a(size_t(M) * K), b(size_t(K) * N), c(M * N);
+  fill_unit(a, 11, 0.5, 1.5);
+  fill_unit(b, 12, 0.5, 1.5);
+  fill_unit(c, 13, 0.5, 1.5);
+  DeviceBuf<float> da(a), db(b), dc(c), d1(std::vector<float>(M * N, 0.f)), d2(std::vector<float>(M * N, 0.f));
+  for (int slices : {1, 3, 8, 16}) {
+    for (float beta : {Mul::Annihilator, Mul::Identity}) {
+      SplitK::Arguments args({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d1.p, N}, {Mul::Identity, beta}, slices);
+      const size_t bytes = SplitK::get_workspace_size(args);
+      DeviceBuf<uint8_t> ws(bytes);
+      SplitK op;
+      bool ok = bytes == sizeof(float) * size_t(M) * N * slices;
+      ok = ok && op.initialize(args, nullptr) == Status::kErrorWorkspaceNull;
+      ok = ok && op.initialize(args, ws.p) == Status::kSuccess && op() == Status::kSuccess;
+      Plain::Arguments pargs({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {Mul::Identity, beta});
+      Plain plain;
+      ok = ok && plain(pargs) == Status::kSuccess;
+      HIP_OK(hipDeviceSynchronize());
+      ok = ok && d1.download() == d2.download();  // the example's own self-check (:270-287)
+      char name[96];
+      std::snprintf(name, sizeof name, "example02 split-K == non-split, slices=%d beta=%s", slices, beta == Mul::Identity ? "one" : "zero");
+      report(ok, name);
+    }
+  }
+  // split_k_slices > 1 on the plain operator is an invalid problem (device/srgemm.h:198-200)
+  Plain::Arguments bad({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {Mul::Identity, Mul::Identity}, 4);
+  report(Plain::can_implement(bad) == Status::kErrorInvalidProblem && Plain().operator()(bad) == Status::kErrorInvalidProblem,
+         "split_k_slices > 1 rejected by Srgemm");
+}
+
+int main() {
+  int devices = 0;
+  if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
+    std::printf("no GPU\n");
+    return 77;
+  }
+  example_minplus_and_known_answer();
+  example_userdefined_xor_and();
+  example_splitk();
+  testbed_sweep<cuasr::plus<float>, cuasr::multiplies<float>, float>("testbed plus-multiplies f32");
+  testbed_sweep<cuasr::minimum<float>, cuasr::plus<float>, float>("testbed minimum-plus f32");
+  testbed_sweep<cuasr::maximum<float>, cuasr::plus<float>, float>("testbed maximum-plus f32");
+  testbed_sweep<cuasr::minimum<float>, cuasr::multiplies<float>, float>("testbed minimum-multiplies f32");
+  testbed_sweep<cuasr::maximum<float>, cuasr::multiplies<float>, float>("testbed maximum-multiplies f32");
+  testbed_sweep<cuasr::minimum<float>, cuasr::maximum<float>, float>("testbed minimum-maximum f32");
+  testbed_sweep<cuasr::maximum<float>, cuasr::minimum<float>, float>("testbed maximum-minimum f32");
+  testbed_sweep<cuasr::binary_or<float>, cuasr::binary_and<float>, float>("testbed or-and f32");
+  testbed_sweep<cuasr::plus<double>, cuasr::multiplies<double>, double>("testbed plus-multiplies f64");
+  testbed_sweep<cuasr::minimum<double>, cuasr::plus<double>, double>("testbed minimum-plus f64");
+  testbed_sweep<cuasr::maximum<double>, cuasr::plus<double>, double>("testbed maximum-plus f64");
+  testbed_sweep<cuasr::minimum<double>, cuasr::multiplies<double>, double>("testbed minimum-multiplies f64");
+  testbed_sweep<cuasr::maximum<double>, cuasr::multiplies<double>, double>("testbed maximum-multiplies f64");
+  testbed_sweep<cuasr::minimum<double>, cuasr::maximum<double>, double>("testbed minimum-maximum f64");
+  testbed_sweep<cuasr::maximum<double>, cuasr::minimum<double>, double>("testbed maximum-minimum f64");
+  testbed_sweep<cuasr::binary_or<double>, cuasr::binary_and<double>, double>("testbed or-and f64");
+  testbed_sweep<cuasr::inf::minimum<float>, cuasr::inf::plus<float>, float>("testbed inf::minimum-plus f32");
+  testbed_sweep<cuasr::inf::maximum<double>, cuasr::inf::plus_for_max<double>, double>("testbed inf::maximum-plus f64");
+  std::printf("%d checks, %d failed\n", g_run, g_fail);
+  return g_fail;
+}

@@ -1,0 +1,23 @@
+"""Runs the C++ operator-API test program (tests/cpp/test_device_api.cpp): the
+reference's testbed sweep, its three examples and its known-answer vector,
+through cuasr::gemm::device::Srgemm / SrgemmSplitKParallel."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+BIN = os.path.join(HERE, "cpp", "test_device_api")
+
+
+def test_cpp_operator_api(lib):
+    if not os.path.exists(BIN):
+        from cuasr_amd import build
+        build.build_cpp_tests()
+    r = subprocess.run([BIN], capture_output=True, text=True, timeout=600)
+    print(r.stdout[-4000:])
+    print(r.stderr[-2000:])
+    assert r.returncode == 0, r.stdout[-4000:]
+    assert "0 failed" in r.stdout
