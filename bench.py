@@ -32,6 +32,9 @@ def main():
     ap.add_argument("--size", type=int, default=4096)
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="also run one plain device copy of this many MiB (a known-size kernel "
+                         "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this library runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -85,6 +88,12 @@ def main():
     ops = 2.0 * n * n * n
     value = ops * args.steps / wall / 1e9
     achieved_tops = ops / (avg_kernel_ms * 1e-3) / 1e12
+
+    if args.copy_calibration:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     desc_kernel = args.kernel
     if args.kernel == "auto":
