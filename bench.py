@@ -27,8 +27,8 @@ SEMIRING_CEILING_TOPS = FP32_VECTOR_PEAK_TFLOPS * (2.0 / 1.5) / 2.0
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=24)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--size", type=int, default=4096)
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -14,7 +14,7 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libcuasr_amd.so")
+LIB_PATH = os.environ.get("CUASR_AMD_LIB") or os.path.join(_HERE, "lib", "libcuasr_amd.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "cuasr_amd.h")
 
 # enums of include/cuasr_amd.h
@@ -22,7 +22,7 @@ OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
        "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
 DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3}
 COLUMN_MAJOR, ROW_MAJOR = 0, 1
-KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3}
+KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3, "direct": 4}
 STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
                 "kErrorInvalidLayout", "kErrorInvalidProblem", "kErrorNotSupported",
                 "kErrorWorkspaceNull", "kErrorInternal", "kErrorArchMismatch",

@@ -11,6 +11,10 @@ launch_fn find_valu_f64(int, int);
 launch_fn find_valu_i32(int, int);
 launch_fn find_valu_u32(int, int);
 launch_fn find_mfma_f32(int, int);
+launch_fn find_direct_f32(int, int);
+launch_fn find_direct_i32(int, int);
+launch_fn find_direct_u32(int, int);
+bool direct_can_run(const Problem &);
 bool mfma_f32_can_run(const Problem &);
 
 launch_fn find_valu(int dtype, int add_op, int mult_op) {
@@ -19,6 +23,15 @@ launch_fn find_valu(int dtype, int add_op, int mult_op) {
     case CUASR_AMD_F64: return find_valu_f64(add_op, mult_op);
     case CUASR_AMD_I32: return find_valu_i32(add_op, mult_op);
     case CUASR_AMD_U32: return find_valu_u32(add_op, mult_op);
+    default: return nullptr;
+  }
+}
+
+launch_fn find_direct(int dtype, int add_op, int mult_op) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return find_direct_f32(add_op, mult_op);
+    case CUASR_AMD_I32: return find_direct_i32(add_op, mult_op);
+    case CUASR_AMD_U32: return find_direct_u32(add_op, mult_op);
     default: return nullptr;
   }
 }
@@ -48,6 +61,12 @@ static bool mfma_usable(const cuasr_amd_srgemm_desc *d) {
   return mfma_f32_can_run(canonical(d));
 }
 
+// the direct-to-LDS tiles need aligned, vector-sized operands as well
+static bool direct_usable(const cuasr_amd_srgemm_desc *d) {
+  if (!find_direct(d->dtype, d->add_op, d->mult_op)) return false;
+  return direct_can_run(canonical(d));
+}
+
 static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (!d) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_U32) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
@@ -60,7 +79,7 @@ static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (d->m < 0 || d->n < 0 || d->k < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->reserved != 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (splitk ? d->split_k_slices < 1 : d->split_k_slices != 1) return CUASR_AMD_ERROR_INVALID_PROBLEM;
-  if (d->kernel < CUASR_AMD_KERNEL_AUTO || d->kernel > CUASR_AMD_KERNEL_MFMA) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->kernel < CUASR_AMD_KERNEL_AUTO || d->kernel > CUASR_AMD_KERNEL_VALU_DIRECT) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   auto min_ld = [](int layout, int rows, int cols) { return (long long)(layout == CUASR_AMD_COLUMN_MAJOR ? rows : cols); };
   if (d->m > 0 && d->k > 0 && d->lda < min_ld(d->layout_a, d->m, d->k)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->n > 0 && d->k > 0 && d->ldb < min_ld(d->layout_b, d->k, d->n)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
@@ -77,6 +96,7 @@ static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (d->kernel == CUASR_AMD_KERNEL_VALU && !find_valu(d->dtype, d->add_op, d->mult_op))
     return CUASR_AMD_ERROR_NOT_SUPPORTED;
   if (d->kernel == CUASR_AMD_KERNEL_MFMA && !mfma_usable(d)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->kernel == CUASR_AMD_KERNEL_VALU_DIRECT && !direct_usable(d)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   return CUASR_AMD_SUCCESS;
 }
 
@@ -107,13 +127,14 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d) {
   return p;
 }
 
-enum Family { kNaive = 1, kValu = 2, kMfma = 3 };
+enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4 };
 
 static int pick_family(const cuasr_amd_srgemm_desc *d) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.
+  if (direct_usable(d)) return kDirect;
   if (find_valu(d->dtype, d->add_op, d->mult_op)) return kValu;
   if (mfma_usable(d)) return kMfma;
   return kNaive;
@@ -122,6 +143,7 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
 static launch_fn family_fn(int family, const cuasr_amd_srgemm_desc *d) {
   switch (family) {
     case kMfma: return find_mfma(d->dtype, d->add_op, d->mult_op);
+    case kDirect: return find_direct(d->dtype, d->add_op, d->mult_op);
     case kValu: return find_valu(d->dtype, d->add_op, d->mult_op);
     default: return find_naive(d->dtype);
   }
@@ -158,6 +180,7 @@ const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc) {
   if (validate(desc, true) != CUASR_AMD_SUCCESS) return nullptr;
   switch (pick_family(desc)) {
     case kMfma: return "mfma";
+    case kDirect: return "valu_direct";
     case kValu: return "valu";
     default: return "naive";
   }

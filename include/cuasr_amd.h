@@ -85,7 +85,9 @@ typedef enum cuasr_amd_kernel {
   CUASR_AMD_KERNEL_AUTO = 0,
   CUASR_AMD_KERNEL_NAIVE = 1, /* one thread per output element               */
   CUASR_AMD_KERNEL_VALU = 2,  /* LDS-staged, register-blocked vector-ALU tile */
-  CUASR_AMD_KERNEL_MFMA = 3   /* matrix-core assisted tile                    */
+  CUASR_AMD_KERNEL_MFMA = 3,  /* matrix-core assisted tile                    */
+  CUASR_AMD_KERNEL_VALU_DIRECT = 4 /* vector-ALU tile fed by direct-to-LDS loads;
+                                      needs 16-byte aligned, vector-sized operands */
 } cuasr_amd_kernel;
 
 /* One element of the problem's type; read through the member `dtype` names. */
@@ -161,7 +163,7 @@ int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
                             void *stream);
 
 /* Name of the kernel family AUTO would choose for this descriptor
- * ("naive", "valu", "mfma"), or NULL if the descriptor is invalid. */
+ * ("naive", "valu", "valu_direct", "mfma"), or NULL if the descriptor is invalid. */
 const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc);
 
 #ifdef __cplusplus

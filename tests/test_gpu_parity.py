@@ -17,6 +17,11 @@ def run(oracle, add, mult, dtype, m, n, k, la, lb, lc, kernel, beta_one, seed=1,
         A = inputs.integers(seed, m, k, -8, 8, npd, order_of(la))
         B = inputs.integers(seed + 1, k, n, -8, 8, npd, order_of(lb))
         C = inputs.integers(seed + 2, m, n, -8, 8, npd, order_of(lc))
+    elif {add, mult} & {"plus", "multiplies", "minimum", "maximum"}:
+        # arithmetic on integers: small values, so nothing overflows (signed overflow is undefined on the CPU side)
+        A = inputs.integers(seed, m, k, 0, 8, npd, order_of(la))
+        B = inputs.integers(seed + 1, k, n, 0, 8, npd, order_of(lb))
+        C = inputs.integers(seed + 2, m, n, 0, 8, npd, order_of(lc))
     else:
         A = inputs.words32(seed, m, k, order_of(la)).astype(npd)
         B = inputs.words32(seed + 1, k, n, order_of(lb)).astype(npd)
@@ -96,3 +101,25 @@ def test_minplus_uniform_1024(oracle, lib):
         cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, 0.0, np.inf, np.inf, 0.0, kernel=kernel)
         torch.cuda.synchronize()
         assert_same_bits(to_host(dD, "f32"), want, kernel)
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f32"), ("plus", "multiplies", "f32"),
+                                ("maximum", "minimum", "f32"), ("bit_xor", "bit_and", "u32"), ("minimum", "plus", "i32")])
+@pytest.mark.parametrize("shape", [(128, 128, 16), (128, 128, 64), (256, 384, 100), (64, 4, 8), (4, 4, 4),
+                                   (516, 260, 52), (132, 388, 1028), (1024, 1024, 1024)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"])
+def test_direct_tile(oracle, lib, sr, shape, layouts):
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    if shape[0] >= 1024 and layouts not in ("ccc", "rcr", "crr"):
+        pytest.skip("large shape: three layout combinations are enough")
+    for beta_one in (False, True):
+        if not beta_one and sr[2] == "i32" and sr[1] == "plus":
+            continue  # plus::Annihilator = INT_MAX: mult(beta, c) overflows on the CPU side (undefined)
+        run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "direct", beta_one)
+
+
+@pytest.mark.parametrize("slices", [1, 3, 8])
+def test_splitk_direct(oracle, lib, slices):
+    run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", "direct", False, splitk=slices)
+    run(oracle, "minimum", "plus", "f32", 100, 60, 332, "col", "col", "col", "direct", True, splitk=slices)
+    run(oracle, "bit_xor", "bit_and", "u32", 260, 132, 520, "col", "row", "row", "direct", True, splitk=slices)
