@@ -131,6 +131,8 @@ enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4 };
 
 static int pick_family(const cuasr_amd_srgemm_desc *d) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
+  // plus-times is the one semiring a matrix instruction computes as is
+  if (d->add_op == kPlus && d->mult_op == kMultiplies && mfma_usable(d)) return kMfma;
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.

@@ -30,17 +30,13 @@
 // (1,1,1,1)) and B likewise, so one ds_read_b128 per lane yields the operand
 // registers of four k-steps: lanes 0..31 fetch their row, lanes 32..63 the
 // ones entry (A), and the other way round for B.
-#include "semiring.h"
+#include "mfma_common.h"
 
 namespace cuasr_amd {
 
-typedef float v4f __attribute__((ext_vector_type(4)));
-typedef float v2f __attribute__((ext_vector_type(2)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
 namespace tropical {
 
-constexpr int BM = 128, BN = 128, BK = 16, KQ = BK / 4;
+using namespace mfma_panel;
 constexpr int ROWS = BM + 1;  // + the ones entry
 
 struct Smem {
@@ -53,63 +49,6 @@ template <bool IS_MIN> __device__ __forceinline__ float sel3(float acc, float x,
 }
 template <bool IS_MIN> __device__ __forceinline__ float sel2(float acc, float x) {
   return IS_MIN ? __builtin_fminf(acc, x) : __builtin_fmaxf(acc, x);
-}
-
-// Global -> registers for one 128 x 16 panel (8 floats per thread).
-//   k contiguous: two 16-byte loads, each 4 consecutive k of one row
-//   x contiguous: two 16-byte loads, each 4 consecutive rows at one k
-// Out-of-range rows / k are clamped to the last valid vector (never used).
-__device__ __forceinline__ void load_panel(v4f (&r)[2], const float *base, long long s_x, long long s_k, int x0,
-                                           int x_end, int k0, int k_end, bool x_contig) {
-  const int tid = threadIdx.x;
-  if (x_contig) {
-    const int xg = tid & 31, kq = (tid >> 5) & 3, half = tid >> 7;
-    const int xx = min(x0 + xg * 4, x_end - 4);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int kk = min(k0 + kq * 4 + half * 2 + j, k_end - 1);
-      r[j] = *reinterpret_cast<const v4f *>(base + (long long)kk * s_k + xx);
-    }
-  } else {
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int f = tid + 256 * q;
-      const int xx = min(x0 + (f >> 2), x_end - 1);
-      const int kk = min(k0 + (f & 3) * 4, k_end - 4);
-      r[q] = *reinterpret_cast<const v4f *>(base + (long long)xx * s_x + kk);
-    }
-  }
-}
-
-__device__ __forceinline__ void store_panel(const v4f (&r)[2], v4f (*dst)[ROWS], bool x_contig) {
-  const int tid = threadIdx.x;
-  if (x_contig) {
-    const int xg = tid & 31, kq = (tid >> 5) & 3, half = tid >> 7;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      v2f t = {r[0][e], r[1][e]};
-      *reinterpret_cast<v2f *>(reinterpret_cast<float *>(&dst[kq][xg * 4 + e]) + half * 2) = t;
-    }
-  } else {
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int f = tid + 256 * q;
-      dst[f & 3][f >> 2] = r[q];
-    }
-  }
-}
-
-__device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int &bm, int &bn) {
-  const int total = tiles_m * tiles_n;
-  // consecutive workgroup ids land on consecutive XCDs (8, one L2 each):
-  // give every XCD one contiguous run of the tile order
-  if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-  constexpr int GROUP = 8;
-  const int width = GROUP * tiles_n;
-  const int group = id / width, first = group * GROUP;
-  const int gsz = min(tiles_m - first, GROUP);
-  bm = first + (id % width) % gsz;
-  bn = (id % width) / gsz;
 }
 
 template <bool IS_MIN>
@@ -162,8 +101,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (ntiles > 0) {
     load_panel(ra, A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_xc);
     load_panel(rb, B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_xc);
-    store_panel(ra, sm.a[0], a_xc);
-    store_panel(rb, sm.b[0], b_xc);
+    store_panel<ROWS>(ra, sm.a[0], a_xc);
+    store_panel<ROWS>(rb, sm.b[0], b_xc);
   }
   __syncthreads();
 
@@ -240,8 +179,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       }
     }
     if (more) {
-      store_panel(ra, sm.a[buf ^ 1], a_xc);
-      store_panel(rb, sm.b[buf ^ 1], b_xc);
+      store_panel<ROWS>(ra, sm.a[buf ^ 1], a_xc);
+      store_panel<ROWS>(rb, sm.b[buf ^ 1], b_xc);
     }
     __syncthreads();
     buf ^= 1;
@@ -289,18 +228,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
-// the loads are 16-byte vectors: aligned bases, leading dimensions that are
-// multiples of 4 and extents of at least one vector along the contiguous
-// direction (so a clamped vector stays inside the matrix)
-static bool can_run(const Problem &p) {
-  auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-  const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
-  if (!al(p.A) || !al(p.B)) return false;
-  if (a_xc ? (p.m % 4 || p.sa_k % 4) : (p.sa_k != 1 || p.k % 4 || p.sa_m % 4)) return false;
-  if (b_xc ? (p.n % 4 || p.sb_k % 4) : (p.sb_k != 1 || p.k % 4 || p.sb_n % 4)) return false;
-  return true;
-}
-
 template <bool IS_MIN> static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   if (!can_run(p)) return hipErrorNotSupported;
@@ -313,12 +240,15 @@ template <bool IS_MIN> static hipError_t launch(const Problem &p, hipStream_t s)
 
 }  // namespace tropical
 
+launch_fn find_mfma_gemm_f32(int add_op, int mult_op);
+
 launch_fn find_mfma_f32(int add_op, int mult_op) {
+  if (launch_fn f = find_mfma_gemm_f32(add_op, mult_op)) return f;
   if (mult_op == kPlus && add_op == kMinimum) return tropical::launch<true>;
   if (mult_op == kPlus && add_op == kMaximum) return tropical::launch<false>;
   return nullptr;
 }
 
-bool mfma_f32_can_run(const Problem &p) { return tropical::can_run(p); }
+bool mfma_f32_can_run(const Problem &p) { return mfma_panel::can_run(p); }
 
 }  // namespace cuasr_amd

@@ -71,7 +71,10 @@ def test_can_implement(lib):
 
 def test_kernel_selection(lib):
     sel = lambda d: lib.cuasr_amd_selected_kernel(ctypes.byref(d))
-    assert sel(desc()) == b"valu"
+    assert sel(desc()) == b"valu_direct"          # min-plus f32, aligned: direct-to-LDS vector-ALU tile
+    assert sel(desc(m=63)) == b"valu"               # not vector-sized: staged tile
+    assert sel(desc(add="plus", mult="multiplies")) == b"mfma"
+    assert sel(desc(dtype="f64")) == b"valu"
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
     assert sel(desc(kernel="mfma")) == b"mfma"
 

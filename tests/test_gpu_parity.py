@@ -123,3 +123,18 @@ def test_splitk_direct(oracle, lib, slices):
     run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", "direct", False, splitk=slices)
     run(oracle, "minimum", "plus", "f32", 100, 60, 332, "col", "col", "col", "direct", True, splitk=slices)
     run(oracle, "bit_xor", "bit_and", "u32", 260, 132, 520, "col", "row", "row", "direct", True, splitk=slices)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 16), (256, 384, 100), (64, 4, 8), (516, 260, 52), (1024, 1024, 1024)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_plus_times_mfma_small_integers(oracle, lib, shape, layouts):
+    """Matrix-core plus-times on small integers: every partial sum is exact in fp32, so any summation
+    order gives the host reference's bits (the reference's own testbed relies on the same fact)."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (False, True):
+        run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", beta_one)
+
+
+def test_plus_times_mfma_splitk(oracle, lib):
+    run(oracle, "plus", "multiplies", "f32", 128, 128, 1000, "row", "col", "row", "mfma", True, splitk=8)
+    run(oracle, "plus", "multiplies", "f32", 100, 60, 332, "col", "col", "col", "mfma", True, splitk=3)
