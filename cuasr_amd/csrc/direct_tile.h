@@ -54,6 +54,13 @@ struct DirectTile {
 #else
   static constexpr int STAGES = (3 * (BM + BN) * BK * 4 * (1024 / THREADS) <= 160 * 1024) ? 3 : 2;
 #endif
+  // k-pairs between two of a wave's loads of the panel two tiles ahead
+#ifdef CUASR_AMD_DIRECT_SPREAD
+  static constexpr int SPREAD = CUASR_AMD_DIRECT_SPREAD;
+#else
+  static constexpr int SPREAD = (BK / 2 - 2) / (LA + LB - 1) > 0 ? (BK / 2 - 2) / (LA + LB - 1) : 1;
+#endif
+  static_assert((LA + LB - 1) * SPREAD < BK / 2, "all loads of a panel must be issued within one k-tile");
   struct Smem {
     T a[STAGES][BK * BM];
     T b[STAGES][BK * BN];
@@ -328,9 +335,11 @@ struct DirectTile {
       const int kc2 = tile_k(t + 2), stage2 = next + 1 == STAGES ? 0 : next + 1;  // tile t+2 and where it goes
       tile_body(std::make_integer_sequence<int, BK / 2>{}, acc, a, b, a_addr, b_addr, [&](auto kp, unsigned &aa, unsigned &ba) {
         constexpr int KP = decltype(kp)::value;
-        // three stages: tile t+2's traffic is spread, one load per k-pair, over the first k-pairs of tile t
-        if constexpr (STAGES == 3 && KP < LA + LB) {
-          if (kc2 > 0) fetch_piece(KP, stage2, kc2);
+        // three stages: tile t+2's traffic is spread over the k-pairs of tile t, one load every
+        // SPREAD k-pairs: a load's address registers are reloaded from scratch right before it, and
+        // the wait for that reload also waits for the previous load, so the loads are kept apart
+        if constexpr (STAGES == 3 && KP % SPREAD == 0 && KP / SPREAD < LA + LB) {
+          if (kc2 > 0) fetch_piece(KP / SPREAD, stage2, kc2);
         }
         if constexpr (KP == BK / 2 - 1) {
           __syncthreads();  // tile t+1 has landed (vmcnt waited first); nobody reads this stage any more

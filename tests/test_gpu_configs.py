@@ -153,16 +153,24 @@ def test_config5a_xor_and_u32_4096(oracle, lib):
 
 
 def test_config5b_plus_times_f32_4096(oracle, lib):
-    """plus-times f32 control semiring, N(0,1) inputs: |d - r| <= 1e-5 * sum_k |a||b|."""
+    """plus-times f32 control semiring, N(0,1) inputs, 4096^3.
+
+    Tolerance: 1e-5 relative.  The matrix-core kernel (the default) sums k in the instruction's
+    order, so it is held to the two forms of "relative" that are meaningful for a dot product
+    whose terms cancel: |d - r| <= 1e-5 * sum_k |a||b| for every element, and
+    ||d - r||_F <= 1e-5 * ||r||_F for the matrix.  (An element-wise bound against |r| itself is
+    not attainable for any change of summation order where the terms cancel to |r| ~ 1.)
+    The vector-ALU tile sums in the host reference's order and is bit-exact."""
     from cuasr_amd import inputs
     n = 4096
     A, B = inputs.normal(601, n, n), inputs.normal(602, n, n)
     C = np.zeros((n, n), dtype=np.float32, order="F")
     want = oracle.srgemm("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0)
+    assert_same_bits(_run("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0, 1.0, "f32", "direct"), want, "vector-ALU plus-times")
     got = _run("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0, 1.0, "f32")
-    rows = slice(0, 256)
-    bound = 1e-5 * (np.abs(A[rows, :]).astype(np.float64) @ np.abs(B).astype(np.float64))
-    assert np.all(np.abs(got[rows, :].astype(np.float64) - want[rows, :].astype(np.float64)) <= bound)
-    big = np.abs(want) >= 1.0
-    rel = np.abs(got[big].astype(np.float64) - want[big]) / np.abs(want[big])
-    assert rel.max() <= 1e-5, rel.max()   # tolerance: 1e-5 relative (fp32 plus-times)
+    diff = got.astype(np.float64) - want.astype(np.float64)
+    import torch
+    # sum_k |a||b| for every element (a bound, so torch's own fp32 product is accurate enough)
+    mag = (torch.from_numpy(np.abs(A)).cuda() @ torch.from_numpy(np.abs(B)).cuda()).cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(diff) <= 1e-5 * mag)
+    assert np.linalg.norm(diff) <= 1e-5 * np.linalg.norm(want.astype(np.float64))
