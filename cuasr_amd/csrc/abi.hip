@@ -136,8 +136,18 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.
-  if (direct_usable(d)) return kDirect;
-  if (find_valu(d->dtype, d->add_op, d->mult_op)) return kValu;
+  // The direct-to-LDS tile is 256 x 128 and the chip holds 512 of them at a time
+  // (two per compute unit).  It is the fastest family when its workgroups fill
+  // whole rounds of 512; a launch that leaves much of a round empty (small or
+  // awkwardly sized outputs, split-K of a small output) is better served by the
+  // smaller tiles of the staged family, whose many short workgroups balance.
+  const Problem c = canonical(d);
+  const long long direct_groups = (long long)((c.m + 255) / 256) * ((c.n + 127) / 128) * d->split_k_slices;
+  const long long rounds = (direct_groups + 511) / 512;
+  const bool fills = direct_groups * 8 >= rounds * 512 * 7;  // >= 7/8 of its rounds
+  const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;
+  if (direct_usable(d) && (fills || !have_valu)) return kDirect;
+  if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
   return kNaive;
 }

@@ -7,7 +7,7 @@
 namespace cuasr_amd {
 
 #define PAIR(ADD, MUL) \
-  if (add_op == ADD && mult_op == MUL) return launch_valu<int32_t, ADD, MUL, 8, 8, 16>;
+  if (add_op == ADD && mult_op == MUL) return launch_valu_sized<int32_t, ADD, MUL, 8, 8, 16, 4, 4>;
 
 launch_fn find_valu_i32(int add_op, int mult_op) {
   PAIR(kPlus, kMultiplies)

@@ -63,6 +63,25 @@ def test_other_semirings(oracle, lib, kernel, sr):
             run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, kernel, True)
 
 
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f64"), ("maximum", "minimum", "f64"),
+                                ("plus", "multiplies", "f32"), ("bit_xor", "bit_and", "u32"), ("minimum", "plus", "i32")])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_valu_full_size_tile(oracle, lib, sr, layouts):
+    """The staged family switches to its quarter-size tile below 256 workgroups; these grids are
+    large enough (>= 1024 tiles) for the full-size tile, ragged edges included."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for shape in [(4096, 4096, 40), (4090, 4100, 19)]:
+        run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", True)
+
+
+def test_valu_splitk_tile_sizes(oracle, lib):
+    """Split-K through both tile sizes of the staged family: 4 tiles x 8 slices (quarter-size tile)
+    and 4 tiles x 256 slices (full-size tile)."""
+    for slices in (8, 256):
+        run(oracle, "minimum", "plus", "f32", 256, 256, 4096, "row", "col", "row", "valu", True, splitk=slices)
+        run(oracle, "maximum", "plus", "f64", 256, 256, 2048, "col", "col", "col", "valu", False, splitk=slices)
+
+
 @pytest.mark.parametrize("kernel", ["naive", "valu"])
 @pytest.mark.parametrize("slices", [1, 3, 8])
 def test_splitk_minplus(oracle, lib, kernel, slices):
