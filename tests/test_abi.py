@@ -71,8 +71,12 @@ def test_can_implement(lib):
 
 def test_kernel_selection(lib):
     sel = lambda d: lib.cuasr_amd_selected_kernel(ctypes.byref(d))
-    assert sel(desc()) == b"valu_direct"          # min-plus f32, aligned: direct-to-LDS vector-ALU tile
-    assert sel(desc(m=63)) == b"valu"               # not vector-sized: staged tile
+    big = dict(m=4096, n=4096, k=4096)
+    assert sel(desc(**big)) == b"valu_direct"      # min-plus f32, aligned, 512 tiles of 256 x 128: direct-to-LDS tile
+    assert sel(desc(m=4095, n=4096, k=4096)) == b"valu"   # not vector-sized: staged tile
+    assert sel(desc()) == b"valu"                   # 64 x 64: one direct tile would leave the chip idle
+    assert sel(desc(m=3072, n=3072, k=64)) == b"valu"     # 288 direct tiles fill 56 % of a round of 512
+    assert sel(desc(m=8192, n=8192, k=64)) == b"valu_direct"
     assert sel(desc(add="plus", mult="multiplies")) == b"mfma"
     assert sel(desc(dtype="f64")) == b"valu"
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
