@@ -62,7 +62,7 @@ launch_fn find_naive(int dtype) {
 // additive identity and folds the slices in ascending order; when the source
 // is not needed it is replaced by the identity and the two-operand epilogue is
 // still applied (reduce_split_k.h:212-227).
-template <typename T, int V>
+template <typename T, int V, bool VOUT>
 __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
   const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
   const long long per_row = (p.n + V - 1) / V;
@@ -75,25 +75,45 @@ __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
   T acc[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) acc[v] = e.ident;
-  if (V > 1) {
-    typedef T vec_t __attribute__((ext_vector_type(V)));
-    for (int s = 0; s < p.slices; ++s) {
-      const vec_t w = *reinterpret_cast<const vec_t *>(ws + s * slice);
+  // eight slices' loads are issued before the first is folded, so a thread has
+  // eight memory requests in flight; the fold itself stays in ascending order
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  constexpr int U = 8;
+  int s = 0;
+  for (; s + U <= p.slices; s += U) {
+    vec_t w[U];
 #pragma unroll
-      for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[v]);
-    }
-  } else {
-    for (int s = 0; s < p.slices; ++s) acc[0] = apply_op<T>(p.add_op, acc[0], ws[s * slice]);
+    for (int u = 0; u < U; ++u) w[u] = *reinterpret_cast<const vec_t *>(ws + (s + u) * slice);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[u][v]);
+  }
+  for (; s < p.slices; ++s) {
+    const vec_t w = *reinterpret_cast<const vec_t *>(ws + s * slice);
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[v]);
   }
   const T *C = reinterpret_cast<const T *>(p.C);
   T *D = reinterpret_cast<T *>(p.D);
+  T out[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) {
-    if (j + v < p.n) {
-      const T src = e.source_needed ? C[(long long)i * p.ldc + j + v] : e.ident;
-      const T lhs = apply_op<T>(p.mult_op, e.alpha, acc[v]);
-      D[(long long)i * p.ldd + j + v] = apply_op<T>(p.add_op, lhs, apply_op<T>(p.mult_op, e.beta, src));
-    }
+    T src = e.ident;
+    if (e.source_needed && j + v < p.n) src = C[(long long)i * p.ldc + j + v];
+    const T lhs = apply_op<T>(p.mult_op, e.alpha, acc[v]);
+    out[v] = apply_op<T>(p.add_op, lhs, apply_op<T>(p.mult_op, e.beta, src));
+  }
+  T *dst = D + (long long)i * p.ldd + j;
+  if (V > 1 && VOUT) {  // one 16-byte store (the host checked alignment and that n is a multiple of V)
+    vec_t o;
+#pragma unroll
+    for (int v = 0; v < V; ++v) o[v] = out[v];
+    *reinterpret_cast<vec_t *>(dst) = o;
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      if (j + v < p.n) dst[v] = out[v];
   }
 }
 
@@ -101,12 +121,18 @@ template <typename T> static hipError_t launch_reduce(const Problem &p, hipStrea
   if (p.m == 0 || p.n == 0) return hipSuccess;
   constexpr int V = 16 / sizeof(T);
   const bool vec = (p.n % V == 0) && (reinterpret_cast<uintptr_t>(p.workspace) % 16 == 0);
-  if (vec) {
+  // small outputs: one element per thread gives V times as many workgroups to spread over the chip
+  const bool small = (long long)p.m * p.n < 256LL * 1024 * V;
+  if (vec && !small) {
     const long long work = (long long)p.m * (p.n / V);
-    hipLaunchKernelGGL((reduce_splitk_kernel<T, V>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
+    const dim3 grid((unsigned)((work + 255) / 256));
+    if (reinterpret_cast<uintptr_t>(p.D) % 16 == 0 && p.ldd % V == 0)
+      hipLaunchKernelGGL((reduce_splitk_kernel<T, V, true>), grid, dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL((reduce_splitk_kernel<T, V, false>), grid, dim3(256), 0, s, p);
   } else {
     const long long work = (long long)p.m * p.n;
-    hipLaunchKernelGGL((reduce_splitk_kernel<T, 1>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
+    hipLaunchKernelGGL((reduce_splitk_kernel<T, 1, false>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
   }
   return hipGetLastError();
 }

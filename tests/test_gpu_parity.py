@@ -82,6 +82,17 @@ def test_valu_splitk_tile_sizes(oracle, lib):
         run(oracle, "maximum", "plus", "f64", 256, 256, 2048, "col", "col", "col", "valu", False, splitk=slices)
 
 
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f64"), ("bit_xor", "bit_and", "u32"),
+                                ("plus", "multiplies", "f32")])
+def test_splitk_large_output(oracle, lib, sr):
+    """Outputs of a million elements and more take the reduction kernel's 16-byte path
+    (smaller ones its one-element-per-thread path); small integers keep plus-times exact."""
+    for layouts in ("rcr", "ccc"):
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        run(oracle, sr[0], sr[1], sr[2], 1024, 1280, 96, la, lb, lc, "auto", True, splitk=3)
+        run(oracle, sr[0], sr[1], sr[2], 1024, 1280, 96, la, lb, lc, "valu", False, splitk=5)
+
+
 @pytest.mark.parametrize("kernel", ["naive", "valu"])
 @pytest.mark.parametrize("slices", [1, 3, 8])
 def test_splitk_minplus(oracle, lib, kernel, slices):
