@@ -357,6 +357,15 @@ struct DirectTile {
       });
       stage = next;
     }
+    // The last k-pair has refilled the fragments for a k-pair that never runs.
+    // Those reads must have returned before the compiler reuses the registers
+    // for anything else (it cannot see that they are still being written).
+    if (nfull > 0) {
+      wait_half<0, 0>(a);
+      wait_half<0, 1>(a);
+      wait_half<0, 0>(b);
+      wait_half<0, 1>(b);
+    }
     const int buf = nfull % STAGES;
     if (rem > 0) {
       const T *pa = sm.a[buf], *pb = sm.b[buf];
