@@ -13,11 +13,13 @@
 //
 // Workgroup 256 threads = 4 waves (2 x 2), output tile 128 x 128, wave tile
 // 64 x 64 = 2 x 2 blocks of 32 x 32 (64 accumulator registers), k-tile 16.
-// LDS per stage: A and B as [k/4][128][4] (4 consecutive k of one row/column
-// per 16 bytes).  The instruction wants k = 2q from lanes 0..31 and k = 2q + 1
-// from lanes 32..63, so a lane reads the two floats (k, k + 2) at its row, the
-// upper half-wave one float further along: one ds_read2_b32 per block row per
-// k-quad feeds two matrix instructions.
+// LDS per stage: A and B k-major, [k][LD] floats.  The instruction wants k = 2q
+// from lanes 0..31 and k = 2q + 1 from lanes 32..63, each lane one float of
+// its row: 32 consecutive floats of LDS row 2q and 32 of row 2q + 1 per read,
+// which no bank layout can make collide.  LD = 160 puts consecutive rows 32
+// banks apart; rows of odd k-quads have bit 4 of the column flipped so that
+// the four k-quads a wave writes at once (k-contiguous operands: 16 rows x 4
+// quads per wave) spread over all banks instead of piling onto 16 of them.
 #include "mfma_common.h"
 
 namespace cuasr_amd {
@@ -25,9 +27,90 @@ namespace gemm_mfma {
 
 using namespace mfma_panel;
 
+constexpr int LD = 160;
+__device__ __forceinline__ int swz(int k) { return ((k >> 2) & 1) << 4; }
+
 struct Smem {
-  v4f a[2][KQ][BM];
-  v4f b[2][KQ][BN];
+  float a[2][BK][LD];
+  float b[2][BK][LD];
+};
+
+// One operand's share of a thread in the global -> LDS copy of a 128 x 16 panel:
+// two 16-byte vectors.
+//   x contiguous: vector j = 4 consecutive x at one k
+//   k contiguous: vector q = 4 consecutive k at one x
+// src[] points at the vectors of the FIRST k-tile (x clamped to the matrix) and
+// advances by `step` per tile; lds[] is the float index inside a stage where
+// element 0 of each vector goes (row stride LD per k for k-contiguous vectors).
+struct Mover {
+  const float *src[2];
+  long long step;
+  int lds[2];
+  bool x_contig;
+
+  __device__ __forceinline__ void init(const float *base, long long s_x, long long s_k, int x0, int x_end, int k0,
+                                       bool xc) {
+    const int tid = threadIdx.x;
+    x_contig = xc;
+    step = (long long)BK * s_k;
+    if (xc) {
+      const int xg = tid & 31, kq = (tid >> 5) & 3, half = tid >> 7;
+      const int xx = min(x0 + xg * 4, x_end - 4);
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int kk = kq * 4 + half * 2 + j;
+        src[j] = base + (long long)(k0 + kk) * s_k + xx;
+        lds[j] = kk * LD + ((xg * 4) ^ swz(kk));
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        // lanes 0..15: 16 consecutive x of k-quad 0, lanes 16..31: the same x of k-quad 1, ...
+        const int f = tid + 256 * q;
+        const int x = ((f >> 6) << 4) | (f & 15), kg = (f >> 4) & 3;
+        const int xx = min(x0 + x, x_end - 1);
+        src[q] = base + (long long)xx * s_x + k0 + kg * 4;
+        lds[q] = kg * 4 * LD + (x ^ swz(kg * 4));
+      }
+    }
+  }
+  // whole k-tile: nothing to clamp along k
+  __device__ __forceinline__ void load(v4f (&r)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) r[j] = *reinterpret_cast<const v4f *>(src[j]);
+  }
+  // ragged last k-tile with `kcount` (< BK) valid k: vectors that start past the end re-read the
+  // last valid one (never used); k-contiguous extents are multiples of 4, so no vector straddles the end
+  __device__ __forceinline__ void load_ragged(v4f (&r)[2], long long s_k, int kcount) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      long long back = 0;
+      if (x_contig) {
+        const int kk = ((tid >> 5) & 3) * 4 + (tid >> 7) * 2 + j;
+        back = (long long)max(kk - (kcount - 1), 0) * s_k;
+      } else {
+        const int kg = ((tid + 256 * j) >> 4) & 3;
+        back = max(kg * 4 - (kcount - 4), 0);
+      }
+      r[j] = *reinterpret_cast<const v4f *>(src[j] - back);
+    }
+  }
+  __device__ __forceinline__ void advance() {
+    src[0] += step;
+    src[1] += step;
+  }
+  __device__ __forceinline__ void store(const v4f (&r)[2], float *stage) const {
+    if (x_contig) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) *reinterpret_cast<v4f *>(stage + lds[j]) = r[j];
+    } else {
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) stage[lds[q] + e * LD] = r[q][e];
+    }
+  }
 };
 
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_kernel(Problem p) {
@@ -48,13 +131,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
 
-  // float index, inside one k-quad of a stage, of this lane's operand pair
-  int a_idx[2], b_idx[2];
+  // float index, inside a stage, of this lane's operand for k-pair 0 of an even / odd k-quad
+  int a_idx[2][2], b_idx[2][2];
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    a_idx[q] = (wm * 64 + q * 32 + (lane & 31)) * 4 + (lane >> 5);
-    b_idx[q] = (wn * 64 + q * 32 + (lane & 31)) * 4 + (lane >> 5);
-  }
+  for (int q = 0; q < 2; ++q)
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+      a_idx[q][o] = (lane >> 5) * LD + ((wm * 64 + q * 32 + (lane & 31)) ^ (o << 4));
+      b_idx[q][o] = (lane >> 5) * LD + ((wn * 64 + q * 32 + (lane & 31)) ^ (o << 4));
+    }
 
   v16f acc[2][2];
 #pragma unroll
@@ -65,12 +150,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int r = 0; r < 16; ++r) acc[bi][bj][r] = p.add_identity.f32;  // 0 for plus
 
   const int ntiles = (ke - kb + BK - 1) / BK;
+  Mover ma, mb;
+  ma.init(A, p.sa_m, p.sa_k, m0, p.m, kb, a_xc);
+  mb.init(B, p.sb_n, p.sb_k, n0, p.n, kb, b_xc);
   v4f ra[2], rb[2];
+  auto fetch = [&](int t) {  // k-tile t into registers
+    const int kcount = min(BK, ke - (kb + t * BK));
+    if (kcount == BK) {
+      ma.load(ra);
+      mb.load(rb);
+    } else {
+      ma.load_ragged(ra, p.sa_k, kcount);
+      mb.load_ragged(rb, p.sb_k, kcount);
+    }
+    ma.advance();
+    mb.advance();
+  };
   if (ntiles > 0) {
-    load_panel(ra, A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_xc);
-    load_panel(rb, B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_xc);
-    store_panel<BM>(ra, sm.a[0], a_xc);
-    store_panel<BN>(rb, sm.b[0], b_xc);
+    fetch(0);
+    ma.store(ra, &sm.a[0][0][0]);
+    mb.store(rb, &sm.b[0][0][0]);
   }
   __syncthreads();
 
@@ -78,26 +177,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   for (int t = 0; t < ntiles; ++t) {
     const int k0 = kb + t * BK;
     const bool more = t + 1 < ntiles;
-    if (more) {
-      load_panel(ra, A, p.sa_m, p.sa_k, m0, p.m, k0 + BK, ke, a_xc);
-      load_panel(rb, B, p.sb_n, p.sb_k, n0, p.n, k0 + BK, ke, b_xc);
-    }
+    if (more) fetch(t + 1);
     // k past the end of a ragged last tile: its products must not count.  The
-    // panels hold clamped (finite or not) data there, so the operands of those
+    // panels hold other (finite or not) data there, so the operands of those
     // k are replaced by zeros: 0 * 0 adds nothing.
     const int kcount = min(BK, ke - k0);
-    const float *pa = reinterpret_cast<const float *>(&sm.a[buf][0][0]);
-    const float *pb = reinterpret_cast<const float *>(&sm.b[buf][0][0]);
+    const float *pa = &sm.a[buf][0][0];
+    const float *pb = &sm.b[buf][0][0];
 #pragma unroll
     for (int kq = 0; kq < KQ; ++kq) {
       float av[2][2], bv[2][2];  // [block][k-pair of the quad]
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        av[q][0] = pa[kq * BM * 4 + a_idx[q]];
-        av[q][1] = pa[kq * BM * 4 + a_idx[q] + 2];
-        bv[q][0] = pb[kq * BN * 4 + b_idx[q]];
-        bv[q][1] = pb[kq * BN * 4 + b_idx[q] + 2];
-      }
+      for (int q = 0; q < 2; ++q)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          av[q][j] = pa[(kq * 4 + 2 * j) * LD + a_idx[q][kq & 1]];
+          bv[q][j] = pb[(kq * 4 + 2 * j) * LD + b_idx[q][kq & 1]];
+        }
       if (kcount < BK) {
 #pragma unroll
         for (int q = 0; q < 2; ++q)
@@ -117,8 +213,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[bi][j], bv[bj][j], acc[bi][bj], 0, 0, 0);
     }
     if (more) {
-      store_panel<BM>(ra, sm.a[buf ^ 1], a_xc);
-      store_panel<BN>(rb, sm.b[buf ^ 1], b_xc);
+      ma.store(ra, &sm.a[buf ^ 1][0][0]);
+      mb.store(rb, &sm.b[buf ^ 1][0][0]);
     }
     __syncthreads();
     buf ^= 1;

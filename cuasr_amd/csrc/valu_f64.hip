@@ -7,7 +7,7 @@
 namespace cuasr_amd {
 
 #define PAIR(ADD, MUL) \
-  if (add_op == ADD && mult_op == MUL) return launch_valu_sized<double, ADD, MUL, 8, 4, 8, 4, 4>;
+  if (add_op == ADD && mult_op == MUL) return launch_valu_sized<double, ADD, MUL, 8, 4, 16, 4, 4>;
 
 launch_fn find_valu_strict(int dtype, int add_op, int mult_op);
 
