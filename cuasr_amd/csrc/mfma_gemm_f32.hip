@@ -131,14 +131,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
 
-  // float index, inside a stage, of this lane's operand for k-pair 0 of an even / odd k-quad
+  // byte offset, inside the LDS panel array, of this lane's operand for k-pair 0 of an even / odd k-quad
   int a_idx[2][2], b_idx[2][2];
 #pragma unroll
   for (int q = 0; q < 2; ++q)
 #pragma unroll
     for (int o = 0; o < 2; ++o) {
-      a_idx[q][o] = (lane >> 5) * LD + ((wm * 64 + q * 32 + (lane & 31)) ^ (o << 4));
-      b_idx[q][o] = (lane >> 5) * LD + ((wn * 64 + q * 32 + (lane & 31)) ^ (o << 4));
+      a_idx[q][o] = 4 * ((lane >> 5) * LD + ((wm * 64 + q * 32 + (lane & 31)) ^ (o << 4)));
+      b_idx[q][o] = 4 * ((lane >> 5) * LD + ((wn * 64 + q * 32 + (lane & 31)) ^ (o << 4)));
     }
 
   v16f acc[2][2];
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   }
   __syncthreads();
 
-  int buf = 0;
+  int buf = 0, stage_step = BK * LD * 4;
   for (int t = 0; t < ntiles; ++t) {
     const int k0 = kb + t * BK;
     const bool more = t + 1 < ntiles;
@@ -182,8 +182,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // panels hold other (finite or not) data there, so the operands of those
     // k are replaced by zeros: 0 * 0 adds nothing.
     const int kcount = min(BK, ke - k0);
-    const float *pa = &sm.a[buf][0][0];
-    const float *pb = &sm.b[buf][0][0];
+    const char *pa = reinterpret_cast<const char *>(&sm.a[0][0][0]);
+    const char *pb = reinterpret_cast<const char *>(&sm.b[0][0][0]);
 #pragma unroll
     for (int kq = 0; kq < KQ; ++kq) {
       float av[2][2], bv[2][2];  // [block][k-pair of the quad]
@@ -191,8 +191,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int q = 0; q < 2; ++q)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          av[q][j] = pa[(kq * 4 + 2 * j) * LD + a_idx[q][kq & 1]];
-          bv[q][j] = pb[(kq * 4 + 2 * j) * LD + b_idx[q][kq & 1]];
+          av[q][j] = *reinterpret_cast<const float *>(pa + (kq * 4 + 2 * j) * LD * 4 + a_idx[q][kq & 1]);
+          bv[q][j] = *reinterpret_cast<const float *>(pb + (kq * 4 + 2 * j) * LD * 4 + b_idx[q][kq & 1]);
         }
       if (kcount < BK) {
 #pragma unroll
@@ -218,6 +218,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
     __syncthreads();
     buf ^= 1;
+    // the lane's read indices follow the stage: one add each instead of an address per read
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int o = 0; o < 2; ++o) {
+        a_idx[q][o] += stage_step;
+        b_idx[q][o] += stage_step;
+      }
+    stage_step = -stage_step;
   }
 
   // ---- epilogue.  Block (bi, bj), register r of lane l holds
