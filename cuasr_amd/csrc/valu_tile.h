@@ -134,36 +134,63 @@ struct ValuTile {
     }
   }
 
-  // Two k-steps at once, row by row: per accumulator two products and two
-  // adds, which the min/max semirings fold into one 3-input instruction.  The
-  // scheduling barrier after each row keeps the products of one row (2*TN
-  // registers) from piling up across rows.
-  static __device__ __forceinline__ void step2(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int kk,
-                                               int ty, int tx) {
+  // ---- whole k-tile, two k-steps at a time (per accumulator two products and
+  // two adds, which the min/max semirings fold into one 3-input instruction;
+  // the scheduling barrier after each row keeps the products of one row from
+  // piling up across rows) and software pipelined: the fragments of k-pair
+  // kp + 1 are read from LDS while k-pair kp is computed (two fragment sets in
+  // registers), so a wave does not stall on LDS latency at every k-pair.
+  // (integer element types keep the rolled loop: unrolled, their tiles take the
+  // compiler ten minutes each, and they are not the throughput cases)
+  static constexpr bool PIPELINED = T(0.5) != T(0);  // floating-point element type
+  struct Frag2 {
     T a[2][TM], b[2][TN];
+  };
+  static __device__ __forceinline__ void load_frag2(Frag2 &f, const T (*as)[LDA], const T (*bs)[LDB], int kk, int ty, int tx) {
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
       for (int h = 0; h < HM; ++h) {
         const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk + s][ty * VW + h * 16 * VW]);
 #pragma unroll
-        for (int e = 0; e < VW; ++e) a[s][h * VW + e] = t[e];
+        for (int e = 0; e < VW; ++e) f.a[s][h * VW + e] = t[e];
       }
 #pragma unroll
       for (int g = 0; g < GN; ++g) {
         const vec_t t = *reinterpret_cast<const vec_t *>(&bs[kk + s][tx * VW + g * 16 * VW]);
 #pragma unroll
-        for (int e = 0; e < VW; ++e) b[s][g * VW + e] = t[e];
+        for (int e = 0; e < VW; ++e) f.b[s][g * VW + e] = t[e];
       }
     }
+  }
+  static __device__ __forceinline__ void compute2(T (&acc)[TM][TN], const Frag2 &f) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const T t0 = Op<MUL>::apply(a[0][i], b[0][j]), t1 = Op<MUL>::apply(a[1][i], b[1][j]);
+        const T t0 = Op<MUL>::apply(f.a[0][i], f.b[0][j]), t1 = Op<MUL>::apply(f.a[1][i], f.b[1][j]);
         acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
       }
       __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  static __device__ __forceinline__ void whole_tile(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int ty, int tx) {
+    if constexpr (PIPELINED) {
+      Frag2 f[2];
+      load_frag2(f[0], as, bs, 0, ty, tx);
+#pragma unroll
+      for (int kp = 0; kp < BK / 2; ++kp) {
+        if (kp + 1 < BK / 2) load_frag2(f[(kp + 1) & 1], as, bs, 2 * kp + 2, ty, tx);
+        __builtin_amdgcn_sched_barrier(0);
+        compute2(acc, f[kp & 1]);
+      }
+    } else {
+#pragma unroll 1
+      for (int kp = 0; kp < BK / 2; ++kp) {
+        Frag2 f;
+        load_frag2(f, as, bs, 2 * kp, ty, tx);
+        compute2(acc, f);
+      }
     }
   }
 
@@ -222,8 +249,7 @@ struct ValuTile {
       }
       const int kcount = min(BK, ke - k0);
       if (kcount == BK) {
-#pragma unroll 1
-        for (int kk = 0; kk < BK; kk += 2) step2(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
+        whole_tile(acc, sm.a[buf], sm.b[buf], ty, tx);
       } else {
 #pragma unroll 1
         for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
