@@ -361,20 +361,25 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
   return hipGetLastError();
 }
 
-// The chip holds 1024 full-size workgroups at a time (four per compute unit).
-// A launch with fewer leaves vector units idle or with a single wave (split-K
-// of a small output, matrices below about 3000 x 3000): such problems run on a
-// quarter-size tile -- four times as many, shorter workgroups, which balance
-// better, at about 7 % less throughput when both sizes fill the chip.
-#ifndef CUASR_AMD_SMALL_TILE_BELOW
-#define CUASR_AMD_SMALL_TILE_BELOW 1024
+// The chip holds 1024 full-size workgroups at a time (four per compute unit),
+// and a launch runs in rounds of that many.  The full-size tile is a few per
+// cent faster than the quarter-size one when its workgroups fill whole rounds
+// (4096^2: exactly one), and much slower when a round is mostly empty (fewer
+// than 1024 workgroups: split-K of a small output, matrices below ~3000^2) or
+// the last round is (5120^2: 1.56 rounds).  The quarter-size tile -- four times
+// as many, shorter workgroups -- balances in all those cases, so the full-size
+// one is used only when at least 95 % of its rounds are filled.
+#ifndef CUASR_AMD_FULL_TILE_FILL_PERCENT
+#define CUASR_AMD_FULL_TILE_FILL_PERCENT 95
 #endif
 
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, int TM_SMALL, int TN_SMALL>
 static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1);
-  if (groups < (long long)(CUASR_AMD_SMALL_TILE_BELOW)) return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK>(p, s);
+  const long long rounds = (groups + 1023) / 1024;
+  if (groups * 100 < rounds * 1024 * (long long)(CUASR_AMD_FULL_TILE_FILL_PERCENT))
+    return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK>(p, s);
   return launch_valu<T, ADD, MUL, TM, TN, BK>(p, s);
 }
 

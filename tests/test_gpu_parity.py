@@ -67,10 +67,10 @@ def test_other_semirings(oracle, lib, kernel, sr):
                                 ("plus", "multiplies", "f32"), ("bit_xor", "bit_and", "u32"), ("minimum", "plus", "i32")])
 @pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
 def test_valu_full_size_tile(oracle, lib, sr, layouts):
-    """The staged family switches to its quarter-size tile below 256 workgroups; these grids are
-    large enough (>= 1024 tiles) for the full-size tile, ragged edges included."""
+    """The staged family uses its quarter-size tile unless the full-size one fills its rounds; these grids are
+    whole rounds of 1024 workgroups (>= 95 % filled) for the full-size tile, ragged edges included."""
     la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
-    for shape in [(4096, 4096, 40), (4090, 4100, 19)]:
+    for shape in [(4096, 4096, 40), (4090, 4000, 19)]:
         run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", True)
 
 
