@@ -79,6 +79,52 @@ struct ValuTile {
     }
   }
 
+  // ---- the same ownership with the addressing done once (VEC only): a thread
+  // keeps one pointer per 16-byte vector, at the vector's place in the first
+  // k-tile with the panel index clamped to the matrix, and moves it one k-tile
+  // along per iteration -- two integer instructions per vector and tile instead
+  // of the index arithmetic of load_panel.  Only a ragged last k-tile needs a
+  // second look at k: vectors past its end re-read its last valid vector.
+  template <int ROWS, int ELEMS> struct Mover {
+    static constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
+    const T *src[VECS];
+    long long step;
+    __device__ __forceinline__ void init(const T *base, long long s_x, long long s_k, int x0, int x_end, int k0,
+                                         bool x_contig) {
+      const int tid = threadIdx.x;
+      step = (long long)BK * s_k;
+#pragma unroll
+      for (int p = 0; p < VECS; ++p) {
+        const int v = tid + 256 * p;
+        const int xx = min(x0 + (x_contig ? (v % XV) * VW : v / KV), x_end - (x_contig ? VW : 1));
+        const int kk = k0 + (x_contig ? v / XV : (v % KV) * VW);
+        src[p] = base + (long long)xx * s_x + (long long)kk * s_k;
+      }
+    }
+    __device__ __forceinline__ void load(T (&r)[ELEMS]) {
+#pragma unroll
+      for (int p = 0; p < VECS; ++p) {
+        const vec_t t = *reinterpret_cast<const vec_t *>(src[p]);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) r[p * VW + e] = t[e];
+        src[p] += step;
+      }
+    }
+    __device__ __forceinline__ void load_ragged(T (&r)[ELEMS], long long s_k, int kcount, bool x_contig) {
+      const int tid = threadIdx.x;
+#pragma unroll
+      for (int p = 0; p < VECS; ++p) {
+        const int v = tid + 256 * p;
+        const int kl = x_contig ? v / XV : (v % KV) * VW;         // the vector's first k inside the tile
+        const int back = max(kl - (kcount - (x_contig ? 1 : VW)), 0);  // steps of k past the last valid vector
+        const vec_t t = *reinterpret_cast<const vec_t *>(src[p] - (long long)back * s_k);
+#pragma unroll
+        for (int e = 0; e < VW; ++e) r[p * VW + e] = t[e];
+        src[p] += step;
+      }
+    }
+  };
+
   // ---- registers -> LDS ([kk][x], k-major), same ownership as load_panel
   template <int ROWS, int LD, int ELEMS>
   static __device__ __forceinline__ void store_panel(const T (&r)[ELEMS], T (*dst)[LD], bool x_contig) {
@@ -232,9 +278,30 @@ struct ValuTile {
 
     const int ntiles = (ke - kb + BK - 1) / BK;
     T ra[A_ELEMS], rb[B_ELEMS];
+    Mover<BM, A_ELEMS> ma;
+    Mover<BN, B_ELEMS> mb;
+    if constexpr (VEC) {
+      ma.init(A, p.sa_m, p.sa_k, m0, p.m, kb, a_xc);
+      mb.init(B, p.sb_n, p.sb_k, n0, p.n, kb, b_xc);
+    }
+    // k-tile starting at k0 into registers
+    auto fetch = [&](int k0) {
+      if constexpr (VEC) {
+        const int kcount = ke - k0;
+        if (kcount >= BK) {
+          ma.load(ra);
+          mb.load(rb);
+        } else {
+          ma.load_ragged(ra, p.sa_k, kcount, a_xc);
+          mb.load_ragged(rb, p.sb_k, kcount, b_xc);
+        }
+      } else {
+        load_panel<BM, A_ELEMS>(ra, A, p.sa_m, p.sa_k, m0, p.m, k0, ke, a_xc);
+        load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, k0, ke, b_xc);
+      }
+    };
     if (ntiles > 0) {
-      load_panel<BM, A_ELEMS>(ra, A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_xc);
-      load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_xc);
+      fetch(kb);
       store_panel<BM, LDA, A_ELEMS>(ra, sm.a[0], a_xc);
       store_panel<BN, LDB, B_ELEMS>(rb, sm.b[0], b_xc);
     }
@@ -243,10 +310,7 @@ struct ValuTile {
     for (int t = 0; t < ntiles; ++t) {
       const int k0 = kb + t * BK;
       const bool more = t + 1 < ntiles;
-      if (more) {
-        load_panel<BM, A_ELEMS>(ra, A, p.sa_m, p.sa_k, m0, p.m, k0 + BK, ke, a_xc);
-        load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, k0 + BK, ke, b_xc);
-      }
+      if (more) fetch(k0 + BK);
       const int kcount = min(BK, ke - k0);
       if (kcount == BK) {
         whole_tile(acc, sm.a[buf], sm.b[buf], ty, tx);
