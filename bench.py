@@ -15,6 +15,7 @@ Other workloads (same JSON shape; one step = one SRGEMM on fixed inputs):
     splitk                    fp32 min-plus, M=N=256, K=65536, --slices S (two kernels per step)
     xorand_u32                GF(2) product on bit-packed uint32 words, 4096^3
     plustimes_f32             fp32 plus-times on the matrix cores, 4096^3, N(0,1)
+    plustimes_f64             fp64 plus-times on the matrix cores, 4096^3, N(0,1)
 """
 import argparse
 import json
@@ -27,7 +28,7 @@ sys.path.insert(0, ROOT)
 
 # MI355X published peaks
 FP32_VECTOR_PEAK = 157.3   # TFLOP/s, FMA counted as 2 flops (also the fp32 matrix-core peak)
-FP64_VECTOR_PEAK = 78.6
+FP64_VECTOR_PEAK = 78.6    # also the fp64 matrix-core peak
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
@@ -144,6 +145,23 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
                     workload=f"plus-times SRGEMM fp32 on the matrix cores, M=N=K={n}, column-major, N(0,1), C = 0",
                     bound="mfma", peak=FP32_VECTOR_PEAK, instr_per_term=None)
 
+    if w == "plustimes_f64":
+        n = args.size or 4096
+        A = inputs.normal(611, n, n).astype(np.float64, order="F")
+        B = inputs.normal(612, n, n).astype(np.float64, order="F")
+        C = np.zeros((n, n), dtype=np.float64, order="F")
+        dA, dB, dC = col_major(A), col_major(B), col_major(C)
+        dD = torch.empty(n, n, dtype=torch.float64, device=dev).t()
+
+        def step(i):
+            cuasr_amd.srgemm("plus", "multiplies", dA, dB, dC, dD, 1.0, 0.0, 0.0, 1.0, dtype="f64", kernel=args.kernel)
+
+        desc = cuasr_amd.make_desc("plus", "multiplies", "f64", dA, dB, dC, dD, 1.0, 0.0, 0.0, 1.0)
+        return dict(step=step, m=n, n=n, k=n, dtype="f64", desc=desc, host=("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0),
+                    metric=f"fp64 plus-times SRGEMM GFLOP/s at {n}^3 (2 flops/term)",
+                    workload=f"plus-times SRGEMM fp64 on the matrix cores, M=N=K={n}, column-major, N(0,1), C = 0",
+                    bound="mfma", peak=FP64_VECTOR_PEAK, instr_per_term=None)
+
     raise SystemExit(f"bench.py: unknown workload {w!r}")
 
 
@@ -153,7 +171,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="apsp",
-                    choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32"])
+                    choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64"])
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")
     ap.add_argument("--kernel", default="auto")

@@ -11,11 +11,13 @@ launch_fn find_valu_f64(int, int);
 launch_fn find_valu_i32(int, int);
 launch_fn find_valu_u32(int, int);
 launch_fn find_mfma_f32(int, int);
+launch_fn find_mfma_f64(int, int);
 launch_fn find_direct_f32(int, int);
 launch_fn find_direct_i32(int, int);
 launch_fn find_direct_u32(int, int);
 bool direct_can_run(const Problem &);
 bool mfma_f32_can_run(const Problem &);
+bool mfma_f64_can_run(const Problem &);
 
 launch_fn find_valu(int dtype, int add_op, int mult_op) {
   switch (dtype) {
@@ -38,6 +40,7 @@ launch_fn find_direct(int dtype, int add_op, int mult_op) {
 
 launch_fn find_mfma(int dtype, int add_op, int mult_op) {
   if (dtype == CUASR_AMD_F32) return find_mfma_f32(add_op, mult_op);
+  if (dtype == CUASR_AMD_F64) return find_mfma_f64(add_op, mult_op);
   return nullptr;
 }
 
@@ -58,7 +61,7 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d);
 // the matrix-core tiles use 16-byte loads and so need aligned, vector-sized operands
 static bool mfma_usable(const cuasr_amd_srgemm_desc *d) {
   if (!find_mfma(d->dtype, d->add_op, d->mult_op)) return false;
-  return mfma_f32_can_run(canonical(d));
+  return d->dtype == CUASR_AMD_F64 ? mfma_f64_can_run(canonical(d)) : mfma_f32_can_run(canonical(d));
 }
 
 // the direct-to-LDS tiles need aligned, vector-sized operands as well

@@ -168,3 +168,44 @@ def test_plus_times_mfma_small_integers(oracle, lib, shape, layouts):
 def test_plus_times_mfma_splitk(oracle, lib):
     run(oracle, "plus", "multiplies", "f32", 128, 128, 1000, "row", "col", "row", "mfma", True, splitk=8)
     run(oracle, "plus", "multiplies", "f32", 100, 60, 332, "col", "col", "col", "mfma", True, splitk=3)
+
+
+@pytest.mark.parametrize("shape", [(128, 128, 16), (256, 384, 100), (64, 4, 8), (516, 260, 50), (130, 66, 6), (1024, 1024, 1024)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_plus_times_mfma_f64_small_integers(oracle, lib, shape, layouts):
+    """fp64 matrix-core plus-times on small integers: every partial sum is exact, so any summation
+    order gives the host reference's bits."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (False, True):
+        run(oracle, "plus", "multiplies", "f64", *shape, la, lb, lc, "mfma", beta_one)
+
+
+def test_plus_times_mfma_f64_splitk(oracle, lib):
+    run(oracle, "plus", "multiplies", "f64", 128, 128, 1000, "row", "col", "row", "mfma", True, splitk=8)
+    run(oracle, "plus", "multiplies", "f64", 100, 60, 332, "col", "col", "col", "mfma", True, splitk=3)
+
+
+def test_plus_times_f64_tolerance(oracle, lib):
+    """fp64 plus-times on N(0,1) data, default kernel (matrix cores): within 1e-12 relative of the host
+    reference -- per element against sum_k |a||b| and in the Frobenius norm; the vector-ALU tile bit-exact."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    m, n, k = 512, 384, 2048
+    A = inputs.normal(701, m, k).astype(np.float64) + 1e-9 * inputs.normal(703, m, k).astype(np.float64)
+    B = inputs.normal(702, k, n).astype(np.float64) + 1e-9 * inputs.normal(704, k, n).astype(np.float64)
+    A, B = np.asfortranarray(A), np.asfortranarray(B)
+    C = np.zeros((m, n), dtype=np.float64, order="F")
+    want = oracle.srgemm("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0)
+    for kernel, exact in (("auto", False), ("valu", True)):
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm("plus", "multiplies", to_device(A), to_device(B), to_device(C), dD, 1.0, 0.0, 0.0, 1.0,
+                         dtype="f64", kernel=kernel)
+        torch.cuda.synchronize()
+        got = to_host(dD, "f64")
+        if exact:
+            assert_same_bits(got, want, "vector-ALU fp64 plus-times")
+        else:
+            diff = np.abs(got - want)
+            assert np.all(diff <= 1e-12 * (np.abs(A) @ np.abs(B)))          # tolerance 1e-12 relative
+            assert np.linalg.norm(diff) <= 1e-12 * np.linalg.norm(want)
