@@ -437,13 +437,13 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
 #define CUASR_AMD_FULL_TILE_FILL_PERCENT 95
 #endif
 
-template <typename T, int ADD, int MUL, int TM, int TN, int BK, int TM_SMALL, int TN_SMALL>
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, int TM_SMALL, int TN_SMALL, int BK_SMALL = BK>
 static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1);
   const long long rounds = (groups + 1023) / 1024;
   if (groups * 100 < rounds * 1024 * (long long)(CUASR_AMD_FULL_TILE_FILL_PERCENT))
-    return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK>(p, s);
+    return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK_SMALL>(p, s);
   return launch_valu<T, ADD, MUL, TM, TN, BK>(p, s);
 }
 
