@@ -139,13 +139,14 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.
-  // The direct-to-LDS tile is 256 x 128 and the chip holds 512 of them at a time
-  // (two per compute unit).  It is the fastest family when its workgroups fill
+  // The direct-to-LDS tile is 256 x 128 (128 x 128 when both operands are k-contiguous)
+  // and the chip holds 512 of them at a time (two per compute unit).  It is the fastest family when its workgroups fill
   // whole rounds of 512; a launch that leaves much of a round empty (small or
   // awkwardly sized outputs, split-K of a small output) is better served by the
   // smaller tiles of the staged family, whose many short workgroups balance.
   const Problem c = canonical(d);
-  const long long direct_groups = (long long)((c.m + 255) / 256) * ((c.n + 127) / 128) * d->split_k_slices;
+  const int tile_m = (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
+  const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + 127) / 128) * d->split_k_slices;
   const long long rounds = (direct_groups + 511) / 512;
   const bool fills = direct_groups * 8 >= rounds * 512 * 7;  // >= 7/8 of its rounds
   const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;

@@ -35,13 +35,16 @@
 
 namespace cuasr_amd {
 
-template <typename T, int ADD, int MUL, bool A_KC, bool B_KC, int TY, int TX>
+// RELAXED = false: 4 waves per SIMD (128 registers), one fragment set refilled in place (see kpair).
+// RELAXED = true:  2 waves per SIMD (256 registers), two fragment sets, two LDS stages of a deeper
+//                  k-tile: half the barriers, no register spills, no counted waits inside a k-pair.
+template <typename T, int ADD, int MUL, bool A_KC, bool B_KC, int TY, int TX, int BK_ = 16, bool RELAXED = false>
 struct DirectTile {
   static_assert(sizeof(T) == 4, "4-byte element types only");
-  static constexpr int BM = 8 * TY, BN = 8 * TX, BK = 16, THREADS = TY * TX, WAVES = THREADS / 64;
+  static constexpr int BM = 8 * TY, BN = 8 * TX, BK = BK_, THREADS = TY * TX, WAVES = THREADS / 64;
   // 1 KiB wave-loads per k-tile each wave issues for the A and the B panel
-  static constexpr int LA = BM / 16 / WAVES, LB = BN / 16 / WAVES;
-  static_assert(LA >= 1 && LB >= 1 && LA * WAVES * 16 == BM && LB * WAVES * 16 == BN, "panel must split evenly over the waves");
+  static constexpr int LA = BM * BK / 256 / WAVES, LB = BN * BK / 256 / WAVES;
+  static_assert(LA >= 1 && LB >= 1 && LA * WAVES * 256 == BM * BK && LB * WAVES * 256 == BN * BK, "panel must split evenly over the waves");
   typedef T vec4 __attribute__((ext_vector_type(4)));
   typedef T vec2 __attribute__((ext_vector_type(2)));
 
@@ -52,7 +55,7 @@ struct DirectTile {
 #ifdef CUASR_AMD_DIRECT_STAGES
   static constexpr int STAGES = CUASR_AMD_DIRECT_STAGES;
 #else
-  static constexpr int STAGES = (3 * (BM + BN) * BK * 4 * (1024 / THREADS) <= 160 * 1024) ? 3 : 2;
+  static constexpr int STAGES = RELAXED ? 2 : (3 * (BM + BN) * BK * 4 * (1024 / THREADS) <= 160 * 1024) ? 3 : 2;
 #endif
   // k-pairs between two of a wave's loads of the panel two tiles ahead
 #ifdef CUASR_AMD_DIRECT_SPREAD
@@ -60,7 +63,7 @@ struct DirectTile {
 #else
   static constexpr int SPREAD = (BK / 2 - 2) / (LA + LB - 1) > 0 ? (BK / 2 - 2) / (LA + LB - 1) : 1;
 #endif
-  static_assert((LA + LB - 1) * SPREAD < BK / 2, "all loads of a panel must be issued within one k-tile");
+  static_assert(RELAXED || (LA + LB - 1) * SPREAD < BK / 2, "all loads of a panel must be issued within one k-tile");
   struct Smem {
     T a[STAGES][BK * BM];
     T b[STAGES][BK * BN];
@@ -243,6 +246,45 @@ struct DirectTile {
     (kpair<KP>(acc, a, b, a_addr, b_addr, hook), ...);
   }
 
+  // ---- RELAXED main loop: fragment set KP & 1 is computed on while set (KP + 1) & 1 is being read.
+  template <int KP> static __device__ __forceinline__ void issue_pair(FragA &a, FragB &b, unsigned a_addr, unsigned b_addr) {
+    refill_half<TY, KP, 0>(a, a_addr);
+    refill_half<TY, KP, 1>(a, a_addr);
+    refill_half<TX, KP, 0>(b, b_addr);
+    refill_half<TX, KP, 1>(b, b_addr);
+  }
+  template <int N> static __device__ __forceinline__ void wait_pair(FragA &a, FragB &b) {
+    wait_half<N, 0>(a);
+    wait_half<N, 1>(a);
+    wait_half<N, 0>(b);
+    wait_half<N, 1>(b);
+  }
+  template <int KP> static __device__ __forceinline__ void relaxed_kpair(T (&acc)[8][8], FragA (&a)[2], FragB (&b)[2], unsigned a_addr, unsigned b_addr) {
+    constexpr int CUR = KP & 1, NXT = CUR ^ 1;
+    // (the counter has 4 bits: with 16 reads per k-pair the wait also covers the first of the new ones)
+    constexpr int READS_ = 2 * reads_per_half<A_KC>() + 2 * reads_per_half<B_KC>(), READS = READS_ < 15 ? READS_ : 15;
+    if constexpr (KP + 1 < BK / 2) {
+      issue_pair<KP + 1>(a[NXT], b[NXT], a_addr, b_addr);
+      wait_pair<READS>(a[CUR], b[CUR]);  // the reads just issued may stay in flight, everything older has landed
+    } else {
+      wait_pair<0>(a[CUR], b[CUR]);
+    }
+    row4<0, 0>(acc, a[CUR], b[CUR]); row4<0, 4>(acc, a[CUR], b[CUR]);
+    row4<1, 0>(acc, a[CUR], b[CUR]); row4<1, 4>(acc, a[CUR], b[CUR]);
+    row4<2, 0>(acc, a[CUR], b[CUR]); row4<2, 4>(acc, a[CUR], b[CUR]);
+    row4<3, 0>(acc, a[CUR], b[CUR]); row4<3, 4>(acc, a[CUR], b[CUR]);
+    row4<4, 0>(acc, a[CUR], b[CUR]); row4<4, 4>(acc, a[CUR], b[CUR]);
+    row4<5, 0>(acc, a[CUR], b[CUR]); row4<5, 4>(acc, a[CUR], b[CUR]);
+    row4<6, 0>(acc, a[CUR], b[CUR]); row4<6, 4>(acc, a[CUR], b[CUR]);
+    row4<7, 0>(acc, a[CUR], b[CUR]); row4<7, 4>(acc, a[CUR], b[CUR]);
+  }
+  template <int... KP>
+  static __device__ __forceinline__ void relaxed_tile(std::integer_sequence<int, KP...>, T (&acc)[8][8], FragA (&a)[2], FragB (&b)[2],
+                                                     unsigned a_addr, unsigned b_addr) {
+    issue_pair<0>(a[0], b[0], a_addr, b_addr);
+    (relaxed_kpair<KP>(acc, a, b, a_addr, b_addr), ...);
+  }
+
   static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
     const int tid = threadIdx.x, tx = tid % TX, ty = tid / TX, lane = tid & 63, wave = tid >> 6;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -313,11 +355,22 @@ struct DirectTile {
     // so each LDS read is issued 50..100 vector instructions before its use.
     // The last k-pair of a tile takes its refills from the other LDS stage,
     // which is why the barrier sits in the middle of that k-pair.
-    FragA a;
-    FragB b;
     // lane's LDS byte address of (stage 0, k-pair 0, x 0) in each panel
     const unsigned a_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][0] + ty * 16;
     const unsigned b_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][0] + tx * 16;
+    if constexpr (RELAXED) {
+      FragA a[2];
+      FragB b[2];
+      for (int t = 0; t < nfull; ++t) {
+        const int stage = t & 1;
+        relaxed_tile(std::make_integer_sequence<int, BK / 2>{}, acc, a, b, a_addr0 + stage * (BK * BM * 4),
+                     b_addr0 + stage * (BK * BN * 4));
+        __syncthreads();     // tile t+1 has landed (vmcnt waited first); nobody reads this stage any more
+        fetch_whole(t + 2);  // ... so tile t+2 may overwrite it
+      }
+    } else {
+    FragA a;
+    FragB b;
     unsigned a_addr = a_addr0, b_addr = b_addr0;
     if (nfull > 0) {
       refill_half<TY, 0, 0>(a, a_addr);
@@ -366,6 +419,7 @@ struct DirectTile {
       wait_half<0, 0>(b);
       wait_half<0, 1>(b);
     }
+    }  // !RELAXED
     const int buf = nfull % STAGES;
     if (rem > 0) {
       const T *pa = sm.a[buf], *pb = sm.b[buf];
@@ -450,6 +504,13 @@ __global__ __launch_bounds__(TY *TX) __attribute__((amdgpu_waves_per_eu(4, 4))) 
   Tile::run(p, sm);
 }
 
+template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void relaxed_srgemm_kernel(Problem p) {
+  using Tile = DirectTile<T, ADD, MUL, A_KC, B_KC, 16, 16, 32, true>;
+  __shared__ typename Tile::Smem sm;
+  Tile::run(p, sm);
+}
+
 // can the direct tile run this (canonical) problem?
 static inline bool direct_ok(const Problem &p) {
   auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
@@ -479,7 +540,29 @@ static inline bool direct_ok(const Problem &p) {
 #define CUASR_AMD_DIRECT_TX 16
 #endif
 
+static inline bool direct_prefers_relaxed(const Problem &p) {
+  return p.sa_k == 1 && p.sa_m != 1 && p.sb_k == 1 && p.sb_n != 1;
+}
+
+template <typename T, int ADD, int MUL> static hipError_t launch_relaxed(const Problem &p, hipStream_t s) {
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  if (!direct_ok(p)) return hipErrorNotSupported;
+  const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
+  if (a_kc && b_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(256), 0, s, p);
+  else if (a_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(256), 0, s, p);
+  else if (b_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, false, true>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, false, false>), grid, dim3(256), 0, s, p);
+  return hipGetLastError();
+}
+
 template <typename T, int ADD, int MUL> static hipError_t launch_direct(const Problem &p, hipStream_t s) {
+  // both operands k-contiguous: the 4-wave tile has to keep more lane addresses than it has
+  // registers for and spills inside its main loop (58.7 vs 70.0 TOPS at 4096^3); the relaxed
+  // tile does not.  Elsewhere the two are within noise of each other.
+  if (direct_prefers_relaxed(p)) return launch_relaxed<T, ADD, MUL>(p, s);
   constexpr int TY = CUASR_AMD_DIRECT_TY, TX = CUASR_AMD_DIRECT_TX, BM = 8 * TY, BN = 8 * TX;
   if (p.m == 0 || p.n == 0) return hipSuccess;
   if (!direct_ok(p)) return hipErrorNotSupported;
