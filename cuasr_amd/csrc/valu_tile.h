@@ -36,6 +36,8 @@ struct ValuTile {
   static constexpr int HM = TM / VW, GN = TN / VW;
   static_assert(A_ELEMS >= VW && B_ELEMS >= VW && HM >= 1 && GN >= 1, "tile too small");
   static_assert(BK % VW == 0 && BK % KU == 0, "BK must hold whole vectors");
+  static_assert(A_ELEMS % VW == 0 && B_ELEMS % VW == 0 && A_ELEMS * 256 == BM * BK && B_ELEMS * 256 == BN * BK,
+                "a panel must split into whole vectors per thread");
   typedef T vec_t __attribute__((ext_vector_type(VW)));
 
   struct Smem {
