@@ -28,7 +28,10 @@ namespace cuasr_amd {
 
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
 struct ValuTile {
-  static constexpr int KU = 2;  // k-steps unrolled together (lets two sums meet in one 3-input min/max)
+  // k-steps taken together: two let a pair of sums meet in one 3-input min/max (4-byte types);
+  // 8-byte types have no 3-input instructions, and one k-step per fragment set halves the
+  // registers the fragments take
+  static constexpr int KU = sizeof(T) == 8 ? 1 : 2;
   static constexpr int VW = 16 / sizeof(T);
   static constexpr int BM = 16 * TM, BN = 16 * TN;
   static constexpr int LDA = BM + VW, LDB = BN + VW;
@@ -192,11 +195,11 @@ struct ValuTile {
   // compiler ten minutes each, and they are not the throughput cases)
   static constexpr bool PIPELINED = T(0.5) != T(0);  // floating-point element type
   struct Frag2 {
-    T a[2][TM], b[2][TN];
+    T a[KU][TM], b[KU][TN];
   };
   static __device__ __forceinline__ void load_frag2(Frag2 &f, const T (*as)[LDA], const T (*bs)[LDB], int kk, int ty, int tx) {
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < KU; ++s) {
 #pragma unroll
       for (int h = 0; h < HM; ++h) {
         const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk + s][ty * VW + h * 16 * VW]);
@@ -216,27 +219,32 @@ struct ValuTile {
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const T t0 = Op<MUL>::apply(f.a[0][i], f.b[0][j]), t1 = Op<MUL>::apply(f.a[1][i], f.b[1][j]);
-        acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
+        if constexpr (KU == 2) {
+          const T t0 = Op<MUL>::apply(f.a[0][i], f.b[0][j]), t1 = Op<MUL>::apply(f.a[1][i], f.b[1][j]);
+          acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
+        } else {
+          acc[i][j] = fold<ADD, MUL>(Op<MUL>::apply(f.a[0][i], f.b[0][j]), acc[i][j]);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
   static __device__ __forceinline__ void whole_tile(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int ty, int tx) {
+    constexpr int STEPS = BK / KU;
     if constexpr (PIPELINED) {
       Frag2 f[2];
       load_frag2(f[0], as, bs, 0, ty, tx);
 #pragma unroll
-      for (int kp = 0; kp < BK / 2; ++kp) {
-        if (kp + 1 < BK / 2) load_frag2(f[(kp + 1) & 1], as, bs, 2 * kp + 2, ty, tx);
+      for (int kp = 0; kp < STEPS; ++kp) {
+        if (kp + 1 < STEPS) load_frag2(f[(kp + 1) & 1], as, bs, KU * (kp + 1), ty, tx);
         __builtin_amdgcn_sched_barrier(0);
         compute2(acc, f[kp & 1]);
       }
     } else {
 #pragma unroll 1
-      for (int kp = 0; kp < BK / 2; ++kp) {
+      for (int kp = 0; kp < STEPS; ++kp) {
         Frag2 f;
-        load_frag2(f, as, bs, 2 * kp, ty, tx);
+        load_frag2(f, as, bs, KU * kp, ty, tx);
         compute2(acc, f);
       }
     }
