@@ -55,6 +55,7 @@ inline cuasr_amd_srgemm_desc make_desc(Args const &a, int kernel) {
 }
 template <typename OperatorClass> struct kernel_of { static int const value = CUASR_AMD_KERNEL_AUTO; };
 template <> struct kernel_of<arch::OpClassMatrixCore> { static int const value = CUASR_AMD_KERNEL_MFMA; };
+template <> struct kernel_of<arch::OpClassVectorAlu> { static int const value = CUASR_AMD_KERNEL_VALU; };
 }  // namespace detail
 
 template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, typename LayoutA_, typename ElementB_,

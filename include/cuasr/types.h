@@ -64,8 +64,9 @@ struct GemmSplitKHorizontalThreadblockSwizzle {};
 }  // namespace gemm
 
 namespace arch {
-struct OpClassSimt {};      ///< vector-ALU kernels (the only class the reference implements)
+struct OpClassSimt {};      ///< the reference's only class; here: the library picks the kernel family
 struct OpClassMatrixCore {};///< matrix-core assisted kernels
+struct OpClassVectorAlu {}; ///< vector-ALU tiles only: bit-exact sequential sums also for plus-times
 struct Gfx950 {};           ///< MI355X
 using Sm50 = Gfx950;        ///< spelled by existing cuASR user code; selects the same kernels
 }  // namespace arch

@@ -8,6 +8,7 @@
 // Prints one line per check; exit status is the number of failures.
 #include <hip/hip_runtime_api.h>
 
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -228,6 +229,34 @@ static void example_splitk() {
          "split_k_slices > 1 rejected by Srgemm");
 }
 
+// The operator class picks the kernel family: OpClassVectorAlu reproduces the host reference bit for
+// bit also for plus-times on non-integer data; the default class may use the matrix cores (rounding
+// differs, |d - r| <= 1e-5 * sum|a||b|).
+static void operator_classes() {
+  using Add = cuasr::plus<float>;
+  using Mul = cuasr::multiplies<float>;
+  using Exact = cuasr::gemm::device::Srgemm<Add, Mul, float, ColumnMajor, float, ColumnMajor, float, ColumnMajor, float,
+                                            cuasr::arch::OpClassVectorAlu>;
+  using Auto = cuasr::gemm::device::Srgemm<Add, Mul, float, ColumnMajor, float, ColumnMajor, float, ColumnMajor, float>;
+  const int M = 256, N = 128, K = 512;
+  std::vector<float> a(size_t(M) * K), b(size_t(K) * N), c(size_t(M) * N), want(size_t(M) * N);
+  fill_unit(a, 21, -1.0, 1.0);
+  fill_unit(b, 22, -1.0, 1.0);
+  fill_unit(c, 23, -1.0, 1.0);
+  cuasr::reference::host::Srgemm<Add, Mul, float, ColumnMajor, float, ColumnMajor, float, ColumnMajor, float, float> ref;
+  ref({M, N, K}, 1.0f, {a.data(), M}, {b.data(), K}, 1.0f, {c.data(), M}, {want.data(), M}, Add::Identity);
+  DeviceBuf<float> da(a), db(b), dc(c), d1(std::vector<float>(size_t(M) * N, 0.f)), d2(std::vector<float>(size_t(M) * N, 0.f));
+  Exact::Arguments e({M, N, K}, {da.p, M}, {db.p, K}, {dc.p, M}, {d1.p, M}, {1.0f, 1.0f});
+  Auto::Arguments u({M, N, K}, {da.p, M}, {db.p, K}, {dc.p, M}, {d2.p, M}, {1.0f, 1.0f});
+  bool ok = Exact()(e) == Status::kSuccess && Auto()(u) == Status::kSuccess;
+  HIP_OK(hipDeviceSynchronize());
+  report(ok && d1.download() == want, "OpClassVectorAlu plus-times bit-exact vs host reference");
+  const std::vector<float> got = d2.download();
+  bool close = ok;
+  for (size_t i = 0; i < got.size() && close; ++i) close = std::fabs(double(got[i]) - double(want[i])) <= 1e-5 * (K + 1);
+  report(close, "default class plus-times within 1e-5 * sum|a||b| of host reference");
+}
+
 int main() {
   int devices = 0;
   if (hipGetDeviceCount(&devices) != hipSuccess || devices == 0) {
@@ -237,6 +266,7 @@ int main() {
   example_minplus_and_known_answer();
   example_userdefined_xor_and();
   example_splitk();
+  operator_classes();
   testbed_sweep<cuasr::plus<float>, cuasr::multiplies<float>, float>("testbed plus-multiplies f32");
   testbed_sweep<cuasr::minimum<float>, cuasr::plus<float>, float>("testbed minimum-plus f32");
   testbed_sweep<cuasr::maximum<float>, cuasr::plus<float>, float>("testbed maximum-plus f32");
