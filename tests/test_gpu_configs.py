@@ -72,10 +72,12 @@ def test_config2_apsp_4096(oracle, lib):
     assert np.array_equal(to_host(cur, "f32").astype(np.float64), fw)
 
 
+@pytest.mark.parametrize("ident", [-np.inf, np.finfo(np.float64).tiny], ids=["minus_inf", "reference_constant"])
 @pytest.mark.parametrize("sr", ["max-plus", "max-min"])
-def test_config3_f64_8192(oracle, lib, sr):
+def test_config3_f64_8192(oracle, lib, sr, ident):
     """fp64 max-plus / max-min at 8192^3, beta = one with a seeded C: a 512 x 512 block against the
-    oracle bit-exact, the full matrix against the naive on-device kernel by checksum."""
+    oracle bit-exact, the full matrix against the naive on-device kernel by checksum; with the
+    accumulator starting from -inf and from the reference's own identity constant."""
     import torch
     import cuasr_amd
     from cuasr_amd import inputs
@@ -85,7 +87,7 @@ def test_config3_f64_8192(oracle, lib, sr):
     C = inputs.uniform(303, n, n, -1.0, 1.0, np.float64)
     add, mult = ("maximum", "plus") if sr == "max-plus" else ("maximum", "minimum")
     one = 0.0 if sr == "max-plus" else np.inf
-    ident = -np.inf
+    # additive identity: -inf, or the reference's maximum<double>::Identity = numeric_limits<double>::min()
     dA, dB, dC = to_device(A), to_device(B), to_device(C)
     dD, dN = to_device(np.zeros_like(C)), to_device(np.zeros_like(C))
     cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype="f64")
@@ -174,3 +176,25 @@ def test_config5b_plus_times_f32_4096(oracle, lib):
     mag = (torch.from_numpy(np.abs(A)).cuda() @ torch.from_numpy(np.abs(B)).cuda()).cpu().numpy().astype(np.float64)
     assert np.all(np.abs(diff) <= 1e-5 * mag)
     assert np.linalg.norm(diff) <= 1e-5 * np.linalg.norm(want.astype(np.float64))
+    big = np.abs(want) >= 1.0
+    print("fp32 plus-times 4096^3: max relative error over |r| >= 1:", float((np.abs(diff[big]) / np.abs(want[big])).max()))
+
+
+def test_config5b_plus_times_f64_4096(oracle, lib):
+    """The fp64 analogue of the plus-times control: N(0,1) inputs, 4096^3, tolerance 1e-12 relative
+    (per element against sum_k |a||b|, and in the Frobenius norm); the vector-ALU tile bit-exact."""
+    import torch
+    from cuasr_amd import inputs
+    n = 4096
+    A = inputs.normal(611, n, n).astype(np.float64, order="F") + 2.0 ** -30 * inputs.normal(613, n, n).astype(np.float64, order="F")
+    B = inputs.normal(612, n, n).astype(np.float64, order="F") + 2.0 ** -30 * inputs.normal(614, n, n).astype(np.float64, order="F")
+    C = np.zeros((n, n), dtype=np.float64, order="F")
+    want = oracle.srgemm("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0)
+    assert_same_bits(_run("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0, 1.0, "f64", "valu"), want, "vector-ALU fp64 plus-times")
+    got = _run("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0, 1.0, "f64")
+    diff = np.abs(got - want)
+    mag = (torch.from_numpy(np.abs(A)).cuda() @ torch.from_numpy(np.abs(B)).cuda()).cpu().numpy()
+    assert np.all(diff <= 1e-12 * mag)
+    assert np.linalg.norm(diff) <= 1e-12 * np.linalg.norm(want)
+    big = np.abs(want) >= 1.0
+    print("fp64 plus-times 4096^3: max relative error over |r| >= 1:", float((diff[big] / np.abs(want[big])).max()))
