@@ -26,7 +26,10 @@
 #endif
 namespace cuasr_amd {
 
-template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
+// VEC: 16-byte global accesses.  CAREFUL (with VEC): operands of any extent, leading dimension and
+// element alignment -- edge vectors and the last k-tile are treated separately (see Mover); without
+// it the host guarantees extents along the contiguous directions that are multiples of the vector.
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC, bool CAREFUL = false>
 struct ValuTile {
   // k-steps taken together: two let a pair of sums meet in one 3-input min/max (4-byte types);
   // 8-byte types have no 3-input instructions, and one k-step per fragment set halves the
@@ -42,6 +45,9 @@ struct ValuTile {
   static_assert(A_ELEMS % VW == 0 && B_ELEMS % VW == 0 && A_ELEMS * 256 == BM * BK && B_ELEMS * 256 == BN * BK,
                 "a panel must split into whole vectors per thread");
   typedef T vec_t __attribute__((ext_vector_type(VW)));
+  // the same vector in global memory, where only element alignment is required (the hardware
+  // takes 16-byte loads and stores at any 4-byte boundary)
+  typedef T gvec_t __attribute__((ext_vector_type(VW), aligned(sizeof(T))));
 
   struct Smem {
     T a[2][BK][LDA];
@@ -86,10 +92,16 @@ struct ValuTile {
 
   // ---- the same ownership with the addressing done once (VEC only): a thread
   // keeps one pointer per 16-byte vector, at the vector's place in the first
-  // k-tile with the panel index clamped to the matrix, and moves it one k-tile
-  // along per iteration -- two integer instructions per vector and tile instead
-  // of the index arithmetic of load_panel.  Only a ragged last k-tile needs a
-  // second look at k: vectors past its end re-read its last valid vector.
+  // k-tile, and moves it one k-tile along per iteration -- two integer
+  // instructions per vector and tile instead of the index arithmetic of
+  // load_panel.  Any extents, leading dimensions and (element) alignment:
+  //   * a vector that lies wholly past the panel's edge points at the last
+  //     whole vector inside the matrix (what it fetches is never used);
+  //   * a vector that straddles the edge of an x-contiguous panel (extent not
+  //     a multiple of VW) reads on into the padding or the next k row: valid
+  //     memory of the same matrix as long as a later k row exists, which is
+  //     why the LAST k-tile of a workgroup is never fetched this way but by
+  //     load_last, element by element with both indices clamped.
   template <int ROWS, int ELEMS> struct Mover {
     static constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
     const T *src[VECS];
@@ -101,7 +113,9 @@ struct ValuTile {
 #pragma unroll
       for (int p = 0; p < VECS; ++p) {
         const int v = tid + 256 * p;
-        const int xx = min(x0 + (x_contig ? (v % XV) * VW : v / KV), x_end - (x_contig ? VW : 1));
+        int xx = x0 + (x_contig ? (v % XV) * VW : v / KV);
+        if (x_contig) xx = xx >= x_end ? x_end - VW : xx;
+        else xx = min(xx, x_end - 1);
         const int kk = k0 + (x_contig ? v / XV : (v % KV) * VW);
         src[p] = base + (long long)xx * s_x + (long long)kk * s_k;
       }
@@ -109,12 +123,13 @@ struct ValuTile {
     __device__ __forceinline__ void load(T (&r)[ELEMS]) {
 #pragma unroll
       for (int p = 0; p < VECS; ++p) {
-        const vec_t t = *reinterpret_cast<const vec_t *>(src[p]);
+        const gvec_t t = *reinterpret_cast<const gvec_t *>(src[p]);
 #pragma unroll
         for (int e = 0; e < VW; ++e) r[p * VW + e] = t[e];
         src[p] += step;
       }
     }
+    // !CAREFUL: ragged last k-tile; vectors past its end re-read its last valid vector
     __device__ __forceinline__ void load_ragged(T (&r)[ELEMS], long long s_k, int kcount, bool x_contig) {
       const int tid = threadIdx.x;
 #pragma unroll
@@ -122,13 +137,38 @@ struct ValuTile {
         const int v = tid + 256 * p;
         const int kl = x_contig ? v / XV : (v % KV) * VW;         // the vector's first k inside the tile
         const int back = max(kl - (kcount - (x_contig ? 1 : VW)), 0);  // steps of k past the last valid vector
-        const vec_t t = *reinterpret_cast<const vec_t *>(src[p] - (long long)back * s_k);
+        const gvec_t t = *reinterpret_cast<const gvec_t *>(src[p] - (long long)back * s_k);
 #pragma unroll
         for (int e = 0; e < VW; ++e) r[p * VW + e] = t[e];
         src[p] += step;
       }
     }
   };
+
+  // The last k-tile (k0 .. k_end, 1 .. BK values of k) of a panel, straight into its LDS stage:
+  // every element with its own clamped indices.  Deliberately NOT inlined: it runs once per
+  // workgroup, and inlined into the main loop its address arithmetic costs the loop 60-80
+  // registers (a wave less per SIMD for the quarter-size tile).
+  template <int ROWS, int LD>
+  static __device__ __attribute__((noinline)) void fill_last(T (*dst)[LD], const T *base, long long s_x, long long s_k, int x0,
+                                                             int x_end, int k0, int k_end, bool x_contig) {
+    const int tid = threadIdx.x;
+    const int xmax = x_end - 1 - x0, kmax = k_end - 1 - k0;
+    const T *tile = base + (long long)x0 * s_x + (long long)k0 * s_k;
+    constexpr int N = ROWS * BK / 256;
+    T r[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {  // all loads in flight together
+      const int el = tid + 256 * i;
+      const int x = x_contig ? el % ROWS : el / BK, kk = x_contig ? el / ROWS : el % BK;
+      r[i] = tile[(long long)min(x, xmax) * s_x + (long long)min(kk, kmax) * s_k];
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int el = tid + 256 * i;
+      dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = r[i];
+    }
+  }
 
   // ---- registers -> LDS ([kk][x], k-major), same ownership as load_panel
   template <int ROWS, int LD, int ELEMS>
@@ -298,7 +338,7 @@ struct ValuTile {
     auto fetch = [&](int k0) {
       if constexpr (VEC) {
         const int kcount = ke - k0;
-        if (kcount >= BK) {
+        if (CAREFUL || kcount >= BK) {
           ma.load(ra);
           mb.load(rb);
         } else {
@@ -310,17 +350,34 @@ struct ValuTile {
         load_panel<BN, B_ELEMS>(rb, B, p.sb_n, p.sb_k, n0, p.n, k0, ke, b_xc);
       }
     };
+    // On the vector path the last k-tile of the workgroup is never fetched through the movers
+    // (see Mover): fill_last puts it straight into its LDS stage -- which is free as soon as the
+    // barrier that ended the previous iteration has been passed, so it is filled ahead of the
+    // compute like a prefetch.
+    auto fill_last_tile = [&](int k0, int stage) {
+      fill_last<BM, LDA>(sm.a[stage], A, p.sa_m, p.sa_k, m0, p.m, k0, ke, a_xc);
+      fill_last<BN, LDB>(sm.b[stage], B, p.sb_n, p.sb_k, n0, p.n, k0, ke, b_xc);
+    };
+    // ... unless nothing about the last tile can reach past the matrix: it is a whole tile and no
+    // vector straddles an edge (x-contiguous extents are multiples of the vector width)
+    const bool careful_last = VEC && CAREFUL && !((ke - kb) % BK == 0 && (!a_xc || p.m % VW == 0) && (!b_xc || p.n % VW == 0));
     if (ntiles > 0) {
-      fetch(kb);
-      store_panel<BM, LDA, A_ELEMS>(ra, sm.a[0], a_xc);
-      store_panel<BN, LDB, B_ELEMS>(rb, sm.b[0], b_xc);
+      if (careful_last && ntiles == 1) {
+        fill_last_tile(kb, 0);
+      } else {
+        fetch(kb);
+        store_panel<BM, LDA, A_ELEMS>(ra, sm.a[0], a_xc);
+        store_panel<BN, LDB, B_ELEMS>(rb, sm.b[0], b_xc);
+      }
     }
     __syncthreads();
     int buf = 0;
     for (int t = 0; t < ntiles; ++t) {
       const int k0 = kb + t * BK;
       const bool more = t + 1 < ntiles;
-      if (more) fetch(k0 + BK);
+      const bool next_is_last = careful_last && t + 2 == ntiles;
+      if (next_is_last) fill_last_tile(k0 + BK, buf ^ 1);
+      else if (more) fetch(k0 + BK);
       const int kcount = min(BK, ke - k0);
       if (kcount == BK) {
         whole_tile(acc, sm.a[buf], sm.b[buf], ty, tx);
@@ -328,7 +385,7 @@ struct ValuTile {
 #pragma unroll 1
         for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
       }
-      if (more) {
+      if (more && !next_is_last) {
         store_panel<BM, LDA, A_ELEMS>(ra, sm.a[buf ^ 1], a_xc);
         store_panel<BN, LDB, B_ELEMS>(rb, sm.b[buf ^ 1], b_xc);
       }
@@ -368,8 +425,8 @@ struct ValuTile {
           for (int c = 0; c < VW; ++c) v[c] = Op<MUL>::apply(e.alpha, v[c]);
           if (e.source_needed) {
             T src[VW];
-            if constexpr (VEC) {
-              const vec_t t = *reinterpret_cast<const vec_t *>(C + (long long)row * p.ldc + col);
+            if (VEC && (!CAREFUL || col + VW <= p.n)) {
+              const gvec_t t = *reinterpret_cast<const gvec_t *>(C + (long long)row * p.ldc + col);
 #pragma unroll
               for (int c = 0; c < VW; ++c) src[c] = t[c];
             } else {
@@ -380,11 +437,11 @@ struct ValuTile {
             for (int c = 0; c < VW; ++c) v[c] = fold_epilogue<ADD, MUL>(v[c], Op<MUL>::apply(e.beta, src[c]));
           }
         }
-        if constexpr (VEC) {
-          vec_t t;
+        if (VEC && (!CAREFUL || col + VW <= p.n)) {
+          gvec_t t;
 #pragma unroll
           for (int c = 0; c < VW; ++c) t[c] = v[c];
-          *reinterpret_cast<vec_t *>(out + (long long)row * ld_out + col) = t;
+          *reinterpret_cast<gvec_t *>(out + (long long)row * ld_out + col) = t;
         } else {
 #pragma unroll
           for (int c = 0; c < VW; ++c)
@@ -396,29 +453,33 @@ struct ValuTile {
   }
 };
 
-template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC>
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC, bool CAREFUL = false>
 __global__ __launch_bounds__(256) WAVES_ATTR void valu_srgemm_kernel(Problem p) {
-  using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC>;
+  using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC, CAREFUL>;
   __shared__ typename Tile::Smem sm;
   Tile::run(p, sm);
 }
 
-// 16-byte access is legal for the whole problem: aligned bases, leading
-// dimensions and contiguous extents that are multiples of the vector width
-template <typename T> static bool vector_friendly(const Problem &p) {
+// Extents along every contiguous direction are multiples of the vector width: no vector straddles
+// an edge, rows of D hold whole vectors (alignment itself is not needed: 16-byte accesses are legal
+// at any element boundary).
+template <typename T> static bool vector_exact(const Problem &p) {
   constexpr int VW = 16 / sizeof(T);
-  auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
-  if (!al(p.A) || !al(p.B)) return false;
-  if (a_xc ? (p.m % VW || p.sa_k % VW) : (p.sa_k != 1 || p.k % VW || p.sa_m % VW)) return false;
-  if (b_xc ? (p.n % VW || p.sb_k % VW) : (p.sb_k != 1 || p.k % VW || p.sb_n % VW)) return false;
-  if (p.n % VW) return false;
-  if (p.workspace) return al(p.workspace);
-  // C is only dereferenced when the source is needed, but whether it is can
-  // depend on a device-side beta; require alignment whenever a pointer is given
-  if (!al(p.D) || p.ldd % VW) return false;
-  if (p.C && (!al(p.C) || p.ldc % VW)) return false;
-  return true;
+  if (a_xc ? p.m % VW : (p.sa_k != 1 || p.k % VW)) return false;
+  if (b_xc ? p.n % VW : (p.sb_k != 1 || p.k % VW)) return false;
+  return p.n % VW == 0 && p.k >= 1;
+}
+// The careful vector path takes any extent; it only needs one whole vector inside each operand
+// along its contiguous direction, for the vectors that lie wholly outside to point at.
+template <typename T> static bool vector_possible(const Problem &p) {
+  constexpr int VW = 16 / sizeof(T);
+  const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
+  if (!a_xc && p.sa_k != 1) return false;  // neither direction contiguous (not produced by the C ABI)
+  if (!b_xc && p.sb_k != 1) return false;
+  if (a_xc && p.m < VW) return false;
+  if (b_xc && p.n < VW) return false;
+  return p.k >= 1;
 }
 
 template <typename T, int ADD, int MUL, int TM, int TN, int BK>
@@ -428,10 +489,12 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
-  if (vector_friendly<T>(p))
-    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true>), grid, dim3(256), 0, s, p);
+  if (vector_exact<T>(p))
+    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, false>), grid, dim3(256), 0, s, p);
+  else if (vector_possible<T>(p))
+    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, true>), grid, dim3(256), 0, s, p);
   else
-    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, false>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, false, false>), grid, dim3(256), 0, s, p);
   return hipGetLastError();
 }
 

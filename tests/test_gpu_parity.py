@@ -209,3 +209,47 @@ def test_plus_times_f64_tolerance(oracle, lib):
             diff = np.abs(got - want)
             assert np.all(diff <= 1e-12 * (np.abs(A) @ np.abs(B)))          # tolerance 1e-12 relative
             assert np.linalg.norm(diff) <= 1e-12 * np.linalg.norm(want)
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f64"), ("plus", "multiplies", "f32"),
+                                ("bit_xor", "bit_and", "u32")])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_unaligned_views(oracle, lib, sr, layouts):
+    """Operands that are interior windows of larger buffers: base pointers aligned to the element only,
+    leading dimensions larger than the extents and odd, extents not multiples of the vector width.
+    Every kernel family AUTO may pick and the staged family itself must reproduce the oracle."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    add, mult, dtype = sr
+    npd = {"f32": np.float32, "f64": np.float64, "u32": np.uint32}[dtype]
+    for (m, n, k) in [(131, 67, 45), (515, 262, 131), (1027, 1030, 77)]:
+        def window(seed, rows, cols, layout):
+            # a (rows x cols) window at offset (3, 1) of a buffer with 5 spare rows and 7 spare columns
+            R, Cc = rows + 5, cols + 7
+            if dtype == "u32":
+                full = inputs.words32(seed, R, Cc, "C")
+            else:
+                full = inputs.integers(seed, R, Cc, -8, 8, npd, "C")
+            host = full[3:3 + rows, 1:1 + cols]
+            if layout == "row":
+                dev = torch.from_numpy(full.view(np.int32) if dtype == "u32" else full).cuda()[3:3 + rows, 1:1 + cols]
+            else:  # column-major window: transpose view of a row-major buffer holding the transpose
+                fullT = np.ascontiguousarray(full.T)
+                dev = torch.from_numpy(fullT.view(np.int32) if dtype == "u32" else fullT).cuda()[1:1 + cols, 3:3 + rows].t()
+            return host, dev
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        A, dA = window(31, m, k, la)
+        B, dB = window(32, k, n, lb)
+        C, dC = window(33, m, n, lc)
+        _, dD0 = window(34, m, n, lc)
+        ident = cuasr_amd.op_identity(add, dtype, True)
+        one = cuasr_amd.op_identity(mult, dtype, True)
+        order = "F" if lc == "col" else "C"
+        want = oracle.srgemm(add, mult, np.asarray(A, order=("F" if la == "col" else "C")), np.asarray(B, order=("F" if lb == "col" else "C")),
+                             np.asarray(C, order=order), one, one, ident)
+        for kernel in ("auto", "valu"):
+            dD = dD0.clone() if False else dD0  # the window of D is written in place
+            cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dtype, kernel=kernel)
+            torch.cuda.synchronize()
+            assert_same_bits(np.asarray(to_host(dD, dtype), order=order), want, f"{sr} {layouts} {m}x{n}x{k} {kernel}")
