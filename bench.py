@@ -35,8 +35,8 @@ HBM_PEAK_GBS = 8000.0
 # this script (profiles/ holds the summaries and the commands); FETCH_SIZE is scaled by 2.0, the
 # factor by which it under-reports a plain device copy of known size, WRITE_SIZE by 1.0.
 MEASURED_TRAFFIC_BYTES = {
-    # direct-to-LDS tile: 2.0 * 404 528 KiB fetched + 77 824 KiB written (268.4 MB algorithmic)
-    ("apsp", 4096, 4096, 4096): (2 * 404528 + 77824) * 1024,
+    # direct-to-LDS tile: 2.0 * 403 136 KiB fetched + 77 824 KiB written (268.4 MB algorithmic)
+    ("apsp", 4096, 4096, 4096): (2 * 403136 + 77824) * 1024,
 }
 
 
