@@ -174,8 +174,12 @@ def make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mul
     desc = SrgemmDesc()
     desc.add_op, desc.mult_op, desc.dtype = OPS[add_op], OPS[mult_op], DTYPES[dtype]
     desc.layout_a, desc.layout_b, desc.layout_c = a.layout, b.layout, d.layout
-    if c.ptr and c.layout != d.layout and min(d.rows, d.cols) > 1:
-        raise ValueError("C and D must share a layout")
+    if c.ptr and c.layout != d.layout:
+        # only a contiguous vector can be read in either layout
+        if min(d.rows, d.cols) > 1 or c.ld != (1 if (c.layout == COLUMN_MAJOR) == (c.rows == 1) else max(c.rows, c.cols)):
+            raise ValueError("C and D must share a layout")
+        c = MatRef(c.ptr, max(c.cols, 1) if d.layout == ROW_MAJOR and c.rows == 1 else
+                   max(c.rows, 1) if d.layout == COLUMN_MAJOR and c.cols == 1 else 1, d.layout, c.rows, c.cols)
     if a.cols != b.rows or (a.rows, b.cols) != (d.rows, d.cols):
         raise ValueError("shape mismatch")
     desc.m, desc.n, desc.k = d.rows, d.cols, a.cols

@@ -1,0 +1,109 @@
+"""Contract details of the operator boundary, on the GPU and through the C ABI: device-resident
+alpha / beta, D aliasing C, launches on a caller's stream, and the shapes the reference's
+cross-implementation tests use (test/regress/Srgemm_test.cu:118-605: tall-skinny, short-wide,
+sub-matrices of larger buffers)."""
+import numpy as np
+import pytest
+
+from helpers import assert_same_bits, to_device, to_host
+
+pytestmark = pytest.mark.gpu
+
+FAMILIES = ["naive", "valu", "direct", "mfma"]
+
+
+def _inputs(m, n, k, seed=5):
+    from cuasr_amd import inputs
+    A = inputs.integers(seed, m, k, -8, 8, np.float32, "F")
+    B = inputs.integers(seed + 1, k, n, -8, 8, np.float32, "F")
+    C = inputs.integers(seed + 2, m, n, -8, 8, np.float32, "F")
+    return A, B, C
+
+
+@pytest.mark.parametrize("kernel", FAMILIES)
+def test_alpha_beta_from_device_memory(oracle, lib, kernel):
+    """alpha_ptr / beta_ptr override the immediate scalars (semiring_linear_combination.h:88-99, :112-115),
+    and whether C is read is decided on the device from the pointed-to beta (:118-125)."""
+    import torch
+    import cuasr_amd
+    m, n, k = 256, 128, 96
+    A, B, C = _inputs(m, n, k)
+    inf = np.float32(np.inf)
+    for beta in (np.float32(0.0), inf):          # min-plus one (C is read) and zero (C is not read)
+        want = oracle.srgemm("minimum", "plus", A, B, C, 2.0, beta, inf)
+        d_alpha = torch.tensor([2.0], dtype=torch.float32, device="cuda")
+        d_beta = torch.tensor([float(beta)], dtype=torch.float32, device="cuda")
+        dD = to_device(np.zeros_like(C))
+        # the immediate scalars are deliberately wrong: the pointers must win
+        cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, 7.0, 3.0, float("inf"), 0.0,
+                         kernel=kernel, alpha_ptr=d_alpha.data_ptr(), beta_ptr=d_beta.data_ptr())
+        torch.cuda.synchronize()
+        assert_same_bits(to_host(dD, "f32"), want, f"{kernel} beta={beta}")
+        if beta == inf:
+            # C is not needed: a null C must be accepted and never dereferenced
+            dD2 = to_device(np.zeros_like(C))
+            cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), None, dD2, 2.0, float("inf"), float("inf"), 0.0,
+                             kernel=kernel)
+            torch.cuda.synchronize()
+            assert_same_bits(to_host(dD2, "f32"), want, f"{kernel} null C")
+
+
+@pytest.mark.parametrize("kernel", FAMILIES)
+@pytest.mark.parametrize("layout", ["F", "C"])
+def test_d_may_alias_c(oracle, lib, kernel, layout):
+    """D = C in place (examples/00_minplus_srgemm/minplus_srgemm.cu:79-80)."""
+    import torch
+    import cuasr_amd
+    m, n, k = 384, 256, 64
+    A, B, C = _inputs(m, n, k, seed=11)
+    A, B, C = (np.asarray(x, order=layout) for x in (A, B, C))
+    want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)
+    dC = to_device(C)
+    cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), dC, dC, 0.0, 0.0, float("inf"), 0.0, kernel=kernel)
+    torch.cuda.synchronize()
+    assert_same_bits(np.asarray(to_host(dC, "f32"), order=layout), want, kernel)
+
+
+def test_launch_on_callers_stream(oracle, lib):
+    """Calls are asynchronous on the stream they are given and ordered by it: a chain of dependent
+    squarings on a side stream, with unrelated work on the default stream in between."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    n = 512
+    D0 = inputs.graph_distances(77, n, density=0.05)
+    host = D0
+    for _ in range(4):
+        host = oracle.srgemm("minimum", "plus", host, host, host, 0.0, 0.0, np.inf)
+    side = torch.cuda.Stream()
+    bufs = [to_device(D0), to_device(np.zeros_like(D0)), to_device(np.zeros_like(D0))]
+    torch.cuda.synchronize()
+    cur = bufs[0]
+    noise = torch.zeros(1 << 20, device="cuda")
+    for i in range(4):
+        dst = bufs[1 + (i & 1)]
+        cuasr_amd.srgemm("minimum", "plus", cur, cur, cur, dst, 0.0, 0.0, float("inf"), 0.0, stream=side)
+        noise += 1.0  # default stream, independent
+        cur = dst
+    side.synchronize()
+    assert_same_bits(to_host(cur, "f32"), host, "4 squarings on a side stream")
+    torch.cuda.synchronize()
+    assert float(noise[0]) == 4.0
+
+
+@pytest.mark.parametrize("shape", [(125, 125, 1000), (1000, 1000, 125), (1, 1000, 1000), (1000, 1, 1000), (1000, 1000, 1),
+                                   (3, 5, 7)])
+@pytest.mark.parametrize("kernel", ["auto", "valu", "naive"])
+def test_reference_cross_implementation_shapes(oracle, lib, shape, kernel):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    m, n, k = shape
+    A = inputs.uniform(21, m, k, 1.5, 100.0)
+    B = inputs.uniform(22, k, n, 1.5, 100.0)
+    C = inputs.uniform(23, m, n, 1.5, 100.0)
+    want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)
+    dD = to_device(np.zeros_like(C))
+    cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, 0.0, 0.0, float("inf"), 0.0, kernel=kernel)
+    torch.cuda.synchronize()
+    assert_same_bits(to_host(dD, "f32"), want, f"{shape} {kernel}")
