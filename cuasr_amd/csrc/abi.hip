@@ -15,7 +15,9 @@ launch_fn find_mfma_f64(int, int);
 launch_fn find_direct_f32(int, int);
 launch_fn find_direct_i32(int, int);
 launch_fn find_direct_u32(int, int);
+launch_fn find_direct_f64(int, int);
 bool direct_can_run(const Problem &);
+bool direct64_can_run(const Problem &);
 bool mfma_f32_can_run(const Problem &);
 bool mfma_f64_can_run(const Problem &);
 
@@ -34,6 +36,7 @@ launch_fn find_direct(int dtype, int add_op, int mult_op) {
     case CUASR_AMD_F32: return find_direct_f32(add_op, mult_op);
     case CUASR_AMD_I32: return find_direct_i32(add_op, mult_op);
     case CUASR_AMD_U32: return find_direct_u32(add_op, mult_op);
+    case CUASR_AMD_F64: return find_direct_f64(add_op, mult_op);
     default: return nullptr;
   }
 }
@@ -67,7 +70,7 @@ static bool mfma_usable(const cuasr_amd_srgemm_desc *d) {
 // the direct-to-LDS tiles need aligned, vector-sized operands as well
 static bool direct_usable(const cuasr_amd_srgemm_desc *d) {
   if (!find_direct(d->dtype, d->add_op, d->mult_op)) return false;
-  return direct_can_run(canonical(d));
+  return d->dtype == CUASR_AMD_F64 ? direct64_can_run(canonical(d)) : direct_can_run(canonical(d));
 }
 
 static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
@@ -140,19 +143,23 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.
   // The direct-to-LDS tile is 256 x 128 (128 x 128 when both operands are k-contiguous)
-  // and the chip holds 512 of them at a time (two per compute unit).  It is the fastest family when its workgroups fill
+  // and the chip holds 512 of them at a time (two per compute unit); for double it is
+  // 128 x 64 and the chip holds 768.  It is the fastest family when its workgroups fill
   // whole rounds of 512; a launch that leaves much of a round empty (small or
   // awkwardly sized outputs, split-K of a small output) is better served by the
   // smaller tiles of the staged family, whose many short workgroups balance.
   const Problem c = canonical(d);
-  const int tile_m = (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
-  const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + 127) / 128) * d->split_k_slices;
-  const long long rounds = (direct_groups + 511) / 512;
-  const bool fills = direct_groups * 8 >= rounds * 512 * 7;  // >= 7/8 of its rounds
+  const bool f64 = d->dtype == CUASR_AMD_F64;  // fp64 direct tile: 128 x 64, three per compute unit
+  const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
+  const int tile_n = f64 ? 64 : 128;
+  const long long slots = f64 ? 768 : 512;
+  const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + tile_n - 1) / tile_n) * d->split_k_slices;
+  const long long rounds = (direct_groups + slots - 1) / slots;
+  const bool fills = direct_groups * 8 >= rounds * slots * 7;  // >= 7/8 of its rounds
   const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;
-  // min-max / max-min: `v_min_f32` / `v_max_f32` do not dual-issue, the arithmetic is 60 % slower than
+  // min-max / max-min on 4-byte types: `v_min_f32` / `v_max_f32` do not dual-issue, the arithmetic is 60 % slower than
   // min-plus and the staged tile's two fragment sets cover it slightly better (47.6 vs 46.1 TOPS at 4096^3)
-  const bool minmax = (d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum);
+  const bool minmax = !f64 && ((d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum));
   if (direct_usable(d) && ((fills && !(minmax && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;

@@ -79,6 +79,7 @@ def test_kernel_selection(lib):
     assert sel(desc(m=8192, n=8192, k=64)) == b"valu_direct"
     assert sel(desc(add="plus", mult="multiplies")) == b"mfma"
     assert sel(desc(dtype="f64")) == b"valu"
+    assert sel(desc(dtype="f64", m=8192, n=8192, k=64)) == b"valu_direct"   # fp64 direct-to-LDS tile, 128 x 64
     assert sel(desc(dtype="f64", add="plus", mult="multiplies")) == b"mfma"   # fp64 matrix cores
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
     assert sel(desc(kernel="mfma")) == b"mfma"

@@ -134,7 +134,8 @@ def test_minplus_uniform_1024(oracle, lib):
 
 
 @pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f32"), ("plus", "multiplies", "f32"),
-                                ("maximum", "minimum", "f32"), ("bit_xor", "bit_and", "u32"), ("minimum", "plus", "i32")])
+                                ("maximum", "minimum", "f32"), ("bit_xor", "bit_and", "u32"), ("minimum", "plus", "i32"),
+                                ("maximum", "plus", "f64"), ("maximum", "minimum", "f64"), ("plus", "multiplies", "f64")])
 @pytest.mark.parametrize("shape", [(128, 128, 16), (128, 128, 64), (256, 384, 100), (64, 4, 8), (4, 4, 4),
                                    (516, 260, 52), (132, 388, 1028), (1024, 1024, 1024)])
 @pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"])
@@ -153,6 +154,8 @@ def test_splitk_direct(oracle, lib, slices):
     run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", "direct", False, splitk=slices)
     run(oracle, "minimum", "plus", "f32", 100, 60, 332, "col", "col", "col", "direct", True, splitk=slices)
     run(oracle, "bit_xor", "bit_and", "u32", 260, 132, 520, "col", "row", "row", "direct", True, splitk=slices)
+    run(oracle, "maximum", "plus", "f64", 260, 132, 520, "col", "row", "row", "direct", True, splitk=slices)
+    run(oracle, "maximum", "minimum", "f64", 128, 64, 1000, "row", "col", "row", "direct", False, splitk=slices)
 
 
 @pytest.mark.parametrize("shape", [(128, 128, 16), (256, 384, 100), (64, 4, 8), (516, 260, 52), (1024, 1024, 1024)])
