@@ -12,7 +12,8 @@ the timed region.
 
 Other workloads (same JSON shape; one step = one SRGEMM on fixed inputs):
     maxplus_f64, maxmin_f64   fp64, M=N=K=8192, column-major, U[-1,1), beta = one with a seeded C
-    splitk                    fp32 min-plus, M=N=256, K=65536, --slices S (two kernels per step)
+    splitk                    fp32 min-plus, M=N=256, K=65536, --slices S (two kernels per step);
+                              --serial runs the serial form (the reference's SplitKSerial = true)
     xorand_u32                GF(2) product on bit-packed uint32 words, 4096^3
     plustimes_f32             fp32 plus-times on the matrix cores, 4096^3, N(0,1)
     plustimes_f64             fp64 plus-times on the matrix cores, 4096^3, N(0,1)
@@ -104,13 +105,16 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         dD = torch.empty(m, n, device=dev)
         ws = torch.empty(cuasr_amd.splitk_workspace_bytes(m, n, args.slices, "f32") // 4, dtype=torch.float32, device=dev)
 
-        def step(i):
-            cuasr_amd.srgemm_splitk("minimum", "plus", dA, dB, dC, dD, args.slices, ws, 0.0, 0.0, inf, 0.0)
+        run = cuasr_amd.srgemm_splitk_serial if args.serial else cuasr_amd.srgemm_splitk
 
+        def step(i):
+            run("minimum", "plus", dA, dB, dC, dD, args.slices, ws, 0.0, 0.0, inf, 0.0)
+
+        form = "serial-form split-K (ordered chain of epilogues)" if args.serial else "split-K"
         return dict(step=step, m=m, n=n, k=k, dtype="f32", desc=None, host=("minimum", "plus", A, B, C, 0.0, 0.0, np.inf),
-                    metric=f"fp32 min-plus split-K SRGEMM GOPS at {m}x{n}x{k}, {args.slices} slices (2 ops/term)",
-                    workload=f"split-K min-plus SRGEMM fp32, M=N={m}, K={k}, K contiguous in A and B, U[0,10), "
-                             f"{args.slices} slices: partial tiles to a workspace, then a min-reduction kernel",
+                    metric=f"fp32 min-plus {form} SRGEMM GOPS at {m}x{n}x{k}, {args.slices} slices (2 ops/term)",
+                    workload=f"{form} min-plus SRGEMM fp32, M=N={m}, K={k}, K contiguous in A and B, U[0,10), "
+                             f"{args.slices} slices: partial tiles to a workspace, then a reduction kernel",
                     bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5, slices=args.slices)
 
     if w == "xorand_u32":
@@ -174,6 +178,7 @@ def main():
                     choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64"])
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")
+    ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",

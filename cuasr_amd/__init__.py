@@ -84,6 +84,10 @@ def load():
         lib.cuasr_amd_splitk_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk.restype = ctypes.c_int
         lib.cuasr_amd_srgemm_splitk.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_splitk_serial_workspace_bytes.restype = ctypes.c_size_t
+        lib.cuasr_amd_splitk_serial_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
+        lib.cuasr_amd_srgemm_splitk_serial.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm_splitk_serial.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
         lib.cuasr_amd_selected_kernel.restype = ctypes.c_char_p
         lib.cuasr_amd_selected_kernel.argtypes = [ctypes.POINTER(SrgemmDesc)]
         _lib = lib
@@ -251,4 +255,31 @@ def srgemm_splitk(add_op, mult_op, A, B, C, D, slices, workspace, alpha=None, be
     st = load().cuasr_amd_srgemm_splitk(ctypes.byref(desc), ctypes.c_void_p(ws or None), _stream_handle(stream))
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_srgemm_splitk")
+    return D
+
+
+def splitk_serial_workspace_bytes(m, n, slices, dtype):
+    desc = SrgemmDesc()
+    desc.m, desc.n, desc.split_k_slices, desc.dtype = m, n, slices, DTYPES[dtype]
+    return int(load().cuasr_amd_splitk_serial_workspace_bytes(ctypes.byref(desc)))
+
+
+def srgemm_splitk_serial(add_op, mult_op, A, B, C, D, slices, workspace, alpha=None, beta=None,
+                         add_identity=None, mult_identity=None, dtype=None, kernel="auto",
+                         stream=None, alpha_ptr=None, beta_ptr=None, infinities=False):
+    """Serial split-K SRGEMM (the reference's ``SplitKSerial = true``): the result is the chain
+    D_0 = add(mult(alpha, acc_0), mult(beta, C)), D_z = add(mult(alpha, acc_z), mult(one, D_{z-1})).
+    ``workspace``: device memory of >= splitk_serial_workspace_bytes (None when slices == 1)."""
+    dtype = dtype or _torch_dtype_name(D)
+    alpha = op_identity(mult_op, dtype, infinities) if alpha is None else alpha
+    beta = op_annihilator(mult_op, dtype, infinities) if beta is None else beta
+    add_identity = op_identity(add_op, dtype, infinities) if add_identity is None else add_identity
+    mult_identity = op_identity(mult_op, dtype, infinities) if mult_identity is None else mult_identity
+    desc = make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,
+                     slices, kernel, alpha_ptr, beta_ptr)
+    ws = workspace.data_ptr() if hasattr(workspace, "data_ptr") else workspace
+    st = load().cuasr_amd_srgemm_splitk_serial(ctypes.byref(desc), ctypes.c_void_p(ws or None),
+                                               _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_srgemm_splitk_serial")
     return D

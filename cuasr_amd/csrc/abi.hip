@@ -227,26 +227,45 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
   return elem_size(desc->dtype) * size_t(desc->m) * size_t(desc->n) * size_t(desc->split_k_slices);
 }
 
-int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
+// Both split-K forms: partial products of the K-slices into the workspace, then one
+// reduction kernel (`serial` picks the ordered replay of the serial form's epilogues).
+static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream, bool serial) {
   const int st = validate(desc, true);
   if (st != CUASR_AMD_SUCCESS) return st;
   if (!workspace) return CUASR_AMD_ERROR_WORKSPACE_NULL;
   if (reinterpret_cast<uintptr_t>(workspace) % elem_size(desc->dtype)) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
   Problem p = canonical(desc);
   p.slices = desc->split_k_slices;
-  // slice extent: whole k-tiles of 16, spread evenly; trailing slices may be
-  // empty and then hold the additive identity
-  const int tile = 16;
+  // slice extent: whole k-tiles, spread evenly; trailing slices may be empty and then
+  // hold the additive identity.  The serial form's result can depend on where the
+  // slices end (alpha multiplies every partial), so it keeps the reference's extent,
+  // ceil(ceil(K / 8) / S) * 8 (include/cuasr/gemm/kernel/srgemm.h:97-100); the parallel
+  // form's cannot, beyond the rounding of sums, and uses this library's k-tile of 16.
+  const int tile = serial ? 8 : 16;
   const long long tiles = (p.k + tile - 1) / tile;
   const long long per = (tiles + p.slices - 1) / p.slices;
   p.k_per_slice = int(per * tile > 0 ? per * tile : tile);
   p.workspace = workspace;
   const launch_fn fn = family_fn(pick_family(desc), desc);
-  const launch_fn red = find_reduce(desc->dtype);
+  const launch_fn red = serial ? find_reduce_serial(desc->dtype) : find_reduce(desc->dtype);
   if (!fn || !red) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
   return red(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+}
+
+int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
+  return run_splitk(desc, workspace, stream, false);
+}
+
+size_t cuasr_amd_splitk_serial_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
+  if (!desc || desc->split_k_slices <= 1) return 0;
+  return cuasr_amd_splitk_workspace_bytes(desc);
+}
+
+int cuasr_amd_srgemm_splitk_serial(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
+  if (desc && desc->split_k_slices == 1) return cuasr_amd_srgemm(desc, stream);  // no workspace, no reduction
+  return run_splitk(desc, workspace, stream, true);
 }
 
 }  // extern "C"

@@ -3,7 +3,8 @@
 //     pair the element type defines, and serves as an on-device cross-check;
 //   * the split-K reduction: D = epilogue(add over slices of workspace, C),
 //     the second kernel of the parallel split-K
-//     (include/cuasr/reduction/kernel/reduce_split_k.h:146-237).
+//     (include/cuasr/reduction/kernel/reduce_split_k.h:146-237), and its
+//     ordered variant that replays the serial split-K's chain of epilogues.
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -117,7 +118,76 @@ __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
   }
 }
 
-template <typename T> static hipError_t launch_reduce(const Problem &p, hipStream_t s) {
+// The ordered fold of the serial split-K.  In the reference the workgroups of one
+// output tile take turns, slice 0 first: slice 0 writes
+// D = add(mult(alpha, acc_0), mult(beta, C)) (or mult(alpha, acc_0) when the source
+// is not needed), every later slice z reads D back as its source with beta replaced
+// by the multiplicative identity and writes D = add(mult(alpha, acc_z), mult(one, D))
+// (include/cuasr/gemm/kernel/srgemm.h:249-320,
+// epilogue/thread/semiring_linear_combination.h:119-134).  Here the slices' raw
+// accumulators are in the workspace and one thread replays that chain for its
+// elements in registers: same operands, same order, one write of D.
+template <typename T, int V, bool VOUT>
+__global__ __launch_bounds__(256) void reduce_serial_kernel(Problem p) {
+  const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
+  const T one = scalar_as<T>(p.mult_identity);
+  // "source needed" as a later slice's epilogue evaluates it, with beta = one
+  const bool chain = e.ident != apply_op<T>(p.mult_op, one, one);
+  const long long per_row = (p.n + V - 1) / V;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= per_row * p.m) return;
+  const int i = int(idx / per_row);
+  const int j = int(idx % per_row) * V;
+  const long long slice = (long long)p.m * p.n;
+  const T *ws = reinterpret_cast<const T *>(p.workspace) + (long long)i * p.n + j;
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const T *C = reinterpret_cast<const T *>(p.C);
+  T out[V];
+  {
+    const vec_t w = *reinterpret_cast<const vec_t *>(ws);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      out[v] = apply_op<T>(p.mult_op, e.alpha, w[v]);
+      if (e.source_needed && j + v < p.n)
+        out[v] = apply_op<T>(p.add_op, out[v], apply_op<T>(p.mult_op, e.beta, C[(long long)i * p.ldc + j + v]));
+    }
+  }
+  auto step = [&](const vec_t &w) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const T lhs = apply_op<T>(p.mult_op, e.alpha, w[v]);
+      out[v] = chain ? apply_op<T>(p.add_op, lhs, apply_op<T>(p.mult_op, one, out[v])) : lhs;
+    }
+  };
+  constexpr int U = 8;  // loads in flight per thread, as in the parallel reduction
+  int s = 1;
+  for (; s + U <= p.slices; s += U) {
+    vec_t w[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) w[u] = *reinterpret_cast<const vec_t *>(ws + (s + u) * slice);
+#pragma unroll
+    for (int u = 0; u < U; ++u) step(w[u]);
+  }
+  for (; s < p.slices; ++s) step(*reinterpret_cast<const vec_t *>(ws + s * slice));
+  T *dst = reinterpret_cast<T *>(p.D) + (long long)i * p.ldd + j;
+  if (V > 1 && VOUT) {
+    vec_t o;
+#pragma unroll
+    for (int v = 0; v < V; ++v) o[v] = out[v];
+    *reinterpret_cast<vec_t *>(dst) = o;
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      if (j + v < p.n) dst[v] = out[v];
+  }
+}
+
+template <typename T, bool SERIAL, int V, bool VOUT> static void launch_one(const Problem &p, dim3 grid, hipStream_t s) {
+  if (SERIAL) hipLaunchKernelGGL((reduce_serial_kernel<T, V, VOUT>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((reduce_splitk_kernel<T, V, VOUT>), grid, dim3(256), 0, s, p);
+}
+
+template <typename T, bool SERIAL> static hipError_t launch_reduce(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   constexpr int V = 16 / sizeof(T);
   const bool vec = (p.n % V == 0) && (reinterpret_cast<uintptr_t>(p.workspace) % 16 == 0);
@@ -126,23 +196,31 @@ template <typename T> static hipError_t launch_reduce(const Problem &p, hipStrea
   if (vec && !small) {
     const long long work = (long long)p.m * (p.n / V);
     const dim3 grid((unsigned)((work + 255) / 256));
-    if (reinterpret_cast<uintptr_t>(p.D) % 16 == 0 && p.ldd % V == 0)
-      hipLaunchKernelGGL((reduce_splitk_kernel<T, V, true>), grid, dim3(256), 0, s, p);
-    else
-      hipLaunchKernelGGL((reduce_splitk_kernel<T, V, false>), grid, dim3(256), 0, s, p);
+    if (reinterpret_cast<uintptr_t>(p.D) % 16 == 0 && p.ldd % V == 0) launch_one<T, SERIAL, V, true>(p, grid, s);
+    else launch_one<T, SERIAL, V, false>(p, grid, s);
   } else {
     const long long work = (long long)p.m * p.n;
-    hipLaunchKernelGGL((reduce_splitk_kernel<T, 1, false>), dim3((unsigned)((work + 255) / 256)), dim3(256), 0, s, p);
+    launch_one<T, SERIAL, 1, false>(p, dim3((unsigned)((work + 255) / 256)), s);
   }
   return hipGetLastError();
 }
 
 launch_fn find_reduce(int dtype) {
   switch (dtype) {
-    case CUASR_AMD_F32: return launch_reduce<float>;
-    case CUASR_AMD_F64: return launch_reduce<double>;
-    case CUASR_AMD_I32: return launch_reduce<int32_t>;
-    case CUASR_AMD_U32: return launch_reduce<uint32_t>;
+    case CUASR_AMD_F32: return launch_reduce<float, false>;
+    case CUASR_AMD_F64: return launch_reduce<double, false>;
+    case CUASR_AMD_I32: return launch_reduce<int32_t, false>;
+    case CUASR_AMD_U32: return launch_reduce<uint32_t, false>;
+    default: return nullptr;
+  }
+}
+
+launch_fn find_reduce_serial(int dtype) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return launch_reduce<float, true>;
+    case CUASR_AMD_F64: return launch_reduce<double, true>;
+    case CUASR_AMD_I32: return launch_reduce<int32_t, true>;
+    case CUASR_AMD_U32: return launch_reduce<uint32_t, true>;
     default: return nullptr;
   }
 }

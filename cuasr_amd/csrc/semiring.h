@@ -138,5 +138,6 @@ launch_fn find_naive(int dtype);
 launch_fn find_valu(int dtype, int add_op, int mult_op);
 launch_fn find_mfma(int dtype, int add_op, int mult_op);
 launch_fn find_reduce(int dtype);
+launch_fn find_reduce_serial(int dtype);
 
 }  // namespace cuasr_amd

@@ -126,30 +126,46 @@ class Srgemm {
           split_k_slices(split_k_slices_) {}
   };
 
-  Srgemm() : ready_(false) {}
+  Srgemm() : workspace_(nullptr), ready_(false) {}
 
-  /// kErrorInvalidProblem when split_k_slices > 1: serial split-K (a
-  /// semaphore-ordered in-place reduction in the reference) is not offered;
-  /// use SrgemmSplitKParallel.
+  /// kErrorInvalidProblem when split_k_slices > 1 and SplitKSerial is false
+  /// (reference: srgemm.h:198-200).
   static Status can_implement(Arguments const &args) {
-    if (args.split_k_slices > 1) return kSplitKSerial ? Status::kErrorNotSupported : Status::kErrorInvalidProblem;
+    if (!kSplitKSerial && args.split_k_slices > 1) return Status::kErrorInvalidProblem;
+    if (args.split_k_slices < 1) return Status::kErrorInvalidProblem;
     cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    d.split_k_slices = 1;  // the slice count is checked above; the rest is the plain problem's check
     return static_cast<Status>(cuasr_amd_srgemm_can_implement(&d));
   }
 
-  static size_t get_workspace_size(Arguments const &) { return 0; }
+  /// Serial split-K: bytes of device workspace `initialize` must be given
+  /// (reference: srgemm.h:218-234).  The reference needs one int per output tile
+  /// for its semaphores; this library needs the slices' partial products,
+  /// sizeof(ElementC) * M * N * split_k_slices, so size the workspace with this
+  /// function, as the reference's callers do.
+  static size_t get_workspace_size(Arguments const &args) {
+    if (!kSplitKSerial || args.split_k_slices <= 1) return 0;
+    cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    return cuasr_amd_splitk_serial_workspace_bytes(&d);
+  }
 
-  Status initialize(Arguments const &args, void * /*workspace*/ = nullptr, hipStream_t /*stream*/ = nullptr) {
+  /// kErrorWorkspaceNull for a serial split-K without workspace (reference:
+  /// srgemm.h:246-251).  Nothing is cleared: the workspace carries no state
+  /// from one run to the next.
+  Status initialize(Arguments const &args, void *workspace = nullptr, hipStream_t /*stream*/ = nullptr) {
     Status s = can_implement(args);
     if (s != Status::kSuccess) return s;
+    if (kSplitKSerial && args.split_k_slices > 1 && !workspace) return Status::kErrorWorkspaceNull;
     desc_ = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    workspace_ = workspace;
     ready_ = true;
     return Status::kSuccess;
   }
 
   /// Lightweight refresh of the operand pointers (reference: srgemm.h:285-300).
-  Status update(Arguments const &args, void * /*workspace*/ = nullptr) {
+  Status update(Arguments const &args, void *workspace = nullptr) {
     if (!ready_) return Status::kErrorInternal;
+    if (kSplitKSerial && args.split_k_slices > 1 && !workspace) return Status::kErrorWorkspaceNull;
     desc_.A = args.ref_A.data();
     desc_.B = args.ref_B.data();
     desc_.C = args.ref_C.data();
@@ -158,11 +174,14 @@ class Srgemm {
     desc_.beta = make_scalar<ElementC>(args.epilogue.beta);
     desc_.alpha_ptr = args.epilogue.alpha_ptr;
     desc_.beta_ptr = args.epilogue.beta_ptr;
+    workspace_ = workspace;
     return Status::kSuccess;
   }
 
   Status run(hipStream_t stream = nullptr) {
     if (!ready_) return Status::kErrorInternal;
+    if (kSplitKSerial && desc_.split_k_slices > 1)
+      return static_cast<Status>(cuasr_amd_srgemm_splitk_serial(&desc_, workspace_, stream));
     return static_cast<Status>(cuasr_amd_srgemm(&desc_, stream));
   }
 
@@ -175,6 +194,7 @@ class Srgemm {
 
  private:
   cuasr_amd_srgemm_desc desc_;
+  void *workspace_;
   bool ready_;
 };
 

@@ -20,6 +20,8 @@
  *                                     include/cuasr/gemm/device/srgemm_splitk_parallel.h:226-235
  *   cuasr_amd_srgemm_splitk           device::SrgemmSplitKParallel::initialize/run
  *                                     include/cuasr/gemm/device/srgemm_splitk_parallel.h:238-357
+ *   cuasr_amd_srgemm_splitk_serial    device::Srgemm<..., SplitKSerial = true>
+ *                                     include/cuasr/gemm/device/srgemm.h:218-282
  *   status codes                      cutlass::Status as used by the reference
  *                                     test/device/testbed.h:24-46
  */
@@ -161,6 +163,24 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
  * (device/srgemm_splitk_parallel.h:247-249). */
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
                             void *stream);
+
+/* Serial split-K (device::Srgemm with SplitKSerial = true,
+ * include/cuasr/gemm/device/srgemm.h:218-282; include/cuasr/gemm/kernel/srgemm.h:249-320).
+ * The result is the reference's chain of epilogues, slice 0 first:
+ *   D_0 = add(mult(alpha, acc_0), mult(beta, C))     (mult(alpha, acc_0) if C is not needed)
+ *   D_z = add(mult(alpha, acc_z), mult(mult_identity, D_{z-1}))   for z = 1 .. slices-1
+ * The reference orders the slices' workgroups with one semaphore per output tile
+ * and reduces in place in D, so its workspace is one int per tile.  Here the
+ * slices run unordered into the workspace and one reduction kernel replays the
+ * chain, so the workspace holds the partial products: callers must size it with
+ * cuasr_amd_splitk_serial_workspace_bytes, which returns
+ * sizeof(element) * m * n * split_k_slices, or 0 when split_k_slices == 1
+ * (then the call is cuasr_amd_srgemm and the workspace may be NULL).
+ * CUASR_AMD_ERROR_WORKSPACE_NULL when split_k_slices > 1 and workspace is NULL
+ * (device/srgemm.h:248-251). */
+size_t cuasr_amd_splitk_serial_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
+int cuasr_amd_srgemm_splitk_serial(const cuasr_amd_srgemm_desc *desc, void *workspace,
+                                   void *stream);
 
 /* Name of the kernel family AUTO would choose for this descriptor
  * ("naive", "valu", "valu_direct", "mfma"), or NULL if the descriptor is invalid. */

@@ -40,6 +40,7 @@ def lib():
         _lib = ctypes.CDLL(_LIB_PATH)
         _lib.oracle_srgemm.restype = ctypes.c_int
         _lib.oracle_srgemm_splitk.restype = ctypes.c_int
+        _lib.oracle_srgemm_splitk_serial.restype = ctypes.c_int
         _lib.oracle_max_threads.restype = ctypes.c_int
     return _lib
 
@@ -129,4 +130,29 @@ def srgemm_splitk(add_op, mult_op, A, B, C, alpha, beta, add_identity,
         int(slices), int(tbk), int(nthreads))
     if rc != 0:
         raise ValueError(f"oracle: unsupported split-K ({dt}, {add_op}, {mult_op})")
+    return D
+
+
+def srgemm_splitk_serial(add_op, mult_op, A, B, C, alpha, beta, add_identity,
+                         mult_identity, slices, tbk=8, out=None, nthreads=0):
+    """CPU model of the serial split-K: the slices' epilogues chained through D."""
+    dt = A.dtype
+    m, k = A.shape
+    _, n = B.shape
+    D = out if out is not None else empty_like_layout(C)
+    pa, lda, la = mat_ref(A)
+    pb, ldb, lb = mat_ref(B)
+    pc, ldc, lc = mat_ref(C)
+    pd, ldd, _ = mat_ref(D)
+    al, be = _scalar(alpha, dt), _scalar(beta, dt)
+    ident, one = _scalar(add_identity, dt), _scalar(mult_identity, dt)
+    rc = lib().oracle_srgemm_splitk_serial(
+        DTYPES[dt], OPS[add_op], OPS[mult_op], m, n, k,
+        al.ctypes.data_as(ctypes.c_void_p), pa, ctypes.c_int64(lda), la,
+        pb, ctypes.c_int64(ldb), lb, be.ctypes.data_as(ctypes.c_void_p),
+        pc, ctypes.c_int64(ldc), pd, ctypes.c_int64(ldd), lc,
+        ident.ctypes.data_as(ctypes.c_void_p), one.ctypes.data_as(ctypes.c_void_p),
+        int(slices), int(tbk), int(nthreads))
+    if rc != 0:
+        raise ValueError(f"oracle: unsupported serial split-K ({dt}, {add_op}, {mult_op})")
     return D

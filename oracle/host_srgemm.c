@@ -40,6 +40,16 @@
  *     source = C if needed else identity; D = add(mult(alpha,acc), mult(beta,source))
  *   include/cuasr/gemm/epilogue/thread/semiring_linear_combination.h:118-125
  *     source needed  <=>  add_identity != mult(beta, mult_identity)
+ *
+ * The serial split-K model follows
+ *   include/cuasr/gemm/kernel/srgemm.h:97-100, :184-189
+ *     slice extent = ceil(ceil(K / tbk) / S) * tbk, slice z ends at min(K, (z+1) * extent)
+ *   include/cuasr/gemm/kernel/srgemm.h:220-225, :249-320
+ *     slices take turns on D in ascending order; slice 0's source is C, a later
+ *     slice's source is D; a slice with no k range keeps acc = identity and still
+ *     runs its epilogue
+ *   include/cuasr/gemm/epilogue/thread/semiring_linear_combination.h:129-134, :152-183
+ *     a later slice's beta is mult_identity; an unneeded source drops the add
  */
 #include <stdint.h>
 #include <stdlib.h>
@@ -86,6 +96,8 @@ typedef struct {
   const void *partials; /* if non-NULL: S row-major m x n slices to reduce   */
   int slices;
   int skip_source_if_unneeded; /* device-style epilogue (reduce kernel model) */
+  int no_source_form;   /* with the above: an unneeded source drops the add,
+                           D = mult(alpha, acc) (the SRGEMM kernel's epilogue) */
 } job_t;
 
 /*
@@ -167,7 +179,8 @@ typedef struct {
                 const T src = need ? C[oc] : ident;                             \
                 const T lhs = MUL(alpha, acc[j][i]);                            \
                 const T rhs = MUL(beta, src);                                   \
-                D[od] = ADD(lhs, rhs);                                          \
+                if (!need && jb->no_source_form) D[od] = lhs;                   \
+                else D[od] = ADD(lhs, rhs);                                     \
               }                                                                 \
           }                                                                     \
         }                                                                       \
@@ -344,5 +357,45 @@ int oracle_srgemm_splitk(int dtype, int add_op, int mult_op, int m, int n, int k
   jb.skip_source_if_unneeded = 1;
   fn(&jb);
   free(ws);
+  return 0;
+}
+
+/* CPU model of the serial split-K: the slices' epilogues applied to D one after
+ * the other, slice 0 first.  tbk is the tile depth the slice extent is rounded
+ * to (8 in every reference default). */
+int oracle_srgemm_splitk_serial(int dtype, int add_op, int mult_op, int m, int n,
+                                int k, const void *alpha, const void *A,
+                                int64_t lda, int layout_a, const void *B,
+                                int64_t ldb, int layout_b, const void *beta,
+                                const void *C, int64_t ldc, void *D, int64_t ldd,
+                                int layout_c, const void *add_identity,
+                                const void *mult_identity, int slices, int tbk,
+                                int nthreads) {
+  kernel_fn fn = lookup(dtype, add_op, mult_op, 0);
+  if (!fn || slices < 1 || tbk < 1) return -1;
+  job_t jb;
+  memset(&jb, 0, sizeof jb);
+  jb.m = m; jb.n = n; jb.k = k;
+  jb.A = A; jb.B = B; jb.D = D;
+  jb.alpha = alpha; jb.add_identity = add_identity;
+  jb.mult_identity = mult_identity;
+  jb.skip_source_if_unneeded = 1;
+  jb.no_source_form = 1;
+  set_threads(nthreads);
+  const int64_t iters = ((int64_t)k + tbk - 1) / tbk;
+  const int64_t ks = ((iters + slices - 1) / slices) * tbk;
+  for (int z = 0; z < slices; ++z) {
+    const int64_t b = z * ks, e = (z + 1) * ks;
+    jb.k_begin = (int)(b < k ? b : k);
+    jb.k_end = (int)(e < k ? e : k);
+    if (z == 0) {
+      jb.C = C; jb.beta = beta;
+      set_strides(&jb, layout_a, lda, layout_b, ldb, layout_c, ldc, ldd);
+    } else {
+      jb.C = D; jb.beta = mult_identity;
+      set_strides(&jb, layout_a, lda, layout_b, ldb, layout_c, ldd, ldd);
+    }
+    fn(&jb);
+  }
   return 0;
 }

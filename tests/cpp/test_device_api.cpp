@@ -70,9 +70,13 @@ template <typename T> struct DeviceBuf {
 template <typename L> static long long ld_of(int rows, int cols) { return std::is_same<L, ColumnMajor>::value ? rows : cols; }
 
 // one testbed case: device operator vs host reference, bit-exact
-template <typename Add, typename Mul, typename T, typename LA, typename LB, typename LC>
-static bool testbed_case(int m, int n, int k, T alpha, T beta) {
-  using Op = cuasr::gemm::device::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T>;
+template <typename Add, typename Mul, typename T, typename LA, typename LB, typename LC, bool SERIAL = false>
+static bool testbed_case(int m, int n, int k, T alpha, T beta, int slices = 1) {
+  using Plain = cuasr::gemm::device::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T>;
+  using Op = cuasr::gemm::device::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T, typename Plain::OperatorClass,
+                                         typename Plain::ArchTag, typename Plain::ThreadblockShape, typename Plain::WarpShape,
+                                         typename Plain::InstructionShape, typename Plain::EpilogueOutputOp,
+                                         typename Plain::ThreadblockSwizzle, Plain::kStages, 1, 1, SERIAL>;
   const long long lda = ld_of<LA>(m, k), ldb = ld_of<LB>(k, n), ldc = ld_of<LC>(m, n);
   std::vector<T> A(size_t(m) * k), B(size_t(k) * n), C(size_t(m) * n), D(size_t(m) * n, T(0)), R(size_t(m) * n, T(0));
   fill_int(A, 2019, -8, 8);
@@ -80,10 +84,11 @@ static bool testbed_case(int m, int n, int k, T alpha, T beta) {
   fill_int(C, 2017, -8, 8);
   A[0] = B[0] = C[0] = T(1);  // as the reference testbed does (testbed.h:142-144)
   DeviceBuf<T> dA(A), dB(B), dC(C), dD(D);
-  typename Op::Arguments args({m, n, k}, {dA.p, lda}, {dB.p, ldb}, {dC.p, ldc}, {dD.p, ldc}, {alpha, beta});
+  typename Op::Arguments args({m, n, k}, {dA.p, lda}, {dB.p, ldb}, {dC.p, ldc}, {dD.p, ldc}, {alpha, beta}, slices);
   Op op;
   if (Op::can_implement(args) != Status::kSuccess) return false;
-  if (op(args) != Status::kSuccess) return false;
+  DeviceBuf<uint8_t> ws(Op::get_workspace_size(args) + 16);  // as the reference testbed does (testbed.h:228-240)
+  if (op(args, ws.p) != Status::kSuccess) return false;
   HIP_OK(hipDeviceSynchronize());
   cuasr::reference::host::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T, T> ref;
   ref({m, n, k}, alpha, {A.data(), lda}, {B.data(), ldb}, beta, {C.data(), ldc}, {R.data(), ldc}, Add::Identity);
@@ -103,6 +108,21 @@ template <typename Add, typename Mul, typename T> static void testbed_sweep(cons
         ok = ok && testbed_case<Add, Mul, T, ColumnMajor, RowMajor, RowMajor>(m, n, k, alpha, Mul::Identity);
         ok = ok && testbed_case<Add, Mul, T, RowMajor, RowMajor, ColumnMajor>(m, n, k, alpha, Mul::Identity);
       }
+  report(ok, name);
+}
+
+// the reference sweep adds split_k_slices = 2, 3, 8 for operators with SplitKSerial (testbed.h:322-338)
+template <typename Add, typename Mul, typename T> static void testbed_sweep_serial(const char *name) {
+  bool ok = true;
+  const int ms[2] = {1, 509}, ns[2] = {1, 510}, ks[2] = {1, 23};
+  for (int slices : {1, 2, 3, 8})
+    for (int m : ms)
+      for (int n : ns)
+        for (int k : ks) {
+          const T alpha = Mul::Identity;
+          ok = ok && testbed_case<Add, Mul, T, ColumnMajor, ColumnMajor, ColumnMajor, true>(m, n, k, alpha, Mul::Annihilator, slices);
+          ok = ok && testbed_case<Add, Mul, T, RowMajor, ColumnMajor, RowMajor, true>(m, n, k, alpha, Mul::Identity, slices);
+        }
   report(ok, name);
 }
 
@@ -223,6 +243,39 @@ static void example_splitk() {
       report(ok, name);
     }
   }
+  // SplitKSerial = true on the plain operator (device/srgemm.h:83, :218-282): the testbed sizes the workspace
+  // with get_workspace_size (testbed.h:228-240); min is idempotent and order-free, so the serial chain
+  // equals the unsplit product bit for bit
+  using Serial = cuasr::gemm::device::Srgemm<Add, Mul, float, RowMajor, float, ColumnMajor, float, RowMajor, float,
+                                             Plain::OperatorClass, Plain::ArchTag, Plain::ThreadblockShape, Plain::WarpShape,
+                                             Plain::InstructionShape, Plain::EpilogueOutputOp, Plain::ThreadblockSwizzle,
+                                             Plain::kStages, 1, 1, true>;
+  static_assert(Serial::kSplitKSerial && !Plain::kSplitKSerial, "kSplitKSerial");
+  for (int slices : {1, 2, 3, 8}) {
+    Serial::Arguments args({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d1.p, N}, {Mul::Identity, Mul::Identity}, slices);
+    const size_t bytes = Serial::get_workspace_size(args);
+    DeviceBuf<uint8_t> ws(bytes ? bytes : 16);
+    Serial op;
+    bool ok = bytes == (slices > 1 ? sizeof(float) * size_t(M) * N * slices : 0);
+    ok = ok && Serial::can_implement(args) == Status::kSuccess;
+    if (slices > 1) ok = ok && op.initialize(args, nullptr) == Status::kErrorWorkspaceNull;
+    ok = ok && op.initialize(args, slices > 1 ? ws.p : nullptr) == Status::kSuccess && op() == Status::kSuccess;
+    Plain::Arguments pargs({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {Mul::Identity, Mul::Identity});
+    Plain plain;
+    ok = ok && plain(pargs) == Status::kSuccess;
+    HIP_OK(hipDeviceSynchronize());
+    ok = ok && d1.download() == d2.download();
+    // update(): new output pointer, workspace handed over again (device/srgemm.h:285-300)
+    DeviceBuf<float> d3(std::vector<float>(M * N, 0.f));
+    Serial::Arguments args3({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d3.p, N}, {Mul::Identity, Mul::Identity}, slices);
+    if (slices > 1) ok = ok && op.update(args3, nullptr) == Status::kErrorWorkspaceNull;
+    ok = ok && op.update(args3, slices > 1 ? ws.p : nullptr) == Status::kSuccess && op.run() == Status::kSuccess;
+    HIP_OK(hipDeviceSynchronize());
+    ok = ok && d3.download() == d2.download();
+    char name[96];
+    std::snprintf(name, sizeof name, "serial split-K (SplitKSerial = true) == non-split, slices=%d", slices);
+    report(ok, name);
+  }
   // split_k_slices > 1 on the plain operator is an invalid problem (device/srgemm.h:198-200)
   Plain::Arguments bad({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {Mul::Identity, Mul::Identity}, 4);
   report(Plain::can_implement(bad) == Status::kErrorInvalidProblem && Plain().operator()(bad) == Status::kErrorInvalidProblem,
@@ -283,6 +336,11 @@ int main() {
   testbed_sweep<cuasr::minimum<double>, cuasr::maximum<double>, double>("testbed minimum-maximum f64");
   testbed_sweep<cuasr::maximum<double>, cuasr::minimum<double>, double>("testbed maximum-minimum f64");
   testbed_sweep<cuasr::binary_or<double>, cuasr::binary_and<double>, double>("testbed or-and f64");
+  testbed_sweep_serial<cuasr::plus<float>, cuasr::multiplies<float>, float>("testbed serial split-K plus-multiplies f32");
+  testbed_sweep_serial<cuasr::minimum<float>, cuasr::plus<float>, float>("testbed serial split-K minimum-plus f32");
+  testbed_sweep_serial<cuasr::maximum<double>, cuasr::plus<double>, double>("testbed serial split-K maximum-plus f64");
+  testbed_sweep_serial<cuasr::maximum<double>, cuasr::minimum<double>, double>("testbed serial split-K maximum-minimum f64");
+  testbed_sweep_serial<cuasr::binary_or<float>, cuasr::binary_and<float>, float>("testbed serial split-K or-and f32");
   testbed_sweep<cuasr::inf::minimum<float>, cuasr::inf::plus<float>, float>("testbed inf::minimum-plus f32");
   testbed_sweep<cuasr::inf::maximum<double>, cuasr::inf::plus_for_max<double>, double>("testbed inf::maximum-plus f64");
   std::printf("%d checks, %d failed\n", g_run, g_fail);

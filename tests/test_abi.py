@@ -20,7 +20,8 @@ def declared_functions():
 def test_exports_match_header(lib):
     names = declared_functions()
     assert {"cuasr_amd_srgemm", "cuasr_amd_srgemm_splitk", "cuasr_amd_splitk_workspace_bytes",
-            "cuasr_amd_srgemm_can_implement"} <= set(names)
+            "cuasr_amd_srgemm_can_implement", "cuasr_amd_srgemm_splitk_serial",
+            "cuasr_amd_splitk_serial_workspace_bytes"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
     assert lib.cuasr_amd_abi_version() == 1
@@ -95,6 +96,19 @@ def test_splitk_host_errors(lib):
     assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
     # the plain entry point refuses split-K descriptors without launching
     assert lib.cuasr_amd_srgemm(ctypes.byref(d), None) == 4
+
+
+def test_serial_splitk_host_errors(lib):
+    # the workspace holds the slices' partial products; none is needed for a single slice (device/srgemm.h:218-234)
+    assert cuasr_amd.splitk_serial_workspace_bytes(256, 256, 8, "f32") == 4 * 256 * 256 * 8
+    assert cuasr_amd.splitk_serial_workspace_bytes(100, 7, 3, "f64") == 8 * 100 * 7 * 3
+    assert cuasr_amd.splitk_serial_workspace_bytes(100, 7, 1, "f64") == 0
+    d = desc(m=256, n=256, k=4096, slices=8)
+    assert lib.cuasr_amd_srgemm_splitk_serial(ctypes.byref(d), None, None) == 6   # kErrorWorkspaceNull (device/srgemm.h:248-251)
+    assert lib.cuasr_amd_srgemm_splitk_serial(ctypes.byref(d), ctypes.c_void_p(0x1002), None) == 1  # misaligned workspace
+    d0 = desc(slices=0)
+    assert lib.cuasr_amd_srgemm_splitk_serial(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
+    assert lib.cuasr_amd_srgemm_splitk_serial(None, None, None) == 4
 
 
 def test_semiring_constants():

@@ -212,3 +212,79 @@ def test_splitk_model(oracle, slices):
     want = oracle.srgemm("plus", "multiplies", Ai, Bi, C, 1.0, 0.0, 0.0)
     got = oracle.srgemm_splitk("plus", "multiplies", Ai, Bi, C, 1.0, 0.0, 0.0, 1.0, slices)
     assert bits(got) == bits(want)
+
+
+def literal_serial_splitk(add, mult, A, B, C, alpha, beta, ident, one, slices, tbk=8):
+    """The serial split-K as the reference's workgroups perform it, in Python scalars: slice z
+    covers k in [z*ks, min(K, (z+1)*ks)) with ks = ceil(ceil(K/tbk)/slices)*tbk
+    (kernel/srgemm.h:97-100, :184-189); its epilogue reads C (z = 0) or D (z > 0, beta replaced
+    by the multiplicative identity) and writes D (kernel/srgemm.h:290-300,
+    semiring_linear_combination.h:129-134); an unneeded source drops the add (:166-183)."""
+    f_add, f_mul = PY_OPS[add], PY_OPS[mult]
+    t = A.dtype.type
+    m, k = A.shape
+    n = B.shape[1]
+    ks = -(-(-(-k // tbk)) // slices) * tbk
+    D = np.zeros((m, n), dtype=A.dtype)
+    with np.errstate(over="ignore", invalid="ignore"):
+        for z in range(slices):
+            b = t(beta) if z == 0 else t(one)
+            need = t(ident) != t(f_mul(b, t(one)))
+            for i in range(m):
+                for j in range(n):
+                    acc = t(ident)
+                    for kk in range(min(k, z * ks), min(k, (z + 1) * ks)):
+                        acc = t(f_add(t(f_mul(A[i, kk], B[kk, j])), acc))
+                    lhs = t(f_mul(t(alpha), acc))
+                    src = C[i, j] if z == 0 else D[i, j]
+                    D[i, j] = t(f_add(lhs, t(f_mul(b, src)))) if need else lhs
+    return D
+
+
+@pytest.mark.parametrize("slices", [1, 2, 3, 5, 8])
+def test_serial_splitk_model_against_literal_chain(oracle, slices):
+    m, n, k = 9, 7, 61
+    inf = np.float32(np.inf)
+    A, B, C = inputs.uniform(11, m, k, -2, 2), inputs.uniform(12, k, n, -2, 2), inputs.uniform(13, m, n, -2, 2)
+    cases = [
+        ("minimum", "plus", 0.25, 0.0, inf, 0.0),          # beta = one: C joins the chain
+        ("minimum", "plus", 0.25, inf, inf, 0.0),          # beta = zero: C is not read
+        ("plus", "multiplies", 1.5, -0.75, 0.0, 1.0),      # rounding depends on the slice boundaries
+        ("minimum", "multiplies", -2.0, 1.0, inf, 1.0),    # alpha < 0: alpha per partial differs from alpha on the total
+        ("maximum", "minimum", 1.0, 0.5, -inf, inf),
+    ]
+    for add, mult, alpha, beta, ident, one in cases:
+        want = literal_serial_splitk(add, mult, A, B, C, alpha, beta, ident, one, slices)
+        got = oracle.srgemm_splitk_serial(add, mult, A, B, C, alpha, beta, ident, one, slices)
+        assert bits(got) == bits(want), (add, mult, slices)
+    Au, Bu, Cu = inputs.words32(14, m, k), inputs.words32(15, k, n), inputs.words32(16, m, n)
+    full = np.uint32(0xFFFFFFFF)
+    want = literal_serial_splitk("bit_xor", "bit_and", Au, Bu, Cu, full, full, 0, full, slices)
+    got = oracle.srgemm_splitk_serial("bit_xor", "bit_and", Au, Bu, Cu, full, full, 0, full, slices)
+    assert bits(got) == bits(want)
+
+
+def test_serial_splitk_model_invariants(oracle):
+    m, n, k = 40, 24, 200
+    inf = np.float32(np.inf)
+    A, B, C = inputs.uniform(1, m, k, 0, 10), inputs.uniform(2, k, n, 0, 10), inputs.uniform(3, m, n, 0, 10)
+    for slices in (1, 2, 3, 8, 16, 40):  # 40 > K/8: trailing slices have no k range
+        for beta in (inf, np.float32(0.0)):
+            # an idempotent, order-free add: the chain equals the unsplit product bit for bit
+            want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, beta, inf)
+            got = oracle.srgemm_splitk_serial("minimum", "plus", A, B, C, 0.0, beta, inf, 0.0, slices)
+            assert bits(got) == bits(want)
+        # an unneeded source is never read: NaN in C must not reach D (the host reference would propagate it)
+        Cn = np.full_like(C, np.nan)
+        got = oracle.srgemm_splitk_serial("minimum", "plus", A, B, Cn, 0.0, inf, inf, 0.0, slices)
+        assert bits(got) == bits(oracle.srgemm("minimum", "plus", A, B, C, 0.0, inf, inf))
+        # D may alias C
+        Cc = C.copy()
+        oracle.srgemm_splitk_serial("minimum", "plus", A, B, Cc, 0.0, 0.0, inf, 0.0, slices, out=Cc)
+        assert bits(Cc) == bits(oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, inf))
+    # plus-times on small integers is exact whatever the slicing; alpha multiplies every partial, beta only C
+    Ai, Bi, Ci = inputs.integers(4, m, k, -8, 8), inputs.integers(5, k, n, -8, 8), inputs.integers(6, m, n, -8, 8)
+    want = oracle.srgemm("plus", "multiplies", Ai, Bi, Ci, 2.0, -3.0, 0.0)
+    for slices in (2, 7):
+        got = oracle.srgemm_splitk_serial("plus", "multiplies", Ai, Bi, Ci, 2.0, -3.0, 0.0, 1.0, slices)
+        assert bits(got) == bits(want)
