@@ -17,6 +17,7 @@ Other workloads (same JSON shape; one step = one SRGEMM on fixed inputs):
     xorand_u32                GF(2) product on bit-packed uint32 words, 4096^3
     plustimes_f32             fp32 plus-times on the matrix cores, 4096^3, N(0,1)
     plustimes_f64             fp64 plus-times on the matrix cores, 4096^3, N(0,1)
+    srgemm                    any --add / --mult / --dtype / --layouts at --size (the reference's benchmark matrix)
 """
 import argparse
 import json
@@ -166,6 +167,39 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
                     workload=f"plus-times SRGEMM fp64 on the matrix cores, M=N=K={n}, column-major, N(0,1), C = 0",
                     bound="mfma", peak=FP64_VECTOR_PEAK, instr_per_term=None)
 
+    if w == "srgemm":
+        # any operator pair / element type / layout combination at one size: the reference's
+        # benchmark matrix (bench/device/harness.h:157-181 counts 2 * N^3 / t the same way)
+        n = args.size or 4096
+        add, mult, dt = args.add, args.mult, args.dtype
+        npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}[dt]
+        la, lb, lc = ["F" if c == "c" else "C" for c in args.layouts]
+        if dt in ("f32", "f64"):
+            A, B, C = (inputs.uniform(701 + i, n, n, -1.0, 1.0, npd, o) for i, o in enumerate((la, lb, lc)))
+        elif dt == "u32":
+            A, B, C = (inputs.words32(701 + i, n, n, o) for i, o in enumerate((la, lb, lc)))
+        else:
+            A, B, C = (inputs.integers(701 + i, n, n, 0, 8, npd, o) for i, o in enumerate((la, lb, lc)))
+        ident = cuasr_amd.op_identity(add, dt, True)
+        one = cuasr_amd.op_identity(mult, dt, True)
+        up = lambda X: (col_major if X.flags.f_contiguous else row_major)(X.view(np.int32) if dt == "u32" else X)
+        dA, dB, dC = up(A), up(B), up(C)
+        tdt = {"f32": torch.float32, "f64": torch.float64, "i32": torch.int32, "u32": torch.int32}[dt]
+        dD = torch.empty(n, n, dtype=tdt, device=dev)
+        dD = dD.t() if lc == "F" else dD
+
+        def step(i):
+            cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dt, kernel=args.kernel)
+
+        desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one)
+        matrix = add == "plus" and mult == "multiplies" and dt in ("f32", "f64")
+        return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=desc, host=(add, mult, A, B, C, one, one, ident),
+                    metric=f"{dt} {add}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
+                    workload=f"{add}-{mult} SRGEMM {dt}, M=N=K={n}, layouts (A, B, C) = {args.layouts} "
+                             "(c = column-major, r = row-major), beta = one with a seeded C",
+                    bound="mfma" if matrix else "valu", peak=FP64_VECTOR_PEAK if dt == "f64" else FP32_VECTOR_PEAK,
+                    instr_per_term=None)
+
     raise SystemExit(f"bench.py: unknown workload {w!r}")
 
 
@@ -175,7 +209,12 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="apsp",
-                    choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64"])
+                    choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64",
+                             "srgemm"])
+    ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
+    ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32"], help="workload srgemm")
+    ap.add_argument("--layouts", default="ccc", help="workload srgemm: layouts of A, B, C (c = column-major, r = row-major)")
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")
     ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")

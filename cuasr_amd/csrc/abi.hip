@@ -160,7 +160,10 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   // min-max / max-min on 4-byte types: `v_min_f32` / `v_max_f32` do not dual-issue, the arithmetic is 60 % slower than
   // min-plus and the staged tile's two fragment sets cover it slightly better (47.6 vs 46.1 TOPS at 4096^3)
   const bool minmax = !f64 && ((d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum));
-  if (direct_usable(d) && ((fills && !(minmax && have_valu)) || !have_valu)) return kDirect;
+  // or-and: the staged tile turns its panels into masks on their way to LDS and spends one
+  // `acc | (a & b)` per term; the direct tile cannot (its panels never pass through registers)
+  const bool masked = d->add_op == kLogicalOr && d->mult_op == kLogicalAnd;
+  if (direct_usable(d) && ((fills && !((minmax || masked) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
   return kNaive;

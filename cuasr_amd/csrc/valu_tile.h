@@ -49,9 +49,44 @@ struct ValuTile {
   // takes 16-byte loads and stores at any 4-byte boundary)
   typedef T gvec_t __attribute__((ext_vector_type(VW), aligned(sizeof(T))));
 
+  // Two semirings whose inner loop does not compute with the operators as written:
+  //   MASKED     or-and.  `lhs && rhs`, `lhs || rhs` (functional.h:212, :252) only look at whether
+  //              an operand is zero, so the panels go to LDS as 32-bit masks (all ones / zero)
+  //              whatever the element type, a term is one `acc | (a & b)` on 32-bit words, and the
+  //              epilogue turns the mask back into the 1 / 0 the operators return.
+  //   ZERO_SIGN  min-times / max-times on floating point.  The hardware min / max give the
+  //              reference's value, but on a tie between +0 and -0 the reference keeps the newer
+  //              product (host_srgemm.h:87 with functional.h:132, :172) and the hardware keeps -0.
+  //              A zero result therefore has the sign of the LAST zero product of the k range,
+  //              which the epilogue looks up for the accumulators that ended at zero.
+  static constexpr bool MASKED = ADD == kLogicalOr && MUL == kLogicalAnd;
+  static constexpr bool ZERO_SIGN = is_fp<T>::value && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum);
+  using S = typename std::conditional<MASKED, uint32_t, T>::type;  // what LDS, fragments and accumulators hold
+  typedef S svec_t __attribute__((ext_vector_type(VW)));
+  static __device__ __forceinline__ S staged(T x) {
+    if constexpr (MASKED) return x != T(0) ? 0xFFFFFFFFu : 0u;
+    else return x;
+  }
+  static __device__ __forceinline__ S term(S acc, S a, S b) {
+    if constexpr (MASKED) return acc | (a & b);
+    else if constexpr (ZERO_SIGN) return Op<ADD>::apply(acc, Op<MUL>::apply(a, b));
+    else return fold<ADD, MUL>(Op<MUL>::apply(a, b), acc);
+  }
+  // ZERO_SIGN: the last product of the k range that is zero (acc itself when there is none: an
+  // empty range, or a zero identity).  Not inlined: it runs for the few accumulators that ended
+  // at zero, after the main loop.
+  static __device__ __attribute__((noinline)) T last_zero_product(const T *a_row, long long sa_k, const T *b_col,
+                                                                 long long sb_k, int kcount, T acc) {
+    for (int kk = kcount - 1; kk >= 0; --kk) {
+      const T prod = a_row[(long long)kk * sa_k] * b_col[(long long)kk * sb_k];
+      if (prod == T(0)) return prod;
+    }
+    return acc;
+  }
+
   struct Smem {
-    T a[2][BK][LDA];
-    T b[2][BK][LDB];
+    S a[2][BK][LDA];
+    S b[2][BK][LDB];
   };
 
   // ---- global -> registers.  ROWS is the panel extent (BM or BN), s_x the
@@ -150,7 +185,7 @@ struct ValuTile {
   // workgroup, and inlined into the main loop its address arithmetic costs the loop 60-80
   // registers (a wave less per SIMD for the quarter-size tile).
   template <int ROWS, int LD>
-  static __device__ __attribute__((noinline)) void fill_last(T (*dst)[LD], const T *base, long long s_x, long long s_k, int x0,
+  static __device__ __attribute__((noinline)) void fill_last(S (*dst)[LD], const T *base, long long s_x, long long s_k, int x0,
                                                              int x_end, int k0, int k_end, bool x_contig) {
     const int tid = threadIdx.x;
     const int xmax = x_end - 1 - x0, kmax = k_end - 1 - k0;
@@ -166,13 +201,13 @@ struct ValuTile {
 #pragma unroll
     for (int i = 0; i < N; ++i) {
       const int el = tid + 256 * i;
-      dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = r[i];
+      dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = staged(r[i]);
     }
   }
 
   // ---- registers -> LDS ([kk][x], k-major), same ownership as load_panel
   template <int ROWS, int LD, int ELEMS>
-  static __device__ __forceinline__ void store_panel(const T (&r)[ELEMS], T (*dst)[LD], bool x_contig) {
+  static __device__ __forceinline__ void store_panel(const T (&r)[ELEMS], S (*dst)[LD], bool x_contig) {
     const int tid = threadIdx.x;
     if constexpr (VEC) {
       constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
@@ -180,47 +215,47 @@ struct ValuTile {
 #pragma unroll
         for (int p = 0; p < VECS; ++p) {
           const int v = tid + 256 * p;
-          vec_t t;
+          svec_t t;
 #pragma unroll
-          for (int e = 0; e < VW; ++e) t[e] = r[p * VW + e];
-          *reinterpret_cast<vec_t *>(&dst[v / XV][(v % XV) * VW]) = t;
+          for (int e = 0; e < VW; ++e) t[e] = staged(r[p * VW + e]);
+          *reinterpret_cast<svec_t *>(&dst[v / XV][(v % XV) * VW]) = t;
         }
       } else {
 #pragma unroll
         for (int p = 0; p < VECS; ++p) {
           const int v = tid + 256 * p;
 #pragma unroll
-          for (int e = 0; e < VW; ++e) dst[(v % KV) * VW + e][v / KV] = r[p * VW + e];
+          for (int e = 0; e < VW; ++e) dst[(v % KV) * VW + e][v / KV] = staged(r[p * VW + e]);
         }
       }
     } else {
 #pragma unroll
       for (int p = 0; p < ELEMS; ++p) {
         const int el = tid + 256 * p;
-        dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = r[p];
+        dst[x_contig ? el / ROWS : el % BK][x_contig ? el % ROWS : el / BK] = staged(r[p]);
       }
     }
   }
 
-  static __device__ __forceinline__ void step(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int kk,
+  static __device__ __forceinline__ void step(S (&acc)[TM][TN], const S (*as)[LDA], const S (*bs)[LDB], int kk,
                                               int ty, int tx) {
-    T a[TM], b[TN];
+    S a[TM], b[TN];
 #pragma unroll
     for (int h = 0; h < HM; ++h) {
-      const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk][ty * VW + h * 16 * VW]);
+      const svec_t t = *reinterpret_cast<const svec_t *>(&as[kk][ty * VW + h * 16 * VW]);
 #pragma unroll
       for (int e = 0; e < VW; ++e) a[h * VW + e] = t[e];
     }
 #pragma unroll
     for (int g = 0; g < GN; ++g) {
-      const vec_t t = *reinterpret_cast<const vec_t *>(&bs[kk][tx * VW + g * 16 * VW]);
+      const svec_t t = *reinterpret_cast<const svec_t *>(&bs[kk][tx * VW + g * 16 * VW]);
 #pragma unroll
       for (int e = 0; e < VW; ++e) b[g * VW + e] = t[e];
     }
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = fold<ADD, MUL>(Op<MUL>::apply(a[i], b[j]), acc[i][j]);
+      for (int j = 0; j < TN; ++j) acc[i][j] = term(acc[i][j], a[i], b[j]);
       __builtin_amdgcn_sched_barrier(0);
     }
   }
@@ -235,31 +270,40 @@ struct ValuTile {
   // compiler ten minutes each, and they are not the throughput cases)
   static constexpr bool PIPELINED = T(0.5) != T(0);  // floating-point element type
   struct Frag2 {
-    T a[KU][TM], b[KU][TN];
+    S a[KU][TM], b[KU][TN];
   };
-  static __device__ __forceinline__ void load_frag2(Frag2 &f, const T (*as)[LDA], const T (*bs)[LDB], int kk, int ty, int tx) {
+  static __device__ __forceinline__ void load_frag2(Frag2 &f, const S (*as)[LDA], const S (*bs)[LDB], int kk, int ty, int tx) {
 #pragma unroll
     for (int s = 0; s < KU; ++s) {
 #pragma unroll
       for (int h = 0; h < HM; ++h) {
-        const vec_t t = *reinterpret_cast<const vec_t *>(&as[kk + s][ty * VW + h * 16 * VW]);
+        const svec_t t = *reinterpret_cast<const svec_t *>(&as[kk + s][ty * VW + h * 16 * VW]);
 #pragma unroll
         for (int e = 0; e < VW; ++e) f.a[s][h * VW + e] = t[e];
       }
 #pragma unroll
       for (int g = 0; g < GN; ++g) {
-        const vec_t t = *reinterpret_cast<const vec_t *>(&bs[kk + s][tx * VW + g * 16 * VW]);
+        const svec_t t = *reinterpret_cast<const svec_t *>(&bs[kk + s][tx * VW + g * 16 * VW]);
 #pragma unroll
         for (int e = 0; e < VW; ++e) f.b[s][g * VW + e] = t[e];
       }
     }
   }
-  static __device__ __forceinline__ void compute2(T (&acc)[TM][TN], const Frag2 &f) {
+  static __device__ __forceinline__ void compute2(S (&acc)[TM][TN], const Frag2 &f) {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        if constexpr (KU == 2) {
+        if constexpr (MASKED || ZERO_SIGN) {
+#pragma unroll
+          for (int s = 0; s < KU; ++s) {
+            acc[i][j] = term(acc[i][j], f.a[s][i], f.b[s][j]);
+            // integer or is associative: left alone, the compiler regroups the terms of a whole
+            // unrolled k-tile into a tree and needs a register for every a & b of it; pinned after
+            // every term, each one is a single v_and_or_b32
+            if constexpr (MASKED) asm volatile("" : "+v"(acc[i][j]));
+          }
+        } else if constexpr (KU == 2) {
           const T t0 = Op<MUL>::apply(f.a[0][i], f.b[0][j]), t1 = Op<MUL>::apply(f.a[1][i], f.b[1][j]);
           acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
         } else {
@@ -269,7 +313,7 @@ struct ValuTile {
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  static __device__ __forceinline__ void whole_tile(T (&acc)[TM][TN], const T (*as)[LDA], const T (*bs)[LDB], int ty, int tx) {
+  static __device__ __forceinline__ void whole_tile(S (&acc)[TM][TN], const S (*as)[LDA], const S (*bs)[LDB], int ty, int tx) {
     constexpr int STEPS = BK / KU;
     if constexpr (PIPELINED) {
       Frag2 f[2];
@@ -320,11 +364,11 @@ struct ValuTile {
     }
     const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
 
-    T acc[TM][TN];
+    S acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j) acc[i][j] = ident;
+      for (int j = 0; j < TN; ++j) acc[i][j] = staged(ident);
 
     const int ntiles = (ke - kb + BK - 1) / BK;
     T ra[A_ELEMS], rb[B_ELEMS];
@@ -419,7 +463,19 @@ struct ValuTile {
         if (col >= p.n) continue;
         T v[VW];
 #pragma unroll
-        for (int c = 0; c < VW; ++c) v[c] = acc[i][g * VW + c];
+        for (int c = 0; c < VW; ++c) {
+          if constexpr (MASKED) {
+            v[c] = acc[i][g * VW + c] ? T(1) : T(0);
+          } else {
+            v[c] = acc[i][g * VW + c];
+            if constexpr (ZERO_SIGN) {
+              if (v[c] == T(0) && ke > kb)
+                v[c] = last_zero_product(A + (long long)row * p.sa_m + (long long)kb * p.sa_k, p.sa_k,
+                                         B + (long long)min(col + c, p.n - 1) * p.sb_n + (long long)kb * p.sb_k, p.sb_k,
+                                         ke - kb, v[c]);
+            }
+          }
+        }
         if (!partial) {
 #pragma unroll
           for (int c = 0; c < VW; ++c) v[c] = Op<MUL>::apply(e.alpha, v[c]);
