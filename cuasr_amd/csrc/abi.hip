@@ -138,7 +138,12 @@ enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4 };
 static int pick_family(const cuasr_amd_srgemm_desc *d) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
   // plus-times is the one semiring a matrix instruction computes as is
-  if (d->add_op == kPlus && d->mult_op == kMultiplies && mfma_usable(d)) return kMfma;
+  // (its tile is 128 x 128: below 128 tiles half the compute units and more stand idle, and the
+  // vector-ALU tiles, which are smaller, are faster -- 1024^3: 31 against 22 TFLOP/s)
+  if (d->add_op == kPlus && d->mult_op == kMultiplies && mfma_usable(d)) {
+    const long long mfma_tiles = (long long)((d->m + 127) / 128) * ((d->n + 127) / 128) * d->split_k_slices;
+    if (mfma_tiles >= 128 || !find_valu(d->dtype, d->add_op, d->mult_op)) return kMfma;
+  }
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.

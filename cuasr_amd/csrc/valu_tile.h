@@ -102,7 +102,7 @@ struct ValuTile {
   template <int ROWS, int ELEMS>
   static __device__ __forceinline__ void load_panel(T (&r)[ELEMS], const T *base, long long s_x, long long s_k,
                                                     int x0, int x_end, int k0, int k_end, bool x_contig) {
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & 255;
     if constexpr (VEC) {
       constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
 #pragma unroll
@@ -143,7 +143,7 @@ struct ValuTile {
     long long step;
     __device__ __forceinline__ void init(const T *base, long long s_x, long long s_k, int x0, int x_end, int k0,
                                          bool x_contig) {
-      const int tid = threadIdx.x;
+      const int tid = threadIdx.x & 255;
       step = (long long)BK * s_k;
 #pragma unroll
       for (int p = 0; p < VECS; ++p) {
@@ -166,7 +166,7 @@ struct ValuTile {
     }
     // !CAREFUL: ragged last k-tile; vectors past its end re-read its last valid vector
     __device__ __forceinline__ void load_ragged(T (&r)[ELEMS], long long s_k, int kcount, bool x_contig) {
-      const int tid = threadIdx.x;
+      const int tid = threadIdx.x & 255;
 #pragma unroll
       for (int p = 0; p < VECS; ++p) {
         const int v = tid + 256 * p;
@@ -187,7 +187,7 @@ struct ValuTile {
   template <int ROWS, int LD>
   static __device__ __attribute__((noinline)) void fill_last(S (*dst)[LD], const T *base, long long s_x, long long s_k, int x0,
                                                              int x_end, int k0, int k_end, bool x_contig) {
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & 255;
     const int xmax = x_end - 1 - x0, kmax = k_end - 1 - k0;
     const T *tile = base + (long long)x0 * s_x + (long long)k0 * s_k;
     constexpr int N = ROWS * BK / 256;
@@ -208,7 +208,7 @@ struct ValuTile {
   // ---- registers -> LDS ([kk][x], k-major), same ownership as load_panel
   template <int ROWS, int LD, int ELEMS>
   static __device__ __forceinline__ void store_panel(const T (&r)[ELEMS], S (*dst)[LD], bool x_contig) {
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x & 255;
     if constexpr (VEC) {
       constexpr int VECS = ELEMS / VW, XV = ROWS / VW, KV = BK / VW;
       if (x_contig) {
@@ -347,30 +347,46 @@ struct ValuTile {
     bn = (id % width) / gsz;
   }
 
-  static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
-    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  // The workgroup's output tile and k range (blockIdx.y is the split-K slice).
+  static __device__ __forceinline__ void tile_and_range(const Problem &p, int &m0, int &n0, int &kb, int &ke) {
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     int bm, bn;
     tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
-    const int m0 = bm * BM, n0 = bn * BN;
-    const T *A = reinterpret_cast<const T *>(p.A);
-    const T *B = reinterpret_cast<const T *>(p.B);
-    const T ident = scalar_as<T>(p.add_identity);
-
-    int kb = 0, ke = p.k;
+    m0 = bm * BM;
+    n0 = bn * BN;
+    kb = 0;
+    ke = p.k;
     if (p.workspace) {
       kb = blockIdx.y * p.k_per_slice;
       ke = min(p.k, kb + p.k_per_slice);
     }
+  }
+
+  static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
+    int m0, n0, kb, ke;
+    tile_and_range(p, m0, n0, kb, ke);
+    S acc[TM][TN];
+    accumulate(p, sm, m0, n0, kb, ke, (ke - kb + BK - 1) / BK, acc);
+    finish(p, acc, m0, n0, kb, ke);
+  }
+
+  // acc = identity, then the terms of k in [kb, ke).  The 256 threads that share `sm` pass
+  // 1 + `sync_tiles` barriers (sync_tiles >= the number of k-tiles of the range, so that groups of
+  // one workgroup whose ranges differ in length stay in step).
+  static __device__ __forceinline__ void accumulate(const Problem &p, Smem &sm, int m0, int n0, int kb, int ke, int sync_tiles,
+                                                    S (&acc)[TM][TN]) {
+    const int tid = threadIdx.x & 255, tx = tid & 15, ty = tid >> 4;
+    const T *A = reinterpret_cast<const T *>(p.A);
+    const T *B = reinterpret_cast<const T *>(p.B);
+    const T ident = scalar_as<T>(p.add_identity);
     const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
 
-    S acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = staged(ident);
 
-    const int ntiles = (ke - kb + BK - 1) / BK;
+    const int ntiles = max((ke - kb + BK - 1) / BK, 0);
     T ra[A_ELEMS], rb[B_ELEMS];
     Mover<BM, A_ELEMS> ma;
     Mover<BN, B_ELEMS> mb;
@@ -416,28 +432,37 @@ struct ValuTile {
     }
     __syncthreads();
     int buf = 0;
-    for (int t = 0; t < ntiles; ++t) {
-      const int k0 = kb + t * BK;
-      const bool more = t + 1 < ntiles;
-      const bool next_is_last = careful_last && t + 2 == ntiles;
-      if (next_is_last) fill_last_tile(k0 + BK, buf ^ 1);
-      else if (more) fetch(k0 + BK);
-      const int kcount = min(BK, ke - k0);
-      if (kcount == BK) {
-        whole_tile(acc, sm.a[buf], sm.b[buf], ty, tx);
-      } else {
+    for (int t = 0; t < sync_tiles; ++t) {
+      if (t < ntiles) {
+        const int k0 = kb + t * BK;
+        const bool more = t + 1 < ntiles;
+        const bool next_is_last = careful_last && t + 2 == ntiles;
+        if (next_is_last) fill_last_tile(k0 + BK, buf ^ 1);
+        else if (more) fetch(k0 + BK);
+        const int kcount = min(BK, ke - k0);
+        if (kcount == BK) {
+          whole_tile(acc, sm.a[buf], sm.b[buf], ty, tx);
+        } else {
 #pragma unroll 1
-        for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
-      }
-      if (more && !next_is_last) {
-        store_panel<BM, LDA, A_ELEMS>(ra, sm.a[buf ^ 1], a_xc);
-        store_panel<BN, LDB, B_ELEMS>(rb, sm.b[buf ^ 1], b_xc);
+          for (int kk = 0; kk < kcount; ++kk) step(acc, sm.a[buf], sm.b[buf], kk, ty, tx);
+        }
+        if (more && !next_is_last) {
+          store_panel<BM, LDA, A_ELEMS>(ra, sm.a[buf ^ 1], a_xc);
+          store_panel<BN, LDB, B_ELEMS>(rb, sm.b[buf ^ 1], b_xc);
+        }
       }
       __syncthreads();
       buf ^= 1;
     }
+  }
 
-    // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or raw partials
+  // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or raw partials; [kb, ke) is the
+  // k range the accumulators cover (ZERO_SIGN looks into it)
+  static __device__ __forceinline__ void finish(const Problem &p, S (&acc)[TM][TN], int m0, int n0, int kb, int ke) {
+    const int tid = threadIdx.x & 255, tx = tid & 15, ty = tid >> 4;
+    const T *A = reinterpret_cast<const T *>(p.A);
+    const T *B = reinterpret_cast<const T *>(p.B);
+    const T ident = scalar_as<T>(p.add_identity);
     T *out;
     long long ld_out;
     const bool partial = p.workspace != nullptr;
@@ -516,6 +541,54 @@ __global__ __launch_bounds__(256) WAVES_ATTR void valu_srgemm_kernel(Problem p) 
   Tile::run(p, sm);
 }
 
+// The same tile with the k range shared out inside the workgroup, for launches that would
+// otherwise leave most of the chip idle (an output of 1024^2 is 256 quarter-size tiles: one
+// workgroup per compute unit, one wave per SIMD, and a single wave issues at little more than a
+// third of the rate two or four reach).  G groups of 256 threads each take a run of whole k-tiles
+// of the workgroup's range, with LDS panels of their own; the groups' accumulators then meet in LDS
+// and group 0 folds them in ascending k order, acc = add(acc, partial) as the split-K reduction does,
+// and runs the epilogue.  Only for adds whose result does not depend on how the terms are grouped
+// (everything but a floating-point sum).
+template <typename T, int ADD> struct order_free : std::integral_constant<bool, !(ADD == kPlus && is_fp<T>::value)> {};
+
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC, bool CAREFUL, int G>
+__global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
+  using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC, CAREFUL>;
+  using S = typename Tile::S;
+  static_assert(order_free<T, ADD>::value, "a floating-point sum depends on the grouping of its terms");
+  static_assert(sizeof(typename Tile::Smem) >= sizeof(S) * TM * TN * 256, "a group's accumulators must fit its panel space");
+  __shared__ typename Tile::Smem sm[G];
+  const int g = threadIdx.x >> 8, tid = threadIdx.x & 255;
+  int m0, n0, kb, ke;
+  Tile::tile_and_range(p, m0, n0, kb, ke);
+  const int tiles = max((ke - kb + BK - 1) / BK, 0), per = (tiles + G - 1) / G;
+  const int gkb = min(ke, kb + g * per * BK), gke = min(ke, gkb + per * BK);
+  S acc[TM][TN];
+  Tile::accumulate(p, sm[g], m0, n0, gkb, gke, per, acc);  // ends with a barrier: every group is done with its panels
+  S *mine = reinterpret_cast<S *>(&sm[g]);
+  if (g > 0) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) mine[(i * TN + j) * 256 + tid] = acc[i][j];
+  }
+  __syncthreads();
+  if (g > 0) return;
+#pragma unroll 1
+  for (int h = 1; h < G; ++h) {
+    const S *part = reinterpret_cast<const S *>(&sm[h]);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const S w = part[(i * TN + j) * 256 + tid];
+        if constexpr (Tile::MASKED) acc[i][j] |= w;
+        else acc[i][j] = Op<ADD>::apply(acc[i][j], w);
+      }
+  }
+  Tile::finish(p, acc, m0, n0, kb, ke);
+}
+
 // Extents along every contiguous direction are multiples of the vector width: no vector straddles
 // an edge, rows of D hold whole vectors (alignment itself is not needed: 16-byte accesses are legal
 // at any element boundary).
@@ -538,13 +611,38 @@ template <typename T> static bool vector_possible(const Problem &p) {
   return p.k >= 1;
 }
 
-template <typename T, int ADD, int MUL, int TM, int TN, int BK>
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, int G>
+static void launch_ksplit(const Problem &p, dim3 grid, hipStream_t s) {
+  if (vector_exact<T>(p))
+    hipLaunchKernelGGL((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, false, G>), grid, dim3(256 * G), 0, s, p);
+  else
+    hipLaunchKernelGGL((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, true, G>), grid, dim3(256 * G), 0, s, p);
+}
+
+// KSPLIT: this tile may share its k range out inside the workgroup when the launch is small.
+template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool KSPLIT = false>
 static hipError_t launch_valu(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   if (p.m == 0 || p.n == 0) return hipSuccess;
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  if constexpr (KSPLIT && order_free<T, ADD>::value) {
+    // 256 compute units: up to 256 workgroups get four groups (1024 threads, four waves per SIMD),
+    // up to 512 two; each group wants a few k-tiles of its own to be worth the fold at the end
+    const long long groups = tiles * grid.y;
+    const long long k_range = p.workspace ? p.k_per_slice : p.k;
+    if (vector_possible<T>(p) && k_range >= 8LL * BK) {
+      if (groups <= 256) {
+        launch_ksplit<T, ADD, MUL, TM, TN, BK, 4>(p, grid, s);
+        return hipGetLastError();
+      }
+      if (groups <= 512) {
+        launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, grid, s);
+        return hipGetLastError();
+      }
+    }
+  }
   if (vector_exact<T>(p))
     hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, false>), grid, dim3(256), 0, s, p);
   else if (vector_possible<T>(p))
@@ -572,7 +670,7 @@ static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1);
   const long long rounds = (groups + 1023) / 1024;
   if (groups * 100 < rounds * 1024 * (long long)(CUASR_AMD_FULL_TILE_FILL_PERCENT))
-    return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK_SMALL>(p, s);
+    return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK_SMALL, true>(p, s);
   return launch_valu<T, ADD, MUL, TM, TN, BK>(p, s);
 }
 

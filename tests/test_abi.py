@@ -78,10 +78,12 @@ def test_kernel_selection(lib):
     assert sel(desc()) == b"valu"                   # 64 x 64: one direct tile would leave the chip idle
     assert sel(desc(m=3072, n=3072, k=64)) == b"valu"     # 288 direct tiles fill 56 % of a round of 512
     assert sel(desc(m=8192, n=8192, k=64)) == b"valu_direct"
-    assert sel(desc(add="plus", mult="multiplies")) == b"mfma"
+    assert sel(desc(add="plus", mult="multiplies", m=2048, n=2048)) == b"mfma"
+    assert sel(desc(add="plus", mult="multiplies", m=1024, n=1024)) == b"valu"   # 64 tiles of 128 x 128 leave the chip idle
     assert sel(desc(dtype="f64")) == b"valu"
     assert sel(desc(dtype="f64", m=8192, n=8192, k=64)) == b"valu_direct"   # fp64 direct-to-LDS tile, 128 x 64
-    assert sel(desc(dtype="f64", add="plus", mult="multiplies")) == b"mfma"   # fp64 matrix cores
+    assert sel(desc(dtype="f64", add="plus", mult="multiplies", m=2048, n=2048)) == b"mfma"   # fp64 matrix cores
+    assert sel(desc(dtype="f64", add="plus", mult="multiplies")) == b"valu"
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
     assert sel(desc(kernel="mfma")) == b"mfma"
 

@@ -256,3 +256,22 @@ def test_unaligned_views(oracle, lib, sr, layouts):
             cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dtype, kernel=kernel)
             torch.cuda.synchronize()
             assert_same_bits(np.asarray(to_host(dD, dtype), order=order), want, f"{sr} {layouts} {m}x{n}x{k} {kernel}")
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f64"), ("bit_xor", "bit_and", "u32"),
+                                ("logical_or", "logical_and", "f32"), ("minimum", "multiplies", "f32"),
+                                ("maximum", "minimum", "f64"), ("minimum", "plus", "i32"), ("plus", "multiplies", "f32")])
+@pytest.mark.parametrize("shape", [(64, 64, 256), (100, 60, 1000), (256, 256, 4099), (512, 512, 512), (1024, 1024, 1024),
+                                   (1000, 1100, 300), (61, 67, 1027)])
+def test_valu_small_launches_share_k_inside_the_workgroup(oracle, lib, sr, shape):
+    """Launches of at most 512 quarter-size tiles with a long enough k range run two or four groups of 256 threads
+    per workgroup, each on a part of the k range (every add but a floating-point sum); results stay the reference's."""
+    for layouts in ("ccc", "rcr", "crr", "rrc"):
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        if shape[0] >= 1000 and layouts in ("crr", "rrc"):
+            continue
+        for beta_one in (False, True):
+            if not beta_one and sr[2] == "i32" and sr[1] == "plus":
+                continue  # plus::Annihilator = INT_MAX: mult(beta, c) overflows on the CPU side (undefined)
+            run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", beta_one)
+    run(oracle, sr[0], sr[1], sr[2], *shape, "row", "col", "row", "valu", True, splitk=3)
