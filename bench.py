@@ -132,7 +132,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         return dict(step=step, m=n, n=n, k=n, dtype="u32", desc=desc, host=("bit_xor", "bit_and", A, B, C, 0xFFFFFFFF, 0, 0),
                     metric=f"uint32 xor-and SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"GF(2) xor-and SRGEMM on bit-packed uint32 words, M=N=K={n}, column-major, random words",
-                    bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=2.0)
+                    bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.0)  # one v_bitop3_b32 per term
 
     if w == "plustimes_f32":
         n = args.size or 4096

@@ -181,8 +181,12 @@ struct DirectTile {
   template <int I, int J0> static __device__ __forceinline__ void row4(T (&acc)[8][8], const FragA &a, const FragB &b) {
 #pragma unroll
     for (int j = J0; j < J0 + 4; ++j) {
-      const T t0 = Op<MUL>::apply(a.get(0, I), b.get(0, j)), t1 = Op<MUL>::apply(a.get(1, I), b.get(1, j));
-      acc[I][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[I][j]));
+      if constexpr (fused_bit_term<ADD, MUL, T>::value) {
+        acc[I][j] = term<ADD, MUL>(term<ADD, MUL>(acc[I][j], a.get(0, I), b.get(0, j)), a.get(1, I), b.get(1, j));
+      } else {
+        const T t0 = Op<MUL>::apply(a.get(0, I), b.get(0, j)), t1 = Op<MUL>::apply(a.get(1, I), b.get(1, j));
+        acc[I][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[I][j]));
+      }
     }
     // pin the row: computed here, not later (arithmetic has no side effect, so
     // only naming it in a volatile statement keeps it from drifting)
@@ -431,7 +435,7 @@ struct DirectTile {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) acc[i][j] = fold<ADD, MUL>(Op<MUL>::apply(a[i], b[j]), acc[i][j]);
+          for (int j = 0; j < 8; ++j) acc[i][j] = term<ADD, MUL>(acc[i][j], a[i], b[j]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }

@@ -83,6 +83,28 @@ template <int ADD, int MUL, typename T> __device__ __forceinline__ T fold(T prod
   else return Op<ADD>::apply(acc, prod);
 }
 
+// One term of the inner product, acc <- add(mult(a, b), acc).  For xor-and and or-and on 32-bit
+// words gfx950's three-input bit operation does the whole term in one instruction, and that
+// instruction issues almost as fast as a two-input one (per wave: v_and_b32 and v_xor_b32 2.1
+// cycles each, v_bitop3_b32 2.6, v_and_or_b32 4.2).  The table is the function's value on
+// a = 0xF0, b = 0xCC, acc = 0xAA.
+template <int ADD, int MUL, typename T> struct fused_bit_term
+    : std::integral_constant<bool, sizeof(T) == 4 && !is_fp<T>::value && MUL == kBitAnd && (ADD == kBitXor || ADD == kBitOr)> {};
+__device__ __forceinline__ uint32_t xor_and_term(uint32_t acc, uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_bitop3_b32(a, b, acc, 0x6a);  // acc ^ (a & b)
+}
+__device__ __forceinline__ uint32_t or_and_term(uint32_t acc, uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_bitop3_b32(a, b, acc, 0xea);  // acc | (a & b)
+}
+template <int ADD, int MUL, typename T> __device__ __forceinline__ T term(T acc, T a, T b) {
+  if constexpr (fused_bit_term<ADD, MUL, T>::value) {
+    if constexpr (ADD == kBitXor) return T(xor_and_term(uint32_t(acc), uint32_t(a), uint32_t(b)));
+    else return T(or_and_term(uint32_t(acc), uint32_t(a), uint32_t(b)));
+  } else {
+    return fold<ADD, MUL>(Op<MUL>::apply(a, b), acc);
+  }
+}
+
 // add(lhs, rhs) of the epilogue, D = add(mult(alpha, acc), mult(beta, C)), same rule
 template <int ADD, int MUL, typename T> __device__ __forceinline__ T fold_epilogue(T lhs, T rhs) {
   if constexpr ((ADD == kMinimum || ADD == kMaximum) && MUL == kMultiplies && is_fp<T>::value) return Op<ADD>::strict(lhs, rhs);

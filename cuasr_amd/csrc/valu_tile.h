@@ -52,8 +52,9 @@ struct ValuTile {
   // Two semirings whose inner loop does not compute with the operators as written:
   //   MASKED     or-and.  `lhs && rhs`, `lhs || rhs` (functional.h:212, :252) only look at whether
   //              an operand is zero, so the panels go to LDS as 32-bit masks (all ones / zero)
-  //              whatever the element type, a term is one `acc | (a & b)` on 32-bit words, and the
-  //              epilogue turns the mask back into the 1 / 0 the operators return.
+  //              whatever the element type, a term is one three-input bit operation `acc | (a & b)`
+  //              on 32-bit words, and the epilogue turns the mask back into the 1 / 0 the operators
+  //              return.
   //   ZERO_SIGN  min-times / max-times on floating point.  The hardware min / max give the
   //              reference's value, but on a tie between +0 and -0 the reference keeps the newer
   //              product (host_srgemm.h:87 with functional.h:132, :172) and the hardware keeps -0.
@@ -67,10 +68,11 @@ struct ValuTile {
     if constexpr (MASKED) return x != T(0) ? 0xFFFFFFFFu : 0u;
     else return x;
   }
+  static constexpr bool FUSED = fused_bit_term<ADD, MUL, T>::value;
   static __device__ __forceinline__ S term(S acc, S a, S b) {
-    if constexpr (MASKED) return acc | (a & b);
+    if constexpr (MASKED) return or_and_term(acc, a, b);
     else if constexpr (ZERO_SIGN) return Op<ADD>::apply(acc, Op<MUL>::apply(a, b));
-    else return fold<ADD, MUL>(Op<MUL>::apply(a, b), acc);
+    else return cuasr_amd::term<ADD, MUL>(acc, a, b);
   }
   // ZERO_SIGN: the last product of the k range that is zero (acc itself when there is none: an
   // empty range, or a zero identity).  Not inlined: it runs for the few accumulators that ended
@@ -294,15 +296,12 @@ struct ValuTile {
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        if constexpr (MASKED || ZERO_SIGN) {
+        if constexpr (MASKED || ZERO_SIGN || FUSED) {
+          // (the bit terms are one opaque instruction each: written as `acc | (a & b)`, integer or
+          // being associative, the compiler regroups the terms of a whole unrolled k-tile into a
+          // tree and needs a register for every a & b of it)
 #pragma unroll
-          for (int s = 0; s < KU; ++s) {
-            acc[i][j] = term(acc[i][j], f.a[s][i], f.b[s][j]);
-            // integer or is associative: left alone, the compiler regroups the terms of a whole
-            // unrolled k-tile into a tree and needs a register for every a & b of it; pinned after
-            // every term, each one is a single v_and_or_b32
-            if constexpr (MASKED) asm volatile("" : "+v"(acc[i][j]));
-          }
+          for (int s = 0; s < KU; ++s) acc[i][j] = term(acc[i][j], f.a[s][i], f.b[s][j]);
         } else if constexpr (KU == 2) {
           const T t0 = Op<MUL>::apply(f.a[0][i], f.b[0][j]), t1 = Op<MUL>::apply(f.a[1][i], f.b[1][j]);
           acc[i][j] = fold<ADD, MUL>(t1, fold<ADD, MUL>(t0, acc[i][j]));
