@@ -555,7 +555,7 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC, CAREFUL>;
   using S = typename Tile::S;
   static_assert(order_free<T, ADD>::value, "a floating-point sum depends on the grouping of its terms");
-  static_assert(sizeof(typename Tile::Smem) >= sizeof(S) * TM * TN * 256, "a group's accumulators must fit its panel space");
+  static_assert(G * sizeof(typename Tile::Smem) >= (G - 1) * sizeof(S) * TM * TN * 256, "the groups' accumulators must fit the panel space");
   __shared__ typename Tile::Smem sm[G];
   const int g = threadIdx.x >> 8, tid = threadIdx.x & 255;
   int m0, n0, kb, ke;
@@ -564,8 +564,10 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   const int gkb = min(ke, kb + g * per * BK), gke = min(ke, gkb + per * BK);
   S acc[TM][TN];
   Tile::accumulate(p, sm[g], m0, n0, gkb, gke, per, acc);  // ends with a barrier: every group is done with its panels
-  S *mine = reinterpret_cast<S *>(&sm[g]);
+  // the panels are dead now: groups 1 .. G-1 leave their accumulators in that space, one after the other
+  S *area = reinterpret_cast<S *>(&sm[0]);
   if (g > 0) {
+    S *mine = area + (g - 1) * (TM * TN * 256);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -575,7 +577,7 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   if (g > 0) return;
 #pragma unroll 1
   for (int h = 1; h < G; ++h) {
-    const S *part = reinterpret_cast<const S *>(&sm[h]);
+    const S *part = area + (h - 1) * (TM * TN * 256);
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -668,6 +670,16 @@ static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1);
   const long long rounds = (groups + 1023) / 1024;
+  if constexpr (order_free<T, ADD>::value) {
+    // 192 .. 256 full-size workgroups (2048^2: exactly 256) are one per compute unit for most of the
+    // chip: two groups per workgroup give every SIMD its two waves, and the full-size tile then runs
+    // at the rate it has on large problems, which the quarter-size tile does not reach
+    const long long k_range = p.workspace ? p.k_per_slice : p.k;
+    if (groups >= 192 && groups <= 256 && k_range >= 8LL * BK && vector_possible<T>(p) && p.m > 0 && p.n > 0) {
+      launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / (p.workspace ? p.slices : 1)), p.workspace ? p.slices : 1), s);
+      return hipGetLastError();
+    }
+  }
   if (groups * 100 < rounds * 1024 * (long long)(CUASR_AMD_FULL_TILE_FILL_PERCENT))
     return launch_valu<T, ADD, MUL, TM_SMALL, TN_SMALL, BK_SMALL, true>(p, s);
   return launch_valu<T, ADD, MUL, TM, TN, BK>(p, s);

@@ -275,3 +275,16 @@ def test_valu_small_launches_share_k_inside_the_workgroup(oracle, lib, sr, shape
                 continue  # plus::Annihilator = INT_MAX: mult(beta, c) overflows on the CPU side (undefined)
             run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", beta_one)
     run(oracle, sr[0], sr[1], sr[2], *shape, "row", "col", "row", "valu", True, splitk=3)
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("maximum", "plus", "f64"), ("bit_xor", "bit_and", "u32"),
+                                ("logical_or", "logical_and", "f32"), ("minimum", "multiplies", "f64"),
+                                ("maximum", "minimum", "f32"), ("plus", "multiplies", "f32")])
+@pytest.mark.parametrize("shape", [(2048, 2048, 260), (1792, 1920, 300), (2048, 1024, 300), (2040, 2047, 517)])
+def test_valu_full_size_tile_two_groups(oracle, lib, sr, shape):
+    """192 .. 256 full-size tiles (one workgroup per compute unit): two groups of 256 threads per workgroup
+    share the k range (every add but a floating-point sum)."""
+    for layouts in ("ccc", "rcr"):
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", True)
+    run(oracle, sr[0], sr[1], sr[2], *shape, "col", "row", "row", "valu", False)
