@@ -59,11 +59,22 @@ launch_fn find_naive(int dtype) {
 }
 
 // ------------------------------------------------------------ split-K reduction
+// One slice's vector of the workspace.  STREAM: a non-temporal load -- the workspace is read once.
+// Two regimes, measured on MI355X: an output of a million elements and more is bound by memory
+// bandwidth, and there few loads in flight per thread (small kernels, many resident waves) and
+// non-temporal loads win (2048^2 x 16 slices: 65.7 us with eight plain loads in flight, 49.1 us
+// with one non-temporal load: 6.2 TB/s); a small output is a handful of workgroups bound by
+// latency, and there eight loads in flight win (256^2 x 64 slices: 9.2 us against 19.8 us).
+template <typename V, bool STREAM> __device__ __forceinline__ V load_slice(const void *at) {
+  if constexpr (STREAM) return __builtin_nontemporal_load(reinterpret_cast<const V *>(at));
+  else return *reinterpret_cast<const V *>(at);
+}
+
 // Each thread owns V consecutive elements of one row.  acc starts at the
 // additive identity and folds the slices in ascending order; when the source
 // is not needed it is replaced by the identity and the two-operand epilogue is
 // still applied (reduce_split_k.h:212-227).
-template <typename T, int V, bool VOUT>
+template <typename T, int V, bool VOUT, int U, bool STREAM>
 __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
   const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
   const long long per_row = (p.n + V - 1) / V;
@@ -76,22 +87,21 @@ __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
   T acc[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) acc[v] = e.ident;
-  // eight slices' loads are issued before the first is folded, so a thread has
-  // eight memory requests in flight; the fold itself stays in ascending order
+  // U slices' loads are issued before the first is folded, so a thread has U memory
+  // requests in flight; the fold itself stays in ascending order
   typedef T vec_t __attribute__((ext_vector_type(V)));
-  constexpr int U = 8;
   int s = 0;
   for (; s + U <= p.slices; s += U) {
     vec_t w[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) w[u] = *reinterpret_cast<const vec_t *>(ws + (s + u) * slice);
+    for (int u = 0; u < U; ++u) w[u] = load_slice<vec_t, STREAM>(ws + (s + u) * slice);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
       for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[u][v]);
   }
   for (; s < p.slices; ++s) {
-    const vec_t w = *reinterpret_cast<const vec_t *>(ws + s * slice);
+    const vec_t w = load_slice<vec_t, STREAM>(ws + s * slice);
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[v] = apply_op<T>(p.add_op, acc[v], w[v]);
   }
@@ -127,7 +137,7 @@ __global__ __launch_bounds__(256) void reduce_splitk_kernel(Problem p) {
 // epilogue/thread/semiring_linear_combination.h:119-134).  Here the slices' raw
 // accumulators are in the workspace and one thread replays that chain for its
 // elements in registers: same operands, same order, one write of D.
-template <typename T, int V, bool VOUT>
+template <typename T, int V, bool VOUT, int U, bool STREAM>
 __global__ __launch_bounds__(256) void reduce_serial_kernel(Problem p) {
   const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
   const T one = scalar_as<T>(p.mult_identity);
@@ -144,7 +154,7 @@ __global__ __launch_bounds__(256) void reduce_serial_kernel(Problem p) {
   const T *C = reinterpret_cast<const T *>(p.C);
   T out[V];
   {
-    const vec_t w = *reinterpret_cast<const vec_t *>(ws);
+    const vec_t w = load_slice<vec_t, STREAM>(ws);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
       out[v] = apply_op<T>(p.mult_op, e.alpha, w[v]);
@@ -159,16 +169,15 @@ __global__ __launch_bounds__(256) void reduce_serial_kernel(Problem p) {
       out[v] = chain ? apply_op<T>(p.add_op, lhs, apply_op<T>(p.mult_op, one, out[v])) : lhs;
     }
   };
-  constexpr int U = 8;  // loads in flight per thread, as in the parallel reduction
-  int s = 1;
+  int s = 1;  // U loads in flight per thread, as in the parallel reduction
   for (; s + U <= p.slices; s += U) {
     vec_t w[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) w[u] = *reinterpret_cast<const vec_t *>(ws + (s + u) * slice);
+    for (int u = 0; u < U; ++u) w[u] = load_slice<vec_t, STREAM>(ws + (s + u) * slice);
 #pragma unroll
     for (int u = 0; u < U; ++u) step(w[u]);
   }
-  for (; s < p.slices; ++s) step(*reinterpret_cast<const vec_t *>(ws + s * slice));
+  for (; s < p.slices; ++s) step(load_slice<vec_t, STREAM>(ws + s * slice));
   T *dst = reinterpret_cast<T *>(p.D) + (long long)i * p.ldd + j;
   if (V > 1 && VOUT) {
     vec_t o;
@@ -183,8 +192,11 @@ __global__ __launch_bounds__(256) void reduce_serial_kernel(Problem p) {
 }
 
 template <typename T, bool SERIAL, int V, bool VOUT> static void launch_one(const Problem &p, dim3 grid, hipStream_t s) {
-  if (SERIAL) hipLaunchKernelGGL((reduce_serial_kernel<T, V, VOUT>), grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((reduce_splitk_kernel<T, V, VOUT>), grid, dim3(256), 0, s, p);
+  constexpr int U = V > 1 ? 1 : 8;      // the 16-byte path is the large-output one
+  constexpr bool STREAM = V > 1;
+  // (the serial form's chain of run-time operators, not memory, bounds it: 65 - 67 us at any depth)
+  if (SERIAL) hipLaunchKernelGGL((reduce_serial_kernel<T, V, VOUT, (V > 1 ? 2 : 8), STREAM>), grid, dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((reduce_splitk_kernel<T, V, VOUT, U, STREAM>), grid, dim3(256), 0, s, p);
 }
 
 template <typename T, bool SERIAL> static hipError_t launch_reduce(const Problem &p, hipStream_t s) {
