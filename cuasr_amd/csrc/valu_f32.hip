@@ -1,7 +1,6 @@
 // Vector-ALU tile kernels for element type float: one instantiation per semiring
-// the reference pre-tunes (include/cuasr/gemm/device/default_srgemm_configuration.h:44-275)
-// and, for integers, the GF(2)-style bitwise pairs of
-// examples/01_userdefined_semiring/userdefined_semiring.cu:56-99.
+// the reference pre-tunes (include/cuasr/gemm/device/default_srgemm_configuration.h:44-275);
+// min-times and max-times live in strict_valu.hip.
 #include "valu_tile.h"
 
 namespace cuasr_amd {
@@ -19,11 +18,6 @@ launch_fn find_valu_f32(int add_op, int mult_op) {
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
   PAIR(kLogicalOr, kLogicalAnd)
-#if 0
-  PAIR(kBitXor, kBitAnd)
-  PAIR(kBitXor, kLogicalAnd)
-  PAIR(kBitOr, kBitAnd)
-#endif
   return find_valu_strict(CUASR_AMD_F32, add_op, mult_op);
 }
 
