@@ -39,6 +39,18 @@ def main():
     sizes = [int(x) for x in args.sizes.split(",")]
     layouts = args.layouts.split(",")
     sink = open(args.json, "w") if args.json else None
+    # the clock takes ~100 ms of load to ramp up: keep the chip busy for a while before the first case
+    warm = torch.rand(4096, 4096, device="cuda")
+    t_end = torch.cuda.Event(enable_timing=True)
+    t_start = torch.cuda.Event(enable_timing=True)
+    t_start.record()
+    while True:
+        for _ in range(20):
+            cuasr_amd.srgemm("minimum", "plus", warm, warm, warm, warm.clone(), 0.0, 0.0, float("inf"), 0.0)
+        t_end.record()
+        torch.cuda.synchronize()
+        if t_start.elapsed_time(t_end) > 300.0:
+            break
     for dt in args.dtypes.split(","):
         npd, tdt = {"f32": (np.float32, torch.float32), "f64": (np.float64, torch.float64)}[dt]
         print(f"\n{dt}: TOPS (2 ops per term), layouts of A and B = {' '.join(layouts)}; C, D column-major; kernel = {args.kernel}")
@@ -55,7 +67,7 @@ def main():
             cells = []
             for n in sizes:
                 A0, B0, C0, D0 = data[n]
-                reps = max(3, min(200, int(2e11 / (2.0 * n ** 3))))
+                reps = max(10, min(200, int(1e12 / (2.0 * n ** 3))))
                 per_layout = []
                 for lay in layouts:
                     A = A0.t() if lay[0] == "n" else A0
