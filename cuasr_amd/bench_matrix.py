@@ -12,6 +12,7 @@ Layouts name A and B as the reference does (n = column-major, t = row-major); C 
 column-major.  Prints a table of TOPS (2 ops per term) and, with --json, one JSON object per case.
 """
 import argparse
+import ctypes
 import json
 import sys
 
@@ -73,7 +74,14 @@ def main():
                     A = A0.t() if lay[0] == "n" else A0
                     B = B0.t() if lay[1] == "n" else B0
                     C, D = C0.t(), D0.t()
-                    run = lambda: cuasr_amd.srgemm(add, mult, A, B, C, D, one, one, ident, one, dtype=dt, kernel=args.kernel)
+                    # the descriptor is built once: at the small sizes a launch is shorter than building it
+                    desc = cuasr_amd.make_desc(add, mult, dt, A, B, C, D, one, one, ident, one, 1, args.kernel)
+                    ref, launch = ctypes.byref(desc), cuasr_amd.load().cuasr_amd_srgemm
+                    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+                    def run():
+                        if launch(ref, stream) != 0:
+                            raise RuntimeError(f"cuasr_amd_srgemm failed for {add}-{mult} {dt} {n} {lay}")
                     for _ in range(max(3, reps // 4)):
                         run()
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -86,7 +94,6 @@ def main():
                     tops = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
                     per_layout.append(tops)
                     if sink:
-                        desc = cuasr_amd.make_desc(add, mult, dt, A, B, C, D, one, one, ident, one)
                         fam = (cuasr_amd.load().cuasr_amd_selected_kernel(desc) or b"?").decode() if args.kernel == "auto" else args.kernel
                         sink.write(json.dumps({"add": add, "mult": mult, "dtype": dt, "n": n, "layout": lay, "ms": round(ms, 5),
                                                "tops": round(tops, 2), "kernel_family": fam}) + "\n")
