@@ -174,6 +174,51 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   return kNaive;
 }
 
+// A large output whose direct-to-LDS tiles do not fill whole rounds (5120^2 is 800 tiles: a round
+// and a half) need not give the fast tile up altogether: the largest top-left block of whole tiles
+// that does fill its rounds runs on the direct tile, and the strips to its right and below it on
+// the staged family.  The three launches write disjoint parts of D and read A, B, C only.
+struct Block { int rows, cols; };
+static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
+  const Block none{0, 0};
+  if (d->kernel != CUASR_AMD_KERNEL_AUTO || d->split_k_slices != 1 || !direct_usable(d)) return none;
+  if (!find_valu(d->dtype, d->add_op, d->mult_op)) return none;
+  const bool f64 = d->dtype == CUASR_AMD_F64;
+  const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;
+  const int tile_n = f64 ? 64 : 128;
+  const long long slots = f64 ? 768 : 512;
+  const int tr = c.m / tile_m, tc = c.n / tile_n;  // whole tiles only
+  long long best = 0;
+  Block b = none;
+  for (int r = 1; r <= tr; ++r) {
+    for (int q = tc; q >= 1; --q) {
+      const long long t = (long long)r * q;
+      if (t <= best) break;  // narrower blocks of this height are smaller still
+      const long long rounds = (t + slots - 1) / slots;
+      if (t * 100 >= rounds * slots * 97) {
+        best = t;
+        b = Block{r * tile_m, q * tile_n};
+        break;
+      }
+    }
+  }
+  // worth three launches only when the block is most of the output
+  if (best * tile_m * tile_n * 10 < (long long)c.m * c.n * 6) return none;
+  return b;
+}
+
+// rows [r0, r0 + rows) x columns [c0, c0 + cols) of the output as a problem of its own
+static Problem sub_problem(const Problem &p, size_t es, int r0, int c0, int rows, int cols) {
+  Problem q = p;
+  q.m = rows;
+  q.n = cols;
+  q.A = static_cast<const char *>(p.A) + (long long)r0 * p.sa_m * (long long)es;
+  q.B = static_cast<const char *>(p.B) + (long long)c0 * p.sb_n * (long long)es;
+  if (p.C) q.C = static_cast<const char *>(p.C) + ((long long)r0 * p.ldc + c0) * (long long)es;
+  q.D = static_cast<char *>(p.D) + ((long long)r0 * p.ldd + c0) * (long long)es;
+  return q;
+}
+
 static launch_fn family_fn(int family, const cuasr_amd_srgemm_desc *d) {
   switch (family) {
     case kMfma: return find_mfma(d->dtype, d->add_op, d->mult_op);
@@ -224,9 +269,25 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   const int st = validate(desc, false);
   if (st != CUASR_AMD_SUCCESS) return st;
   const Problem p = canonical(desc);
-  const launch_fn fn = family_fn(pick_family(desc), desc);
+  const int family = pick_family(desc);
+  const launch_fn fn = family_fn(family, desc);
   if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
-  return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (family == kValu) {
+    const bool f32_minmax = desc->dtype != CUASR_AMD_F64 && ((desc->add_op == kMaximum && desc->mult_op == kMinimum) ||
+                                                              (desc->add_op == kMinimum && desc->mult_op == kMaximum));
+    const bool masked = desc->add_op == kLogicalOr && desc->mult_op == kLogicalAnd;
+    const Block b = (f32_minmax || masked) ? Block{0, 0} : direct_block(desc, p);  // those two prefer the staged tile anyway
+    const launch_fn direct = b.rows ? find_direct(desc->dtype, desc->add_op, desc->mult_op) : nullptr;
+    if (direct) {
+      const size_t es = elem_size(desc->dtype);
+      hipError_t e = direct(sub_problem(p, es, 0, 0, b.rows, b.cols), s);
+      if (e == hipSuccess && b.cols < p.n) e = fn(sub_problem(p, es, 0, b.cols, b.rows, p.n - b.cols), s);
+      if (e == hipSuccess && b.rows < p.m) e = fn(sub_problem(p, es, b.rows, 0, p.m - b.rows, p.n), s);
+      return e == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+    }
+  }
+  return fn(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
 
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {

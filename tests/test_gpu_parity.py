@@ -288,3 +288,15 @@ def test_valu_full_size_tile_two_groups(oracle, lib, sr, shape):
         la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
         run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "valu", True)
     run(oracle, sr[0], sr[1], sr[2], *shape, "col", "row", "row", "valu", False)
+
+
+@pytest.mark.parametrize("case", [("minimum", "plus", "f32", 5120, 5120, 24, "ccc"), ("minimum", "plus", "f32", 5120, 4736, 20, "rcr"),
+                                  ("bit_xor", "bit_and", "u32", 4608, 5248, 16, "crr"), ("maximum", "plus", "f64", 4480, 3264, 12, "ccc"),
+                                  ("plus", "multiplies", "f32", 5124, 5000, 8, "ccr")])
+def test_large_output_in_two_regions(oracle, lib, case):
+    """Outputs whose direct-to-LDS tiles do not fill whole rounds run a top-left block on that tile and the two
+    remaining strips on the staged tiles: three launches, disjoint parts of D."""
+    add, mult, dtype, m, n, k, layouts = case
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (True, False):
+        run(oracle, add, mult, dtype, m, n, k, la, lb, lc, "auto", beta_one)
