@@ -12,7 +12,8 @@
 // plus-times.
 //
 // Workgroup 256 threads = 4 waves (2 x 2), output tile 128 x 128, wave tile
-// 64 x 64 = 2 x 2 blocks of 32 x 32 (64 accumulator registers), k-tile 16.
+// 64 x 64 = 2 x 2 blocks of 32 x 32 (64 accumulator registers), k-tile 16; or
+// output tile 128 x 256, wave tile 64 x 128 (128 accumulator registers).
 // LDS per stage: A and B k-major, [k][LD] floats.  The instruction wants k = 2q
 // from lanes 0..31 and k = 2q + 1 from lanes 32..63, each lane one float of
 // its row: 32 consecutive floats of LDS row 2q and 32 of row 2q + 1 per read,
@@ -30,9 +31,12 @@ using namespace mfma_panel;
 constexpr int LD = 160;
 __device__ __forceinline__ int swz(int k) { return ((k >> 2) & 1) << 4; }
 
-struct Smem {
+// NB: 128-column halves of the B panel.  1: output tile 128 x 128, wave tile 64 x 64.  2: output
+// tile 128 x 256, wave tile 64 x 128 -- six LDS reads per sixteen matrix instructions instead of
+// four per eight, and a quarter less global traffic per flop; for outputs that fill its rounds.
+template <int NB> struct Smem {
   float a[2][BK][LD];
-  float b[2][BK][LD];
+  float b[2][NB][BK][LD];
 };
 
 // One operand's share of a thread in the global -> LDS copy of a 128 x 16 panel:
@@ -113,8 +117,10 @@ struct Mover {
   }
 };
 
+template <int NB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_kernel(Problem p) {
-  __shared__ Smem sm;
+  constexpr int BN = 128 * NB, WN = 64 * NB, QB = 2 * NB;  // tile columns, wave columns, 32-column blocks per wave
+  __shared__ Smem<NB> sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -132,61 +138,74 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const bool a_xc = p.sa_m == 1, b_xc = p.sb_n == 1;
 
   // byte offset, inside the LDS panel array, of this lane's operand for k-pair 0 of an even / odd k-quad
-  int a_idx[2][2], b_idx[2][2];
+  int a_idx[2][2], b_idx[QB][2];
 #pragma unroll
-  for (int q = 0; q < 2; ++q)
+  for (int o = 0; o < 2; ++o) {
 #pragma unroll
-    for (int o = 0; o < 2; ++o) {
-      a_idx[q][o] = 4 * ((lane >> 5) * LD + ((wm * 64 + q * 32 + (lane & 31)) ^ (o << 4)));
-      b_idx[q][o] = 4 * ((lane >> 5) * LD + ((wn * 64 + q * 32 + (lane & 31)) ^ (o << 4)));
+    for (int q = 0; q < 2; ++q) a_idx[q][o] = 4 * ((lane >> 5) * LD + ((wm * 64 + q * 32 + (lane & 31)) ^ (o << 4)));
+#pragma unroll
+    for (int q = 0; q < QB; ++q) {
+      const int c = wn * WN + q * 32;  // the block's first column inside the tile: half c / 128, column c % 128 of it
+      b_idx[q][o] = 4 * ((c >> 7) * BK * LD + (lane >> 5) * LD + (((c & 127) + (lane & 31)) ^ (o << 4)));
     }
+  }
 
-  v16f acc[2][2];
+  v16f acc[2][QB];
 #pragma unroll
   for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
+    for (int bj = 0; bj < QB; ++bj)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[bi][bj][r] = p.add_identity.f32;  // 0 for plus
 
   const int ntiles = (ke - kb + BK - 1) / BK;
-  Mover ma, mb;
+  Mover ma, mb[NB];
   ma.init(A, p.sa_m, p.sa_k, m0, p.m, kb, a_xc);
-  mb.init(B, p.sb_n, p.sb_k, n0, p.n, kb, b_xc);
-  v4f ra[2], rb[2];
+#pragma unroll
+  for (int h = 0; h < NB; ++h) mb[h].init(B, p.sb_n, p.sb_k, n0 + 128 * h, p.n, kb, b_xc);
+  v4f ra[2], rb[NB][2];
   // k-tile t into registers; `whole` says at compile time whether it has all BK values of k
   // (one code path per call site: merged paths made the compiler wait for the first three loads
   // of a tile before issuing the fourth)
   auto fetch = [&](int t, auto whole) {
     if constexpr (decltype(whole)::value) {
       ma.load(ra);
-      mb.load(rb);
+#pragma unroll
+      for (int h = 0; h < NB; ++h) mb[h].load(rb[h]);
     } else {
       const int kcount = ke - (kb + t * BK);
       ma.load_ragged(ra, p.sa_k, kcount);
-      mb.load_ragged(rb, p.sb_k, kcount);
+#pragma unroll
+      for (int h = 0; h < NB; ++h) mb[h].load_ragged(rb[h], p.sb_k, kcount);
     }
     ma.advance();
-    mb.advance();
+#pragma unroll
+    for (int h = 0; h < NB; ++h) mb[h].advance();
+  };
+  auto store = [&](int stage) {
+    ma.store(ra, &sm.a[stage][0][0]);
+#pragma unroll
+    for (int h = 0; h < NB; ++h) mb[h].store(rb[h], &sm.b[stage][h][0][0]);
   };
   const int nfull = max(ke - kb, 0) / BK;
   if (ntiles > 0) {
     if (nfull > 0) fetch(0, std::true_type{});
     else fetch(0, std::false_type{});
-    ma.store(ra, &sm.a[0][0][0]);
-    mb.store(rb, &sm.b[0][0][0]);
+    store(0);
   }
   __syncthreads();
 
-  int buf = 0, stage_step = BK * LD * 4;
+  int buf = 0, a_step = BK * LD * 4, b_step = NB * BK * LD * 4;
+  constexpr int STORE_AT = KQ - 2;
   // One k-tile: the next tile's global loads, this tile's matrix instructions, the next tile's
   // LDS stores, a barrier.  RAGGED (the last tile of a k range that is not a multiple of BK): k
   // past the end must not count.  The panels hold other (finite or not) data there, so the
   // operands of those k are replaced by zeros: 0 * 0 adds nothing.  Kept out of the steady-state
-  // loop, whose body then has no branch (125.6 -> 130.3 TFLOP/s at 4096^3).  The instruction
-  // order inside a tile is the compiler's: pinning the global loads to the top of the tile, or the
-  // LDS reads a k-quad ahead of their use, both measured slower (122 and 114 TFLOP/s) -- two
-  // workgroups share each SIMD, and one's stalls are the other's matrix-pipe time.
+  // loop, whose body then has no branch (125.6 -> 130.3 TFLOP/s at 4096^3).  Order inside a tile:
+  // the next tile's global loads first, its LDS stores after the third of the four k-quads, so
+  // that they run under the last quad's matrix instructions instead of between them and the
+  // barrier (2048^3: 88.6 -> 110.3 TFLOP/s, 6144^3: 117.7 -> 127.7); the LDS reads stay where the
+  // compiler puts them -- a k-quad ahead of their use measured slower (114 TFLOP/s at 4096^3).
   // NEXT: what follows this tile -- 2 a whole tile, 1 a ragged one, 0 nothing
   auto tile = [&](int t, auto ragged, auto next) {
     constexpr bool RAGGED = decltype(ragged)::value;
@@ -194,52 +213,55 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr bool more = NEXT != 0;
     if constexpr (NEXT == 2) fetch(t + 1, std::true_type{});
     if constexpr (NEXT == 1) fetch(t + 1, std::false_type{});
+    __builtin_amdgcn_sched_barrier(0);
     const int kcount = ke - (kb + t * BK);
     const char *pa = reinterpret_cast<const char *>(&sm.a[0][0][0]);
-    const char *pb = reinterpret_cast<const char *>(&sm.b[0][0][0]);
+    const char *pb = reinterpret_cast<const char *>(&sm.b[0][0][0][0]);
 #pragma unroll
     for (int kq = 0; kq < KQ; ++kq) {
-      float av[2][2], bv[2][2];  // [block][k-pair of the quad]
+      float av[2][2], bv[QB][2];  // [block][k-pair of the quad]
 #pragma unroll
-      for (int q = 0; q < 2; ++q)
+      for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          av[q][j] = *reinterpret_cast<const float *>(pa + (kq * 4 + 2 * j) * LD * 4 + a_idx[q][kq & 1]);
-          bv[q][j] = *reinterpret_cast<const float *>(pb + (kq * 4 + 2 * j) * LD * 4 + b_idx[q][kq & 1]);
-        }
+        for (int q = 0; q < 2; ++q) av[q][j] = *reinterpret_cast<const float *>(pa + (kq * 4 + 2 * j) * LD * 4 + a_idx[q][kq & 1]);
+#pragma unroll
+        for (int q = 0; q < QB; ++q) bv[q][j] = *reinterpret_cast<const float *>(pb + (kq * 4 + 2 * j) * LD * 4 + b_idx[q][kq & 1]);
+      }
       if constexpr (RAGGED) {
 #pragma unroll
-        for (int q = 0; q < 2; ++q)
+        for (int j = 0; j < 2; ++j) {
+          const bool valid = kq * 4 + 2 * j + (lane >> 5) < kcount;
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            const bool valid = kq * 4 + 2 * j + (lane >> 5) < kcount;
-            av[q][j] = valid ? av[q][j] : 0.0f;
-            bv[q][j] = valid ? bv[q][j] : 0.0f;
-          }
+          for (int q = 0; q < 2; ++q) av[q][j] = valid ? av[q][j] : 0.0f;
+#pragma unroll
+          for (int q = 0; q < QB; ++q) bv[q][j] = valid ? bv[q][j] : 0.0f;
+        }
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
-          for (int bj = 0; bj < 2; ++bj)
+          for (int bj = 0; bj < QB; ++bj)
             acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[bi][j], bv[bj][j], acc[bi][bj], 0, 0, 0);
-    }
-    if constexpr (more) {
-      ma.store(ra, &sm.a[buf ^ 1][0][0]);
-      mb.store(rb, &sm.b[buf ^ 1][0][0]);
+      if (kq == STORE_AT) {
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (more) store(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     __syncthreads();
     buf ^= 1;
     // the lane's read indices follow the stage: one add each instead of an address per read
 #pragma unroll
-    for (int q = 0; q < 2; ++q)
+    for (int o = 0; o < 2; ++o) {
 #pragma unroll
-      for (int o = 0; o < 2; ++o) {
-        a_idx[q][o] += stage_step;
-        b_idx[q][o] += stage_step;
-      }
-    stage_step = -stage_step;
+      for (int q = 0; q < 2; ++q) a_idx[q][o] += a_step;
+#pragma unroll
+      for (int q = 0; q < QB; ++q) b_idx[q][o] += b_step;
+    }
+    a_step = -a_step;
+    b_step = -b_step;
   };
   using whole_next = std::integral_constant<int, 2>;
   using ragged_next = std::integral_constant<int, 1>;
@@ -273,8 +295,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
   for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
-      const int col = n0 + wn * 64 + bj * 32 + (lane & 31);
+    for (int bj = 0; bj < QB; ++bj) {
+      const int col = n0 + wn * WN + bj * 32 + (lane & 31);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + wm * 64 + bi * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
@@ -293,10 +315,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   if (!can_run(p)) return hipErrorNotSupported;
-  const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+  const long long tiles_m = (p.m + BM - 1) / BM, slices = p.workspace ? p.slices : 1;
+  const long long tiles = tiles_m * ((p.n + 127) / 128), wide = tiles_m * ((p.n + 255) / 256);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
-  hipLaunchKernelGGL(gemm_mfma_kernel, grid, dim3(256), 0, s, p);
+  // the 128 x 256 tile when its workgroups fill >= 7/8 of whole rounds of 512 (two per compute unit)
+  const long long rounds = (wide * slices + 511) / 512;
+  if (wide * slices * 8 >= rounds * 512 * 7)
+    hipLaunchKernelGGL(gemm_mfma_kernel<2>, dim3((unsigned)wide, (unsigned)slices), dim3(256), 0, s, p);
+  else
+    hipLaunchKernelGGL(gemm_mfma_kernel<1>, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
   return hipGetLastError();
 }
 
