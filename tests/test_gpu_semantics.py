@@ -107,3 +107,59 @@ def test_reference_cross_implementation_shapes(oracle, lib, shape, kernel):
     cuasr_amd.srgemm("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, 0.0, 0.0, float("inf"), 0.0, kernel=kernel)
     torch.cuda.synchronize()
     assert_same_bits(to_host(dD, "f32"), want, f"{shape} {kernel}")
+
+
+def test_calls_can_be_captured_in_a_graph(oracle, lib):
+    """Nothing in a call allocates, frees or synchronises, so a stream capture may contain it: two squarings, a
+    parallel and a serial split-K are captured once and replayed on new inputs, with eager work and
+    synchronisations between the replays; every replay must equal the eager result."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    n, k = 192, 640
+    inf = float("inf")
+    d_in = torch.empty(n, n, device="cuda").t()            # column-major, as the repeated-squaring step uses it
+    d_mid, d_out = torch.empty(n, n, device="cuda").t(), torch.empty(n, n, device="cuda").t()
+    a = torch.empty(n, k, device="cuda")                    # k contiguous in both operands: the split-K example's layout
+    b = torch.empty(n, k, device="cuda").t()
+    s_par, s_ser = torch.empty(n, n, device="cuda"), torch.empty(n, n, device="cuda")
+    ws = torch.empty(n * n * 4, dtype=torch.float32, device="cuda")
+
+    def work():
+        cuasr_amd.srgemm("minimum", "plus", d_in, d_in, d_in, d_mid, 0.0, 0.0, inf, 0.0)
+        cuasr_amd.srgemm("minimum", "plus", d_mid, d_mid, d_mid, d_out, 0.0, 0.0, inf, 0.0)
+        cuasr_amd.srgemm_splitk("minimum", "plus", a, b, d_out.t(), s_par, 4, ws, 0.0, 0.0, inf, 0.0)
+        cuasr_amd.srgemm_splitk_serial("minimum", "plus", a, b, d_out.t(), s_ser, 3, ws, 0.0, 0.0, inf, 0.0)
+
+    def load(seed):
+        D = inputs.graph_distances(seed, n, density=0.2, lo=1.0, hi=9.0)
+        A, B = inputs.uniform(seed + 1, n, k, 0.0, 10.0, order="C"), inputs.uniform(seed + 2, k, n, 0.0, 10.0, order="F")
+        d_in.copy_(torch.from_numpy(np.ascontiguousarray(D.T)).cuda().t())
+        a.copy_(torch.from_numpy(A).cuda())
+        b.copy_(torch.from_numpy(np.ascontiguousarray(B.T)).cuda().t())
+        return D, A, B
+
+    load(100)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    for seed in (200, 300, 400):
+        D, A, B = load(seed)
+        # eager work of the program's own between the replays
+        scratch = torch.rand(256, 256, device="cuda") @ torch.rand(256, 256, device="cuda")
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        del scratch
+        D1 = oracle.srgemm("minimum", "plus", D, D, D, 0.0, 0.0, np.inf)
+        D2 = oracle.srgemm("minimum", "plus", D1, D1, D1, 0.0, 0.0, np.inf)
+        assert_same_bits(d_out.cpu().numpy(), D2, f"graph replay, seed {seed}: squarings")
+        C = np.ascontiguousarray(D2.T)                      # d_out.t() is the transpose, row-major
+        want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)
+        assert_same_bits(s_par.cpu().numpy(), want, f"graph replay, seed {seed}: split-K")
+        assert_same_bits(s_ser.cpu().numpy(), want, f"graph replay, seed {seed}: serial split-K")
