@@ -184,6 +184,9 @@ static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO || d->split_k_slices != 1 || !direct_usable(d)) return none;
   if (!find_valu(d->dtype, d->add_op, d->mult_op)) return none;
   const bool f64 = d->dtype == CUASR_AMD_F64;
+  // min-max / max-min on 4-byte types and or-and prefer the staged tile at any size (pick_family)
+  const bool f32_minmax = !f64 && ((d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum));
+  if (f32_minmax || (d->add_op == kLogicalOr && d->mult_op == kLogicalAnd)) return none;
   const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;
   const int tile_n = f64 ? 64 : 128;
   const long long slots = f64 ? 768 : 512;
@@ -260,7 +263,7 @@ const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc) {
   switch (pick_family(desc)) {
     case kMfma: return "mfma";
     case kDirect: return "valu_direct";
-    case kValu: return "valu";
+    case kValu: return direct_block(desc, canonical(desc)).rows ? "valu_direct+valu" : "valu";  // a block + two strips
     default: return "naive";
   }
 }
@@ -274,10 +277,7 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (family == kValu) {
-    const bool f32_minmax = desc->dtype != CUASR_AMD_F64 && ((desc->add_op == kMaximum && desc->mult_op == kMinimum) ||
-                                                              (desc->add_op == kMinimum && desc->mult_op == kMaximum));
-    const bool masked = desc->add_op == kLogicalOr && desc->mult_op == kLogicalAnd;
-    const Block b = (f32_minmax || masked) ? Block{0, 0} : direct_block(desc, p);  // those two prefer the staged tile anyway
+    const Block b = direct_block(desc, p);
     const launch_fn direct = b.rows ? find_direct(desc->dtype, desc->add_op, desc->mult_op) : nullptr;
     if (direct) {
       const size_t es = elem_size(desc->dtype);

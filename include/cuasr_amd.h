@@ -183,7 +183,9 @@ int cuasr_amd_srgemm_splitk_serial(const cuasr_amd_srgemm_desc *desc, void *work
                                    void *stream);
 
 /* Name of the kernel family AUTO would choose for this descriptor
- * ("naive", "valu", "valu_direct", "mfma"), or NULL if the descriptor is invalid. */
+ * ("naive", "valu", "valu_direct", "mfma"; "valu_direct+valu" when a block of the output runs on
+ * the direct-to-LDS tile and the strips around it on the staged one), or NULL if the descriptor
+ * is invalid. */
 const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc);
 
 #ifdef __cplusplus

@@ -86,6 +86,8 @@ def test_kernel_selection(lib):
     assert sel(desc(dtype="f64", add="plus", mult="multiplies")) == b"valu"
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
     assert sel(desc(kernel="mfma")) == b"mfma"
+    assert sel(desc(m=5120, n=5120, k=64)) == b"valu_direct+valu"   # 800 direct tiles: one full round + two strips
+    assert sel(desc(m=3072, n=3072, k=64)) == b"valu"               # 288 direct tiles fill no round
 
 
 def test_splitk_host_errors(lib):
