@@ -88,6 +88,13 @@ def load():
         lib.cuasr_amd_splitk_serial_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk_serial.restype = ctypes.c_int
         lib.cuasr_amd_srgemm_splitk_serial.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_fwgemm.restype = ctypes.c_int
+        lib.cuasr_amd_fwgemm.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_void_p]
+        lib.cuasr_amd_apsp_workspace_bytes.restype = ctypes.c_size_t
+        lib.cuasr_amd_apsp_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.cuasr_amd_apsp_squaring.restype = ctypes.c_int
+        lib.cuasr_amd_apsp_squaring.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                                ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
         lib.cuasr_amd_selected_kernel.restype = ctypes.c_char_p
         lib.cuasr_amd_selected_kernel.argtypes = [ctypes.POINTER(SrgemmDesc)]
         _lib = lib
@@ -283,3 +290,49 @@ def srgemm_splitk_serial(add_op, mult_op, A, B, C, D, slices, workspace, alpha=N
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_srgemm_splitk_serial")
     return D
+
+
+def _column_major(t, what):
+    """(pointer, leading dimension) of a column-major 2-D device tensor."""
+    ref = MatRef.of(t)
+    if ref.layout != COLUMN_MAJOR:
+        raise ValueError(f"{what} must be column-major")
+    return ctypes.c_void_p(ref.ptr), ctypes.c_int64(ref.ld)
+
+
+def fwgemm(A, B, dist, parent, kernel="auto", stream=None):
+    """dist = min(dist, A (x) B) with parent[i, j] = the k that gave each new
+    minimum, in place (test/regress/include/fwgpu/cpu_srgemm.hpp:20-48).  All
+    four are column-major device tensors; parent is int32."""
+    import torch
+    if parent.dtype != torch.int32:
+        raise ValueError("parent must be int32")
+    (m, k), n = A.shape, B.shape[1]
+    pa, lda = _column_major(A, "A")
+    pb, ldb = _column_major(B, "B")
+    pd, ldc = _column_major(dist, "dist")
+    pp, ldp = _column_major(parent, "parent")
+    st = load().cuasr_amd_fwgemm(DTYPES[_torch_dtype_name(dist)], m, n, k, pa, lda, pb, ldb, pd, ldc, pp, ldp,
+                                 KERNELS[kernel], _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_fwgemm")
+    return dist, parent
+
+
+def apsp_workspace_bytes(n, dtype):
+    return int(load().cuasr_amd_apsp_workspace_bytes(DTYPES[dtype], n))
+
+
+def apsp_squaring(dist, parent, workspace, iterations=0, stream=None):
+    """All-pairs shortest paths by repeated squaring, in place on the n x n
+    column-major ``dist`` and int32 ``parent``; ``workspace`` is a device tensor
+    of at least apsp_workspace_bytes(n, dtype) bytes."""
+    n = dist.shape[0]
+    pd, ld = _column_major(dist, "dist")
+    pp, ldp = _column_major(parent, "parent")
+    ws = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
+    st = load().cuasr_amd_apsp_squaring(DTYPES[_torch_dtype_name(dist)], n, pd, ld, pp, ldp, ws, int(iterations),
+                                        _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_apsp_squaring")
+    return dist, parent

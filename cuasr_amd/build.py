@@ -24,7 +24,8 @@ def sources():
 
 # the vector-ALU tiles may assume NaN-free data: it lets min/max map to single
 # (3-input) instructions without re-canonicalising every accumulator
-PER_FILE = {"valu_": ["-fno-honor-nans"], "mfma_f32": ["-fno-honor-nans"], "direct_": ["-fno-honor-nans"]}
+PER_FILE = {"valu_": ["-fno-honor-nans"], "mfma_f32": ["-fno-honor-nans"], "direct_": ["-fno-honor-nans"],
+            "fwgemm": ["-fno-honor-nans"]}
 
 
 def _compile(src):

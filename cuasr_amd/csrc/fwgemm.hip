@@ -1,0 +1,337 @@
+// Min-plus product that also records where each new minimum came from
+// (the building block of all-pairs shortest paths with path recovery), and the
+// repeated-squaring driver on top of it.  Semantics: cpu_fwgemm_naive,
+// test/regress/include/fwgpu/cpu_srgemm.hpp:20-48 -- for every (row, col), scan
+// k ascending, take prod = A[row,k] + B[k,col], and on prod < dist replace dist
+// by prod and parent by k.  All four matrices are column-major.
+//
+// The result does not depend on the scan order when stated as: let v be the
+// smallest product; if v < dist then dist = v and parent = the smallest k whose
+// product equals v; otherwise nothing changes.  The tile kernel uses that form:
+//   - per chunk of BK k-values it keeps a plain min-plus accumulator (1.5
+//     vector instructions per term, as in the SRGEMM tiles),
+//   - after the chunk, "chunk minimum < running minimum" (strict) moves the
+//     running minimum and records the chunk index: 3 instructions per BK terms,
+//   - the epilogue re-reads the recorded chunk of every improved element and
+//     takes the first k whose product equals the minimum.  The product is the
+//     same single addition of the same operands, so equality is exact, and the
+//     stored distance is that product, which keeps the sign of a zero as the
+//     sequential scan would.
+// Operands must be free of NaN and of -infinity (+infinity marks "no edge").
+#include "semiring.h"
+
+#include <limits>
+
+namespace cuasr_amd {
+namespace {
+
+struct FwArgs {
+  int m, n, k;
+  const void *A; int64_t lda;
+  const void *B; int64_t ldb;
+  void *dist; int64_t ldc;
+  int32_t *parent; int64_t ldp;
+};
+
+// cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
+// folded into a hardware minimum when NaNs need not be honoured, and that minimum
+// prefers -0 to +0, where the reference's comparison keeps whichever came first
+template <typename T> __device__ __forceinline__ T pick(bool cond, T a, T b) {
+  asm("" : "+v"(a));
+  return cond ? a : b;
+}
+
+// one thread per element, the literal scan; any extent, any leading dimension
+template <typename T>
+__global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
+  const int row = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int col = blockIdx.y * 4 + (threadIdx.x >> 6);
+  if (row >= g.m || col >= g.n) return;
+  const T *a = static_cast<const T *>(g.A) + row;
+  const T *b = static_cast<const T *>(g.B) + col * g.ldb;
+  T *d = static_cast<T *>(g.dist) + row + col * g.ldc;
+  int32_t *pp = g.parent + row + col * g.ldp;
+  T curr = *d;
+  int32_t p = *pp;
+  for (int i = 0; i < g.k; ++i) {
+    const T prod = a[i * g.lda] + b[i];
+    const bool lower = prod < curr;
+    curr = pick(lower, prod, curr);
+    p = lower ? i : p;
+  }
+  *d = curr;
+  *pp = p;
+}
+
+template <typename T> struct vec4_of;
+template <> struct vec4_of<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct vec4_of<double> { typedef double type __attribute__((ext_vector_type(4))); };
+
+// 256 threads as 16 x 16; each owns TM x TN outputs in groups of four rows /
+// columns that lie 64 apart, so a workgroup covers (16 TM) x (16 TN).
+// GUARD = false: whole tiles, 16-byte aligned columns of A and B (vector loads).
+// GUARD = true : any extents and alignment; out-of-range operands read as
+//                +infinity, whose products never improve anything.
+template <typename T, int TM, int TN, int SN, int BK, bool GUARD>
+__global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
+  typedef typename vec4_of<T>::type V4;
+  constexpr int BM = 16 * TM, BN = 16 * TN, PAD = 4;
+  constexpr int NA = BM * BK / 4 / 256, NB = BN * BK / 4 / 256;
+  static_assert(TM % 4 == 0 && TN % SN == 0 && SN % 4 == 0 && BK % 4 == 0 && BK % 2 == 0 && NA >= 1 && NB >= 1, "tile shape");
+  __shared__ __attribute__((aligned(16))) T as[2][BK][BM + PAD];
+  __shared__ __attribute__((aligned(16))) T bs[2][BK][BN + PAD];
+
+  const T *A = static_cast<const T *>(g.A);
+  const T *B = static_cast<const T *>(g.B);
+  const int tid = threadIdx.x & 255;
+  const int tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const T inf = std::numeric_limits<T>::infinity();
+
+  auto row_of = [&](int i) { return m0 + (i >> 2) * 64 + tx * 4 + (i & 3); };
+  auto col_of = [&](int j) { return n0 + (j >> 2) * 64 + ty * 4 + (j & 3); };
+
+  V4 ra[NA], rb[NB];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int p = 0; p < NA; ++p) {
+      const int v = tid + p * 256, r = (v % (BM / 4)) * 4, kk = v / (BM / 4);
+      if constexpr (!GUARD) {
+        ra[p] = *reinterpret_cast<const V4 *>(A + (m0 + r) + int64_t(k0 + kk) * g.lda);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          ra[p][e] = (m0 + r + e < g.m && k0 + kk < g.k) ? A[(m0 + r + e) + int64_t(k0 + kk) * g.lda] : inf;
+      }
+    }
+#pragma unroll
+    for (int p = 0; p < NB; ++p) {
+      const int v = tid + p * 256, kk = (v % (BK / 4)) * 4, c = v / (BK / 4);
+      if constexpr (!GUARD) {
+        rb[p] = *reinterpret_cast<const V4 *>(B + (k0 + kk) + int64_t(n0 + c) * g.ldb);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          rb[p][e] = (n0 + c < g.n && k0 + kk + e < g.k) ? B[(k0 + kk + e) + int64_t(n0 + c) * g.ldb] : inf;
+      }
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < NA; ++p) {
+      const int v = tid + p * 256, r = (v % (BM / 4)) * 4, kk = v / (BM / 4);
+      *reinterpret_cast<V4 *>(&as[buf][kk][r]) = ra[p];
+    }
+#pragma unroll
+    for (int p = 0; p < NB; ++p) {
+      const int v = tid + p * 256, kk = (v % (BK / 4)) * 4, c = v / (BK / 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) bs[buf][kk + e][c] = rb[p][e];
+    }
+  };
+
+  struct Frag {
+    T a[2][4], b[2][SN];
+  };
+  auto load_frag = [&](Frag &f, int buf, int kk, int qi, int qj) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      *reinterpret_cast<V4 *>(&f.a[u][0]) = *reinterpret_cast<const V4 *>(&as[buf][kk + u][qi * 64 + tx * 4]);
+#pragma unroll
+      for (int q = 0; q < SN / 4; ++q)
+        *reinterpret_cast<V4 *>(&f.b[u][q * 4]) =
+            *reinterpret_cast<const V4 *>(&bs[buf][kk + u][(qj * (SN / 4) + q) * 64 + ty * 4]);
+    }
+  };
+
+  T acc[TM][TN];
+  int32_t chunk[TM][TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int r = row_of(i), c = col_of(j);
+      chunk[i][j] = -1;
+      if constexpr (!GUARD) acc[i][j] = static_cast<const T *>(g.dist)[r + int64_t(c) * g.ldc];
+      else acc[i][j] = (r < g.m && c < g.n) ? static_cast<const T *>(g.dist)[r + int64_t(c) * g.ldc] : -inf;
+    }
+
+  const int tiles = (g.k + BK - 1) / BK;
+  if (tiles > 0) {
+    fetch(0);
+    stage(0);
+  }
+  __syncthreads();
+  for (int t = 0; t < tiles; ++t) {
+    const int cur = t & 1;
+    if (t + 1 < tiles) fetch((t + 1) * BK);
+    // one block of 4 x SN outputs at a time, so that only its chunk minima are live
+#pragma unroll
+    for (int qi = 0; qi < TM / 4; ++qi)
+#pragma unroll
+      for (int qj = 0; qj < TN / SN; ++qj) {
+        T best[4][SN];
+        // two k-values per step (a 3-input minimum per pair of products); the next
+        // step's fragments are read from LDS while this one is computed, and the
+        // scheduling barriers keep the reads of later steps from being hoisted
+        // (a whole tile's fragments do not fit in registers)
+        Frag f[2];
+        load_frag(f[0], cur, 0, qi, qj);
+#pragma unroll
+        for (int kp = 0; kp < BK / 2; ++kp) {
+          if (kp + 1 < BK / 2) load_frag(f[(kp + 1) & 1], cur, 2 * (kp + 1), qi, qj);
+          __builtin_amdgcn_sched_barrier(0);
+          const Frag &x = f[kp & 1];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int j = 0; j < SN; ++j) {
+              const T p0 = x.a[0][i] + x.b[0][j], p1 = x.a[1][i] + x.b[1][j];
+              best[i][j] = kp == 0 ? hw_min<T>(p0, p1) : hw_min<T>(hw_min<T>(best[i][j], p0), p1);
+              // ties the arithmetic to this place in the instruction order: without it
+              // instruction selection emits it next to its only use, after every read
+              asm volatile("" : "+v"(best[i][j]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < SN; ++j) {
+            T &running = acc[qi * 4 + i][qj * SN + j];
+            int32_t &where = chunk[qi * 4 + i][qj * SN + j];
+            const bool lower = best[i][j] < running;
+            running = lower ? best[i][j] : running;
+            where = lower ? t : where;
+          }
+      }
+    if (t + 1 < tiles) stage(cur ^ 1);
+    __syncthreads();
+  }
+
+  // improved elements: the first k of the recorded chunk whose product is the minimum
+  T *dist = static_cast<T *>(g.dist);
+  // the element addresses are formed again from a thread index the compiler cannot
+  // match with the prologue's: keeping 2 x TM x TN addresses live across the loop
+  // would push the accumulators out of the register file
+  int tx2 = tx, ty2 = ty;
+  asm volatile("" : "+v"(tx2), "+v"(ty2));
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int c = n0 + (j >> 2) * 64 + ty2 * 4 + (j & 3);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int r = m0 + (i >> 2) * 64 + tx2 * 4 + (i & 3);
+      const int ch = chunk[i][j];
+      if (ch < 0) continue;
+      if constexpr (GUARD) {
+        if (r >= g.m || c >= g.n) continue;
+      }
+      const int k0 = ch * BK;
+      const T *ap = A + r + int64_t(k0) * g.lda;
+      const T *bp = B + k0 + int64_t(c) * g.ldb;
+      const T want = acc[i][j];
+      T value = want;
+      int first = 0;
+#pragma unroll 4
+      for (int kk = BK - 1; kk >= 0; --kk) {
+        bool in = true;
+        if constexpr (GUARD) in = k0 + kk < g.k;
+        const T prod = in ? ap[int64_t(kk) * g.lda] + bp[kk] : inf;
+        const bool hit = in && prod == want;
+        first = hit ? kk : first;
+        value = pick(hit, prod, value);
+      }
+      dist[r + int64_t(c) * g.ldc] = value;
+      g.parent[r + int64_t(c) * g.ldp] = k0 + first;
+    }
+  }
+}
+
+template <typename T, int TM, int TN, int SN, int BK>
+hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
+  constexpr int BM = 16 * TM, BN = 16 * TN;
+  const bool whole = g.m % BM == 0 && g.n % BN == 0 && g.k % BK == 0;
+  const size_t vec = 4 * sizeof(T);
+  const bool aligned = reinterpret_cast<uintptr_t>(g.A) % vec == 0 && reinterpret_cast<uintptr_t>(g.B) % vec == 0 &&
+                       g.lda % 4 == 0 && g.ldb % 4 == 0;
+  dim3 grid((g.m + BM - 1) / BM, (g.n + BN - 1) / BN);
+  if (whole && aligned)
+    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false>), grid, dim3(256), 0, stream, g);
+  else
+    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true>), grid, dim3(256), 0, stream, g);
+  return hipGetLastError();
+}
+
+template <typename T> hipError_t launch_naive(const FwArgs &g, hipStream_t stream) {
+  dim3 grid((g.m + 63) / 64, (g.n + 3) / 4);
+  hipLaunchKernelGGL(fwgemm_naive_kernel<T>, grid, dim3(256), 0, stream, g);
+  return hipGetLastError();
+}
+
+int check(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, const void *dist,
+          int64_t ldc, const int32_t *parent, int64_t ldp, int kernel) {
+  if (dtype != CUASR_AMD_F32 && dtype != CUASR_AMD_F64) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
+  if (m < 0 || n < 0 || k < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (lda < (m > 1 ? m : 1) || ldb < (k > 1 ? k : 1) || ldc < (m > 1 ? m : 1) || ldp < (m > 1 ? m : 1))
+    return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (kernel != CUASR_AMD_KERNEL_AUTO && kernel != CUASR_AMD_KERNEL_NAIVE && kernel != CUASR_AMD_KERNEL_VALU)
+    return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (m == 0 || n == 0) return CUASR_AMD_SUCCESS;
+  if (!dist || !parent || (k > 0 && (!A || !B))) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  const size_t es = dtype == CUASR_AMD_F64 ? 8 : 4;
+  if (reinterpret_cast<uintptr_t>(A) % es || reinterpret_cast<uintptr_t>(B) % es ||
+      reinterpret_cast<uintptr_t>(dist) % es || reinterpret_cast<uintptr_t>(parent) % 4)
+    return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+  return CUASR_AMD_SUCCESS;
+}
+
+}  // namespace
+}  // namespace cuasr_amd
+
+using namespace cuasr_amd;
+
+extern "C" int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb,
+                                void *dist, int64_t ldc, int32_t *parent, int64_t ldp, int kernel, void *stream) {
+  const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
+  if (st != CUASR_AMD_SUCCESS || m == 0 || n == 0 || k == 0) return st;
+  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // a launch of a few workgroups is better spread over one thread per element
+  const bool tiny = int64_t(m) * n < 64 * 64;
+  const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
+  hipError_t e;
+  if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 8, 16>(g, s);
+  else e = naive ? launch_naive<double>(g, s) : launch_tile<double, 4, 8, 4, 16>(g, s);
+  return e == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+}
+
+extern "C" size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n) {
+  if (n <= 0 || (dtype != CUASR_AMD_F32 && dtype != CUASR_AMD_F64)) return 0;
+  return size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * size_t(n) * size_t(n);
+}
+
+extern "C" int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
+                                       void *workspace, int iterations, void *stream) {
+  const int64_t ldw = n > 0 ? n : 1;
+  const int st = check(dtype, n, n, n, workspace, ldw, workspace, ldw, dist, ld, parent, ldp, CUASR_AMD_KERNEL_AUTO);
+  if (n > 0 && !workspace) return CUASR_AMD_ERROR_WORKSPACE_NULL;
+  if (st != CUASR_AMD_SUCCESS) return st;
+  if (iterations < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (n == 0) return CUASR_AMD_SUCCESS;
+  if (iterations == 0)  // paths of up to n - 1 edges: ceil(log2(n - 1)) squarings
+    for (int64_t reach = 1; reach < n - 1; reach *= 2) ++iterations;
+  const size_t es = dtype == CUASR_AMD_F64 ? 8 : 4;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  for (int it = 0; it < iterations; ++it) {
+    // the product reads a snapshot, so no workgroup sees another's updates
+    if (hipMemcpy2DAsync(workspace, size_t(n) * es, dist, size_t(ld) * es, size_t(n) * es, size_t(n),
+                         hipMemcpyDeviceToDevice, s) != hipSuccess)
+      return CUASR_AMD_ERROR_INTERNAL;
+    const int r = cuasr_amd_fwgemm(dtype, n, n, n, workspace, n, workspace, n, dist, ld, parent, ldp,
+                                   CUASR_AMD_KERNEL_AUTO, stream);
+    if (r != CUASR_AMD_SUCCESS) return r;
+  }
+  return CUASR_AMD_SUCCESS;
+}

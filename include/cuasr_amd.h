@@ -182,6 +182,37 @@ size_t cuasr_amd_splitk_serial_workspace_bytes(const cuasr_amd_srgemm_desc *desc
 int cuasr_amd_srgemm_splitk_serial(const cuasr_amd_srgemm_desc *desc, void *workspace,
                                    void *stream);
 
+/* Min-plus product with predecessor tracking, the step of an all-pairs
+ * shortest-path computation that can rebuild its paths
+ * (cpu_fwgemm_naive, test/regress/include/fwgpu/cpu_srgemm.hpp:20-48; the
+ * reference has this on the CPU only).  A (m x k), B (k x n), dist and parent
+ * (m x n) are column-major device matrices with leading dimensions in elements;
+ * dtype is CUASR_AMD_F32 or CUASR_AMD_F64, parent holds int32.  In place, for
+ * every (row, col):
+ *   scan k ascending; prod = A[row,k] + B[k,col];
+ *   if (prod < dist[row,col]) { dist[row,col] = prod; parent[row,col] = k; }
+ * Elements that do not improve keep both values.  Results are bit-identical to
+ * that scan for operands free of NaN and -infinity (+infinity = no edge).
+ * A and B must not overlap dist.  kernel: CUASR_AMD_KERNEL_AUTO, _NAIVE (one
+ * thread per element) or _VALU (LDS-staged tile).  Errors as for cuasr_amd_srgemm. */
+int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda,
+                     const void *B, int64_t ldb, void *dist, int64_t ldc,
+                     int32_t *parent, int64_t ldp, int kernel, void *stream);
+
+/* All-pairs shortest paths by repeated squaring on an n x n distance matrix
+ * (the application README.md:338-342 of the reference motivates): `iterations`
+ * times, dist is copied into the workspace and cuasr_amd_fwgemm(workspace,
+ * workspace, dist, parent) is run; iterations = 0 means ceil(log2(n - 1)), which
+ * covers every path.  parent[i,j] = k says the shortest i -> j path found is the
+ * i -> k path followed by the k -> j path; an entry the caller initialised (say
+ * to -1) and that never changed means the direct edge.  The workspace holds
+ * cuasr_amd_apsp_workspace_bytes(dtype, n) = sizeof(element) * n * n bytes;
+ * CUASR_AMD_ERROR_WORKSPACE_NULL without it.  Asynchronous on the stream, no
+ * allocation, no host synchronisation. */
+size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n);
+int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *parent,
+                            int64_t ldp, void *workspace, int iterations, void *stream);
+
 /* Name of the kernel family AUTO would choose for this descriptor
  * ("naive", "valu", "valu_direct", "mfma"; "valu_direct+valu" when a block of the output runs on
  * the direct-to-LDS tile and the strips around it on the staged one), or NULL if the descriptor

@@ -156,3 +156,25 @@ def srgemm_splitk_serial(add_op, mult_op, A, B, C, alpha, beta, add_identity,
     if rc != 0:
         raise ValueError(f"oracle: unsupported serial split-K ({dt}, {add_op}, {mult_op})")
     return D
+
+
+def fwgemm(A, B, dist, parent, nthreads=0):
+    """Min-plus product with predecessor tracking, in place on ``dist`` and
+    ``parent`` (column-major float32/float64 and int32 arrays), following
+    test/regress/include/fwgpu/cpu_srgemm.hpp:20-48."""
+    dt = A.dtype
+    m, k = A.shape
+    _, n = B.shape
+    if m == 0 or n == 0 or k == 0:
+        return dist, parent          # an empty scan changes nothing
+    refs = [mat_ref(x) for x in (A, B, dist, parent)]
+    if any(r[2] != COLUMN_MAJOR for r in refs) or parent.dtype != np.int32 or dist.shape != (m, n):
+        raise ValueError("oracle.fwgemm: column-major operands and an int32 parent matrix")
+    (pa, lda, _), (pb, ldb, _), (pd, ldc, _), (pp, ldp, _) = refs
+    fn = lib().oracle_fwgemm
+    fn.restype = ctypes.c_int
+    rc = fn(DTYPES[dt], m, n, k, pa, ctypes.c_int64(lda), pb, ctypes.c_int64(ldb),
+            pd, ctypes.c_int64(ldc), pp, ctypes.c_int64(ldp), int(nthreads))
+    if rc != 0:
+        raise ValueError(f"oracle.fwgemm: unsupported element type {dt}")
+    return dist, parent

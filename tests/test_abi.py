@@ -21,7 +21,8 @@ def test_exports_match_header(lib):
     names = declared_functions()
     assert {"cuasr_amd_srgemm", "cuasr_amd_srgemm_splitk", "cuasr_amd_splitk_workspace_bytes",
             "cuasr_amd_srgemm_can_implement", "cuasr_amd_srgemm_splitk_serial",
-            "cuasr_amd_splitk_serial_workspace_bytes"} <= set(names)
+            "cuasr_amd_splitk_serial_workspace_bytes", "cuasr_amd_fwgemm", "cuasr_amd_apsp_squaring",
+            "cuasr_amd_apsp_workspace_bytes"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
     assert lib.cuasr_amd_abi_version() == 1
@@ -113,6 +114,22 @@ def test_serial_splitk_host_errors(lib):
     d0 = desc(slices=0)
     assert lib.cuasr_amd_srgemm_splitk_serial(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
     assert lib.cuasr_amd_srgemm_splitk_serial(None, None, None) == 4
+
+
+def test_fwgemm_host_errors(lib):
+    P = ctypes.c_void_p
+    call = lambda dtype=0, m=64, n=64, k=64, a=0x1000, lda=64, b=0x1000, ldb=64, d=0x1000, ldc=64, p=0x1000, ldp=64, kern=0: \
+        lib.cuasr_amd_fwgemm(dtype, m, n, k, P(a), lda, P(b), ldb, P(d), ldc, P(p), ldp, kern, None)
+    assert call(dtype=2) == 2                 # float and double only
+    assert call(m=-1) == 4 and call(lda=10) == 4 and call(ldb=63) == 4 and call(ldc=1) == 4 and call(ldp=0) == 4
+    assert call(d=0) == 4 and call(p=0) == 4 and call(a=0) == 4
+    assert call(a=0x1002) == 1 and call(dtype=1, d=0x1004) == 1 and call(p=0x1001) == 1
+    assert call(kern=3) == 5                  # no matrix-core form
+    assert call(m=0) == 0 and call(n=0, d=0) == 0 and call(k=0, a=0, b=0) == 0   # nothing to do, nothing launched
+    assert cuasr_amd.apsp_workspace_bytes(1000, "f32") == 4 * 1000 * 1000
+    assert cuasr_amd.apsp_workspace_bytes(10, "f64") == 800 and cuasr_amd.apsp_workspace_bytes(0, "f32") == 0
+    sq = lambda n=64, ws=0x1000, it=0, dtype=0: lib.cuasr_amd_apsp_squaring(dtype, n, P(0x1000), max(n, 1), P(0x1000), max(n, 1), P(ws), it, None)
+    assert sq(ws=0) == 6 and sq(it=-1) == 4 and sq(dtype=3) == 2 and sq(n=0) == 0
 
 
 def test_semiring_constants():

@@ -1,0 +1,163 @@
+"""GPU parity of the min-plus product with predecessor tracking and of the
+repeated-squaring driver, through the C ABI, against the CPU oracle
+(test/regress/include/fwgpu/cpu_srgemm.hpp:20-48).  Distances are compared
+bit for bit, parents exactly."""
+import numpy as np
+import pytest
+
+import cuasr_amd
+from cuasr_amd import inputs
+from helpers import assert_same_bits, to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def operands(seed, m, n, k, dtype, ties, pad=(0, 0, 0, 0), inf_share=0.2):
+    """Column-major A, B, dist, parent as views with the given extra leading-dimension rows."""
+    rng = np.random.default_rng(seed)
+    def mat(r, c, lo, hi, extra):
+        buf = np.full((r + extra, c), 1.0, dtype=dtype, order="F")
+        v = rng.integers(lo, hi, (r, c)).astype(dtype) if ties else (rng.random((r, c)) * 10).astype(dtype)
+        v[rng.random((r, c)) < inf_share] = np.inf
+        buf[:r] = v
+        return buf
+    A, B = mat(m, k, 0, 6, pad[0]), mat(k, n, 0, 6, pad[1])
+    dist = mat(m, n, 2, 9, pad[2])
+    parent = np.full((m + pad[3], n), -7, dtype=np.int32, order="F")
+    return A, B, dist, parent
+
+
+def run_case(oracle, m, n, k, dtype, ties, kernel, pad=(0, 0, 0, 0), seed=0):
+    A, B, dist, parent = operands(seed + m + 3 * n + 5 * k, m, n, k, dtype, ties, pad)
+    dA, dB, dD, dP = (to_device(x) for x in (A, B, dist, parent))
+    cuasr_amd.fwgemm(dA[:m], dB[:k], dD[:m], dP[:m], kernel=kernel)
+    want_d, want_p = dist.copy(order="F"), parent.copy(order="F")
+    oracle.fwgemm(A[:m], B[:k], want_d[:m], want_p[:m])
+    got_d, got_p = dD.cpu().numpy(), dP.cpu().numpy()
+    what = f"{np.dtype(dtype).name} {m}x{n}x{k} {kernel} ties={ties} pad={pad}"
+    assert_same_bits(got_d, want_d, "dist " + what)          # rows beyond m (the padding) untouched as well
+    bad = np.argwhere(got_p != want_p)
+    assert len(bad) == 0, f"parent {what}: {len(bad)} differ, first {bad[0]}: {got_p[tuple(bad[0])]} != {want_p[tuple(bad[0])]}"
+    return want_p[:m]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kernel", ["naive", "valu"])
+@pytest.mark.parametrize("ties", [True, False])
+def test_whole_tiles(oracle, dtype, kernel, ties):
+    for m, n, k in [(128, 128, 64), (256, 384, 160), (128, 256, 16)]:
+        p = run_case(oracle, m, n, k, dtype, ties, kernel)
+        assert (p == -7).any() and (p >= 0).any()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kernel", ["naive", "valu", "auto"])
+def test_ragged_extents_and_leading_dimensions(oracle, dtype, kernel):
+    for m, n, k in [(1, 1, 1), (5, 7, 3), (129, 127, 17), (200, 130, 95), (63, 300, 33), (257, 65, 1)]:
+        run_case(oracle, m, n, k, dtype, True, kernel)
+        run_case(oracle, m, n, k, dtype, False, kernel, pad=(3, 1, 2, 5))
+    # whole tiles, but leading dimensions that break the vector alignment
+    run_case(oracle, 128, 128, 32, dtype, True, kernel, pad=(1, 2, 0, 0))
+    run_case(oracle, 128, 128, 32, dtype, True, kernel, pad=(4, 4, 8, 12))
+
+
+def test_first_of_many_equal_products(oracle):
+    """Every product equal: the first k wins where it improves, nothing moves where it does not."""
+    m = n = 128
+    k = 96
+    A = np.ones((m, k), np.float32, order="F")
+    B = np.ones((k, n), np.float32, order="F")
+    dist = np.asfortranarray(np.where(np.add.outer(np.arange(m), np.arange(n)) % 2 == 0, 5.0, 2.0).astype(np.float32))
+    parent = np.full((m, n), -1, np.int32, order="F")
+    dA, dB, dD, dP = (to_device(x) for x in (A, B, dist, parent))
+    cuasr_amd.fwgemm(dA, dB, dD, dP, kernel="valu")
+    got_d, got_p = dD.cpu().numpy(), dP.cpu().numpy()
+    assert np.array_equal(got_d, np.full((m, n), 2.0, np.float32))
+    assert np.array_equal(got_p, np.where(dist == 5.0, 0, -1))
+    # the minimum sits in a later chunk for some elements and is met again afterwards
+    A[:, :40] = 3.0
+    A[::2, 70] = 0.5
+    dA, dD, dP = to_device(A), to_device(dist), to_device(parent)
+    cuasr_amd.fwgemm(dA, dB, dD, dP, kernel="valu")
+    want_d, want_p = dist.copy(order="F"), parent.copy(order="F")
+    oracle.fwgemm(A, B, want_d, want_p)
+    assert_same_bits(dD.cpu().numpy(), want_d, "dist")
+    assert np.array_equal(dP.cpu().numpy(), want_p)
+    assert set(np.unique(want_p)) == {-1, 40, 70}
+
+
+def test_signed_zero_products(oracle):
+    """A product that is -0 does not beat a +0 found earlier (and the other way round); the stored
+    distance is the first of them, as in the sequential scan."""
+    m, n, k = 128, 128, 32
+    rng = np.random.default_rng(5)
+    A = np.asfortranarray(rng.choice(np.array([0.0, -0.0, 1.0], np.float32), (m, k)))
+    B = np.asfortranarray(rng.choice(np.array([0.0, -0.0, 2.0], np.float32), (k, n)))
+    dist = np.full((m, n), 1.0, np.float32, order="F")
+    parent = np.full((m, n), -1, np.int32, order="F")
+    for kernel in ("naive", "valu"):
+        dA, dB, dD, dP = (to_device(x) for x in (A, B, dist, parent))
+        cuasr_amd.fwgemm(dA, dB, dD, dP, kernel=kernel)
+        want_d, want_p = dist.copy(order="F"), parent.copy(order="F")
+        oracle.fwgemm(A, B, want_d, want_p)
+        assert_same_bits(dD.cpu().numpy(), want_d, "dist " + kernel)
+        assert np.array_equal(dP.cpu().numpy(), want_p)
+    assert np.signbit(want_d).any() and (~np.signbit(want_d)).any()
+
+
+def test_large_square_step_properties():
+    """4096^3 (the size of the headline workload): too large for the CPU scan, so check what the
+    definition fixes -- dist equals the min-plus SRGEMM bit for bit, improved elements carry a parent
+    whose product is the new distance and no earlier k gives it, others keep distance and parent."""
+    import torch
+    n = 4096
+    D = inputs.graph_distances(3, n)
+    dA = to_device(D)
+    dD, dP = dA.clone(), torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    cuasr_amd.fwgemm(dA, dA, dD, dP)
+    ref = torch.empty_like(dA)
+    cuasr_amd.srgemm("minimum", "plus", dA, dA, dA, ref, alpha=0.0, beta=0.0, add_identity=float("inf"))
+    assert torch.equal(dD, ref)
+    improved = dD < dA
+    assert torch.equal(dP >= 0, improved)
+    rows, cols = torch.nonzero(improved, as_tuple=True)
+    pick = torch.randperm(rows.numel(), device="cuda")[:20000]
+    r, c = rows[pick], cols[pick]
+    p = dP[r, c].long()
+    assert torch.equal(dA[r, p] + dA[p, c], dD[r, c])
+    # no smaller k reaches the same value: compare with the first-occurrence argmin over all k
+    first = torch.stack([(dA[ri, :] + dA[:, ci]).eq(dD[ri, ci]).nonzero()[0, 0] for ri, ci in zip(r[:200], c[:200])])
+    assert torch.equal(first, p[:200])
+
+
+def test_apsp_squaring_rebuilds_shortest_paths(oracle):
+    import torch
+    from scipy.sparse.csgraph import floyd_warshall as scipy_fw
+    rng = np.random.default_rng(21)
+    n = 300
+    W = np.where(rng.random((n, n)) < 0.03, rng.integers(1, 50, (n, n)), np.inf).astype(np.float32)
+    np.fill_diagonal(W, 0)
+    dD = to_device(np.asfortranarray(W))
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_squaring(dD, dP, ws)
+    dist, parent = dD.cpu().numpy(), dP.cpu().numpy()
+    assert np.array_equal(dist.astype(np.float64), scipy_fw(W.astype(np.float64)))
+    # the same iterations on the CPU give the same parents
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    for _ in range(9):                                    # ceil(log2(299))
+        snap = want_d.copy(order="F")
+        oracle.fwgemm(snap, snap, want_d, want_p)
+    assert_same_bits(dist, want_d, "dist")
+    assert np.array_equal(parent, want_p)
+
+    def expand(i, j):
+        k = parent[i, j]
+        return [] if k < 0 else expand(i, k) + [int(k)] + expand(k, j)
+    rng2 = np.random.default_rng(1)
+    for i, j in rng2.integers(0, n, (300, 2)):
+        if i == j or np.isinf(dist[i, j]):
+            assert parent[i, j] == -1
+            continue
+        hops = [i] + expand(i, j) + [j]
+        assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]

@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 from cuasr_amd import inputs
+from helpers import assert_same_bits
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -288,3 +289,87 @@ def test_serial_splitk_model_invariants(oracle):
     for slices in (2, 7):
         got = oracle.srgemm_splitk_serial("plus", "multiplies", Ai, Bi, Ci, 2.0, -3.0, 0.0, 1.0, slices)
         assert bits(got) == bits(want)
+
+
+# ---- min-plus product with predecessor tracking (test/regress/include/fwgpu/cpu_srgemm.hpp:20-48) ----
+
+def fw_inputs(seed, m, n, k, dtype, ties=True):
+    """Small-integer weights (many equal products), some +inf, leading dimensions larger than the extents."""
+    rng = np.random.default_rng(seed)
+    def mat(r, c, lo, hi, pad):
+        buf = np.full((r + pad, c), np.nan, dtype=dtype, order="F")
+        v = rng.integers(lo, hi, (r, c)).astype(dtype) if ties else rng.random((r, c)).astype(dtype) * 10
+        v[rng.random((r, c)) < 0.2] = np.inf
+        buf[:r] = v
+        return buf[:r]
+    A, B = mat(m, k, 0, 6, 3), mat(k, n, 0, 6, 1)
+    dist = mat(m, n, 2, 9, 2)
+    parent = np.full((m + 5, n), -7, dtype=np.int32, order="F")[:m]
+    return A, B, dist, parent
+
+
+def fw_expected(A, B, dist, parent):
+    """Independent statement: the smallest product, where it first occurs (numpy's argmin returns the
+    first occurrence), taken only when strictly smaller than the old distance."""
+    prods = A[:, :, None] + B[None, :, :]              # m x k x n
+    best = prods.min(axis=1) if A.shape[1] else np.full(dist.shape, np.inf, dist.dtype)
+    where = prods.argmin(axis=1) if A.shape[1] else np.zeros(dist.shape, np.int64)
+    better = best < dist
+    return np.where(better, best, dist), np.where(better, where, parent).astype(np.int32)
+
+
+def test_fwgemm_hand_worked_graph(oracle):
+    inf = np.inf
+    D = np.asfortranarray(np.array([[0, 1, inf], [inf, 0, 2], [1, inf, 0]], dtype=np.float32))
+    dist, parent = D.copy(order="F"), np.full((3, 3), -1, np.int32, order="F")
+    oracle.fwgemm(D, D, dist, parent)
+    # 0 -> 2 through 1 (1 + 2), 1 -> 0 through 2 (2 + 1), 2 -> 1 through 0 (1 + 1)
+    assert dist.tolist() == [[0, 1, 3], [3, 0, 2], [1, 2, 0]]
+    assert parent.tolist() == [[-1, -1, 1], [2, -1, -1], [-1, 0, -1]]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (5, 7, 3), (33, 20, 41), (64, 64, 64), (3, 2, 0)])
+def test_fwgemm_first_strict_minimum(oracle, dtype, shape):
+    for ties in (True, False):
+        A, B, dist, parent = fw_inputs(shape[0] * 7 + shape[2], *shape, dtype, ties)
+        want_d, want_p = fw_expected(A, B, dist, parent)
+        got_d, got_p = dist.copy(order="F"), parent.copy(order="F")
+        oracle.fwgemm(A, B, got_d, got_p)
+        assert_same_bits(got_d, want_d.astype(dtype), "dist")
+        assert np.array_equal(got_p, want_p)
+        # dist is the min-plus SRGEMM with the old distances as C
+        if shape[2] > 0:
+            srgemm = oracle.srgemm("minimum", "plus", A, B, dist, 0.0, 0.0, np.inf)
+            assert_same_bits(got_d, srgemm, "dist vs srgemm")
+        if ties and min(shape) > 4:
+            assert (want_p == -7).any() and (want_p >= 0).any()   # both branches were taken
+
+
+def expand_path(parent, i, j):
+    """Vertices strictly between i and j on the path the parent matrix encodes."""
+    k = parent[i, j]
+    if k < 0:
+        return []
+    return expand_path(parent, i, k) + [int(k)] + expand_path(parent, k, j)
+
+
+def test_fwgemm_squaring_gives_shortest_paths(oracle):
+    from scipy.sparse.csgraph import floyd_warshall as scipy_fw
+    rng = np.random.default_rng(11)
+    n = 48
+    W = np.where(rng.random((n, n)) < 0.15, rng.integers(1, 20, (n, n)), np.inf).astype(np.float32)
+    np.fill_diagonal(W, 0)
+    dist, parent = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    for _ in range(6):                                      # 2^6 >= n - 1 edges
+        snap = dist.copy(order="F")
+        oracle.fwgemm(snap, snap, dist, parent)
+    assert np.array_equal(dist.astype(np.float64), scipy_fw(W.astype(np.float64)))
+    for i in range(n):
+        for j in range(n):
+            if i == j or np.isinf(dist[i, j]):
+                assert parent[i, j] == -1
+                continue
+            hops = [i] + expand_path(parent, i, j) + [j]
+            assert all(np.isfinite(W[a, b]) for a, b in zip(hops, hops[1:]))    # every hop is an edge
+            assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]   # and the path has that length
