@@ -167,6 +167,35 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
                     workload=f"plus-times SRGEMM fp64 on the matrix cores, M=N=K={n}, column-major, N(0,1), C = 0",
                     bound="mfma", peak=FP64_VECTOR_PEAK, instr_per_term=None)
 
+    if w == "fwgemm":
+        # one step of all-pairs shortest paths WITH predecessor tracking: the library snapshots dist (and
+        # its transpose) into the workspace and runs the min-plus product that records the first k of
+        # every improvement
+        n = args.size or 4096
+        D0 = inputs.graph_distances(2024, n, density=0.10, lo=1.0, hi=100.0)
+        d0 = col_major(D0)
+        dist = torch.empty(n, n, device=dev).t()
+        parent = torch.empty(n, n, dtype=torch.int32, device=dev).t()
+        ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32") // 4, dtype=torch.float32, device=dev)
+        squarings = max(1, int(np.ceil(np.log2(max(2, n - 1)))))
+
+        def restart():
+            dist.copy_(d0)
+            parent.fill_(-1)
+
+        def step(i):
+            if i % squarings == 0:   # a new job every `squarings` steps, so every job's first (improving) steps are timed
+                restart()
+            cuasr_amd.apsp_squaring(dist, parent, ws, iterations=1)
+
+        return dict(step=step, reset=restart, m=n, n=n, k=n, dtype="f32", desc=None, host=(D0,), family="fwgemm_tile",
+                    fw=dict(dist=dist, parent=parent, ws=ws, squarings=squarings),
+                    metric=f"fp32 min-plus product with predecessor tracking GOPS at {n}^3 (2 ops/term)",
+                    workload=f"APSP repeated-squaring step with predecessor tracking (cpu_fwgemm_naive semantics), fp32, "
+                             f"M=N=K={n}, column-major, 10% edges U[1,100), rest +inf; a step = snapshot of dist and its "
+                             f"transpose into the workspace + product; a new job (dist, parent reset) every {squarings} steps",
+                    bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5)
+
     if w == "srgemm":
         # any operator pair / element type / layout combination at one size: the reference's
         # benchmark matrix (bench/device/harness.h:157-181 counts 2 * N^3 / t the same way)
@@ -210,7 +239,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="apsp",
                     choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64",
-                             "srgemm"])
+                             "srgemm", "fwgemm"])
     ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
     ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32"], help="workload srgemm")
@@ -268,7 +297,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
 
-    family = args.kernel
+    family = wl.get("family", args.kernel)
     if args.kernel == "auto" and wl["desc"] is not None:
         family = (cuasr_amd.load().cuasr_amd_selected_kernel(wl["desc"]) or b"?").decode()
 
@@ -323,6 +352,24 @@ def main():
                 "sample": f"{squarings} repeated squarings of the same {n}x{n} input (M=N=K={n} each), "
                           f"{cpu_s:.2f} s wall on {threads} OpenMP threads",
                 "gpu_final_matrix_bit_exact_vs_oracle": exact,
+            }
+        elif args.workload == "fwgemm":
+            D0, fw = wl["host"][0], wl["fw"]
+            rows = int(min(n, max(32, 0.5e11 / (2.0 * n * k))))  # the literal scan runs at a few GOPS
+            hd, hp = np.asfortranarray(D0[:rows]), np.full((rows, n), -1, dtype=np.int32, order="F")
+            t1 = time.perf_counter()
+            oracle.fwgemm(np.asfortranarray(D0[:rows]), D0, hd, hp)
+            cpu_s = time.perf_counter() - t1
+            wl["reset"]()
+            step(1)  # one squaring from the initial graph (index 1: no restart)
+            torch.cuda.synchronize()
+            gd, gp = fw["dist"].cpu().numpy()[:rows], fw["parent"].cpu().numpy()[:rows]
+            exact = bool(np.ascontiguousarray(gd).tobytes() == np.ascontiguousarray(hd).tobytes() and (gp == hp).all())
+            out["cpu_baseline"] = {
+                "value": round(2.0 * rows * n * k / cpu_s / 1e9, 2), "unit": "GOPS", "cores": threads, "kind": "port",
+                "sample": f"the first {rows} rows of the first squaring ({rows} x {n} x {k}), {cpu_s:.2f} s wall on "
+                          f"{threads} OpenMP threads",
+                "gpu_rows_bit_exact_vs_oracle": exact,
             }
         else:
             add, mult, A, B, C, alpha, beta, ident = wl["host"]

@@ -31,6 +31,10 @@ struct FwArgs {
   const void *B; int64_t ldb;
   void *dist; int64_t ldc;
   int32_t *parent; int64_t ldp;
+  // optional second image of A with k contiguous (At[row * ldat + k] = A[row, k]); the tile
+  // kernel's lookup of the first minimising k then reads one run of memory per element
+  // instead of one element from each of BK columns
+  const void *At; int64_t ldat;
 };
 
 // cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
@@ -72,7 +76,7 @@ template <> struct vec4_of<double> { typedef double type __attribute__((ext_vect
 // GUARD = false: whole tiles, 16-byte aligned columns of A and B (vector loads).
 // GUARD = true : any extents and alignment; out-of-range operands read as
 //                +infinity, whose products never improve anything.
-template <typename T, int TM, int TN, int SN, int BK, bool GUARD>
+template <typename T, int TM, int TN, int SN, int BK, bool GUARD, bool HAS_AT>
 __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   typedef typename vec4_of<T>::type V4;
   constexpr int BM = 16 * TM, BN = 16 * TN, PAD = 4;
@@ -217,6 +221,66 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   // would push the accumulators out of the register file
   int tx2 = tx, ty2 = ty;
   asm volatile("" : "+v"(tx2), "+v"(ty2));
+  if constexpr (!GUARD) {
+    // Whole, aligned tiles.  Every lane looks at a chunk of its own, so each load of a
+    // column-major A touches 64 cache lines per wave: with most elements improved (the
+    // first squarings of a sparse graph) those BK scattered loads per element cost as much
+    // as the product itself.  With the k-contiguous image of A an element's operands are
+    // two runs of BK values.  Two elements at a time have all of their operands requested
+    // before any is used.  An element that did not improve reads chunk 0 (valid memory)
+    // and stores nothing; a pair with no improved lane in the whole wave is skipped.
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int c = n0 + (j >> 2) * 64 + ty2 * 4 + (j & 3);
+#pragma unroll
+      for (int i = 0; i < TM; i += 2) {
+        const int r = m0 + (i >> 2) * 64 + tx2 * 4 + (i & 3);  // and r + 1
+        const int ch[2] = {chunk[i][j], chunk[i + 1][j]};
+        if (__builtin_amdgcn_ballot_w64(ch[0] >= 0 || ch[1] >= 0) == 0) continue;
+        T pa[2][BK];
+        V4 pb[2][BK / 4];
+        const T *At = static_cast<const T *>(g.At);
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int k0 = (ch[e] < 0 ? 0 : ch[e]) * BK;
+          const T *ap = A + (r + e) + int64_t(k0) * g.lda;
+          const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(c) * g.ldb);
+          if constexpr (HAS_AT) {
+            const V4 *atp = reinterpret_cast<const V4 *>(At + k0 + int64_t(r + e) * g.ldat);
+#pragma unroll
+            for (int q = 0; q < BK / 4; ++q) {
+              const V4 v = atp[q];
+#pragma unroll
+              for (int x = 0; x < 4; ++x) pa[e][q * 4 + x] = v[x];
+            }
+          } else {
+#pragma unroll
+            for (int kk = 0; kk < BK; ++kk) pa[e][kk] = ap[int64_t(kk) * g.lda];
+          }
+#pragma unroll
+          for (int q = 0; q < BK / 4; ++q) pb[e][q] = bp[q];
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const T want = acc[i + e][j];
+          T value = want;
+          int first = 0;
+#pragma unroll
+          for (int kk = BK - 1; kk >= 0; --kk) {
+            const T prod = pa[e][kk] + pb[e][kk >> 2][kk & 3];
+            const bool hit = prod == want;
+            first = hit ? kk : first;
+            value = pick(hit, prod, value);
+          }
+          if (ch[e] >= 0) {
+            dist[(r + e) + int64_t(c) * g.ldc] = value;
+            g.parent[(r + e) + int64_t(c) * g.ldp] = ch[e] * BK + first;
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int c = n0 + (j >> 2) * 64 + ty2 * 4 + (j & 3);
@@ -229,7 +293,8 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
         if (r >= g.m || c >= g.n) continue;
       }
       const int k0 = ch * BK;
-      const T *ap = A + r + int64_t(k0) * g.lda;
+      const T *ap = HAS_AT ? static_cast<const T *>(g.At) + k0 + int64_t(r) * g.ldat : A + r + int64_t(k0) * g.lda;
+      const int64_t a_step = HAS_AT ? 1 : g.lda;
       const T *bp = B + k0 + int64_t(c) * g.ldb;
       const T want = acc[i][j];
       T value = want;
@@ -238,7 +303,7 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
       for (int kk = BK - 1; kk >= 0; --kk) {
         bool in = true;
         if constexpr (GUARD) in = k0 + kk < g.k;
-        const T prod = in ? ap[int64_t(kk) * g.lda] + bp[kk] : inf;
+        const T prod = in ? ap[int64_t(kk) * a_step] + bp[kk] : inf;
         const bool hit = in && prod == want;
         first = hit ? kk : first;
         value = pick(hit, prod, value);
@@ -257,11 +322,40 @@ hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   const bool aligned = reinterpret_cast<uintptr_t>(g.A) % vec == 0 && reinterpret_cast<uintptr_t>(g.B) % vec == 0 &&
                        g.lda % 4 == 0 && g.ldb % 4 == 0;
   dim3 grid((g.m + BM - 1) / BM, (g.n + BN - 1) / BN);
-  if (whole && aligned)
-    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false>), grid, dim3(256), 0, stream, g);
-  else
-    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true>), grid, dim3(256), 0, stream, g);
+  if (g.At) {
+    const bool at_aligned = reinterpret_cast<uintptr_t>(g.At) % vec == 0 && g.ldat % 4 == 0;
+    if (whole && aligned && at_aligned)
+      hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, true>), grid, dim3(256), 0, stream, g);
+    else
+      hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, true>), grid, dim3(256), 0, stream, g);
+  } else if (whole && aligned) {
+    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, false>), grid, dim3(256), 0, stream, g);
+  } else {
+    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, false>), grid, dim3(256), 0, stream, g);
+  }
   return hipGetLastError();
+}
+
+// dist (leading dimension ld) -> w, a packed column-major copy, and wt, its transpose
+// (wt[k + row * n] = dist[row, k]), in one pass over 64 x 64 blocks
+template <typename T>
+__global__ void __launch_bounds__(256) snapshot_kernel(const T *src, int64_t ld, T *w, T *wt, int n) {
+  __shared__ T tile[64][65];
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int j = ty; j < 64; j += 4) {
+    const int r = r0 + tx, c = c0 + j;
+    if (r < n && c < n) {
+      const T v = src[r + int64_t(c) * ld];
+      w[r + int64_t(c) * n] = v;
+      tile[j][tx] = v;
+    }
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int r = r0 + i, c = c0 + tx;
+    if (r < n && c < n) wt[c + int64_t(r) * n] = tile[tx][i];
+  }
 }
 
 template <typename T> hipError_t launch_naive(const FwArgs &g, hipStream_t stream) {
@@ -292,11 +386,12 @@ int check(int dtype, int m, int n, int k, const void *A, int64_t lda, const void
 
 using namespace cuasr_amd;
 
-extern "C" int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb,
-                                void *dist, int64_t ldc, int32_t *parent, int64_t ldp, int kernel, void *stream) {
+namespace {
+int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, void *dist,
+               int64_t ldc, int32_t *parent, int64_t ldp, const void *At, int64_t ldat, int kernel, void *stream) {
   const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
   if (st != CUASR_AMD_SUCCESS || m == 0 || n == 0 || k == 0) return st;
-  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp};
+  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, At, ldat};
   hipStream_t s = static_cast<hipStream_t>(stream);
   // a launch of a few workgroups is better spread over one thread per element
   const bool tiny = int64_t(m) * n < 64 * 64;
@@ -306,10 +401,16 @@ extern "C" int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, i
   else e = naive ? launch_naive<double>(g, s) : launch_tile<double, 4, 8, 4, 16>(g, s);
   return e == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
+}  // namespace
+
+extern "C" int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb,
+                                void *dist, int64_t ldc, int32_t *parent, int64_t ldp, int kernel, void *stream) {
+  return fwgemm_run(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, nullptr, 0, kernel, stream);
+}
 
 extern "C" size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n) {
   if (n <= 0 || (dtype != CUASR_AMD_F32 && dtype != CUASR_AMD_F64)) return 0;
-  return size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * size_t(n) * size_t(n);
+  return 2 * size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * size_t(n) * size_t(n);  // the snapshot and its transpose
 }
 
 extern "C" int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
@@ -324,13 +425,20 @@ extern "C" int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld,
     for (int64_t reach = 1; reach < n - 1; reach *= 2) ++iterations;
   const size_t es = dtype == CUASR_AMD_F64 ? 8 : 4;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  void *transposed = static_cast<char *>(workspace) + es * size_t(n) * size_t(n);
   for (int it = 0; it < iterations; ++it) {
-    // the product reads a snapshot, so no workgroup sees another's updates
-    if (hipMemcpy2DAsync(workspace, size_t(n) * es, dist, size_t(ld) * es, size_t(n) * es, size_t(n),
-                         hipMemcpyDeviceToDevice, s) != hipSuccess)
-      return CUASR_AMD_ERROR_INTERNAL;
-    const int r = cuasr_amd_fwgemm(dtype, n, n, n, workspace, n, workspace, n, dist, ld, parent, ldp,
-                                   CUASR_AMD_KERNEL_AUTO, stream);
+    // the product reads a snapshot, so no workgroup sees another's updates; the snapshot's
+    // transpose serves the lookup of the first minimising k
+    const dim3 grid((n + 63) / 64, (n + 63) / 64);
+    if (dtype == CUASR_AMD_F64)
+      hipLaunchKernelGGL(snapshot_kernel<double>, grid, dim3(256), 0, s, static_cast<const double *>(dist), ld,
+                         static_cast<double *>(workspace), static_cast<double *>(transposed), n);
+    else
+      hipLaunchKernelGGL(snapshot_kernel<float>, grid, dim3(256), 0, s, static_cast<const float *>(dist), ld,
+                         static_cast<float *>(workspace), static_cast<float *>(transposed), n);
+    if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    const int r = fwgemm_run(dtype, n, n, n, workspace, n, workspace, n, dist, ld, parent, ldp, transposed, n,
+                             CUASR_AMD_KERNEL_AUTO, stream);
     if (r != CUASR_AMD_SUCCESS) return r;
   }
   return CUASR_AMD_SUCCESS;

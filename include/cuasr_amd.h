@@ -206,8 +206,9 @@ int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda,
  * covers every path.  parent[i,j] = k says the shortest i -> j path found is the
  * i -> k path followed by the k -> j path; an entry the caller initialised (say
  * to -1) and that never changed means the direct edge.  The workspace holds
- * cuasr_amd_apsp_workspace_bytes(dtype, n) = sizeof(element) * n * n bytes;
- * CUASR_AMD_ERROR_WORKSPACE_NULL without it.  Asynchronous on the stream, no
+ * cuasr_amd_apsp_workspace_bytes(dtype, n) = 2 * sizeof(element) * n * n bytes
+ * (the snapshot and its transpose, in which the search for the first minimising
+ * k reads contiguous memory); CUASR_AMD_ERROR_WORKSPACE_NULL without it.  Asynchronous on the stream, no
  * allocation, no host synchronisation. */
 size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n);
 int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *parent,

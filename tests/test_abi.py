@@ -126,8 +126,8 @@ def test_fwgemm_host_errors(lib):
     assert call(a=0x1002) == 1 and call(dtype=1, d=0x1004) == 1 and call(p=0x1001) == 1
     assert call(kern=3) == 5                  # no matrix-core form
     assert call(m=0) == 0 and call(n=0, d=0) == 0 and call(k=0, a=0, b=0) == 0   # nothing to do, nothing launched
-    assert cuasr_amd.apsp_workspace_bytes(1000, "f32") == 4 * 1000 * 1000
-    assert cuasr_amd.apsp_workspace_bytes(10, "f64") == 800 and cuasr_amd.apsp_workspace_bytes(0, "f32") == 0
+    assert cuasr_amd.apsp_workspace_bytes(1000, "f32") == 2 * 4 * 1000 * 1000   # the snapshot and its transpose
+    assert cuasr_amd.apsp_workspace_bytes(10, "f64") == 1600 and cuasr_amd.apsp_workspace_bytes(0, "f32") == 0
     sq = lambda n=64, ws=0x1000, it=0, dtype=0: lib.cuasr_amd_apsp_squaring(dtype, n, P(0x1000), max(n, 1), P(0x1000), max(n, 1), P(ws), it, None)
     assert sq(ws=0) == 6 and sq(it=-1) == 4 and sq(dtype=3) == 2 and sq(n=0) == 0
 

@@ -130,22 +130,23 @@ def test_large_square_step_properties():
     assert torch.equal(first, p[:200])
 
 
-def test_apsp_squaring_rebuilds_shortest_paths(oracle):
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [300, 256])   # ragged tiles; whole, aligned tiles (the vector lookup in the transposed snapshot)
+def test_apsp_squaring_rebuilds_shortest_paths(oracle, n, dtype):
     import torch
     from scipy.sparse.csgraph import floyd_warshall as scipy_fw
-    rng = np.random.default_rng(21)
-    n = 300
-    W = np.where(rng.random((n, n)) < 0.03, rng.integers(1, 50, (n, n)), np.inf).astype(np.float32)
+    rng = np.random.default_rng(21 + n)
+    W = np.where(rng.random((n, n)) < 0.03, rng.integers(1, 50, (n, n)), np.inf).astype(dtype)
     np.fill_diagonal(W, 0)
     dD = to_device(np.asfortranarray(W))
     dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
-    ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32" if dtype == np.float32 else "f64"), dtype=torch.uint8, device="cuda")
     cuasr_amd.apsp_squaring(dD, dP, ws)
     dist, parent = dD.cpu().numpy(), dP.cpu().numpy()
     assert np.array_equal(dist.astype(np.float64), scipy_fw(W.astype(np.float64)))
     # the same iterations on the CPU give the same parents
     want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
-    for _ in range(9):                                    # ceil(log2(299))
+    for _ in range(int(np.ceil(np.log2(n - 1)))):
         snap = want_d.copy(order="F")
         oracle.fwgemm(snap, snap, want_d, want_p)
     assert_same_bits(dist, want_d, "dist")
