@@ -92,6 +92,11 @@ def load():
         lib.cuasr_amd_fwgemm.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_int64] * 4 + [ctypes.c_int, ctypes.c_void_p]
         lib.cuasr_amd_apsp_workspace_bytes.restype = ctypes.c_size_t
         lib.cuasr_amd_apsp_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.cuasr_amd_apsp_blocked_workspace_bytes.restype = ctypes.c_size_t
+        lib.cuasr_amd_apsp_blocked_workspace_bytes.argtypes = [ctypes.c_int, ctypes.c_int]
+        lib.cuasr_amd_apsp_blocked.restype = ctypes.c_int
+        lib.cuasr_amd_apsp_blocked.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                               ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
         lib.cuasr_amd_apsp_squaring.restype = ctypes.c_int
         lib.cuasr_amd_apsp_squaring.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
                                                 ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
@@ -335,4 +340,23 @@ def apsp_squaring(dist, parent, workspace, iterations=0, stream=None):
                                         _stream_handle(stream))
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_apsp_squaring")
+    return dist, parent
+
+
+def apsp_blocked_workspace_bytes(n, dtype):
+    return int(load().cuasr_amd_apsp_blocked_workspace_bytes(DTYPES[dtype], n))
+
+
+def apsp_blocked(dist, parent, workspace, stream=None):
+    """All-pairs shortest paths by blocked Floyd-Warshall with predecessor
+    tracking, in place on the n x n column-major ``dist`` and int32 ``parent``;
+    ``workspace`` is a device tensor of at least
+    apsp_blocked_workspace_bytes(n, dtype) bytes."""
+    n = dist.shape[0]
+    pd, ld = _column_major(dist, "dist")
+    pp, ldp = _column_major(parent, "parent")
+    ws = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
+    st = load().cuasr_amd_apsp_blocked(DTYPES[_torch_dtype_name(dist)], n, pd, ld, pp, ldp, ws, _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_apsp_blocked")
     return dist, parent

@@ -35,6 +35,8 @@ struct FwArgs {
   // kernel's lookup of the first minimising k then reads one run of memory per element
   // instead of one element from each of BK columns
   const void *At; int64_t ldat;
+  int k_base;                               // recorded parents are k_base + k
+  int skip_r0, skip_r1, skip_c0, skip_c1;   // outputs in these rows or these columns are left alone
 };
 
 // cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
@@ -51,6 +53,7 @@ __global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
   const int row = blockIdx.x * 64 + (threadIdx.x & 63);
   const int col = blockIdx.y * 4 + (threadIdx.x >> 6);
   if (row >= g.m || col >= g.n) return;
+  if ((row >= g.skip_r0 && row < g.skip_r1) || (col >= g.skip_c0 && col < g.skip_c1)) return;
   const T *a = static_cast<const T *>(g.A) + row;
   const T *b = static_cast<const T *>(g.B) + col * g.ldb;
   T *d = static_cast<T *>(g.dist) + row + col * g.ldc;
@@ -61,7 +64,7 @@ __global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
     const T prod = a[i * g.lda] + b[i];
     const bool lower = prod < curr;
     curr = pick(lower, prod, curr);
-    p = lower ? i : p;
+    p = lower ? g.k_base + i : p;
   }
   *d = curr;
   *pp = p;
@@ -90,6 +93,8 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   const int tid = threadIdx.x & 255;
   const int tx = tid & 15, ty = tid >> 4;
   const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  // (the host only passes ranges whose ends fall on tile boundaries or beyond the matrix)
+  if ((m0 < g.skip_r1 && m0 + BM > g.skip_r0) || (n0 < g.skip_c1 && n0 + BN > g.skip_c0)) return;
   const T inf = std::numeric_limits<T>::infinity();
 
   auto row_of = [&](int i) { return m0 + (i >> 2) * 64 + tx * 4 + (i & 3); };
@@ -274,7 +279,7 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
           }
           if (ch[e] >= 0) {
             dist[(r + e) + int64_t(c) * g.ldc] = value;
-            g.parent[(r + e) + int64_t(c) * g.ldp] = ch[e] * BK + first;
+            g.parent[(r + e) + int64_t(c) * g.ldp] = g.k_base + ch[e] * BK + first;
           }
         }
       }
@@ -309,7 +314,7 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
         value = pick(hit, prod, value);
       }
       dist[r + int64_t(c) * g.ldc] = value;
-      g.parent[r + int64_t(c) * g.ldp] = k0 + first;
+      g.parent[r + int64_t(c) * g.ldp] = g.k_base + k0 + first;
     }
   }
 }
@@ -336,25 +341,81 @@ hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// dist (leading dimension ld) -> w, a packed column-major copy, and wt, its transpose
-// (wt[k + row * n] = dist[row, k]), in one pass over 64 x 64 blocks
+// src (rows x cols, column-major, leading dimension ld) -> w, a column-major copy with leading
+// dimension ldw, and wt, its transpose (wt[c + r * ldwt] = src[r, c]), in one pass over
+// 64 x 64 blocks; either destination may be null
 template <typename T>
-__global__ void __launch_bounds__(256) snapshot_kernel(const T *src, int64_t ld, T *w, T *wt, int n) {
+__global__ void __launch_bounds__(256) snapshot_kernel(const T *src, int64_t ld, T *w, int64_t ldw, T *wt, int64_t ldwt,
+                                                       int rows, int cols) {
   __shared__ T tile[64][65];
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int j = ty; j < 64; j += 4) {
     const int r = r0 + tx, c = c0 + j;
-    if (r < n && c < n) {
+    if (r < rows && c < cols) {
       const T v = src[r + int64_t(c) * ld];
-      w[r + int64_t(c) * n] = v;
+      if (w) w[r + int64_t(c) * ldw] = v;
       tile[j][tx] = v;
     }
   }
+  if (!wt) return;
   __syncthreads();
   for (int i = ty; i < 64; i += 4) {
     const int r = r0 + i, c = c0 + tx;
-    if (r < n && c < n) wt[c + int64_t(r) * n] = tile[tx][i];
+    if (r < rows && c < cols) wt[c + int64_t(r) * ldwt] = tile[tx][i];
+  }
+}
+
+template <typename T>
+hipError_t snapshot(const void *src, int64_t ld, void *w, int64_t ldw, void *wt, int64_t ldwt, int rows, int cols,
+                    hipStream_t s) {
+  const dim3 grid((rows + 63) / 64, (cols + 63) / 64);
+  hipLaunchKernelGGL(snapshot_kernel<T>, grid, dim3(256), 0, s, static_cast<const T *>(src), ld, static_cast<T *>(w), ldw,
+                     static_cast<T *>(wt), ldwt, rows, cols);
+  return hipGetLastError();
+}
+
+// Floyd-Warshall inside one diagonal block of at most FW_BLOCK x FW_BLOCK, held in LDS: k ascending,
+// d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent = k_base + k.  Row k and column k do not
+// change in step k (the block's diagonal is not negative), so every step reads a settled state.
+constexpr int FW_BLOCK = 128;
+template <typename T>
+__global__ void __launch_bounds__(1024) fw_diagonal_kernel(T *d, int64_t ld, int32_t *parent, int64_t ldp, int bb, int k_base) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char fw_lds[];
+  T *blk = reinterpret_cast<T *>(fw_lds);  // [FW_BLOCK][FW_BLOCK], column-major
+  const int i = threadIdx.x & (FW_BLOCK - 1), j0 = threadIdx.x >> 7;  // 8 columns per pass, 16 passes
+  const T inf = std::numeric_limits<T>::infinity();
+  T cur[FW_BLOCK / 8];
+  int32_t par[FW_BLOCK / 8];
+#pragma unroll
+  for (int q = 0; q < FW_BLOCK / 8; ++q) {
+    const int j = j0 + 8 * q;
+    cur[q] = (i < bb && j < bb) ? d[i + int64_t(j) * ld] : inf;
+    par[q] = -1;
+    blk[i + j * FW_BLOCK] = cur[q];
+  }
+  __syncthreads();
+  for (int k = 0; k < bb; ++k) {
+    const T dik = blk[i + k * FW_BLOCK];
+#pragma unroll
+    for (int q = 0; q < FW_BLOCK / 8; ++q) {
+      const T cand = dik + blk[k + (j0 + 8 * q) * FW_BLOCK];
+      const bool lower = cand < cur[q];
+      cur[q] = pick(lower, cand, cur[q]);
+      par[q] = lower ? k_base + k : par[q];
+    }
+    __syncthreads();  // everybody has read the state of step k
+#pragma unroll
+    for (int q = 0; q < FW_BLOCK / 8; ++q) blk[i + (j0 + 8 * q) * FW_BLOCK] = cur[q];
+    __syncthreads();
+  }
+#pragma unroll
+  for (int q = 0; q < FW_BLOCK / 8; ++q) {
+    const int j = j0 + 8 * q;
+    if (i < bb && j < bb && par[q] >= 0) {
+      d[i + int64_t(j) * ld] = cur[q];
+      parent[i + int64_t(j) * ldp] = par[q];
+    }
   }
 }
 
@@ -387,11 +448,16 @@ int check(int dtype, int m, int n, int k, const void *A, int64_t lda, const void
 using namespace cuasr_amd;
 
 namespace {
+struct FwExtra {
+  const void *At = nullptr; int64_t ldat = 0;
+  int k_base = 0, skip_r0 = 0, skip_r1 = 0, skip_c0 = 0, skip_c1 = 0;
+};
 int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, void *dist,
-               int64_t ldc, int32_t *parent, int64_t ldp, const void *At, int64_t ldat, int kernel, void *stream) {
+               int64_t ldc, int32_t *parent, int64_t ldp, const FwExtra &x, int kernel, void *stream) {
   const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
   if (st != CUASR_AMD_SUCCESS || m == 0 || n == 0 || k == 0) return st;
-  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, At, ldat};
+  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, x.At, x.ldat, x.k_base,
+                 x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1};
   hipStream_t s = static_cast<hipStream_t>(stream);
   // a launch of a few workgroups is better spread over one thread per element
   const bool tiny = int64_t(m) * n < 64 * 64;
@@ -405,7 +471,7 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
 
 extern "C" int cuasr_amd_fwgemm(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb,
                                 void *dist, int64_t ldc, int32_t *parent, int64_t ldp, int kernel, void *stream) {
-  return fwgemm_run(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, nullptr, 0, kernel, stream);
+  return fwgemm_run(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, FwExtra{}, kernel, stream);
 }
 
 extern "C" size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n) {
@@ -429,16 +495,89 @@ extern "C" int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld,
   for (int it = 0; it < iterations; ++it) {
     // the product reads a snapshot, so no workgroup sees another's updates; the snapshot's
     // transpose serves the lookup of the first minimising k
-    const dim3 grid((n + 63) / 64, (n + 63) / 64);
-    if (dtype == CUASR_AMD_F64)
-      hipLaunchKernelGGL(snapshot_kernel<double>, grid, dim3(256), 0, s, static_cast<const double *>(dist), ld,
-                         static_cast<double *>(workspace), static_cast<double *>(transposed), n);
-    else
-      hipLaunchKernelGGL(snapshot_kernel<float>, grid, dim3(256), 0, s, static_cast<const float *>(dist), ld,
-                         static_cast<float *>(workspace), static_cast<float *>(transposed), n);
-    if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
-    const int r = fwgemm_run(dtype, n, n, n, workspace, n, workspace, n, dist, ld, parent, ldp, transposed, n,
+    const hipError_t e = dtype == CUASR_AMD_F64 ? snapshot<double>(dist, ld, workspace, n, transposed, n, n, n, s)
+                                                : snapshot<float>(dist, ld, workspace, n, transposed, n, n, n, s);
+    if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    FwExtra x;
+    x.At = transposed;
+    x.ldat = n;
+    const int r = fwgemm_run(dtype, n, n, n, workspace, n, workspace, n, dist, ld, parent, ldp, x,
                              CUASR_AMD_KERNEL_AUTO, stream);
+    if (r != CUASR_AMD_SUCCESS) return r;
+  }
+  return CUASR_AMD_SUCCESS;
+}
+
+// ---- blocked Floyd-Warshall ------------------------------------------------------------------
+
+extern "C" size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n) {
+  if (n <= 0 || (dtype != CUASR_AMD_F32 && dtype != CUASR_AMD_F64)) return 0;
+  const size_t nn = (size_t(n) + 3) & ~size_t(3);
+  return 3 * size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * FW_BLOCK * nn;  // block row, block column, transposed block column
+}
+
+extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
+                                      void *workspace, void *stream) {
+  const int64_t nn = (int64_t(n) + 3) & ~int64_t(3);
+  const int st = check(dtype, n, n, n, workspace, nn > 0 ? nn : 1, workspace, nn > 0 ? nn : 1, dist, ld, parent, ldp,
+                       CUASR_AMD_KERNEL_AUTO);
+  if (n > 0 && !workspace) return CUASR_AMD_ERROR_WORKSPACE_NULL;
+  if (st != CUASR_AMD_SUCCESS) return st;
+  if (n == 0) return CUASR_AMD_SUCCESS;
+  if (reinterpret_cast<uintptr_t>(workspace) % 16) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+  const bool f64 = dtype == CUASR_AMD_F64;
+  const size_t es = f64 ? 8 : 4;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  char *D = static_cast<char *>(dist);
+  char *R = static_cast<char *>(workspace);             // block row,    FW_BLOCK x n,  leading dimension FW_BLOCK
+  char *C = R + es * FW_BLOCK * size_t(nn);             // block column, n x FW_BLOCK,  leading dimension nn
+  char *Ct = C + es * FW_BLOCK * size_t(nn);            // updated block column with k contiguous, leading dimension FW_BLOCK
+  const size_t lds = es * FW_BLOCK * FW_BLOCK;
+  static bool lds_set = false;  // the fp64 block needs 128 KiB of LDS, above the default limit of a launch
+  if (!lds_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(fw_diagonal_kernel<double>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, int(8 * FW_BLOCK * FW_BLOCK)) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void *>(fw_diagonal_kernel<float>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, int(4 * FW_BLOCK * FW_BLOCK)) != hipSuccess)
+      return CUASR_AMD_ERROR_INTERNAL;
+    lds_set = true;
+  }
+  for (int k0 = 0; k0 < n; k0 += FW_BLOCK) {
+    const int bb = n - k0 < FW_BLOCK ? n - k0 : FW_BLOCK;
+    char *Dkk = D + es * (size_t(k0) + size_t(k0) * size_t(ld));
+    int32_t *Pkk = parent + size_t(k0) + size_t(k0) * size_t(ldp);
+    // 1. the diagonal block, closed in LDS
+    if (f64)
+      hipLaunchKernelGGL(fw_diagonal_kernel<double>, dim3(1), dim3(1024), lds, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
+    else
+      hipLaunchKernelGGL(fw_diagonal_kernel<float>, dim3(1), dim3(1024), lds, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
+    if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    // 2. snapshots of block row and block column (the products below read these, so that no
+    //    workgroup sees another's updates)
+    char *Drow = D + es * size_t(k0), *Dcol = D + es * size_t(k0) * size_t(ld);
+    hipError_t e = f64 ? snapshot<double>(Drow, ld, R, FW_BLOCK, nullptr, 0, bb, n, s)
+                       : snapshot<float>(Drow, ld, R, FW_BLOCK, nullptr, 0, bb, n, s);
+    if (e == hipSuccess)
+      e = f64 ? snapshot<double>(Dcol, ld, C, nn, nullptr, 0, n, bb, s) : snapshot<float>(Dcol, ld, C, nn, nullptr, 0, n, bb, s);
+    if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    // 3. block row <- (closed diagonal block) x (block row); block column <- (block column) x (closed diagonal block)
+    FwExtra x;
+    x.k_base = k0;
+    int r = fwgemm_run(dtype, bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp, x,
+                       CUASR_AMD_KERNEL_AUTO, stream);
+    if (r != CUASR_AMD_SUCCESS) return r;
+    r = fwgemm_run(dtype, n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp, x,
+                   CUASR_AMD_KERNEL_AUTO, stream);
+    if (r != CUASR_AMD_SUCCESS) return r;
+    // 4. everything outside block row and block column <- (block column) x (block row), read in place
+    //    (those panels are not written in this step); the column's k-contiguous image serves the lookups
+    e = f64 ? snapshot<double>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s) : snapshot<float>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s);
+    if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    x.At = Ct;
+    x.ldat = FW_BLOCK;
+    x.skip_r0 = x.skip_c0 = k0;
+    x.skip_r1 = x.skip_c1 = k0 + bb;
+    r = fwgemm_run(dtype, n, n, bb, Dcol, ld, Drow, ld, dist, ld, parent, ldp, x, CUASR_AMD_KERNEL_AUTO, stream);
     if (r != CUASR_AMD_SUCCESS) return r;
   }
   return CUASR_AMD_SUCCESS;

@@ -214,6 +214,29 @@ size_t cuasr_amd_apsp_workspace_bytes(int dtype, int n);
 int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *parent,
                             int64_t ldp, void *workspace, int iterations, void *stream);
 
+/* All-pairs shortest paths by blocked Floyd-Warshall with predecessor tracking:
+ * n^3 products instead of the n^3 * log2(n) of repeated squaring.  The reference
+ * has no such routine; it is built from the reference's block, the product of
+ * cpu_fwgemm_naive (test/regress/include/fwgpu/cpu_srgemm.hpp:20-48), for the
+ * application its README names (README.md:338-342).  For every diagonal block of
+ * 128 vertices: Floyd-Warshall inside the block; block row and block column
+ * through the closed block; every other element through block column x block
+ * row.  dist (n x n, column-major, leading dimension ld) and parent (int32, ldp)
+ * are updated in place: on return dist holds the shortest distances and
+ * parent[i,j] = k says the path found is the i -> k path followed by the k -> j
+ * path (an entry the caller initialised, say to -1, that never changed: the
+ * direct edge).  Weights must be free of NaN and -infinity, +infinity = no
+ * edge, no negative cycles.  Sums along a path are formed in the blocked order,
+ * so on weights whose sums round, distances can differ in the last bits from
+ * those of cuasr_amd_apsp_squaring (both are sums of the same edges).  The
+ * workspace holds cuasr_amd_apsp_blocked_workspace_bytes(dtype, n) bytes
+ * (3 * 128 * n elements, n rounded up to a multiple of 4) and is 16-byte
+ * aligned; CUASR_AMD_ERROR_WORKSPACE_NULL without it.  Asynchronous on the
+ * stream, no allocation, no host synchronisation. */
+size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n);
+int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, int32_t *parent,
+                           int64_t ldp, void *workspace, void *stream);
+
 /* Name of the kernel family AUTO would choose for this descriptor
  * ("naive", "valu", "valu_direct", "mfma"; "valu_direct+valu" when a block of the output runs on
  * the direct-to-LDS tile and the strips around it on the staged one), or NULL if the descriptor

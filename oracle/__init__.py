@@ -178,3 +178,22 @@ def fwgemm(A, B, dist, parent, nthreads=0):
     if rc != 0:
         raise ValueError(f"oracle.fwgemm: unsupported element type {dt}")
     return dist, parent
+
+
+def apsp_blocked(dist, parent, block=128):
+    """Blocked Floyd-Warshall with predecessor tracking, in place on a square
+    column-major ``dist`` (float32/float64) and an int32 ``parent``; the order of
+    operations is the device driver's (see host_blocked_fw.c)."""
+    n = dist.shape[0]
+    if n == 0:
+        return dist, parent
+    refs = [mat_ref(x) for x in (dist, parent)]
+    if any(r[2] != COLUMN_MAJOR for r in refs) or parent.dtype != np.int32 or dist.shape != (n, n) or parent.shape != (n, n):
+        raise ValueError("oracle.apsp_blocked: square column-major dist and an int32 parent matrix")
+    (pd, ld, _), (pp, ldp, _) = refs
+    fn = lib().oracle_apsp_blocked
+    fn.restype = ctypes.c_int
+    rc = fn(DTYPES[dist.dtype], n, pd, ctypes.c_int64(ld), pp, ctypes.c_int64(ldp), int(block))
+    if rc != 0:
+        raise ValueError(f"oracle.apsp_blocked: failed ({rc})")
+    return dist, parent

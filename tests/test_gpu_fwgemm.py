@@ -162,3 +162,83 @@ def test_apsp_squaring_rebuilds_shortest_paths(oracle, n, dtype):
             continue
         hops = [i] + expand(i, j) + [j]
         assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]
+
+
+def _check_paths(W, dist, parent, seed, count=300):
+    n = W.shape[0]
+
+    def expand(i, j):
+        k = parent[i, j]
+        return [] if k < 0 else expand(i, k) + [int(k)] + expand(k, j)
+    rng = np.random.default_rng(seed)
+    for i, j in rng.integers(0, n, (count, 2)):
+        if i == j or np.isinf(dist[i, j]):
+            assert parent[i, j] == -1
+            continue
+        hops = [i] + expand(i, j) + [j]
+        assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,pad", [(1, 0), (100, 0), (128, 0), (300, 3), (384, 0), (513, 1)])
+def test_apsp_blocked_floyd_warshall(oracle, n, pad, dtype):
+    """Blocked Floyd-Warshall: distances equal to scipy's on integer weights (every order of
+    additions is exact), dist and parent bit-identical to the oracle's blocked iteration, and the
+    paths rebuilt from parent sum to the distances."""
+    import torch
+    from scipy.sparse.csgraph import floyd_warshall as scipy_fw
+    rng = np.random.default_rng(77 + n)
+    W = np.where(rng.random((n, n)) < max(0.02, 3.0 / n), rng.integers(1, 60, (n, n)), np.inf).astype(dtype)
+    np.fill_diagonal(W, 0)
+    host = np.full((n + pad, n), 7.0, dtype=dtype, order="F")     # leading dimension n + pad
+    host[:n] = W
+    dD = to_device(host)
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    name = "f32" if dtype == np.float32 else "f64"
+    ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, name), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_blocked(dD[:n], dP, ws)
+    got, parent = dD.cpu().numpy(), dP.cpu().numpy()
+    assert (got[n:] == 7.0).all()                                # the padding rows are untouched
+    dist = got[:n]
+    assert np.array_equal(dist.astype(np.float64), scipy_fw(W.astype(np.float64)))
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(want_d, want_p, 128)
+    assert_same_bits(np.ascontiguousarray(dist), np.ascontiguousarray(want_d), "dist")
+    assert np.array_equal(parent, want_p)
+    _check_paths(W, dist, parent, n)
+
+
+def test_apsp_blocked_on_rounding_weights_matches_the_oracle_bit_for_bit(oracle):
+    """Real-valued weights: sums round, so the result depends on the order of additions; the
+    device and the oracle use the same order.  Against repeated squaring only closeness holds."""
+    import torch
+    n = 640
+    rng = np.random.default_rng(5)
+    W = np.where(rng.random((n, n)) < 0.02, rng.random((n, n)) * 10 + 0.1, np.inf).astype(np.float32)
+    np.fill_diagonal(W, 0)
+    dD = to_device(np.asfortranarray(W))
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_blocked(dD, dP, ws)
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(want_d, want_p, 128)
+    dist, parent = dD.cpu().numpy(), dP.cpu().numpy()
+    assert_same_bits(np.ascontiguousarray(dist), np.ascontiguousarray(want_d), "dist")
+    assert np.array_equal(parent, want_p)
+    sq = to_device(np.asfortranarray(W))
+    sqp = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    ws2 = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_squaring(sq, sqp, ws2)
+    ref = sq.cpu().numpy()
+    finite = np.isfinite(ref)
+    assert np.array_equal(finite, np.isfinite(dist))
+    assert np.allclose(dist[finite], ref[finite], rtol=1e-5, atol=0)
+    # paths rebuilt from parent are real paths of (almost) the recorded length
+    def expand(i, j):
+        k = parent[i, j]
+        return [] if k < 0 else expand(i, k) + [int(k)] + expand(k, j)
+    for i, j in rng.integers(0, n, (200, 2)):
+        if i == j or not finite[i, j]:
+            continue
+        hops = [i] + expand(i, j) + [j]
+        assert abs(sum(float(W[a, b]) for a, b in zip(hops, hops[1:])) - dist[i, j]) <= 1e-4 * dist[i, j]

@@ -373,3 +373,81 @@ def test_fwgemm_squaring_gives_shortest_paths(oracle):
             hops = [i] + expand_path(parent, i, j) + [j]
             assert all(np.isfinite(W[a, b]) for a, b in zip(hops, hops[1:]))    # every hop is an edge
             assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]   # and the path has that length
+
+
+# ---- blocked Floyd-Warshall (oracle/host_blocked_fw.c) -------------------------------------
+
+def literal_floyd_warshall(W):
+    """The textbook triple loop, k outermost, with the intermediate vertex as predecessor."""
+    n = W.shape[0]
+    d, p = W.copy(), np.full((n, n), -1, np.int32)
+    for k in range(n):
+        cand = d[:, k:k + 1] + d[k:k + 1, :]
+        better = cand < d
+        d[better], p[better] = cand[better], k
+    return d, p
+
+
+def test_blocked_fw_hand_worked_graph(oracle):
+    inf = np.inf
+    # 0 -> 1 -> 2 -> 3 is a chain of unit edges, 0 -> 3 costs 10 directly
+    W = np.array([[0, 1, inf, 10], [inf, 0, 1, inf], [inf, inf, 0, 1], [inf, inf, inf, 0]], dtype=np.float32)
+    for block in (1, 2, 3, 4, 128):
+        dist, parent = np.asfortranarray(W), np.full((4, 4), -1, np.int32, order="F")
+        oracle.apsp_blocked(dist, parent, block)
+        assert dist.tolist() == [[0, 1, 2, 3], [inf, 0, 1, 2], [inf, inf, 0, 1], [inf, inf, inf, 0]], block
+        assert [0] + expand_path(parent, 0, 3) + [3] == [0, 1, 2, 3], block
+        assert parent[0, 1] == -1 and parent[3, 0] == -1
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,block", [(1, 4), (7, 3), (31, 8), (50, 16), (96, 32), (130, 128), (150, 64)])
+def test_blocked_fw_on_integer_weights(oracle, n, block, dtype):
+    """Integer weights: every order of additions is exact, so the distances equal scipy's
+    Floyd-Warshall and the textbook loop's; parents need not (ties), but must describe paths
+    of exactly the distance."""
+    from scipy.sparse.csgraph import floyd_warshall as scipy_fw
+    rng = np.random.default_rng(1000 * n + block)
+    W = np.where(rng.random((n, n)) < max(0.05, 2.5 / n), rng.integers(1, 30, (n, n)), np.inf).astype(dtype)
+    np.fill_diagonal(W, 0)
+    dist, parent = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(dist, parent, block)
+    assert np.array_equal(dist.astype(np.float64), scipy_fw(W.astype(np.float64)))
+    assert np.array_equal(dist, literal_floyd_warshall(W)[0])
+    for i in range(n):
+        for j in range(n):
+            if i == j or np.isinf(dist[i, j]):
+                assert parent[i, j] == -1
+                continue
+            hops = [i] + expand_path(parent, i, j) + [j]
+            assert all(np.isfinite(W[a, b]) for a, b in zip(hops, hops[1:]))
+            assert sum(W[a, b] for a, b in zip(hops, hops[1:])) == dist[i, j]
+
+
+def test_blocked_fw_with_one_block_is_the_textbook_loop(oracle):
+    """A block as large as the matrix leaves the in-block loop (the products that follow find
+    nothing to improve on exact sums): distances and parents of the textbook algorithm."""
+    rng = np.random.default_rng(3)
+    n = 40
+    W = np.where(rng.random((n, n)) < 0.2, rng.integers(1, 12, (n, n)), np.inf).astype(np.float32)
+    np.fill_diagonal(W, 0)
+    dist, parent = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(dist, parent, n)
+    want_d, want_p = literal_floyd_warshall(W)
+    assert np.array_equal(dist, want_d) and np.array_equal(parent, want_p)
+
+
+def test_blocked_fw_leading_dimensions(oracle):
+    rng = np.random.default_rng(4)
+    n = 37
+    W = np.where(rng.random((n, n)) < 0.2, rng.integers(1, 9, (n, n)), np.inf).astype(np.float64)
+    np.fill_diagonal(W, 0)
+    big = np.full((n + 5, n), -3.0, order="F")
+    big[:n] = W
+    pbig = np.full((n + 2, n), -9, np.int32, order="F")
+    pbig[:n] = -1
+    oracle.apsp_blocked(big[:n], pbig[:n], 16)
+    dist, parent = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(dist, parent, 16)
+    assert np.array_equal(big[:n], dist) and np.array_equal(pbig[:n], parent)
+    assert (big[n:] == -3.0).all() and (pbig[n:] == -9).all()
