@@ -196,6 +196,30 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
                              f"transpose into the workspace + product; a new job (dist, parent reset) every {squarings} steps",
                     bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5)
 
+    if w == "apsp_blocked":
+        # a whole all-pairs shortest-path job with predecessor tracking by blocked Floyd-Warshall:
+        # one step = reset dist and parent, then the n / 128 block steps (2 * n^3 operations in all)
+        n = args.size or 4096
+        D0 = inputs.graph_distances(2024, n, density=0.10, lo=1.0, hi=100.0)
+        d0 = col_major(D0)
+        dist = torch.empty(n, n, device=dev).t()
+        parent = torch.empty(n, n, dtype=torch.int32, device=dev).t()
+        ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, "f32"), dtype=torch.uint8, device=dev)
+
+        def step(i):
+            dist.copy_(d0)
+            parent.fill_(-1)
+            cuasr_amd.apsp_blocked(dist, parent, ws)
+
+        return dict(step=step, m=n, n=n, k=n, dtype="f32", desc=None, host=(D0,), family="fwgemm_tile + fw_diagonal",
+                    fw=dict(dist=dist, parent=parent),
+                    metric=f"fp32 all-pairs shortest paths with predecessors, blocked Floyd-Warshall, GOPS at n={n} "
+                           "(2 ops/term, 2*n^3 per job)",
+                    workload=f"whole APSP job with predecessor tracking by blocked Floyd-Warshall (128-vertex blocks), fp32, "
+                             f"n={n}, column-major, 10% edges U[1,100), rest +inf; a step = reset of dist and parent + "
+                             f"{(n + 127) // 128} block steps",
+                    bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5)
+
     if w == "srgemm":
         # any operator pair / element type / layout combination at one size: the reference's
         # benchmark matrix (bench/device/harness.h:157-181 counts 2 * N^3 / t the same way)
@@ -239,7 +263,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="apsp",
                     choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64",
-                             "srgemm", "fwgemm"])
+                             "srgemm", "fwgemm", "apsp_blocked"])
     ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
     ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32"], help="workload srgemm")
@@ -352,6 +376,27 @@ def main():
                 "sample": f"{squarings} repeated squarings of the same {n}x{n} input (M=N=K={n} each), "
                           f"{cpu_s:.2f} s wall on {threads} OpenMP threads",
                 "gpu_final_matrix_bit_exact_vs_oracle": exact,
+            }
+        elif args.workload == "apsp_blocked":
+            # the oracle's blocked iteration on a smaller graph of the same kind (the CPU needs
+            # minutes at full size); the GPU runs that graph too and must match it bit for bit
+            nc = min(n, 2048)
+            Dc = inputs.graph_distances(2024, nc, density=0.10, lo=1.0, hi=100.0)
+            hd, hp = Dc.copy(order="F"), np.full((nc, nc), -1, dtype=np.int32, order="F")   # (a copy: the oracle works in place)
+            t1 = time.perf_counter()
+            oracle.apsp_blocked(hd, hp, 128)
+            cpu_s = time.perf_counter() - t1
+            gd = torch.from_numpy(np.ascontiguousarray(Dc.T)).to("cuda:0").t()
+            gp = torch.full((nc, nc), -1, dtype=torch.int32, device="cuda:0").t()
+            gws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(nc, "f32"), dtype=torch.uint8, device="cuda:0")
+            cuasr_amd.apsp_blocked(gd, gp, gws)
+            torch.cuda.synchronize()
+            exact = bool(np.ascontiguousarray(gd.cpu().numpy()).tobytes() == np.ascontiguousarray(hd).tobytes()
+                         and (gp.cpu().numpy() == hp).all())
+            out["cpu_baseline"] = {
+                "value": round(2.0 * nc ** 3 / cpu_s / 1e9, 2), "unit": "GOPS", "cores": threads, "kind": "port",
+                "sample": f"the same job at n={nc} ({cpu_s:.2f} s wall on {threads} OpenMP threads)",
+                "gpu_dist_and_parent_bit_exact_vs_oracle": exact,
             }
         elif args.workload == "fwgemm":
             D0, fw = wl["host"][0], wl["fw"]

@@ -164,6 +164,20 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
       if constexpr (!GUARD) acc[i][j] = static_cast<const T *>(g.dist)[r + int64_t(c) * g.ldc];
       else acc[i][j] = (r < g.m && c < g.n) ? static_cast<const T *>(g.dist)[r + int64_t(c) * g.ldc] : -inf;
     }
+  if constexpr (!GUARD) {
+    // a lane's rows come in runs of four: one 16-byte load per run when dist allows it
+    const size_t vb = 4 * sizeof(T);
+    if (reinterpret_cast<uintptr_t>(g.dist) % vb == 0 && g.ldc % 4 == 0) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; i += 4) {
+          const V4 v = *reinterpret_cast<const V4 *>(static_cast<const T *>(g.dist) + row_of(i) + int64_t(col_of(j)) * g.ldc);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) acc[i + x][j] = v[x];
+        }
+    }
+  }
 
   const int tiles = (g.k + BK - 1) / BK;
   if (tiles > 0) {
@@ -404,9 +418,14 @@ __global__ void __launch_bounds__(1024) fw_diagonal_kernel(T *d, int64_t ld, int
       cur[q] = pick(lower, cand, cur[q]);
       par[q] = lower ? k_base + k : par[q];
     }
-    __syncthreads();  // everybody has read the state of step k
+    // Step k + 1 reads row k + 1 and column k + 1 only, so only those are published.  They
+    // differ from what step k reads (row k, column k) except at the two crossings, which
+    // step k does not change: one barrier per step is enough.
+    const int kn = k + 1;
+    const bool my_row = i == kn;
 #pragma unroll
-    for (int q = 0; q < FW_BLOCK / 8; ++q) blk[i + (j0 + 8 * q) * FW_BLOCK] = cur[q];
+    for (int q = 0; q < FW_BLOCK / 8; ++q)
+      if (my_row || j0 + 8 * q == kn) blk[i + (j0 + 8 * q) * FW_BLOCK] = cur[q];
     __syncthreads();
   }
 #pragma unroll
@@ -460,7 +479,10 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
                  x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1};
   hipStream_t s = static_cast<hipStream_t>(stream);
   // a launch of a few workgroups is better spread over one thread per element
-  const bool tiny = int64_t(m) * n < 64 * 64;
+  // ... and so is one of fewer tiles than half the compute units (a block row or column of
+  // the blocked Floyd-Warshall): the tile kernel's workgroups would each run alone on a unit
+  const int64_t tiles = ((int64_t(m) + 127) / 128) * ((int64_t(n) + 127) / 128);
+  const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 128;
   const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
   hipError_t e;
   if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 8, 16>(g, s);

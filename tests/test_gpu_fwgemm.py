@@ -180,7 +180,9 @@ def _check_paths(W, dist, parent, seed, count=300):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("n,pad", [(1, 0), (100, 0), (128, 0), (300, 3), (384, 0), (513, 1)])
+@pytest.mark.parametrize("n,pad", [(1, 0), (100, 0), (128, 0), (300, 3), (384, 0), (513, 1),
+                                   # 128 tiles and more: the tiled product with the block row / column tiles skipped
+                                   (1536, 0), (1500, 4), (1475, 1)])
 def test_apsp_blocked_floyd_warshall(oracle, n, pad, dtype):
     """Blocked Floyd-Warshall: distances equal to scipy's on integer weights (every order of
     additions is exact), dist and parent bit-identical to the oracle's blocked iteration, and the
@@ -242,3 +244,24 @@ def test_apsp_blocked_on_rounding_weights_matches_the_oracle_bit_for_bit(oracle)
             continue
         hops = [i] + expand(i, j) + [j]
         assert abs(sum(float(W[a, b]) for a, b in zip(hops, hops[1:])) - dist[i, j]) <= 1e-4 * dist[i, j]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [1536, 1501])
+def test_apsp_squaring_two_steps_on_the_tiled_kernel(oracle, n, dtype):
+    """Outputs of 128 tiles and more run on the tiled kernel, whose search for the first
+    minimising k reads the transposed snapshot: two squarings, dist and parent bit for bit."""
+    import torch
+    rng = np.random.default_rng(n)
+    W = np.where(rng.random((n, n)) < 0.01, rng.integers(1, 9, (n, n)), np.inf).astype(dtype)   # many ties
+    np.fill_diagonal(W, 0)
+    dD = to_device(np.asfortranarray(W))
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32" if dtype == np.float32 else "f64"), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_squaring(dD, dP, ws, iterations=2)
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    for _ in range(2):
+        snap = want_d.copy(order="F")
+        oracle.fwgemm(snap, snap, want_d, want_p)
+    assert_same_bits(np.ascontiguousarray(dD.cpu().numpy()), np.ascontiguousarray(want_d), "dist")
+    assert np.array_equal(dP.cpu().numpy(), want_p)
