@@ -21,6 +21,7 @@
 #include "semiring.h"
 
 #include <limits>
+#include <type_traits>
 
 namespace cuasr_amd {
 namespace {
@@ -389,53 +390,87 @@ hipError_t snapshot(const void *src, int64_t ld, void *w, int64_t ldw, void *wt,
   return hipGetLastError();
 }
 
-// Floyd-Warshall inside one diagonal block of at most FW_BLOCK x FW_BLOCK, held in LDS: k ascending,
-// d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent = k_base + k.  Row k and column k do not
-// change in step k (the block's diagonal is not negative), so every step reads a settled state.
+// Floyd-Warshall inside one diagonal block of at most FW_BLOCK x FW_BLOCK: k ascending,
+// d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent = k_base + k.  One workgroup of 1024
+// threads holds the block in registers, a 4 x 4 patch per thread.  Step k needs column k and row k
+// only, and they do not change during step k (the block's diagonal is not negative): every step
+// reads them from two 128-element LDS buffers and publishes column k + 1 and row k + 1 into the
+// other pair, so one barrier per step is enough and a thread reads two vectors per 16 updates.
 constexpr int FW_BLOCK = 128;
 template <typename T>
 __global__ void __launch_bounds__(1024) fw_diagonal_kernel(T *d, int64_t ld, int32_t *parent, int64_t ldp, int bb, int k_base) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char fw_lds[];
-  T *blk = reinterpret_cast<T *>(fw_lds);  // [FW_BLOCK][FW_BLOCK], column-major
-  const int i = threadIdx.x & (FW_BLOCK - 1), j0 = threadIdx.x >> 7;  // 8 columns per pass, 16 passes
+  typedef typename vec4_of<T>::type V4;
+  __shared__ __attribute__((aligned(32))) T colbuf[2][FW_BLOCK];  // d[i][k] for the step that reads this buffer
+  __shared__ __attribute__((aligned(32))) T rowbuf[2][FW_BLOCK];  // d[k][j]
+  const int ti = threadIdx.x & 31, tj = threadIdx.x >> 5;  // rows 4 ti .. 4 ti + 3, columns 4 tj .. 4 tj + 3
   const T inf = std::numeric_limits<T>::infinity();
-  T cur[FW_BLOCK / 8];
-  int32_t par[FW_BLOCK / 8];
+  T cur[4][4];  // [row in patch][column in patch]
+  int32_t par[4][4];
 #pragma unroll
-  for (int q = 0; q < FW_BLOCK / 8; ++q) {
-    const int j = j0 + 8 * q;
-    cur[q] = (i < bb && j < bb) ? d[i + int64_t(j) * ld] : inf;
-    par[q] = -1;
-    blk[i + j * FW_BLOCK] = cur[q];
-  }
-  __syncthreads();
-  for (int k = 0; k < bb; ++k) {
-    const T dik = blk[i + k * FW_BLOCK];
+  for (int b = 0; b < 4; ++b)
 #pragma unroll
-    for (int q = 0; q < FW_BLOCK / 8; ++q) {
-      const T cand = dik + blk[k + (j0 + 8 * q) * FW_BLOCK];
-      const bool lower = cand < cur[q];
-      cur[q] = pick(lower, cand, cur[q]);
-      par[q] = lower ? k_base + k : par[q];
+    for (int a = 0; a < 4; ++a) {
+      const int i = 4 * ti + a, j = 4 * tj + b;
+      cur[a][b] = (i < bb && j < bb) ? d[i + int64_t(j) * ld] : inf;
+      par[a][b] = -1;
     }
-    // Step k + 1 reads row k + 1 and column k + 1 only, so only those are published.  They
-    // differ from what step k reads (row k, column k) except at the two crossings, which
-    // step k does not change: one barrier per step is enough.
-    const int kn = k + 1;
-    const bool my_row = i == kn;
+  // S = kn & 3, the row / column of the patch that is published, is a compile-time constant
+  // (the step loop is unrolled by four): indexed by a run-time value the patch would be
+  // moved to scratch memory, and every step would wait for memory
+  auto publish = [&](int kn, int buf, auto sc) {
+    constexpr int S = decltype(sc)::value;
+    if ((kn >> 2) == ti) {  // my patch holds row kn
+      V4 v;
 #pragma unroll
-    for (int q = 0; q < FW_BLOCK / 8; ++q)
-      if (my_row || j0 + 8 * q == kn) blk[i + (j0 + 8 * q) * FW_BLOCK] = cur[q];
+      for (int b = 0; b < 4; ++b) v[b] = cur[S][b];
+      *reinterpret_cast<V4 *>(&rowbuf[buf][4 * tj]) = v;
+    }
+    if ((kn >> 2) == tj) {  // my patch holds column kn
+      V4 v;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) v[a] = cur[a][S];
+      *reinterpret_cast<V4 *>(&colbuf[buf][4 * ti]) = v;
+    }
+  };
+  auto step = [&](int k, auto uc) {
+    constexpr int U = decltype(uc)::value;  // k & 3
+    const int buf = U & 1;
+    const V4 ci = *reinterpret_cast<const V4 *>(&colbuf[buf][4 * ti]);
+    const V4 rj = *reinterpret_cast<const V4 *>(&rowbuf[buf][4 * tj]);
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const T cand = ci[a] + rj[b];
+        const bool lower = cand < cur[a][b];
+        cur[a][b] = pick(lower, cand, cur[a][b]);
+        par[a][b] = lower ? k_base + k : par[a][b];
+      }
+    // the other pair of buffers: nobody reads it before the barrier, and nobody is still
+    // reading it from the step before (everybody has passed that step's barrier)
+    publish(k + 1, buf ^ 1, std::integral_constant<int, (U + 1) & 3>{});
     __syncthreads();
+  };
+  publish(0, 0, std::integral_constant<int, 0>{});
+  __syncthreads();
+  // steps beyond bb (up to the next multiple of four) read rows and columns of the padding,
+  // which hold +infinity and improve nothing
+  for (int k4 = 0; k4 < bb; k4 += 4) {
+    step(k4 + 0, std::integral_constant<int, 0>{});
+    step(k4 + 1, std::integral_constant<int, 1>{});
+    step(k4 + 2, std::integral_constant<int, 2>{});
+    step(k4 + 3, std::integral_constant<int, 3>{});
   }
 #pragma unroll
-  for (int q = 0; q < FW_BLOCK / 8; ++q) {
-    const int j = j0 + 8 * q;
-    if (i < bb && j < bb && par[q] >= 0) {
-      d[i + int64_t(j) * ld] = cur[q];
-      parent[i + int64_t(j) * ldp] = par[q];
+  for (int b = 0; b < 4; ++b)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const int i = 4 * ti + a, j = 4 * tj + b;
+      if (i < bb && j < bb && par[a][b] >= 0) {
+        d[i + int64_t(j) * ld] = cur[a][b];
+        parent[i + int64_t(j) * ldp] = par[a][b];
+      }
     }
-  }
 }
 
 template <typename T> hipError_t launch_naive(const FwArgs &g, hipStream_t stream) {
@@ -554,25 +589,15 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
   char *R = static_cast<char *>(workspace);             // block row,    FW_BLOCK x n,  leading dimension FW_BLOCK
   char *C = R + es * FW_BLOCK * size_t(nn);             // block column, n x FW_BLOCK,  leading dimension nn
   char *Ct = C + es * FW_BLOCK * size_t(nn);            // updated block column with k contiguous, leading dimension FW_BLOCK
-  const size_t lds = es * FW_BLOCK * FW_BLOCK;
-  static bool lds_set = false;  // the fp64 block needs 128 KiB of LDS, above the default limit of a launch
-  if (!lds_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(fw_diagonal_kernel<double>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, int(8 * FW_BLOCK * FW_BLOCK)) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(fw_diagonal_kernel<float>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, int(4 * FW_BLOCK * FW_BLOCK)) != hipSuccess)
-      return CUASR_AMD_ERROR_INTERNAL;
-    lds_set = true;
-  }
   for (int k0 = 0; k0 < n; k0 += FW_BLOCK) {
     const int bb = n - k0 < FW_BLOCK ? n - k0 : FW_BLOCK;
     char *Dkk = D + es * (size_t(k0) + size_t(k0) * size_t(ld));
     int32_t *Pkk = parent + size_t(k0) + size_t(k0) * size_t(ldp);
-    // 1. the diagonal block, closed in LDS
+    // 1. the diagonal block, closed by one workgroup
     if (f64)
-      hipLaunchKernelGGL(fw_diagonal_kernel<double>, dim3(1), dim3(1024), lds, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
+      hipLaunchKernelGGL(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
     else
-      hipLaunchKernelGGL(fw_diagonal_kernel<float>, dim3(1), dim3(1024), lds, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
+      hipLaunchKernelGGL(fw_diagonal_kernel<float>, dim3(1), dim3(1024), 0, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
     if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     // 2. snapshots of block row and block column (the products below read these, so that no
     //    workgroup sees another's updates)
