@@ -520,7 +520,7 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
   const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 128;
   const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
   hipError_t e;
-  if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 8, 16>(g, s);
+  if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 4, 16>(g, s);
   else e = naive ? launch_naive<double>(g, s) : launch_tile<double, 4, 8, 4, 16>(g, s);
   return e == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
