@@ -265,3 +265,33 @@ def test_apsp_squaring_two_steps_on_the_tiled_kernel(oracle, n, dtype):
         oracle.fwgemm(snap, snap, want_d, want_p)
     assert_same_bits(np.ascontiguousarray(dD.cpu().numpy()), np.ascontiguousarray(want_d), "dist")
     assert np.array_equal(dP.cpu().numpy(), want_p)
+
+
+def test_apsp_4096_blocked_and_squaring_agree():
+    """Full size, integer weights (every order of additions exact): blocked Floyd-Warshall and
+    repeated squaring are different algorithms and must find the same distances; both parent
+    matrices must describe paths of exactly those lengths; squaring once more changes nothing."""
+    import torch
+    n = 4096
+    rng = np.random.default_rng(4096)
+    W = np.where(rng.random((n, n)) < 0.002, rng.integers(1, 100, (n, n)), np.inf).astype(np.float32)
+    np.fill_diagonal(W, 0)
+    dW = to_device(np.asfortranarray(W))
+    results = []
+    for solver, size in ((cuasr_amd.apsp_blocked, cuasr_amd.apsp_blocked_workspace_bytes),
+                         (cuasr_amd.apsp_squaring, cuasr_amd.apsp_workspace_bytes)):
+        d = dW.clone()                       # (clone keeps the column-major strides)
+        p = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+        ws = torch.empty(size(n, "f32"), dtype=torch.uint8, device="cuda")
+        solver(d, p, ws)
+        results.append((d, p, ws))
+    (db, pb, _), (ds, ps, ws) = results
+    assert torch.equal(db, ds)
+    assert bool(torch.isfinite(db).float().mean() > 0.5)          # the graph is mostly connected
+    # a fixed point: one more squaring step improves nothing
+    before, pbefore = ds.clone(), ps.clone()
+    cuasr_amd.apsp_squaring(ds, ps, ws, iterations=1)
+    assert torch.equal(ds, before) and torch.equal(ps, pbefore)
+    dist = db.cpu().numpy()
+    for parent in (pb.cpu().numpy(), pbefore.cpu().numpy()):
+        _check_paths(W, dist, parent, seed=9, count=400)
