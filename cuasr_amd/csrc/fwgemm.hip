@@ -247,8 +247,8 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
     // first squarings of a sparse graph) those BK scattered loads per element cost as much
     // as the product itself.  With the k-contiguous image of A an element's operands are
     // two runs of BK values.  Two elements at a time have all of their operands requested
-    // before any is used.  An element that did not improve reads chunk 0 (valid memory)
-    // and stores nothing; a pair with no improved lane in the whole wave is skipped.
+    // before any is used.  An element that did not improve stores nothing; a pair with no
+    // improved lane in the whole wave is skipped.
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int c = n0 + (j >> 2) * 64 + ty2 * 4 + (j & 3);
@@ -262,11 +262,14 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
         const T *At = static_cast<const T *>(g.At);
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const int k0 = (ch[e] < 0 ? 0 : ch[e]) * BK;
+          // a lane whose element did not improve reads the first BK values of the operand (one
+          // place for all such lanes, so that they add next to nothing to the traffic)
+          const bool improved = ch[e] >= 0;
+          const int k0 = (improved ? ch[e] : 0) * BK;
           const T *ap = A + (r + e) + int64_t(k0) * g.lda;
-          const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(c) * g.ldb);
+          const V4 *bp = reinterpret_cast<const V4 *>(improved ? B + k0 + int64_t(c) * g.ldb : B);
           if constexpr (HAS_AT) {
-            const V4 *atp = reinterpret_cast<const V4 *>(At + k0 + int64_t(r + e) * g.ldat);
+            const V4 *atp = reinterpret_cast<const V4 *>(improved ? At + k0 + int64_t(r + e) * g.ldat : At);
 #pragma unroll
             for (int q = 0; q < BK / 4; ++q) {
               const V4 v = atp[q];
