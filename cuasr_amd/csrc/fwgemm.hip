@@ -242,64 +242,78 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   int tx2 = tx, ty2 = ty;
   asm volatile("" : "+v"(tx2), "+v"(ty2));
   if constexpr (!GUARD) {
-    // Whole, aligned tiles.  Every lane looks at a chunk of its own, so each load of a
-    // column-major A touches 64 cache lines per wave: with most elements improved (the
-    // first squarings of a sparse graph) those BK scattered loads per element cost as much
-    // as the product itself.  With the k-contiguous image of A an element's operands are
-    // two runs of BK values.  Two elements at a time have all of their operands requested
-    // before any is used.  An element that did not improve stores nothing; a pair with no
-    // improved lane in the whole wave is skipped.
-#pragma unroll
+    // Whole, aligned tiles.  Improved elements are few in most launches and scattered over the
+    // lanes, so they are first collected in a queue in LDS (the panels are no longer needed),
+    // one column j of the lanes' outputs at a time (at most 256 x TM entries), and the queue is
+    // then worked off by all 256 threads, one element per thread and turn: no lane waits for an
+    // element that did not improve.  Every lane looks at a chunk of its own, so each load of a
+    // column-major A touches 64 cache lines per wave; with the k-contiguous image of A an
+    // element's operands are two runs of BK values.
+    constexpr int CAP = 256 * TM;
+    static_assert(sizeof(as) >= 2 * CAP * sizeof(int) && sizeof(bs) >= CAP * sizeof(T), "the queue must fit in the panels");
+    __shared__ int q_count;
+    int *q_pos = reinterpret_cast<int *>(&as[0][0][0]);  // row | column << 8, inside the tile
+    int *q_ch = q_pos + CAP;                             // chunk
+    T *q_want = reinterpret_cast<T *>(&bs[0][0][0]);     // the minimum found
+    const T *At = static_cast<const T *>(g.At);
+#pragma unroll 1
     for (int j = 0; j < TN; ++j) {
-      const int c = n0 + (j >> 2) * 64 + ty2 * 4 + (j & 3);
+      __syncthreads();  // everybody is done with the panels / with the queue of the column before
+      if (tid == 0) q_count = 0;
+      __syncthreads();
 #pragma unroll
-      for (int i = 0; i < TM; i += 2) {
-        const int r = m0 + (i >> 2) * 64 + tx2 * 4 + (i & 3);  // and r + 1
-        const int ch[2] = {chunk[i][j], chunk[i + 1][j]};
-        if (__builtin_amdgcn_ballot_w64(ch[0] >= 0 || ch[1] >= 0) == 0) continue;
-        T pa[2][BK];
-        V4 pb[2][BK / 4];
-        const T *At = static_cast<const T *>(g.At);
+      for (int i = 0; i < TM; ++i) {
+        // (j is a run-time value here: the accumulators are read through a select chain over
+        // the TN columns, which is cheap next to the loop it replaces)
+        int ch = -1;
+        T want = T(0);
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          // a lane whose element did not improve reads the first BK values of the operand (one
-          // place for all such lanes, so that they add next to nothing to the traffic)
-          const bool improved = ch[e] >= 0;
-          const int k0 = (improved ? ch[e] : 0) * BK;
-          const T *ap = A + (r + e) + int64_t(k0) * g.lda;
-          const V4 *bp = reinterpret_cast<const V4 *>(improved ? B + k0 + int64_t(c) * g.ldb : B);
-          if constexpr (HAS_AT) {
-            const V4 *atp = reinterpret_cast<const V4 *>(improved ? At + k0 + int64_t(r + e) * g.ldat : At);
-#pragma unroll
-            for (int q = 0; q < BK / 4; ++q) {
-              const V4 v = atp[q];
-#pragma unroll
-              for (int x = 0; x < 4; ++x) pa[e][q * 4 + x] = v[x];
-            }
-          } else {
-#pragma unroll
-            for (int kk = 0; kk < BK; ++kk) pa[e][kk] = ap[int64_t(kk) * g.lda];
+        for (int jj = 0; jj < TN; ++jj)
+          if (jj == j) {
+            ch = chunk[i][jj];
+            want = acc[i][jj];
           }
+        if (ch >= 0) {
+          const int slot = atomicAdd(&q_count, 1);
+          q_pos[slot] = ((i >> 2) * 64 + tx2 * 4 + (i & 3)) | (((j >> 2) * 64 + ty2 * 4 + (j & 3)) << 8);
+          q_ch[slot] = ch;
+          q_want[slot] = want;
+        }
+      }
+      __syncthreads();
+      const int count = q_count;
+      for (int e = tid; e < count; e += 256) {
+        const int pos = q_pos[e], r = m0 + (pos & 255), c = n0 + (pos >> 8), k0 = q_ch[e] * BK;
+        const T want = q_want[e];
+        T pa[BK];
+        V4 pb[BK / 4];
+        const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(c) * g.ldb);
+        if constexpr (HAS_AT) {
+          const V4 *atp = reinterpret_cast<const V4 *>(At + k0 + int64_t(r) * g.ldat);
 #pragma unroll
-          for (int q = 0; q < BK / 4; ++q) pb[e][q] = bp[q];
+          for (int q = 0; q < BK / 4; ++q) {
+            const V4 v = atp[q];
+#pragma unroll
+            for (int x = 0; x < 4; ++x) pa[q * 4 + x] = v[x];
+          }
+        } else {
+          const T *ap = A + r + int64_t(k0) * g.lda;
+#pragma unroll
+          for (int kk = 0; kk < BK; ++kk) pa[kk] = ap[int64_t(kk) * g.lda];
         }
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const T want = acc[i + e][j];
-          T value = want;
-          int first = 0;
+        for (int q = 0; q < BK / 4; ++q) pb[q] = bp[q];
+        T value = want;
+        int first = 0;
 #pragma unroll
-          for (int kk = BK - 1; kk >= 0; --kk) {
-            const T prod = pa[e][kk] + pb[e][kk >> 2][kk & 3];
-            const bool hit = prod == want;
-            first = hit ? kk : first;
-            value = pick(hit, prod, value);
-          }
-          if (ch[e] >= 0) {
-            dist[(r + e) + int64_t(c) * g.ldc] = value;
-            g.parent[(r + e) + int64_t(c) * g.ldp] = g.k_base + ch[e] * BK + first;
-          }
+        for (int kk = BK - 1; kk >= 0; --kk) {
+          const T prod = pa[kk] + pb[kk >> 2][kk & 3];
+          const bool hit = prod == want;
+          first = hit ? kk : first;
+          value = pick(hit, prod, value);
         }
+        dist[r + int64_t(c) * g.ldc] = value;
+        g.parent[r + int64_t(c) * g.ldp] = g.k_base + k0 + first;
       }
     }
     return;
