@@ -49,10 +49,9 @@ template <typename T> __device__ __forceinline__ T pick(bool cond, T a, T b) {
 }
 
 // one thread per element, the literal scan; any extent, any leading dimension
-template <typename T>
-__global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
-  const int row = blockIdx.x * 64 + (threadIdx.x & 63);
-  const int col = blockIdx.y * 4 + (threadIdx.x >> 6);
+template <typename T> __device__ __forceinline__ void fwgemm_naive_block(const FwArgs &g, int bx, int by) {
+  const int row = bx * 64 + (threadIdx.x & 63);
+  const int col = by * 4 + (threadIdx.x >> 6);
   if (row >= g.m || col >= g.n) return;
   if ((row >= g.skip_r0 && row < g.skip_r1) || (col >= g.skip_c0 && col < g.skip_c1)) return;
   const T *a = static_cast<const T *>(g.A) + row;
@@ -69,6 +68,26 @@ __global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
   }
   *d = curr;
   *pp = p;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
+  fwgemm_naive_block<T>(g, blockIdx.x, blockIdx.y);
+}
+
+// two independent products in one launch (the block row and the block column of a blocked
+// Floyd-Warshall step, each too small to fill the chip): the first blocks0 workgroups work on
+// g0, the others on g1
+template <typename T>
+__global__ void __launch_bounds__(256) fwgemm_naive_pair_kernel(FwArgs g0, FwArgs g1, int blocks0) {
+  const int b = blockIdx.x;
+  if (b < blocks0) {
+    const int gx = (g0.m + 63) / 64;
+    fwgemm_naive_block<T>(g0, b % gx, b / gx);
+  } else {
+    const int gx = (g1.m + 63) / 64;
+    fwgemm_naive_block<T>(g1, (b - blocks0) % gx, (b - blocks0) / gx);
+  }
 }
 
 template <typename T> struct vec4_of;
@@ -624,15 +643,32 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
     if (e == hipSuccess)
       e = f64 ? snapshot<double>(Dcol, ld, C, nn, nullptr, 0, n, bb, s) : snapshot<float>(Dcol, ld, C, nn, nullptr, 0, n, bb, s);
     if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
-    // 3. block row <- (closed diagonal block) x (block row); block column <- (block column) x (closed diagonal block)
+    // 3. block row <- (closed diagonal block) x (block row); block column <- (block column) x (closed
+    //    diagonal block).  Neither touches the diagonal block itself (it is closed), so the two are
+    //    independent, and while each is too small to fill the chip they share one launch.
     FwExtra x;
     x.k_base = k0;
-    int r = fwgemm_run(dtype, bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp, x,
-                       CUASR_AMD_KERNEL_AUTO, stream);
-    if (r != CUASR_AMD_SUCCESS) return r;
-    r = fwgemm_run(dtype, n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp, x,
-                   CUASR_AMD_KERNEL_AUTO, stream);
-    if (r != CUASR_AMD_SUCCESS) return r;
+    int r;
+    if ((int64_t(n) + 127) / 128 < 128) {
+      const FwArgs g0{bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp,
+                      nullptr, 0, k0, 0, 0, k0, k0 + bb};
+      const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
+                      nullptr, 0, k0, k0, k0 + bb, 0, 0};
+      const int blocks0 = ((bb + 63) / 64) * ((n + 3) / 4), blocks1 = ((n + 63) / 64) * ((bb + 3) / 4);
+      if (f64) hipLaunchKernelGGL(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      else hipLaunchKernelGGL(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    } else {
+      FwExtra xr = x, xc = x;
+      xr.skip_c0 = xc.skip_r0 = k0;
+      xr.skip_c1 = xc.skip_r1 = k0 + bb;
+      r = fwgemm_run(dtype, bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp, xr,
+                     CUASR_AMD_KERNEL_AUTO, stream);
+      if (r != CUASR_AMD_SUCCESS) return r;
+      r = fwgemm_run(dtype, n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp, xc,
+                     CUASR_AMD_KERNEL_AUTO, stream);
+      if (r != CUASR_AMD_SUCCESS) return r;
+    }
     // 4. everything outside block row and block column <- (block column) x (block row), read in place
     //    (those panels are not written in this step); the column's k-contiguous image serves the lookups
     e = f64 ? snapshot<double>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s) : snapshot<float>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s);

@@ -16,7 +16,8 @@
  *        d[i][j] > d[i][k] + d[k][j]  =>  d[i][j] = that sum, parent = k0 + k;
  *     2. R = copy of block row k0 (b x n), C = copy of block column k0 (n x b);
  *     3. block row    <- fwgemm(R[:, k0:k0+b], R)   (parents offset by k0),
- *        block column <- fwgemm(C, C[k0:k0+b, :]);
+ *        block column <- fwgemm(C, C[k0:k0+b, :]),
+ *        both leaving the diagonal block, which is closed, as it is;
  *     4. every element outside block row and block column k0
  *                     <- fwgemm(block column, block row).
  *
@@ -77,9 +78,9 @@
       for (int j = 0; j < bb; ++j)                                                          \
         for (int i = 0; i < n; ++i) C[i + (size_t)j * n] = D[i + (k0 + j) * ld];            \
       NAME##_product(bb, n, bb, R + (size_t)k0 * b, b, R, b, D + k0, ld, P + k0, ldp, k0,   \
-                     0, 0, 0, 0);                                                           \
+                     0, 0, k0, k0 + bb);                                                    \
       NAME##_product(n, bb, bb, C, n, C + k0, n, D + k0 * ld, ld, P + k0 * ldp, ldp, k0,    \
-                     0, 0, 0, 0);                                                           \
+                     k0, k0 + bb, 0, 0);                                                    \
       NAME##_product(n, n, bb, D + k0 * ld, ld, D + k0, ld, D, ld, P, ldp, k0,              \
                      k0, k0 + bb, k0, k0 + bb);                                             \
     }                                                                                       \
