@@ -38,6 +38,9 @@ struct FwArgs {
   const void *At; int64_t ldat;
   int k_base;                               // recorded parents are k_base + k
   int skip_r0, skip_r1, skip_c0, skip_c1;   // outputs in these rows or these columns are left alone
+  // one-thread-per-element kernel only: every output it computes is also stored transposed,
+  // out_t[col + row * ld_out_t] (the k-contiguous image a later product's lookups read)
+  void *out_t; int64_t ld_out_t;
 };
 
 // cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
@@ -68,6 +71,7 @@ template <typename T> __device__ __forceinline__ void fwgemm_naive_block(const F
   }
   *d = curr;
   *pp = p;
+  if (g.out_t) static_cast<T *>(g.out_t)[col + int64_t(row) * g.ld_out_t] = curr;
 }
 
 template <typename T>
@@ -426,6 +430,24 @@ hipError_t snapshot(const void *src, int64_t ld, void *w, int64_t ldw, void *wt,
   return hipGetLastError();
 }
 
+// two copies in one launch: the first blocks0 workgroups copy (src0 -> w0), the others (src1 -> w1)
+template <typename T>
+__global__ void __launch_bounds__(256) snapshot_pair_kernel(const T *src0, T *w0, int64_t ldw0, int rows0, int cols0,
+                                                            const T *src1, T *w1, int64_t ldw1, int rows1, int cols1,
+                                                            int64_t ld, int blocks0) {
+  int b = blockIdx.x;
+  const bool first = b < blocks0;
+  if (!first) b -= blocks0;
+  const T *src = first ? src0 : src1;
+  T *w = first ? w0 : w1;
+  const int64_t ldw = first ? ldw0 : ldw1;
+  const int rows = first ? rows0 : rows1, cols = first ? cols0 : cols1;
+  const int gx = (rows + 63) / 64;
+  const int r = (b % gx) * 64 + (threadIdx.x & 63), c0 = (b / gx) * 64 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  for (int c = c0; c < cols && c < (b / gx) * 64 + 64; c += 4) w[r + int64_t(c) * ldw] = src[r + int64_t(c) * ld];
+}
+
 // Floyd-Warshall inside one diagonal block of at most FW_BLOCK x FW_BLOCK: k ascending,
 // d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent = k_base + k.  One workgroup of 1024
 // threads holds the block in registers, a 4 x 4 patch per thread.  Step k needs column k and row k
@@ -638,11 +660,19 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
     // 2. snapshots of block row and block column (the products below read these, so that no
     //    workgroup sees another's updates)
     char *Drow = D + es * size_t(k0), *Dcol = D + es * size_t(k0) * size_t(ld);
-    hipError_t e = f64 ? snapshot<double>(Drow, ld, R, FW_BLOCK, nullptr, 0, bb, n, s)
-                       : snapshot<float>(Drow, ld, R, FW_BLOCK, nullptr, 0, bb, n, s);
-    if (e == hipSuccess)
-      e = f64 ? snapshot<double>(Dcol, ld, C, nn, nullptr, 0, n, bb, s) : snapshot<float>(Dcol, ld, C, nn, nullptr, 0, n, bb, s);
-    if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    {
+      const int sb0 = ((bb + 63) / 64) * ((n + 63) / 64), sb1 = ((n + 63) / 64) * ((bb + 63) / 64);
+      if (f64)
+        hipLaunchKernelGGL(snapshot_pair_kernel<double>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const double *>(Drow),
+                           reinterpret_cast<double *>(R), int64_t(FW_BLOCK), bb, n, reinterpret_cast<const double *>(Dcol),
+                           reinterpret_cast<double *>(C), nn, n, bb, ld, sb0);
+      else
+        hipLaunchKernelGGL(snapshot_pair_kernel<float>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const float *>(Drow),
+                           reinterpret_cast<float *>(R), int64_t(FW_BLOCK), bb, n, reinterpret_cast<const float *>(Dcol),
+                           reinterpret_cast<float *>(C), nn, n, bb, ld, sb0);
+      if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    }
+    hipError_t e = hipSuccess;
     // 3. block row <- (closed diagonal block) x (block row); block column <- (block column) x (closed
     //    diagonal block).  Neither touches the diagonal block itself (it is closed), so the two are
     //    independent, and while each is too small to fill the chip they share one launch.
@@ -651,9 +681,11 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
     int r;
     if ((int64_t(n) + 127) / 128 < 128) {
       const FwArgs g0{bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp,
-                      nullptr, 0, k0, 0, 0, k0, k0 + bb};
+                      nullptr, 0, k0, 0, 0, k0, k0 + bb, nullptr, 0};
+      // (the column product also writes the updated column's k-contiguous image for step 4; the rows
+      // of the diagonal block, which it skips, are not read there)
       const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
-                      nullptr, 0, k0, k0, k0 + bb, 0, 0};
+                      nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK};
       const int blocks0 = ((bb + 63) / 64) * ((n + 3) / 4), blocks1 = ((n + 63) / 64) * ((bb + 3) / 4);
       if (f64) hipLaunchKernelGGL(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
       else hipLaunchKernelGGL(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
@@ -668,11 +700,11 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
       r = fwgemm_run(dtype, n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp, xc,
                      CUASR_AMD_KERNEL_AUTO, stream);
       if (r != CUASR_AMD_SUCCESS) return r;
+      e = f64 ? snapshot<double>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s) : snapshot<float>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s);
+      if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     }
     // 4. everything outside block row and block column <- (block column) x (block row), read in place
     //    (those panels are not written in this step); the column's k-contiguous image serves the lookups
-    e = f64 ? snapshot<double>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s) : snapshot<float>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s);
-    if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     x.At = Ct;
     x.ldat = FW_BLOCK;
     x.skip_r0 = x.skip_c0 = k0;
