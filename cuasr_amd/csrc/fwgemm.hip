@@ -54,7 +54,8 @@ template <typename T> __device__ __forceinline__ T pick(bool cond, T a, T b) {
 // one thread per element, the literal scan; any extent, any leading dimension
 template <typename T> __device__ __forceinline__ void fwgemm_naive_block(const FwArgs &g, int bx, int by) {
   const int row = bx * 64 + (threadIdx.x & 63);
-  const int col = by * 4 + (threadIdx.x >> 6);
+  // (a wave's 64 threads share a column: saying so keeps B's addresses in scalar registers)
+  const int col = __builtin_amdgcn_readfirstlane(by * 4 + (threadIdx.x >> 6));
   if (row >= g.m || col >= g.n) return;
   if ((row >= g.skip_r0 && row < g.skip_r1) || (col >= g.skip_c0 && col < g.skip_c1)) return;
   const T *a = static_cast<const T *>(g.A) + row;
@@ -63,7 +64,23 @@ template <typename T> __device__ __forceinline__ void fwgemm_naive_block(const F
   int32_t *pp = g.parent + row + col * g.ldp;
   T curr = *d;
   int32_t p = *pp;
-  for (int i = 0; i < g.k; ++i) {
+  int i = 0;
+  for (; i + 8 <= g.k; i += 8) {  // eight k at a time, their operands requested together
+    T av[8], bv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      av[u] = a[(i + u) * g.lda];
+      bv[u] = b[i + u];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const T prod = av[u] + bv[u];
+      const bool lower = prod < curr;
+      curr = pick(lower, prod, curr);
+      p = lower ? g.k_base + i + u : p;
+    }
+  }
+  for (; i < g.k; ++i) {
     const T prod = a[i * g.lda] + b[i];
     const bool lower = prod < curr;
     curr = pick(lower, prod, curr);
