@@ -65,15 +65,15 @@ template <typename T> __device__ __forceinline__ void fwgemm_naive_block(const F
   T curr = *d;
   int32_t p = *pp;
   int i = 0;
-  for (; i + 8 <= g.k; i += 8) {  // eight k at a time, their operands requested together
-    T av[8], bv[8];
+  for (; i + 16 <= g.k; i += 16) {  // sixteen k at a time, their operands requested together
+    T av[16], bv[16];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 16; ++u) {
       av[u] = a[(i + u) * g.lda];
       bv[u] = b[i + u];
     }
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < 16; ++u) {
       const T prod = av[u] + bv[u];
       const bool lower = prod < curr;
       curr = pick(lower, prod, curr);
