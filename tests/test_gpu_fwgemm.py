@@ -295,3 +295,57 @@ def test_apsp_4096_blocked_and_squaring_agree():
     dist = db.cpu().numpy()
     for parent in (pb.cpu().numpy(), pbefore.cpu().numpy()):
         _check_paths(W, dist, parent, seed=9, count=400)
+
+
+def test_apsp_drivers_can_be_captured_in_a_graph(oracle):
+    """Neither driver allocates, frees, copies through the runtime or synchronises: a stream capture
+    may contain them.  Both are captured once and replayed on new graphs, with eager work and
+    synchronisations between the replays; every replay must equal the oracle bit for bit."""
+    import torch
+    n = 300
+    src = torch.empty(n, n, device="cuda").t()
+    d_blk, d_sq = torch.empty(n, n, device="cuda").t(), torch.empty(n, n, device="cuda").t()
+    p_blk = torch.empty(n, n, dtype=torch.int32, device="cuda").t()
+    p_sq = torch.empty(n, n, dtype=torch.int32, device="cuda").t()
+    w_blk = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    w_sq = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+
+    def work():
+        d_blk.copy_(src); d_sq.copy_(src)
+        p_blk.fill_(-1); p_sq.fill_(-1)
+        cuasr_amd.apsp_blocked(d_blk, p_blk, w_blk)
+        cuasr_amd.apsp_squaring(d_sq, p_sq, w_sq, iterations=3)
+
+    def load(seed):
+        rng = np.random.default_rng(seed)
+        W = np.where(rng.random((n, n)) < 0.03, rng.random((n, n)) * 9 + 0.5, np.inf).astype(np.float32)
+        np.fill_diagonal(W, 0)
+        src.copy_(torch.from_numpy(np.ascontiguousarray(W.T)).cuda().t())
+        return W
+
+    load(1)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        work()
+    for seed in (2, 3, 4):
+        W = load(seed)
+        scratch = torch.rand(256, 256, device="cuda") @ torch.rand(256, 256, device="cuda")   # eager work in between
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        del scratch
+        want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+        oracle.apsp_blocked(want_d, want_p, 128)
+        assert_same_bits(np.ascontiguousarray(d_blk.cpu().numpy()), np.ascontiguousarray(want_d), f"blocked, seed {seed}")
+        assert np.array_equal(p_blk.cpu().numpy(), want_p)
+        want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+        for _ in range(3):
+            snap = want_d.copy(order="F")
+            oracle.fwgemm(snap, snap, want_d, want_p)
+        assert_same_bits(np.ascontiguousarray(d_sq.cpu().numpy()), np.ascontiguousarray(want_d), f"squaring, seed {seed}")
+        assert np.array_equal(p_sq.cpu().numpy(), want_p)
