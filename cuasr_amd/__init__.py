@@ -80,6 +80,8 @@ def load():
         lib.cuasr_amd_srgemm_can_implement.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm.restype = ctypes.c_int
         lib.cuasr_amd_srgemm.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p]
+        lib.cuasr_amd_srgemm_batched.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm_batched.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_int] + [ctypes.c_int64] * 4 + [ctypes.c_void_p]
         lib.cuasr_amd_splitk_workspace_bytes.restype = ctypes.c_size_t
         lib.cuasr_amd_splitk_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk.restype = ctypes.c_int
@@ -241,6 +243,22 @@ def srgemm(add_op, mult_op, A, B, C, D, alpha=None, beta=None, add_identity=None
     st = load().cuasr_amd_srgemm(ctypes.byref(desc), _stream_handle(stream))
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_srgemm")
+    return D
+
+
+def srgemm_batched(add_op, mult_op, A, B, C, D, alpha, beta, add_identity, mult_identity, dtype=None,
+                   kernel="auto", stream=None):
+    """A batch of SRGEMMs: A, B, C, D are 3-D CUDA tensors (batch, rows, cols) whose 2-D slices are
+    row- or column-major matrices; a first dimension of stride 0 (``expand``) shares an operand."""
+    dtype = dtype or _torch_dtype_name(D)
+    batch = D.shape[0]
+    if batch == 0:
+        return D
+    desc = make_desc(add_op, mult_op, dtype, A[0], B[0], C[0], D[0], alpha, beta, add_identity, mult_identity, 1, kernel)
+    st = load().cuasr_amd_srgemm_batched(ctypes.byref(desc), batch, A.stride(0), B.stride(0), C.stride(0), D.stride(0),
+                                         _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_srgemm_batched")
     return D
 
 

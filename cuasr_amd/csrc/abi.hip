@@ -290,6 +290,32 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   return fn(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
 
+// A batch as a sequence of launches on the stream (each validated like a single call): right for
+// matrices large enough to fill the chip; a batch of many small products would want the batch index
+// in the grid instead.
+int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a, int64_t stride_b,
+                             int64_t stride_c, int64_t stride_d, void *stream) {
+  if (!desc || batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0 || stride_d < 0)
+    return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  const int st = validate(desc, false);
+  if (st != CUASR_AMD_SUCCESS) return st;
+  // the outputs must not overlap: at least the span of one matrix apart
+  const bool col = desc->layout_c == CUASR_AMD_COLUMN_MAJOR;
+  const int64_t outer = col ? desc->n : desc->m, inner = col ? desc->m : desc->n;
+  if (batch > 1 && outer > 0 && inner > 0 && stride_d < (outer - 1) * desc->ldd + inner) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  const int64_t es = int64_t(elem_size(desc->dtype));
+  for (int i = 0; i < batch; ++i) {
+    cuasr_amd_srgemm_desc one = *desc;
+    if (one.A) one.A = static_cast<const char *>(desc->A) + es * stride_a * i;
+    if (one.B) one.B = static_cast<const char *>(desc->B) + es * stride_b * i;
+    if (one.C) one.C = static_cast<const char *>(desc->C) + es * stride_c * i;
+    if (one.D) one.D = static_cast<char *>(desc->D) + es * stride_d * i;
+    const int r = cuasr_amd_srgemm(&one, stream);
+    if (r != CUASR_AMD_SUCCESS) return r;
+  }
+  return CUASR_AMD_SUCCESS;
+}
+
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
   if (!desc || desc->m < 0 || desc->n < 0 || desc->split_k_slices < 1) return 0;
   if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_U32) return 0;

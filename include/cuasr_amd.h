@@ -153,6 +153,17 @@ int cuasr_amd_srgemm_can_implement(const cuasr_amd_srgemm_desc *desc);
  * split_k_slices > 1 (device/srgemm.h:198-200). */
 int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream);
 
+/* A batch of SRGEMMs that share one descriptor: product i works on the
+ * descriptor's A, B, C, D advanced by i * stride_a, i * stride_b, i * stride_c,
+ * i * stride_d ELEMENTS (the reference only names batched operation as an aim,
+ * README.md:11, and has no such call).  Stride 0 shares an operand between all
+ * products; the outputs must lie at least one matrix apart, strides must not be
+ * negative (CUASR_AMD_ERROR_INVALID_PROBLEM otherwise).  The products are
+ * launched one after the other on the stream, each chosen and validated like a
+ * single cuasr_amd_srgemm; the first failure is returned. */
+int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a,
+                             int64_t stride_b, int64_t stride_c, int64_t stride_d, void *stream);
+
 /* Bytes of device workspace the split-K call needs:
  * sizeof(element) * m * n * split_k_slices. */
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);

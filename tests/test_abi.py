@@ -22,7 +22,8 @@ def test_exports_match_header(lib):
     assert {"cuasr_amd_srgemm", "cuasr_amd_srgemm_splitk", "cuasr_amd_splitk_workspace_bytes",
             "cuasr_amd_srgemm_can_implement", "cuasr_amd_srgemm_splitk_serial",
             "cuasr_amd_splitk_serial_workspace_bytes", "cuasr_amd_fwgemm", "cuasr_amd_apsp_squaring",
-            "cuasr_amd_apsp_workspace_bytes", "cuasr_amd_apsp_blocked", "cuasr_amd_apsp_blocked_workspace_bytes"} <= set(names)
+            "cuasr_amd_apsp_workspace_bytes", "cuasr_amd_apsp_blocked", "cuasr_amd_apsp_blocked_workspace_bytes",
+            "cuasr_amd_srgemm_batched"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
     assert lib.cuasr_amd_abi_version() == 1
@@ -133,6 +134,24 @@ def test_fwgemm_host_errors(lib):
     assert cuasr_amd.apsp_blocked_workspace_bytes(1001, "f32") == 3 * 4 * 128 * 1004 and cuasr_amd.apsp_blocked_workspace_bytes(0, "f64") == 0
     bl = lambda n=64, ws=0x1000, dtype=0, ld=None: lib.cuasr_amd_apsp_blocked(dtype, n, P(0x1000), ld or max(n, 1), P(0x1000), max(n, 1), P(ws), None)
     assert bl(ws=0) == 6 and bl(dtype=2) == 2 and bl(n=0) == 0 and bl(ld=10) == 4 and bl(ws=0x1004) == 1   # all before any launch
+
+
+def test_batched_host_errors(lib):
+    """Argument checks of the batched call; nothing here launches (a batch of 0 is valid and empty)."""
+    d = cuasr_amd.SrgemmDesc()
+    d.add_op, d.mult_op, d.dtype = cuasr_amd.OPS["minimum"], cuasr_amd.OPS["plus"], cuasr_amd.DTYPES["f32"]
+    d.m = d.n = d.k = 64
+    d.split_k_slices = 1
+    d.A = d.B = d.C = d.D = 0x1000
+    d.lda = d.ldb = d.ldc = d.ldd = 64
+    call = lambda batch=0, sa=4096, sb=4096, sc=4096, sd=4096: lib.cuasr_amd_srgemm_batched(
+        ctypes.byref(d), batch, sa, sb, sc, sd, None)
+    assert call() == 0
+    assert call(batch=-1) == 4 and call(sa=-1) == 4 and call(sd=-4096) == 4
+    assert call(batch=2, sd=4095) == 4 and call(batch=2, sd=0) == 4      # outputs would overlap
+    assert lib.cuasr_amd_srgemm_batched(None, 0, 0, 0, 0, 0, None) == 4
+    d.split_k_slices = 2
+    assert call() == 4                                                     # as the single call
 
 
 def test_semiring_constants():

@@ -1,0 +1,53 @@
+"""GPU parity of the batched call (a sequence of products sharing one descriptor) through the C ABI:
+every product bit-identical to the oracle's SRGEMM on the same operands."""
+import numpy as np
+import pytest
+
+import cuasr_amd
+from helpers import assert_same_bits
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case", [
+    ("minimum", "plus", np.float32, 0.0, 0.0, np.inf, 0.0),
+    ("maximum", "minimum", np.float64, np.inf, np.inf, -np.inf, np.inf),
+    ("plus", "multiplies", np.float64, 1.0, 1.0, 0.0, 1.0),
+])
+def test_batched_products_match_the_oracle(oracle, case):
+    import torch
+    add, mult, dtype, alpha, beta, ident, one = case
+    batch, m, n, k = 5, 96, 80, 70
+    rng = np.random.default_rng(17)
+    # small integers: the plus-times sums are exact whatever their order
+    A = rng.integers(0, 7, (batch, m, k)).astype(dtype)
+    B = rng.integers(0, 7, (k, n)).astype(dtype)                      # one B for the whole batch (stride 0)
+    C = rng.integers(0, 9, (batch, m, n + 3)).astype(dtype)           # padded rows: leading dimension n + 3
+    dA = torch.from_numpy(A).cuda()
+    dB = torch.from_numpy(B).cuda().unsqueeze(0).expand(batch, k, n)
+    dC = torch.from_numpy(C).cuda()
+    dD = torch.full((batch, m, n + 3), -5, dtype=dA.dtype, device="cuda")
+    cuasr_amd.srgemm_batched(add, mult, dA, dB, dC[:, :, :n], dD[:, :, :n], alpha, beta, ident, one, kernel="valu")
+    got = dD.cpu().numpy()
+    assert (got[:, :, n:] == -5).all()                                 # the padding is untouched
+    for i in range(batch):
+        want = oracle.srgemm(add, mult, A[i], B, np.ascontiguousarray(C[i][:, :n]), alpha, beta, ident)
+        assert_same_bits(np.ascontiguousarray(got[i][:, :n]), want, f"{add}-{mult} product {i}")
+
+
+def test_batched_empty_batch_and_column_major(oracle):
+    import torch
+    batch, m, n, k = 3, 64, 64, 32
+    rng = np.random.default_rng(3)
+    A = rng.random((batch, k, m)).astype(np.float32)                   # slices are column-major m x k matrices
+    B = rng.random((batch, n, k)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).cuda().transpose(1, 2), torch.from_numpy(B).cuda().transpose(1, 2)
+    dD = torch.zeros(batch, n, m, device="cuda").transpose(1, 2)
+    inf = float("inf")
+    cuasr_amd.srgemm_batched("minimum", "plus", dA, dB, dD, dD, 0.0, inf, inf, 0.0)   # beta = annihilator: C unread
+    got = dD.cpu().numpy()
+    for i in range(batch):
+        want = oracle.srgemm("minimum", "plus", np.asfortranarray(A[i].T), np.asfortranarray(B[i].T),
+                             np.zeros((m, n), np.float32, order="F"), 0.0, np.inf, np.inf)
+        assert_same_bits(np.ascontiguousarray(got[i]), np.ascontiguousarray(want), f"product {i}")
+    cuasr_amd.srgemm_batched("minimum", "plus", dA[:0], dB[:0], dD[:0], dD[:0], 0.0, inf, inf, 0.0)   # nothing to do
