@@ -589,10 +589,11 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
                  x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1};
   hipStream_t s = static_cast<hipStream_t>(stream);
   // a launch of a few workgroups is better spread over one thread per element
-  // ... and so is one of fewer tiles than half the compute units (a block row or column of
-  // the blocked Floyd-Warshall): the tile kernel's workgroups would each run alone on a unit
+  // ... and so is one of few tiles (the tile kernel's workgroups would each run alone on a
+  // compute unit): measured on square problems, the two kernels meet at about 100 tiles
+  // (1024^3: 193 against 270 us, 1280^3: 356 against 334, 1408^3: 466 against 366)
   const int64_t tiles = ((int64_t(m) + 127) / 128) * ((int64_t(n) + 127) / 128);
-  const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 128;
+  const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 96;
   const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
   hipError_t e;
   if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 4, 16>(g, s);
