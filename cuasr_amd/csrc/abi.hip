@@ -341,7 +341,15 @@ static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *
   const long long per = (tiles + p.slices - 1) / p.slices;
   p.k_per_slice = int(per * tile > 0 ? per * tile : tile);
   p.workspace = workspace;
-  const launch_fn fn = family_fn(pick_family(desc), desc);
+  // The direct-to-LDS tiles store partial tiles as 16-byte vectors; family selection looks at the
+  // operands only, so a workspace that is element-aligned but not 16-byte aligned is sorted out here:
+  // AUTO goes on to the staged family (or the naive kernel), a forced direct tile is refused.
+  int family = pick_family(desc);
+  if (family == kDirect && !(desc->dtype == CUASR_AMD_F64 ? direct64_can_run(p) : direct_can_run(p))) {
+    if (desc->kernel != CUASR_AMD_KERNEL_AUTO) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+    family = find_valu(desc->dtype, desc->add_op, desc->mult_op) ? kValu : kNaive;
+  }
+  const launch_fn fn = family_fn(family, desc);
   const launch_fn red = serial ? find_reduce_serial(desc->dtype) : find_reduce(desc->dtype);
   if (!fn || !red) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);

@@ -171,7 +171,11 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
 /* Two launches on `stream`: partial products of `split_k_slices` K-slices into
  * `workspace`, then a reduction with the semiring's add and the epilogue.
  * CUASR_AMD_ERROR_WORKSPACE_NULL when workspace is NULL
- * (device/srgemm_splitk_parallel.h:247-249). */
+ * (device/srgemm_splitk_parallel.h:247-249).  The workspace must be aligned to
+ * the element size; a workspace that is not 16-byte aligned keeps AUTO off the
+ * direct-to-LDS tiles (they store 16-byte vectors), and a forced
+ * CUASR_AMD_KERNEL_VALU_DIRECT is then refused with
+ * CUASR_AMD_ERROR_MISALIGNED_OPERAND. */
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
                             void *stream);
 

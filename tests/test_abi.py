@@ -104,6 +104,17 @@ def test_splitk_host_errors(lib):
     assert lib.cuasr_amd_srgemm(ctypes.byref(d), None) == 4
 
 
+def test_splitk_workspace_alignment_host_side(lib):
+    """A workspace aligned to the element but not to 16 bytes: refused for a forced direct-to-LDS tile
+    (which stores 16-byte vectors) before anything is launched; 2-byte misalignment refused for every family."""
+    d = desc(m=512, n=512, k=4096, slices=8, kernel="direct")
+    assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d), ctypes.c_void_p(0x1004), None) == 1
+    assert lib.cuasr_amd_srgemm_splitk_serial(ctypes.byref(d), ctypes.c_void_p(0x1004), None) == 1
+    d = desc(m=512, n=512, k=4096, slices=8, dtype="f64", add="maximum", kernel="direct")
+    assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d), ctypes.c_void_p(0x1008), None) == 1
+    assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(desc(slices=8)), ctypes.c_void_p(0x1002), None) == 1
+
+
 def test_serial_splitk_host_errors(lib):
     # the workspace holds the slices' partial products; none is needed for a single slice (device/srgemm.h:218-234)
     assert cuasr_amd.splitk_serial_workspace_bytes(256, 256, 8, "f32") == 4 * 256 * 256 * 8

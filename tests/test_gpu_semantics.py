@@ -163,3 +163,34 @@ def test_calls_can_be_captured_in_a_graph(oracle, lib):
         want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)
         assert_same_bits(s_par.cpu().numpy(), want, f"graph replay, seed {seed}: split-K")
         assert_same_bits(s_ser.cpu().numpy(), want, f"graph replay, seed {seed}: serial split-K")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("serial", [False, True])
+def test_splitk_workspace_aligned_to_the_element_only(oracle, lib, dtype, serial):
+    """A split-K workspace at an element boundary that is not a 16-byte boundary: the descriptor is one the
+    direct-to-LDS tile is chosen for (1024 x 1024 x 4096 in 16 slices fills its rounds, operands aligned),
+    so AUTO has to notice the workspace and fall back to a family that stores element-wise."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    npd = {"f32": np.float32, "f64": np.float64}[dtype]
+    m, n, k, slices = 1024, 1024, 4096, 16
+    A = inputs.uniform(61, m, k, 0.0, 10.0, npd, "F")
+    B = inputs.uniform(62, k, n, 0.0, 10.0, npd, "F")
+    C = inputs.uniform(63, m, n, 0.0, 10.0, npd, "F")
+    want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)   # min is order-free: both split-K forms equal the plain product
+    es = np.dtype(npd).itemsize
+    nbytes = cuasr_amd.splitk_workspace_bytes(m, n, slices, dtype)
+    raw = torch.empty(nbytes + 16, dtype=torch.uint8, device="cuda")
+    assert raw.data_ptr() % 16 == 0
+    run = cuasr_amd.srgemm_splitk_serial if serial else cuasr_amd.srgemm_splitk
+    import ctypes
+    for offset in (0, es):
+        dD = to_device(np.zeros_like(C))
+        desc = cuasr_amd.make_desc("minimum", "plus", dtype, to_device(A), to_device(B), to_device(C), dD, 0.0, 0.0, float("inf"), 0.0, slices)
+        assert lib.cuasr_amd_selected_kernel(ctypes.byref(desc)) == b"valu_direct"   # what the operands alone would get
+        run("minimum", "plus", to_device(A), to_device(B), to_device(C), dD, slices, raw.data_ptr() + offset,
+            0.0, 0.0, float("inf"), 0.0, dtype=dtype)
+        torch.cuda.synchronize()
+        assert_same_bits(to_host(dD, dtype), want, f"{dtype} workspace offset {offset}")
