@@ -86,6 +86,8 @@ def load():
         lib.cuasr_amd_splitk_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk.restype = ctypes.c_int
         lib.cuasr_amd_srgemm_splitk.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_srgemm_splitk_static.restype = ctypes.c_int
+        lib.cuasr_amd_srgemm_splitk_static.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p]
         lib.cuasr_amd_splitk_serial_workspace_bytes.restype = ctypes.c_size_t
         lib.cuasr_amd_splitk_serial_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk_serial.restype = ctypes.c_int
@@ -285,6 +287,28 @@ def srgemm_splitk(add_op, mult_op, A, B, C, D, slices, workspace, alpha=None, be
     st = load().cuasr_amd_srgemm_splitk(ctypes.byref(desc), ctypes.c_void_p(ws or None), _stream_handle(stream))
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_srgemm_splitk")
+    return D
+
+
+STATIC_WORKSPACE_BYTES = 16 << 20  # CUASR_AMD_STATIC_WORKSPACE_BYTES
+
+
+def srgemm_splitk_static(add_op, mult_op, A, B, C, D, slices, alpha=None, beta=None,
+                         add_identity=None, mult_identity=None, dtype=None, kernel="auto",
+                         stream=None, alpha_ptr=None, beta_ptr=None, infinities=False):
+    """Parallel split-K SRGEMM whose partial tiles go to the library's own fixed device array
+    (STATIC_WORKSPACE_BYTES per GPU) instead of a caller workspace: the call allocates nothing.
+    Calls that may overlap on one GPU share that array and must be ordered by the caller."""
+    dtype = dtype or _torch_dtype_name(D)
+    alpha = op_identity(mult_op, dtype, infinities) if alpha is None else alpha
+    beta = op_annihilator(mult_op, dtype, infinities) if beta is None else beta
+    add_identity = op_identity(add_op, dtype, infinities) if add_identity is None else add_identity
+    mult_identity = op_identity(mult_op, dtype, infinities) if mult_identity is None else mult_identity
+    desc = make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,
+                     slices, kernel, alpha_ptr, beta_ptr)
+    st = load().cuasr_amd_srgemm_splitk_static(ctypes.byref(desc), _stream_handle(stream))
+    if st != SUCCESS:
+        raise CuasrError(st, "cuasr_amd_srgemm_splitk_static")
     return D
 
 

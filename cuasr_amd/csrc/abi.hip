@@ -2,6 +2,8 @@
 // kernel-family selection and launch.  Host-side counterpart of
 // include/cuasr/gemm/device/srgemm.h:196-356 and
 // include/cuasr/gemm/device/srgemm_splitk_parallel.h:220-357.
+#include <atomic>
+
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -251,7 +253,7 @@ const char *cuasr_amd_status_string(int status) {
     case CUASR_AMD_ERROR_INTERNAL: return "internal error";
     case CUASR_AMD_ERROR_ARCH_MISMATCH: return "architecture mismatch";
     case CUASR_AMD_ERROR_INSUFFICIENT_DRIVER: return "insufficient driver";
-    case CUASR_AMD_ERROR_MEMORY_ALLOCATION: return "memory allocation failed";
+    case CUASR_AMD_ERROR_MEMORY_ALLOCATION: return "memory allocation failed (or: larger than the library's fixed workspace)";
     default: return "invalid status";
   }
 }
@@ -359,6 +361,39 @@ static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *
 
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
   return run_splitk(desc, workspace, stream, false);
+}
+
+// ---- split-K for callers that cannot allocate: the workspace is a fixed array in the library's
+// own device image, one copy per GPU, shared by every call on that GPU.
+static __device__ __align__(256) unsigned char scratch[CUASR_AMD_STATIC_WORKSPACE_BYTES];
+
+// Device address of `scratch` on the current GPU.  The array's name is only a host-side handle
+// for the symbol; the address is asked for once per device, with that device current, and kept.
+static void *static_workspace(void) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void *> table[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  void *ptr = table[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return nullptr;
+    table[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  }
+  return ptr;
+}
+
+int cuasr_amd_srgemm_splitk_static(const cuasr_amd_srgemm_desc *desc, void *stream) {
+  const int st = validate(desc, true);
+  if (st != CUASR_AMD_SUCCESS) return st;
+  // the partial tiles of all slices must fit (no overflow: m * n < 2^62, and the quotient bounds the rest)
+  const unsigned long long elems = (unsigned long long)desc->m * (unsigned long long)desc->n;
+  const unsigned long long room = CUASR_AMD_STATIC_WORKSPACE_BYTES / elem_size(desc->dtype);
+  if (elems > room || elems * (unsigned long long)desc->split_k_slices > room) return CUASR_AMD_ERROR_MEMORY_ALLOCATION;
+  void *ws = static_workspace();
+  if (!ws) return CUASR_AMD_ERROR_INTERNAL;
+  // nothing in the array has to start at zero: the slice kernels write every element of the
+  // slices the reduction reads (empty trailing slices are filled with the additive identity)
+  return run_splitk(desc, ws, stream, false);
 }
 
 size_t cuasr_amd_splitk_serial_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {

@@ -179,6 +179,23 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
                             void *stream);
 
+/* Split-K for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart
+ * in the reference, whose split-K always takes the caller's workspace
+ * (device/srgemm_splitk_parallel.h:238-249).  Same result as
+ * cuasr_amd_srgemm_splitk, bit for bit; the partial tiles go to a fixed array of
+ * CUASR_AMD_STATIC_WORKSPACE_BYTES inside the library's device image (one copy
+ * per GPU, held until the process ends) instead of a caller workspace.  The call
+ * makes no hipMalloc / hipFree and no allocating library call; its first use on
+ * a device looks the array's address up once (make that first call outside a
+ * graph capture).  CUASR_AMD_ERROR_MEMORY_ALLOCATION when
+ * sizeof(element) * m * n * split_k_slices exceeds the array.  All calls on one
+ * GPU share the array: calls that may overlap in time on one GPU (different
+ * streams, several host threads) race on it and must be ordered by the caller;
+ * calls on one stream are ordered by the stream. */
+#define CUASR_AMD_STATIC_WORKSPACE_BYTES (16u << 20)
+int cuasr_amd_srgemm_splitk_static(const cuasr_amd_srgemm_desc *desc, void *stream);
+
 /* Serial split-K (device::Srgemm with SplitKSerial = true,
  * include/cuasr/gemm/device/srgemm.h:218-282; include/cuasr/gemm/kernel/srgemm.h:249-320).
  * The result is the reference's chain of epilogues, slice 0 first:

@@ -23,7 +23,7 @@ def test_exports_match_header(lib):
             "cuasr_amd_srgemm_can_implement", "cuasr_amd_srgemm_splitk_serial",
             "cuasr_amd_splitk_serial_workspace_bytes", "cuasr_amd_fwgemm", "cuasr_amd_apsp_squaring",
             "cuasr_amd_apsp_workspace_bytes", "cuasr_amd_apsp_blocked", "cuasr_amd_apsp_blocked_workspace_bytes",
-            "cuasr_amd_srgemm_batched"} <= set(names)
+            "cuasr_amd_srgemm_batched", "cuasr_amd_srgemm_splitk_static"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
     assert lib.cuasr_amd_abi_version() == 1
@@ -113,6 +113,19 @@ def test_splitk_workspace_alignment_host_side(lib):
     d = desc(m=512, n=512, k=4096, slices=8, dtype="f64", add="maximum", kernel="direct")
     assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d), ctypes.c_void_p(0x1008), None) == 1
     assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(desc(slices=8)), ctypes.c_void_p(0x1002), None) == 1
+
+
+def test_static_splitk_host_errors(lib):
+    """cuasr_amd_srgemm_splitk_static checks the descriptor and the size of the partial tiles against
+    the library's fixed array before it touches the device."""
+    call = lambda d: lib.cuasr_amd_srgemm_splitk_static(ctypes.byref(d), None)
+    assert cuasr_amd.STATIC_WORKSPACE_BYTES == 16 << 20
+    assert lib.cuasr_amd_srgemm_splitk_static(None, None) == 4
+    assert call(desc(slices=0)) == 4
+    assert call(desc(ptr=0x10002, slices=2)) == 1
+    assert call(desc(m=1024, n=1024, k=64, slices=5)) == 10        # 20 MiB of partial tiles: kErrorMemoryAllocation
+    assert call(desc(m=2048, n=2048, k=64, slices=1, dtype="f64")) == 10
+    assert call(desc(m=46341, n=46341, k=8, slices=2 ** 31 - 1)) == 10   # products past 64 bits are still refused
 
 
 def test_serial_splitk_host_errors(lib):
