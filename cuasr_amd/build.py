@@ -40,7 +40,17 @@ def _compile(src):
     return obj, err
 
 
+def generate():
+    """The hand-scheduled main loops of the direct-to-LDS tile: asm text written by csrc/gen_direct_asm.py."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("gen_direct_asm", os.path.join(CSRC, "gen_direct_asm.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.generate(os.path.join(CSRC, "gen"))
+
+
 def build(jobs=None, verbose=True):
+    generate()
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)

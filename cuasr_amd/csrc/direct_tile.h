@@ -31,6 +31,7 @@
 #pragma once
 #include <utility>
 
+#include "direct_asm.h"
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -362,7 +363,54 @@ struct DirectTile {
     // lane's LDS byte address of (stage 0, k-pair 0, x 0) in each panel
     const unsigned a_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][0] + ty * 16;
     const unsigned b_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][0] + tx * 16;
-    if constexpr (RELAXED) {
+    typedef typename AsmLoop<T, ADD, MUL, A_KC, B_KC>::type Loop;
+    if constexpr (!RELAXED && !std::is_void<Loop>::value && TY == 32 && TX == 16 && BK == 16 && STAGES == 3) {
+      // The hand-scheduled main loop (direct_asm.h): accumulators and fragments live in fixed registers,
+      // one asm statement per k-tile.  It fetches whole tiles only; a ragged last tile is fetched here,
+      // by the same route as in the prologue, two tiles ahead like every other.
+      static_assert(LA == 2 && LB == 1, "the generated loop moves two pieces of A and one of B per wave");
+      if (nfull > 0) {
+        AsmRegs r;
+        float ident_bits;
+        __builtin_memcpy(&ident_bits, &ident, 4);
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) r.acc[v][e] = ident_bits;
+#pragma unroll
+        for (int v = 0; v < 3; ++v) r.frag[v] = asm_v16(0.0f);
+        // lane's global byte offsets inside a whole k-tile (the x clamp is part of xa / xb)
+        const unsigned off_a0 = tile_offset<A_KC, BM>((wave * LA + 0) * 64 + lane, xa[0], a_kbytes, BK);
+        const unsigned off_a1 = tile_offset<A_KC, BM>((wave * LA + 1) * 64 + lane, xa[1], a_kbytes, BK);
+        const unsigned off_b0 = tile_offset<B_KC, BN>((wave * LB + 0) * 64 + lane, xb[0], b_kbytes, BK);
+        // LDS byte address of this wave's first piece of each panel in stage 0 (wave-uniform)
+        const unsigned m0_a0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][(wave * LA) * 256]);
+        const unsigned m0_b0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][(wave * LB) * 256]);
+        constexpr unsigned A_STAGE = BK * BM * 4, B_STAGE = BK * BN * 4;
+        unsigned a_addr = a_addr0, b_addr = b_addr0;
+        Loop::prime(r, a_addr, b_addr);
+        int stage = 0;
+        for (int t = 0; t < nfull; ++t) {
+          const int next = stage + 1 == STAGES ? 0 : stage + 1, stage2 = next + 1 == STAGES ? 0 : next + 1;
+          if (t + 2 == nfull && rem > 0) {
+#pragma unroll
+            for (int q = 0; q < LA + LB; ++q) fetch_piece(q, stage2, rem);
+          }
+          Loop::tile(r, a_addr, b_addr, (unsigned)((next - stage) * (int)A_STAGE), (unsigned)((next - stage) * (int)B_STAGE),
+                     nfull - (t + 2), m0_a0 + stage2 * A_STAGE, m0_b0 + stage2 * B_STAGE, off_a0, off_a1, off_b0, base_a, base_b);
+          base_a += a_step;
+          base_b += b_step;
+          stage = next;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float bits = r.acc[i >> 1][(i & 1) * 8 + j];
+            __builtin_memcpy(&acc[i][j], &bits, 4);
+          }
+      }
+    } else if constexpr (RELAXED) {
       FragA a[2];
       FragB b[2];
       for (int t = 0; t < nfull; ++t) {
@@ -460,12 +508,12 @@ struct DirectTile {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const int row = m0 + own<A_KC, TY>(i, ty);
-      if (row < p.m) {
+      if ((unsigned)row < (unsigned)p.m) {  // unsigned: an index that is not one cannot pass
         if constexpr (!B_KC) {
 #pragma unroll
           for (int g = 0; g < 2; ++g) {
             const int col = n0 + g * 4 * TX + tx * 4;
-            if (col < p.n) {  // n is a multiple of 4 here: the whole group is inside
+            if ((unsigned)col < (unsigned)p.n) {  // n is a multiple of 4 here: the whole group is inside
               vec4 v;
 #pragma unroll
               for (int c = 0; c < 4; ++c) v[c] = acc[i][g * 4 + c];
@@ -485,7 +533,7 @@ struct DirectTile {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int col = n0 + own<true, TX>(j, tx);
-            if (col < p.n) {
+            if ((unsigned)col < (unsigned)p.n) {
               T v = acc[i][j];
               if (!partial) {
                 v = Op<MUL>::apply(e.alpha, v);
