@@ -33,13 +33,53 @@ FP32_VECTOR_PEAK = 157.3   # TFLOP/s, FMA counted as 2 flops (also the fp32 matr
 FP64_VECTOR_PEAK = 78.6    # also the fp64 matrix-core peak
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script (profiles/ holds the summaries and the commands); FETCH_SIZE is scaled by 2.0, the
-# factor by which it under-reports a plain device copy of known size, WRITE_SIZE by 1.0.
-MEASURED_TRAFFIC_BYTES = {
-    # direct-to-LDS tile: 2.0 * 403 136 KiB fetched + 77 824 KiB written (268.4 MB algorithmic)
-    ("apsp", 4096, 4096, 4096): (2 * 403136 + 77824) * 1024,
-}
+# HBM bytes per launch of the dominant kernel come from profiles/traffic.json, which the profiling
+# run writes (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads for
+# a plain copy of known size): {"<workload>:<m>x<n>x<k>": {"bytes": ..., "kernel": ..., "commit": ...}}.
+# An entry is used only for the kernel family it was measured on.
+def measured_traffic(workload, m, n, k, family):
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            e = json.load(f).get(f"{workload}:{m}x{n}x{k}")
+    except (OSError, ValueError):
+        return None
+    if not e or e.get("kernel_family") != family:
+        return None
+    return e
+
+
+def settle(step, torch, min_ms=200.0, cap_ms=1500.0):
+    """Launch until the clock has settled: at least min_ms of GPU time and three consecutive launches
+    within 1 % of each other (the engine clock ramps over the first tens of milliseconds of load)."""
+    total, last = 0.0, []
+    i = 0
+    while total < cap_ms:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step(i)
+        e1.record()
+        e1.synchronize()
+        ms = e0.elapsed_time(e1)
+        total += ms
+        last = (last + [ms])[-3:]
+        i += 1
+        if total >= min_ms and len(last) == 3 and max(last) <= 1.01 * min(last):
+            break
+    return i
+
+
+def timed(step, steps, torch):
+    """steps launches, HIP events on the launch stream around each: (wall seconds, [ms per launch])."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        step(i)
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
 
 
 def build_workload(args, np, torch, cuasr_amd, inputs):
@@ -60,11 +100,14 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         d_in = col_major(D0)
         bufs = [torch.empty(n, n, device=dev).t() for _ in range(2)]
         state = {"cur": d_in}
+        squarings = max(1, int(np.ceil(np.log2(n))))
 
         def reset():
             state["cur"] = d_in
 
         def step(i):
+            if i % squarings == 0:   # a new job: the timed steps are whole runs of log2(n) squarings of the input graph
+                state["cur"] = d_in
             dst = bufs[i & 1]
             cuasr_amd.srgemm("minimum", "plus", state["cur"], state["cur"], state["cur"], dst, 0.0, 0.0, inf, 0.0,
                              kernel=args.kernel)
@@ -74,7 +117,8 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         return dict(step=step, reset=reset, state=state, m=n, n=n, k=n, dtype="f32", desc=desc, host=(D0,),
                     metric=f"fp32 min-plus SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"APSP repeated-squaring step, min-plus SRGEMM fp32, M=N=K={n}, column-major, "
-                             "D_out = min(D, D (x) D), 10% edges U[1,100), rest +inf, alpha=beta=0.0f (semiring one)",
+                             "D_out = min(D, D (x) D), 10% edges U[1,100), rest +inf, alpha=beta=0.0f (semiring one); "
+                             f"consecutive steps square the previous result, a new job from the input graph every {squarings} steps",
                     bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5)
 
     if w in ("maxplus_f64", "maxmin_f64"):
@@ -92,6 +136,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
 
         desc = cuasr_amd.make_desc(add, mult, "f64", dA, dB, dC, dD, one, one, -inf, one)
         return dict(step=step, m=n, n=n, k=n, dtype="f64", desc=desc, host=(add, mult, A, B, C, one, one, -np.inf),
+                    result=lambda: dD.cpu().numpy(),
                     metric=f"fp64 {add[:3]}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"fp64 {add}-{mult} SRGEMM, M=N=K={n}, column-major, U[-1,1), beta = one with a seeded C",
                     bound="valu", peak=FP64_VECTOR_PEAK, instr_per_term=2.0)
@@ -111,8 +156,17 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         def step(i):
             run("minimum", "plus", dA, dB, dC, dD, args.slices, ws, 0.0, 0.0, inf, 0.0)
 
+        import ctypes
+        rdesc = cuasr_amd.make_desc("minimum", "plus", "f32", dA, dB, dC, dD, 0.0, 0.0, inf, 0.0, args.slices)
+
+        def reduce_step(i):   # the reduction kernel alone, on the partial tiles the last step left in the workspace
+            st = cuasr_amd.load().cuasr_amd_reduce_splitk(ctypes.byref(rdesc), ctypes.c_void_p(ws.data_ptr()),
+                                                          ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+            assert st == 0, st
+
         form = "serial-form split-K (ordered chain of epilogues)" if args.serial else "split-K"
         return dict(step=step, m=m, n=n, k=k, dtype="f32", desc=None, host=("minimum", "plus", A, B, C, 0.0, 0.0, np.inf),
+                    result=lambda: dD.cpu().numpy(), reduce_step=reduce_step,
                     metric=f"fp32 min-plus {form} SRGEMM GOPS at {m}x{n}x{k}, {args.slices} slices (2 ops/term)",
                     workload=f"{form} min-plus SRGEMM fp32, M=N={m}, K={k}, K contiguous in A and B, U[0,10), "
                              f"{args.slices} slices: partial tiles to a workspace, then a reduction kernel",
@@ -130,6 +184,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
 
         desc = cuasr_amd.make_desc("bit_xor", "bit_and", "u32", dA, dB, dC, dD, 0xFFFFFFFF, 0, 0, 0xFFFFFFFF)
         return dict(step=step, m=n, n=n, k=n, dtype="u32", desc=desc, host=("bit_xor", "bit_and", A, B, C, 0xFFFFFFFF, 0, 0),
+                    result=lambda: dD.cpu().numpy(),
                     metric=f"uint32 xor-and SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"GF(2) xor-and SRGEMM on bit-packed uint32 words, M=N=K={n}, column-major, random words",
                     bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.0)  # one v_bitop3_b32 per term
@@ -146,6 +201,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
 
         desc = cuasr_amd.make_desc("plus", "multiplies", "f32", dA, dB, dC, dD, 1.0, 0.0, 0.0, 1.0)
         return dict(step=step, m=n, n=n, k=n, dtype="f32", desc=desc, host=("plus", "multiplies", A, B, C, 1.0, 0.0, 0.0),
+                    result=lambda: dD.cpu().numpy(),
                     metric=f"fp32 plus-times SRGEMM GFLOP/s at {n}^3 (2 flops/term)",
                     workload=f"plus-times SRGEMM fp32 on the matrix cores, M=N=K={n}, column-major, N(0,1), C = 0",
                     bound="mfma", peak=FP32_VECTOR_PEAK, instr_per_term=None)
@@ -247,6 +303,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one)
         matrix = add == "plus" and mult == "multiplies" and dt in ("f32", "f64")
         return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=desc, host=(add, mult, A, B, C, one, one, ident),
+                    result=lambda: dD.cpu().numpy(),
                     metric=f"{dt} {add}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"{add}-{mult} SRGEMM {dt}, M=N=K={n}, layouts (A, B, C) = {args.layouts} "
                              "(c = column-major, r = row-major), beta = one with a seeded C",
@@ -254,6 +311,104 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
                     instr_per_term=None)
 
     raise SystemExit(f"bench.py: unknown workload {w!r}")
+
+
+def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
+    """The other BASELINE configs, timed in the same process (a few launches each) and checked against the
+    oracle on a sample: [{workload, ms, tops, frac, kernel_family, bit_exact | within_tolerance}]."""
+    out = []
+
+    def ns(**kw):
+        a = argparse.Namespace(**vars(base_args))
+        a.kernel, a.size, a.serial = "auto", 0, False
+        for k, v in kw.items():
+            setattr(a, k, v)
+        return a
+
+    def family_of(wl, fallback):
+        if wl["desc"] is None:
+            return fallback
+        return (cuasr_amd.load().cuasr_amd_selected_kernel(wl["desc"]) or b"?").decode()
+
+    def measure(wl, budget_ms=60.0):
+        step = wl["step"]
+        for i in range(3):
+            step(i)
+        _, first = timed(step, 2, torch)
+        steps = int(max(3, min(300, budget_ms / max(min(first), 1e-3))))
+        _, ms = timed(step, steps, torch)
+        return sum(ms) / len(ms), steps
+
+    def entry(wl, ms, steps, family, **check):
+        tops = 2.0 * wl["m"] * wl["n"] * wl["k"] / (ms * 1e-3) / 1e12
+        e = {"workload": wl["workload"], "ms": round(ms, 4), "launches": steps, "tops": round(tops, 2),
+             "frac": round(tops / wl["peak"], 4), "peak": wl["peak"], "bound": wl["bound"], "kernel_family": family}
+        e.update(check)
+        return e
+
+    def rows_of(X, rows):
+        return np.ascontiguousarray(X[:rows]) if X.flags.c_contiguous else np.asfortranarray(X[:rows])
+
+    # C1: min-plus f32 1024^3, column-major (the srgemm workload: beta = one with a seeded C)
+    wl = build_workload(ns(workload="srgemm", add="minimum", mult="plus", dtype="f32", layouts="ccc", size=1024), np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    wl["step"](0)
+    torch.cuda.synchronize()
+    want = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident)
+    out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(wl["result"]().tobytes() == np.ascontiguousarray(want).tobytes())))
+
+    # C3: fp64 max-plus and max-min 8192^3; a 512 x 512 block against the oracle
+    for w in ("maxplus_f64", "maxmin_f64"):
+        wl = build_workload(ns(workload=w), np, torch, cuasr_amd, inputs)
+        ms, steps = measure(wl, 150.0)
+        add, mult, A, B, C, alpha, beta, ident = wl["host"]
+        r0, c0 = 3 * 512 + 17, 9 * 512 + 5
+        want = oracle.srgemm(add, mult, np.asfortranarray(A[r0:r0 + 512, :]), np.asfortranarray(B[:, c0:c0 + 512]),
+                             np.asfortranarray(C[r0:r0 + 512, c0:c0 + 512]), alpha, beta, ident)
+        got = wl["result"]()[r0:r0 + 512, c0:c0 + 512]
+        out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(np.asfortranarray(got).tobytes() == np.asfortranarray(want).tobytes()),
+                         checked="512 x 512 block of the output"))
+        del wl
+        torch.cuda.empty_cache()
+
+    # C4: split-K 256 x 256 x 65536, 8 and 64 slices; the reduction kernel on its own as well
+    want = None
+    for slices in (8, 64):
+        wl = build_workload(ns(workload="splitk", slices=slices), np, torch, cuasr_amd, inputs)
+        ms, steps = measure(wl)
+        add, mult, A, B, C, alpha, beta, ident = wl["host"]
+        if want is None:
+            want = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident)
+        red_step = wl["reduce_step"]
+        _, rms = timed(red_step, 50, torch)
+        rms = sorted(rms)[len(rms) // 2]
+        red_bytes = (slices + 2) * wl["m"] * wl["n"] * 4      # S partial tiles + C read, D written
+        out.append(entry(wl, ms, steps, "valu (64x64x32 staged tile) + reduce_splitk_kernel",
+                         bit_exact=bool(wl["result"]().tobytes() == np.ascontiguousarray(want).tobytes()),
+                         split_k_slices=slices, reduce_kernel_ms=round(rms, 5), reduce_kernel_bytes=red_bytes,
+                         reduce_kernel_gbs=round(red_bytes / (rms * 1e-3) / 1e9, 1),
+                         reduce_note="partial tiles of this size stay in the last-level caches: an effective rate, not an HBM rate"))
+
+    # C5a: xor-and on bit-packed uint32 words, 4096^3; the first 256 rows against the oracle
+    wl = build_workload(ns(workload="xorand_u32"), np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    want = oracle.srgemm(add, mult, rows_of(A, 256), B, rows_of(C, 256), alpha, beta, ident)
+    got = wl["result"]().view(np.uint32)[:256]
+    out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(np.asfortranarray(got).tobytes() == np.asfortranarray(want).tobytes()),
+                     checked="first 256 rows of the output"))
+
+    # C5b: plus-times f32 on the matrix cores, 4096^3; |d - r| <= 1e-5 * sum |a||b| on the first 256 rows
+    wl = build_workload(ns(workload="plustimes_f32"), np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    want = oracle.srgemm(add, mult, rows_of(A, 256), B, rows_of(C, 256), alpha, beta, ident).astype(np.float64)
+    bound = 1e-5 * (np.abs(A[:256]).astype(np.float64) @ np.abs(B).astype(np.float64))
+    got = wl["result"]()[:256].astype(np.float64)
+    out.append(entry(wl, ms, steps, family_of(wl, "?"), within_tolerance=bool((np.abs(got - want) <= bound).all()),
+                     tolerance="|d - r| <= 1e-5 * sum_k |a||b|, first 256 rows"))
+    return out
 
 
 def main():
@@ -273,6 +428,7 @@ def main():
     ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="headline only: do not time the other configs (extra.configs)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="also run one plain device copy of this many MiB (a known-size kernel "
                          "to scale rocprofv3 FETCH_SIZE / WRITE_SIZE readings by)")
@@ -295,21 +451,13 @@ def main():
     step = wl["step"]
     m, n, k = wl["m"], wl["n"], wl["k"]
 
+    settled = settle(step, torch)      # whatever --warmup says: a short warm-up must not time the clock ramp
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
     if "reset" in wl:
         wl["reset"]()
-    # HIP events on the stream the kernels are launched on (torch's current stream)
-    ev = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    ev[0].record()
-    for i in range(args.steps):
-        step(i)
-        ev[i + 1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    kernel_ms = [ev[i].elapsed_time(ev[i + 1]) for i in range(args.steps)]
+    wall, kernel_ms = timed(step, args.steps, torch)
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
     ops = 2.0 * m * n * k
     value = ops * args.steps / wall / 1e9
@@ -328,11 +476,15 @@ def main():
     roof = {
         "bound": wl["bound"], "achieved": round(achieved_tops, 3), "peak": wl["peak"], "unit": "TFLOP/s",
         "frac": round(achieved_tops / wl["peak"], 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get((args.workload, m, n, k)),
+        "traffic": None,
         "kernel_ms_avg": round(avg_kernel_ms, 4), "kernel_ms_min": round(min(kernel_ms), 4),
         "note": "achieved = 2*M*N*K per launch / mean launch duration (HIP events on the launch stream); "
                 "peak = published vector / matrix peak of the element type (FMA = 2 flops).",
     }
+    traffic = measured_traffic(args.workload, m, n, k, family)
+    if traffic:
+        roof["traffic"] = traffic["bytes"]
+        roof["traffic_source"] = f"profiles/traffic.json: {traffic.get('kernel', '?')} at commit {traffic.get('commit', '?')}"
     if wl["instr_per_term"]:
         # a semiring term that needs i vector instructions for its 2 ops cannot beat peak / i
         ceiling = wl["peak"] / wl["instr_per_term"]
@@ -342,7 +494,7 @@ def main():
                         "semiring_ceiling = peak / that."
     out = {
         "metric": wl["metric"], "value": round(value, 1), "unit": "GOPS", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
+        "warmup": args.warmup, "settle_launches": settled, "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": wl["dtype"], "data": "synthetic",
         "config": {"workload": wl["workload"], "m": m, "n": n, "k": k, "kernel_family": family},
         "roofline": roof,
@@ -429,6 +581,13 @@ def main():
                 "sample": f"the first {rows} rows of the output ({rows} x {n} x {k}), {cpu_s:.2f} s wall on "
                           f"{threads} OpenMP threads",
             }
+    if args.workload == "apsp" and not args.size and not args.no_extra and args.kernel == "auto":
+        import oracle
+        del wl
+        torch.cuda.empty_cache()
+        out["extra"] = {"configs": extra_configs(np, torch, cuasr_amd, inputs, oracle, args),
+                        "note": "the other BASELINE configs at full size, same process, mean launch time by HIP events; "
+                                "frac = tops / peak of the element type's vector (valu) or matrix (mfma) unit"}
     print(json.dumps(out), flush=True)
 
 

@@ -86,6 +86,8 @@ def load():
         lib.cuasr_amd_splitk_workspace_bytes.argtypes = [ctypes.POINTER(SrgemmDesc)]
         lib.cuasr_amd_srgemm_splitk.restype = ctypes.c_int
         lib.cuasr_amd_srgemm_splitk.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_reduce_splitk.restype = ctypes.c_int
+        lib.cuasr_amd_reduce_splitk.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p, ctypes.c_void_p]
         lib.cuasr_amd_srgemm_splitk_static.restype = ctypes.c_int
         lib.cuasr_amd_srgemm_splitk_static.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_void_p]
         lib.cuasr_amd_splitk_serial_workspace_bytes.restype = ctypes.c_size_t

@@ -326,7 +326,8 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
 
 // Both split-K forms: partial products of the K-slices into the workspace, then one
 // reduction kernel (`serial` picks the ordered replay of the serial form's epilogues).
-static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream, bool serial) {
+// `stages`: 1 = the slice kernel, 2 = the reduction kernel, 3 = both.
+static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream, bool serial, int stages = 3) {
   const int st = validate(desc, true);
   if (st != CUASR_AMD_SUCCESS) return st;
   if (!workspace) return CUASR_AMD_ERROR_WORKSPACE_NULL;
@@ -355,12 +356,17 @@ static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *
   const launch_fn red = serial ? find_reduce_serial(desc->dtype) : find_reduce(desc->dtype);
   if (!fn || !red) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
-  return red(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+  if ((stages & 1) && fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+  if ((stages & 2) && red(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+  return CUASR_AMD_SUCCESS;
 }
 
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
   return run_splitk(desc, workspace, stream, false);
+}
+
+int cuasr_amd_reduce_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream) {
+  return run_splitk(desc, workspace, stream, false, 2);
 }
 
 // ---- split-K for callers that cannot allocate: the workspace is a fixed array in the library's

@@ -179,6 +179,16 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
 int cuasr_amd_srgemm_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace,
                             void *stream);
 
+/* The second kernel of the parallel split-K on its own (reduction::kernel::ReduceSplitK,
+ * include/cuasr/reduction/kernel/reduce_split_k.h:56-238, which the reference launches
+ * at device/srgemm_splitk_parallel.h:348): folds the `split_k_slices` partial tiles
+ * that a slice kernel left in `workspace` (slice z at workspace + z * m * n elements,
+ * row-major in the orientation the slice kernel wrote them) with the semiring's add,
+ * slice 0 first, and applies the epilogue D = add(mult(alpha, acc), mult(beta, C)).
+ * For callers that produce or keep the partial tiles themselves, and for timing the
+ * reduction alone.  Arguments and errors as cuasr_amd_srgemm_splitk. */
+int cuasr_amd_reduce_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *stream);
+
 /* Split-K for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart
  * in the reference, whose split-K always takes the caller's workspace

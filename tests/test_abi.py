@@ -23,7 +23,7 @@ def test_exports_match_header(lib):
             "cuasr_amd_srgemm_can_implement", "cuasr_amd_srgemm_splitk_serial",
             "cuasr_amd_splitk_serial_workspace_bytes", "cuasr_amd_fwgemm", "cuasr_amd_apsp_squaring",
             "cuasr_amd_apsp_workspace_bytes", "cuasr_amd_apsp_blocked", "cuasr_amd_apsp_blocked_workspace_bytes",
-            "cuasr_amd_srgemm_batched", "cuasr_amd_srgemm_splitk_static"} <= set(names)
+            "cuasr_amd_srgemm_batched", "cuasr_amd_srgemm_splitk_static", "cuasr_amd_reduce_splitk"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
     assert lib.cuasr_amd_abi_version() == 1
@@ -100,6 +100,10 @@ def test_splitk_host_errors(lib):
     assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d), None, None) == 6
     d0 = desc(slices=0)
     assert lib.cuasr_amd_srgemm_splitk(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
+    # the reduction kernel on its own checks its arguments the same way
+    assert lib.cuasr_amd_reduce_splitk(ctypes.byref(d), None, None) == 6
+    assert lib.cuasr_amd_reduce_splitk(ctypes.byref(d0), ctypes.c_void_p(0x1000), None) == 4
+    assert lib.cuasr_amd_reduce_splitk(ctypes.byref(d), ctypes.c_void_p(0x1002), None) == 1
     # the plain entry point refuses split-K descriptors without launching
     assert lib.cuasr_amd_srgemm(ctypes.byref(d), None) == 4
 

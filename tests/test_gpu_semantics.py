@@ -194,3 +194,34 @@ def test_splitk_workspace_aligned_to_the_element_only(oracle, lib, dtype, serial
             0.0, 0.0, float("inf"), 0.0, dtype=dtype)
         torch.cuda.synchronize()
         assert_same_bits(to_host(dD, dtype), want, f"{dtype} workspace offset {offset}")
+
+
+def test_reduction_kernel_on_its_own(oracle, lib):
+    """cuasr_amd_reduce_splitk folds partial tiles that are already in the workspace: after a split-K call it
+    reproduces that call's output into another D, and on hand-made partial tiles it gives their fold
+    (reduction/kernel/reduce_split_k.h:162-227: slices in ascending order, then the epilogue with C)."""
+    import ctypes
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    m, n, k, slices = 200, 120, 1040, 5
+    A = inputs.uniform(71, m, k, 0.0, 10.0, np.float32, "C")
+    B = inputs.uniform(72, k, n, 0.0, 10.0, np.float32, "C")
+    C = inputs.uniform(73, m, n, 0.0, 10.0, np.float32, "C")
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    ws = torch.empty(slices * m * n, dtype=torch.float32, device="cuda")
+    d1, d2 = to_device(np.zeros_like(C)), to_device(np.zeros_like(C))
+    cuasr_amd.srgemm_splitk("minimum", "plus", dA, dB, dC, d1, slices, ws, 0.0, 0.0, float("inf"), 0.0)
+    desc = cuasr_amd.make_desc("minimum", "plus", "f32", dA, dB, dC, d2, 0.0, 0.0, float("inf"), 0.0, slices)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert lib.cuasr_amd_reduce_splitk(ctypes.byref(desc), ctypes.c_void_p(ws.data_ptr()), stream) == 0
+    torch.cuda.synchronize()
+    want = oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf)
+    assert_same_bits(to_host(d1, "f32"), want, "split-K")
+    assert_same_bits(to_host(d2, "f32"), want, "reduction alone")
+    # hand-made partial tiles (row-major output: slice z at ws + z * m * n): D = min(min_z partial_z, C)
+    parts = np.stack([inputs.uniform(80 + z, m, n, 0.0, 10.0, np.float32, "C") for z in range(slices)])
+    ws.copy_(torch.from_numpy(parts.reshape(-1)).cuda())
+    assert lib.cuasr_amd_reduce_splitk(ctypes.byref(desc), ctypes.c_void_p(ws.data_ptr()), stream) == 0
+    torch.cuda.synchronize()
+    assert_same_bits(to_host(d2, "f32"), np.minimum(parts.min(axis=0), C), "hand-made partial tiles")
