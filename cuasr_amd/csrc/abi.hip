@@ -164,13 +164,14 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   const long long rounds = (direct_groups + slots - 1) / slots;
   const bool fills = direct_groups * 8 >= rounds * slots * 7;  // >= 7/8 of its rounds
   const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;
-  // min-max / max-min on 4-byte types: `v_min_f32` / `v_max_f32` do not dual-issue, the arithmetic is 60 % slower than
-  // min-plus and the staged tile's two fragment sets cover it slightly better (47.6 vs 46.1 TOPS at 4096^3)
-  const bool minmax = !f64 && ((d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum));
   // or-and: the staged tile turns its panels into masks on their way to LDS and spends one
   // `acc | (a & b)` per term; the direct tile cannot (its panels never pass through registers)
   const bool masked = d->add_op == kLogicalOr && d->mult_op == kLogicalAnd;
-  if (direct_usable(d) && ((fills && !((minmax || masked) && have_valu)) || !have_valu)) return kDirect;
+  // both operands k-contiguous, 4-byte types: the direct tile has no hand-scheduled loop for that pair of
+  // panel forms (two k-quad operands do not fit 128 registers) and its 2-wave variant is slower than the
+  // staged tile (4096^3 min-plus: 70.4 against 72.9 TOPS)
+  const bool both_kc = !f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
+  if (direct_usable(d) && ((fills && !((both_kc || masked) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
   return kNaive;
@@ -186,9 +187,9 @@ static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO || d->split_k_slices != 1 || !direct_usable(d)) return none;
   if (!find_valu(d->dtype, d->add_op, d->mult_op)) return none;
   const bool f64 = d->dtype == CUASR_AMD_F64;
-  // min-max / max-min on 4-byte types and or-and prefer the staged tile at any size (pick_family)
-  const bool f32_minmax = !f64 && ((d->add_op == kMaximum && d->mult_op == kMinimum) || (d->add_op == kMinimum && d->mult_op == kMaximum));
-  if (f32_minmax || (d->add_op == kLogicalOr && d->mult_op == kLogicalAnd)) return none;
+  // or-and and 4-byte operands that are both k-contiguous prefer the staged tile at any size (pick_family)
+  if (d->add_op == kLogicalOr && d->mult_op == kLogicalAnd) return none;
+  if (!f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) return none;
   const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;
   const int tile_n = f64 ? 64 : 128;
   const long long slots = f64 ? 768 : 512;

@@ -4,6 +4,10 @@
 //
 //   AsmLoop<T, ADD, MUL, A_KC, B_KC>::type   the loop for that element type, semiring and pair of
 //                                            panel forms, or void where there is none
+//
+// The operators are those of semiring.h: floating-point minimum / maximum are the hardware instructions
+// (the data is free of NaN and of -0, the same contract as the compiled tiles), sums and products are
+// single rounded operations (no fused multiply-add), and plus-times adds its products in ascending k.
 #pragma once
 #include "semiring.h"
 
@@ -19,32 +23,106 @@ struct AsmRegs {
   asm_v16 frag[3];
 };
 
-#define CUASR_MUL2_ADD3(MULOP, ADD3OP, acc, t0, t1, q0, p0, q1, p1)                                           \
-  MULOP " " t0 ", " q0 ", " p0 "\n" MULOP " " t1 ", " q1 ", " p1 "\n" ADD3OP " " acc ", " acc ", " t0 ", " t1 "\n"
-#define CUASR_BITOP3(TABLE, acc, t0, t1, q0, p0, q1, p1)                                                      \
-  "v_bitop3_b32 " acc ", " q0 ", " p0 ", " acc " bitop3:" TABLE "\nv_bitop3_b32 " acc ", " q1 ", " p1 ", " acc " bitop3:" TABLE "\n"
+template <typename T, int ADD, int MUL, bool A_KC, bool B_KC> struct AsmLoop { typedef void type; };
 
-// ---- one struct per (semiring, pair of panel forms)
-#define CUASR_ASM_FORMS(NAME)                                 \
-  CUASR_ASM_ONE(NAME##_kx, "gen/direct_asm_kx_prime.inc", "gen/direct_asm_kx_tile.inc") \
-  CUASR_ASM_ONE(NAME##_xx, "gen/direct_asm_xx_prime.inc", "gen/direct_asm_xx_tile.inc") \
-  CUASR_ASM_ONE(NAME##_xk, "gen/direct_asm_xk_prime.inc", "gen/direct_asm_xk_tile.inc")
+#define CUASR_ASM_CAT_(a, b) a##b
+#define CUASR_ASM_CAT(a, b) CUASR_ASM_CAT_(a, b)
+// acc <- ADD3(acc, MUL(q0, p0), MUL(q1, p1)): two products and one three-input fold
+#define CUASR_MUL2_FOLD3(MULOP, ADD3OP, acc, t0, t1, q0, p0, q1, p1) \
+  MULOP " " t0 ", " q0 ", " p0 "\n" MULOP " " t1 ", " q1 ", " p1 "\n" ADD3OP " " acc ", " acc ", " t0 ", " t1 "\n"
+// acc <- (acc + q0 * p0) + q1 * p1, every operation rounded on its own, ascending k
+#define CUASR_MUL2_ADD2(MULOP, ADDOP, acc, t0, t1, q0, p0, q1, p1) \
+  MULOP " " t0 ", " q0 ", " p0 "\n" MULOP " " t1 ", " q1 ", " p1 "\n" ADDOP " " acc ", " t0 ", " acc "\n" ADDOP " " acc ", " t1 ", " acc "\n"
+// acc <- f(q, p, acc) twice, f a three-input bit function given by its truth table
+#define CUASR_BITOP3(TABLE, acc, t0, t1, q0, p0, q1, p1) \
+  "v_bitop3_b32 " acc ", " q0 ", " p0 ", " acc " bitop3:" TABLE "\nv_bitop3_b32 " acc ", " q1 ", " p1 ", " acc " bitop3:" TABLE "\n"
+#define CUASR_ASM_SELECT(T, ADD, MUL, NAME)                                                            \
+  template <> struct AsmLoop<T, ADD, MUL, true, false> { typedef asm_loops::NAME##_kx type; };        \
+  template <> struct AsmLoop<T, ADD, MUL, false, false> { typedef asm_loops::NAME##_xx type; };       \
+  template <> struct AsmLoop<T, ADD, MUL, false, true> { typedef asm_loops::NAME##_xk type; };
 
 namespace asm_loops {
 
-#define CUASR_TERM2(acc, t0, t1, q0, p0, q1, p1) CUASR_MUL2_ADD3("v_add_f32", "v_min3_f32", acc, t0, t1, q0, p0, q1, p1)
-#define CUASR_ASM_STRUCT min_plus_f32_kx
-#define CUASR_ASM_PRIME_INC "gen/direct_asm_kx_prime.inc"
-#define CUASR_ASM_TILE_INC "gen/direct_asm_kx_tile.inc"
-#include "direct_asm_instance.h"
-#undef CUASR_ASM_STRUCT
-#undef CUASR_ASM_PRIME_INC
-#undef CUASR_ASM_TILE_INC
+#define CUASR_ASM_SEMIRING min_plus_f32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_f32", "v_min3_f32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING max_plus_f32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_f32", "v_max3_f32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING max_min_f32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_min_f32", "v_max3_f32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING min_max_f32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_max_f32", "v_min3_f32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING plus_times_f32
+#define CUASR_TERM2(...) CUASR_MUL2_ADD2("v_mul_f32", "v_add_f32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING min_plus_i32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_u32", "v_min3_i32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING max_plus_i32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_u32", "v_max3_i32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING min_plus_u32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_u32", "v_min3_u32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING max_plus_u32
+#define CUASR_TERM2(...) CUASR_MUL2_FOLD3("v_add_u32", "v_max3_u32", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING xor_and_b32   // acc ^ (q & p): table = value on q = 0xF0, p = 0xCC, acc = 0xAA
+#define CUASR_TERM2(...) CUASR_BITOP3("0x6a", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM2
+
+#define CUASR_ASM_SEMIRING or_and_b32    // acc | (q & p)
+#define CUASR_TERM2(...) CUASR_BITOP3("0xea", __VA_ARGS__)
+#include "direct_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
 #undef CUASR_TERM2
 
 }  // namespace asm_loops
 
-template <typename T, int ADD, int MUL, bool A_KC, bool B_KC> struct AsmLoop { typedef void type; };
-template <> struct AsmLoop<float, kMinimum, kPlus, true, false> { typedef asm_loops::min_plus_f32_kx type; };
+CUASR_ASM_SELECT(float, kMinimum, kPlus, min_plus_f32)
+CUASR_ASM_SELECT(float, kMaximum, kPlus, max_plus_f32)
+CUASR_ASM_SELECT(float, kMaximum, kMinimum, max_min_f32)
+CUASR_ASM_SELECT(float, kMinimum, kMaximum, min_max_f32)
+CUASR_ASM_SELECT(float, kPlus, kMultiplies, plus_times_f32)
+CUASR_ASM_SELECT(int32_t, kMinimum, kPlus, min_plus_i32)
+CUASR_ASM_SELECT(int32_t, kMaximum, kPlus, max_plus_i32)
+CUASR_ASM_SELECT(uint32_t, kMinimum, kPlus, min_plus_u32)
+CUASR_ASM_SELECT(uint32_t, kMaximum, kPlus, max_plus_u32)
+CUASR_ASM_SELECT(int32_t, kBitXor, kBitAnd, xor_and_b32)
+CUASR_ASM_SELECT(uint32_t, kBitXor, kBitAnd, xor_and_b32)
+CUASR_ASM_SELECT(int32_t, kBitOr, kBitAnd, or_and_b32)
+CUASR_ASM_SELECT(uint32_t, kBitOr, kBitAnd, or_and_b32)
 
 }  // namespace cuasr_amd

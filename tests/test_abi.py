@@ -132,6 +132,19 @@ def test_static_splitk_host_errors(lib):
     assert call(desc(m=46341, n=46341, k=8, slices=2 ** 31 - 1)) == 10   # products past 64 bits are still refused
 
 
+def test_library_sources_never_allocate():
+    """No entry point allocates or frees device memory: nothing in the library's sources names an allocating call."""
+    import glob
+    import os
+    src = os.path.join(os.path.dirname(cuasr_amd.LIB_PATH), "..", "csrc")
+    files = glob.glob(os.path.join(src, "*.hip")) + glob.glob(os.path.join(src, "*.h"))
+    assert len(files) > 10
+    for f in files:
+        text = open(f).read()
+        for word in ("hipMalloc", "hipFree", "hipHostMalloc", "hipExtMalloc", "hipMemPool", "malloc("):
+            assert word not in text, (f, word)
+
+
 def test_serial_splitk_host_errors(lib):
     # the workspace holds the slices' partial products; none is needed for a single slice (device/srgemm.h:218-234)
     assert cuasr_amd.splitk_serial_workspace_bytes(256, 256, 8, "f32") == 4 * 256 * 256 * 8
