@@ -149,17 +149,16 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
   // pipeline, so the matrix-core assisted tropical tile is no faster than the
   // vector-ALU tile; it stays selectable but is not the default.
-  // The direct-to-LDS tile is 256 x 128 (128 x 128 when both operands are k-contiguous)
-  // and the chip holds 512 of them at a time (two per compute unit); for double it is
-  // 128 x 64 and the chip holds 768.  It is the fastest family when its workgroups fill
+  // The direct-to-LDS tile is 256 x 128 (128 x 128 when both operands are k-contiguous, and
+  // for double) and the chip holds 512 of them at a time (two per compute unit).  It is the fastest family when its workgroups fill
   // whole rounds of 512; a launch that leaves much of a round empty (small or
   // awkwardly sized outputs, split-K of a small output) is better served by the
   // smaller tiles of the staged family, whose many short workgroups balance.
   const Problem c = canonical(d);
-  const bool f64 = d->dtype == CUASR_AMD_F64;  // fp64 direct tile: 128 x 64, three per compute unit
+  const bool f64 = d->dtype == CUASR_AMD_F64;  // fp64 direct tile: 128 x 128, two per compute unit like the 4-byte one
   const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
-  const int tile_n = f64 ? 64 : 128;
-  const long long slots = f64 ? 768 : 512;
+  const int tile_n = 128;
+  const long long slots = 512;
   const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + tile_n - 1) / tile_n) * d->split_k_slices;
   const long long rounds = (direct_groups + slots - 1) / slots;
   const bool fills = direct_groups * 8 >= rounds * slots * 7;  // >= 7/8 of its rounds
@@ -190,9 +189,9 @@ static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
   // or-and and 4-byte operands that are both k-contiguous prefer the staged tile at any size (pick_family)
   if (d->add_op == kLogicalOr && d->mult_op == kLogicalAnd) return none;
   if (!f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) return none;
-  const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;
-  const int tile_n = f64 ? 64 : 128;
-  const long long slots = f64 ? 768 : 512;
+  const int tile_m = f64 ? 128 : 256;
+  const int tile_n = 128;
+  const long long slots = 512;
   const int tr = c.m / tile_m, tc = c.n / tile_n;  // whole tiles only
   long long best = 0;
   Block b = none;

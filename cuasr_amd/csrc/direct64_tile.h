@@ -1,52 +1,37 @@
 // Direct-to-LDS vector-ALU SRGEMM tile for 8-byte element types on gfx950.
 //
-// The fp64 counterpart of direct_tile.h's relaxed variant (same role in the
-// reference: threadblock/srmma_pipelined.h:153-288, warp/srmma_simt.h:190-199,
-// thread/srmma_sm50.h:118-146, kernel/srgemm.h:156-321).  fp64 vector
-// instructions issue at 16 lanes per clock and there is no 3-input fp64
-// min/max, so a term costs two instructions whatever the tile; what the tile
-// can add is occupancy: the isolated 8x4 inner loop fed from LDS measures
-// 28.4 TOPS at 2 waves per SIMD, 31.7 at 3 and 33.1 at 4.  The staged tile
-// (valu_tile.h) needs ~216 registers for its staging registers, pointers and
-// LDS store addresses and stays at 2 waves.  Here panels go global -> LDS
-// without passing through registers, which leaves accumulators (64 registers),
-// two fragment sets of one k-step (2 x 24) and a handful of addresses: 3 waves.
+// Same role as direct_tile.h (in the reference: threadblock/srmma_pipelined.h:153-288,
+// warp/srmma_simt.h:190-199, thread/srmma_sm50.h:118-146, kernel/srgemm.h:156-321).  fp64 vector
+// instructions issue at 16 lanes per clock and there is no 3-input fp64 min/max, so a term costs two
+// instructions whatever the tile; what the tile can add is occupancy: an fp64 instruction issues every
+// ~4.5 cycles per SIMD at 4 waves, 4.6 at 3, 4.9 at 2 (LDS reads, waits and scalar instructions hide
+// beneath them).  Panels go global -> LDS without passing through registers, and the main loop is
+// hand-scheduled asm (direct_asm.h): accumulators (64 registers), ONE set of fragments of a k-pair (48)
+// refilled in place and four temporaries stay inside 128 registers = 4 waves per SIMD.
 //
-//   workgroup 256 threads (16 x 16), output tile 128 x 64, thread tile 8 x 4,
-//   k-tile 16, two LDS stages (48 KiB; three workgroups per compute unit).
+//   workgroup 512 threads (16 x 32), output tile 128 x 128, thread tile 8 x 4, k-tile 16,
+//   two LDS stages (64 KiB; two workgroups per compute unit = 16 waves).
 //
-// LDS forms (the image equals the lane fetch order of the 16-byte loads):
+// LDS forms (the image equals the lane fetch order of the 16-byte loads), X = 128 for both panels:
 //   x-contiguous operand: [k][X]       one 16-byte read = 2 x at one k
-//   k-contiguous operand: [k/2][X][2]  one 8-byte read  = one x at one k
-// Thread t of 16 along a panel owns, of its 8 (A) or 4 (B) rows/columns,
-//   x-contiguous: pairs  x = (i/2)*32 + 2t + i%2      k-contiguous: x = 16 i + t.
-// LDS reads are issued as asm with counted waits (see direct_tile.h for why):
-// the set for k-step s+1 is read while step s is computed.
+//   k-contiguous operand: [k/2][X][2]  one 16-byte read = both k of a pair at one x
+// Thread t of XT along a panel owns, of its 8 (A) or 4 (B) rows / columns,
+//   x-contiguous: x = (i / 2) * 2 XT + 2 t + i % 2        k-contiguous: x = XT * i + t.
 // Needs 16-byte aligned operands with even leading dimensions and extents
 // (see direct64_ok); everything else goes to the staged tile.
 #pragma once
 #include <utility>
+#include "direct_asm.h"
 #include "semiring.h"
 
 namespace cuasr_amd {
 
-template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
-struct Direct64Tile {
-  static_assert(sizeof(T) == 8, "8-byte element types only");
-  static constexpr int BM = 128, BN = 64, BK = 16, WAVES = 4, STAGES = 2;
-  // 1 KiB wave-loads per k-tile each wave issues for the A and the B panel
-  static constexpr int LA = BM * BK * 8 / 1024 / WAVES, LB = BN * BK * 8 / 1024 / WAVES;  // 4, 2
-  typedef T vec2 __attribute__((ext_vector_type(2)));
-
-  struct Smem {
-    T a[STAGES][BK * BM];
-    T b[STAGES][BK * BN];
-  };
-
-  // ---- global -> LDS.  A panel's LDS image has X*BK/2 positions of 16 bytes; a position's
-  // global address is (uniform base of this k-tile) + (per-lane byte offset, 32 bits: the host
-  // checks that a tile spans less than 2 GiB).  Indices past the matrix edge or past the last
-  // valid k of a ragged tile are clamped to the last valid vector (never used).
+// what the tile shares with nothing else: the global -> LDS addressing and the tile order
+struct Direct64Base {
+  // A panel's LDS image has X * 16 / 2 positions of 16 bytes; a position's global address is
+  // (uniform base of this k-tile) + (per-lane byte offset, 32 bits: the host checks that a tile
+  // spans less than 2 GiB).  Indices past the matrix edge or past the last valid k of a ragged
+  // tile are clamped to the last valid vector (never used).
   template <bool KC, int X>
   static __device__ __forceinline__ unsigned tile_offset(int pos, long long s_x, unsigned s_k_bytes, int x0, int x_end, int kcount) {
     if constexpr (KC) {
@@ -57,98 +42,10 @@ struct Direct64Tile {
       return (unsigned)x * 8u + (unsigned)k * s_k_bytes;
     }
   }
-  static __device__ __forceinline__ void dma16(const char *src, T *lds_wave_base) {
+  template <typename T> static __device__ __forceinline__ void dma16(const char *src, T *lds_wave_base) {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
                                      (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
   }
-
-  // ---- LDS -> registers: the fragments of one k-step.
-  template <bool KC, int N, int DUMMY = 0> struct Frag;
-  template <int N, int DUMMY> struct Frag<true, N, DUMMY> {
-    T v[N];
-    __device__ __forceinline__ T get(int i) const { return v[i]; }
-  };
-  template <int N, int DUMMY> struct Frag<false, N, DUMMY> {
-    vec2 v[N / 2];
-    __device__ __forceinline__ T get(int i) const { return v[i >> 1][i & 1]; }
-  };
-  typedef Frag<A_KC, 8> FragA;
-  typedef Frag<B_KC, 4> FragB;
-  template <bool KC, int N> static constexpr int reads() { return KC ? N : N / 2; }
-
-  // `addr` is the lane's LDS byte address of (stage, k 0, its first x); X the panel width
-  template <int X, int K, int I, int N> static __device__ __forceinline__ void read_one(Frag<true, N> &f, unsigned addr) {
-    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(f.v[I]) : "v"(addr), "n"(((K >> 1) * X + I * 16) * 16 + (K & 1) * 8));
-  }
-  template <int X, int K, int I, int N> static __device__ __forceinline__ void read_one(Frag<false, N> &f, unsigned addr) {
-    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f.v[I]) : "v"(addr), "n"((K * X + I * 32) * 8));
-  }
-  template <int X, int K, bool KC, int N, int... I>
-  static __device__ __forceinline__ void read_all(Frag<KC, N> &f, unsigned addr, std::integer_sequence<int, I...>) {
-    (read_one<X, K, I>(f, addr), ...);
-  }
-  template <int X, int K, bool KC, int N> static __device__ __forceinline__ void read_frag(Frag<KC, N> &f, unsigned addr) {
-    read_all<X, K>(f, addr, std::make_integer_sequence<int, reads<KC, N>()>{});
-  }
-  // wait until at most CNT LDS reads are in flight; the fragments named become valid
-  template <int CNT> static __device__ __forceinline__ void wait(Frag<true, 8> &f) {
-    asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(f.v[0]), "+v"(f.v[1]), "+v"(f.v[2]), "+v"(f.v[3]), "+v"(f.v[4]), "+v"(f.v[5]), "+v"(f.v[6]), "+v"(f.v[7]) : "n"(CNT));
-  }
-  template <int CNT> static __device__ __forceinline__ void wait(Frag<false, 8> &f) {
-    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f.v[0]), "+v"(f.v[1]), "+v"(f.v[2]), "+v"(f.v[3]) : "n"(CNT));
-  }
-  template <int CNT> static __device__ __forceinline__ void wait(Frag<true, 4> &f) {
-    asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(f.v[0]), "+v"(f.v[1]), "+v"(f.v[2]), "+v"(f.v[3]) : "n"(CNT));
-  }
-  template <int CNT> static __device__ __forceinline__ void wait(Frag<false, 4> &f) {
-    asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(f.v[0]), "+v"(f.v[1]) : "n"(CNT));
-  }
-
-  // tile-local index of the thread's i-th row / column
-  template <bool KC> static __device__ __forceinline__ int own(int i, int t) {
-    return KC ? i * 16 + t : (i >> 1) * 32 + t * 2 + (i & 1);
-  }
-  // the same fragments for a single k through ordinary loads (ragged last k-tile: nothing is in flight by then)
-  template <bool KC, int N, int X> static __device__ __forceinline__ void load_frag1(T (&f)[N], const T *panel, int kk, int t) {
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int x = own<KC>(i, t);
-      f[i] = KC ? panel[((kk >> 1) * X + x) * 2 + (kk & 1)] : panel[kk * X + x];
-    }
-  }
-
-  static __device__ __forceinline__ void compute(T (&acc)[8][4], const FragA &a, const FragB &b) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = fold<ADD, MUL>(Op<MUL>::apply(a.get(i), b.get(j)), acc[i][j]);
-      // pin the row: computed here, not later (only naming it in a volatile statement keeps it from drifting)
-      asm volatile("" : "+v"(acc[i][0]), "+v"(acc[i][1]), "+v"(acc[i][2]), "+v"(acc[i][3]));
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  }
-  template <int K> static __device__ __forceinline__ void kstep(T (&acc)[8][4], FragA (&a)[2], FragB (&b)[2], unsigned a_addr, unsigned b_addr) {
-    constexpr int CUR = K & 1, NXT = CUR ^ 1;
-    constexpr int READS = reads<A_KC, 8>() + reads<B_KC, 4>();  // at most 12: fits the 4-bit counter
-    if constexpr (K + 1 < BK) {
-      read_frag<BM, K + 1>(a[NXT], a_addr);
-      read_frag<BN, K + 1>(b[NXT], b_addr);
-      wait<READS>(a[CUR]);  // the reads just issued may stay in flight, everything older has landed
-      wait<READS>(b[CUR]);
-    } else {
-      wait<0>(a[CUR]);
-      wait<0>(b[CUR]);
-    }
-    compute(acc, a[CUR], b[CUR]);
-  }
-  template <int... K>
-  static __device__ __forceinline__ void whole_tile(std::integer_sequence<int, K...>, T (&acc)[8][4], FragA (&a)[2], FragB (&b)[2],
-                                                   unsigned a_addr, unsigned b_addr) {
-    read_frag<BM, 0>(a[0], a_addr);
-    read_frag<BN, 0>(b[0], b_addr);
-    (kstep<K>(acc, a, b, a_addr, b_addr), ...);
-  }
-
   static __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int &bm, int &bn) {
     const int total = tiles_m * tiles_n;
     // consecutive workgroup ids land on consecutive XCDs (8, one L2 each):
@@ -161,12 +58,40 @@ struct Direct64Tile {
     bm = first + (id % width) % gsz;
     bn = (id % width) / gsz;
   }
+};
+
+template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
+struct Direct64Tile {
+  static_assert(sizeof(T) == 8, "8-byte element types only");
+  typedef Direct64Base Base;
+  typedef typename AsmLoop<T, ADD, MUL, A_KC, B_KC>::type Loop;
+  static constexpr int TY = 16, TX = 32, BM = 8 * TY, BN = 4 * TX, BK = 16, THREADS = TY * TX, WAVES = THREADS / 64, STAGES = 2;
+  static constexpr int LA = BM * BK * 8 / 1024 / WAVES, LB = BN * BK * 8 / 1024 / WAVES;  // 2, 2
+  static_assert(LA == 2 && LB == 2, "the generated loop moves two pieces of each panel per wave");
+  typedef T vec2 __attribute__((ext_vector_type(2)));
+
+  struct Smem {
+    T a[STAGES][BK * BM];
+    T b[STAGES][BK * BN];
+  };
+
+  template <bool KC, int XT> static __device__ __forceinline__ int own(int i, int t) {
+    return KC ? i * XT + t : (i >> 1) * 2 * XT + t * 2 + (i & 1);
+  }
+  template <bool KC, int N, int XT> static __device__ __forceinline__ void load_frag1(T (&f)[N], const T *panel, int kk, int t) {
+    constexpr int X = N * XT;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int x = own<KC, XT>(i, t);
+      f[i] = KC ? panel[((kk >> 1) * X + x) * 2 + (kk & 1)] : panel[kk * X + x];
+    }
+  }
 
   static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
-    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, tx = tid % TX, ty = tid / TX, lane = tid & 63, wave = tid >> 6;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     int bm, bn;
-    tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
+    Base::tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
     const int m0 = bm * BM, n0 = bn * BN;
     const T *A = reinterpret_cast<const T *>(p.A);
     const T *B = reinterpret_cast<const T *>(p.B);
@@ -182,23 +107,27 @@ struct Direct64Tile {
     const char *base_b = reinterpret_cast<const char *>(B + (long long)n0 * p.sb_n + (long long)kb * p.sb_k);
     const long long a_step = (long long)BK * p.sa_k * 8, b_step = (long long)BK * p.sb_k * 8;
     const unsigned a_kbytes = (unsigned)p.sa_k * 8u, b_kbytes = (unsigned)p.sb_k * 8u;
-    // k-tile with kcount valid k into an LDS stage: each wave 4 x 1 KiB of A and 2 x 1 KiB of B
+    auto off_a = [&](int q, int kcount) { return Base::template tile_offset<A_KC, BM>((wave * LA + q) * 64 + lane, p.sa_m, a_kbytes, m0, p.m, kcount); };
+    auto off_b = [&](int q, int kcount) { return Base::template tile_offset<B_KC, BN>((wave * LB + q) * 64 + lane, p.sb_n, b_kbytes, n0, p.n, kcount); };
+    // k-tile with kcount valid k into an LDS stage (compiler-issued: prologue and a ragged last tile)
     auto fetch = [&](int stage, int kcount) {
       if (kcount > 0) {
 #pragma unroll
-        for (int q = 0; q < LA; ++q) {
-          const int pos = (wave * LA + q) * 64 + lane;
-          dma16(base_a + tile_offset<A_KC, BM>(pos, p.sa_m, a_kbytes, m0, p.m, kcount), &sm.a[stage][(wave * LA + q) * 128]);
-        }
+        for (int q = 0; q < LA; ++q) Base::dma16<T>(base_a + off_a(q, kcount), &sm.a[stage][(wave * LA + q) * 128]);
 #pragma unroll
-        for (int q = 0; q < LB; ++q) {
-          const int pos = (wave * LB + q) * 64 + lane;
-          dma16(base_b + tile_offset<B_KC, BN>(pos, p.sb_n, b_kbytes, n0, p.n, kcount), &sm.b[stage][(wave * LB + q) * 128]);
-        }
+        for (int q = 0; q < LB; ++q) Base::dma16<T>(base_b + off_b(q, kcount), &sm.b[stage][(wave * LB + q) * 128]);
       }
-      base_a += a_step;
-      base_b += b_step;
     };
+
+    const int nfull = (ke - kb) / BK, rem = (ke - kb) - nfull * BK;  // whole k-tiles, then one ragged tile
+    auto tile_k = [&](int t) { return t < nfull ? BK : (t == nfull ? rem : 0); };
+    fetch(0, tile_k(0));
+    base_a += a_step;
+    base_b += b_step;
+    __syncthreads();
+    fetch(1, tile_k(1));
+    base_a += a_step;
+    base_b += b_step;  // base_a / base_b now point at tile 2
 
     T acc[8][4];
 #pragma unroll
@@ -206,31 +135,52 @@ struct Direct64Tile {
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = ident;
 
-    const int nfull = (ke - kb) / BK, rem = (ke - kb) - nfull * BK;  // whole k-tiles, then one ragged tile
-    auto tile_k = [&](int t) { return t < nfull ? BK : (t == nfull ? rem : 0); };
-    fetch(0, tile_k(0));
-    __syncthreads();
-    fetch(1, tile_k(1));
-
-    // lane's LDS byte address of (stage 0, k 0, its first x) in each panel
-    const unsigned a_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][0] + ty * 16;
-    const unsigned b_addr0 = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][0] + tx * 16;
-    FragA a[2];
-    FragB b[2];
-    for (int t = 0; t < nfull; ++t) {
-      const int stage = t & 1;
-      whole_tile(std::make_integer_sequence<int, BK>{}, acc, a, b, a_addr0 + stage * (BK * BM * 8), b_addr0 + stage * (BK * BN * 8));
-      __syncthreads();                 // tile t+1 has landed (vmcnt waited first); nobody reads this stage any more
-      fetch(stage, tile_k(t + 2));     // ... so tile t+2 may overwrite it
+    if (nfull > 0) {
+      AsmRegs r;
+      const unsigned long long ident_bits = __builtin_bit_cast(unsigned long long, ident);
+      const float ident_lo = __builtin_bit_cast(float, (unsigned)ident_bits), ident_hi = __builtin_bit_cast(float, (unsigned)(ident_bits >> 32));
+#pragma unroll
+      for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) r.acc[v][e] = (e & 1) ? ident_hi : ident_lo;
+#pragma unroll
+      for (int v = 0; v < 3; ++v) r.frag[v] = asm_v16(0.0f);
+      const unsigned oa0 = off_a(0, BK), oa1 = off_a(1, BK), ob0 = off_b(0, BK), ob1 = off_b(1, BK);
+      // LDS byte address of this wave's first piece of each panel in stage 0 (wave-uniform)
+      const unsigned m0_a0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][(wave * LA) * 128]);
+      const unsigned m0_b0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][(wave * LB) * 128]);
+      constexpr unsigned A_STAGE = BK * BM * 8, B_STAGE = BK * BN * 8;
+      unsigned a_addr = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.a[0][0] + ty * 16;
+      unsigned b_addr = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&sm.b[0][0] + tx * 16;
+      Loop::prime(r, a_addr, b_addr);
+      for (int t = 0; t < nfull; ++t) {
+        const int stage = t & 1;
+        // the statement's barrier hands stage `stage` back; the tile two ahead goes there: a whole one
+        // from inside the statement, a ragged one from here right after it
+        Loop::tile(r, a_addr, b_addr, stage ? 0u - A_STAGE : A_STAGE, stage ? 0u - B_STAGE : B_STAGE, nfull - (t + 2),
+                   m0_a0 + stage * A_STAGE, m0_b0 + stage * B_STAGE, oa0, oa1, ob0, ob1, base_a, base_b);
+        if (t + 2 == nfull) fetch(stage, rem);
+        base_a += a_step;
+        base_b += b_step;
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const unsigned lo = __builtin_bit_cast(unsigned, (float)r.acc[i >> 1][(i & 1) * 8 + 2 * j]);
+          const unsigned hi = __builtin_bit_cast(unsigned, (float)r.acc[i >> 1][(i & 1) * 8 + 2 * j + 1]);
+          acc[i][j] = __builtin_bit_cast(T, ((unsigned long long)hi << 32) | lo);
+        }
     }
     if (rem > 0) {
+      if (nfull == 0) __syncthreads();  // (with whole tiles before it, the last statement's barrier covers the ragged tile)
       const int buf = nfull & 1;
       const T *pa = sm.a[buf], *pb = sm.b[buf];
 #pragma unroll 1
       for (int kk = 0; kk < rem; ++kk) {
         T fa[8], fb[4];
-        load_frag1<A_KC, 8, BM>(fa, pa, kk, ty);
-        load_frag1<B_KC, 4, BN>(fb, pb, kk, tx);
+        load_frag1<A_KC, 8, TY>(fa, pa, kk, ty);
+        load_frag1<B_KC, 4, TX>(fb, pb, kk, tx);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
@@ -258,13 +208,13 @@ struct Direct64Tile {
     const T *C = reinterpret_cast<const T *>(p.C);
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int row = m0 + own<A_KC>(i, ty);
-      if (row < p.m) {
+      const int row = m0 + own<A_KC, TY>(i, ty);
+      if ((unsigned)row < (unsigned)p.m) {
         if constexpr (!B_KC) {
 #pragma unroll
           for (int g = 0; g < 2; ++g) {
-            const int col = n0 + g * 32 + tx * 2;
-            if (col < p.n) {  // n is even here: the pair is inside
+            const int col = n0 + g * 2 * TX + tx * 2;
+            if ((unsigned)col < (unsigned)p.n) {  // n is even here: the pair is inside
               vec2 v = {acc[i][2 * g], acc[i][2 * g + 1]};
               if (!partial) {
 #pragma unroll
@@ -281,8 +231,8 @@ struct Direct64Tile {
         } else {
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const int col = n0 + own<true>(j, tx);
-            if (col < p.n) {
+            const int col = n0 + own<true, TX>(j, tx);
+            if ((unsigned)col < (unsigned)p.n) {
               T v = acc[i][j];
               if (!partial) {
                 v = Op<MUL>::apply(e.alpha, v);
@@ -298,13 +248,8 @@ struct Direct64Tile {
   }
 };
 
-#ifndef CUASR_AMD_DIRECT64_WAVES
-#define CUASR_AMD_DIRECT64_WAVES 3
-#endif
-
 template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CUASR_AMD_DIRECT64_WAVES, CUASR_AMD_DIRECT64_WAVES)))
-void direct64_srgemm_kernel(Problem p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void direct64_srgemm_kernel(Problem p) {
   using Tile = Direct64Tile<T, ADD, MUL, A_KC, B_KC>;
   __shared__ typename Tile::Smem sm;
   Tile::run(p, sm);
@@ -333,17 +278,18 @@ static inline bool direct64_ok(const Problem &p) {
 }
 
 template <typename T, int ADD, int MUL> static hipError_t launch_direct64(const Problem &p, hipStream_t s) {
+  static_assert(!std::is_void<typename AsmLoop<T, ADD, MUL, false, false>::type>::value, "no main loop for this semiring");
   if (p.m == 0 || p.n == 0) return hipSuccess;
   if (!direct64_ok(p)) return hipErrorNotSupported;
-  const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 63) / 64);
+  const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
-  if (a_kc && b_kc) hipLaunchKernelGGL((direct64_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(256), 0, s, p);
-  else if (a_kc) hipLaunchKernelGGL((direct64_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(256), 0, s, p);
-  else if (b_kc) hipLaunchKernelGGL((direct64_srgemm_kernel<T, ADD, MUL, false, true>), grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((direct64_srgemm_kernel<T, ADD, MUL, false, false>), grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  if (a_kc && b_kc) launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(512), 0, s, p);
+  else if (a_kc) launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(512), 0, s, p);
+  else if (b_kc) launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, false, true>), grid, dim3(512), 0, s, p);
+  else launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, false, false>), grid, dim3(512), 0, s, p);
+  return take_launch_status();
 }
 
 }  // namespace cuasr_amd

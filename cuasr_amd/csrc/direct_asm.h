@@ -15,9 +15,10 @@ namespace cuasr_amd {
 
 typedef float asm_v16 __attribute__((ext_vector_type(16)));
 
-// The registers a loop lives in: acc[i / 2][(i % 2) * 8 + j] is accumulator (i, j) and sits in v(8 i + j);
-// frag is v64 .. v111, the fragments carried from one k-tile to the next.  Element types other than float
-// travel as bit patterns.
+// The registers a loop lives in.  4-byte types: acc[i / 2][(i % 2) * 8 + j] is accumulator (i, j) of the 8 x 8
+// tile and sits in v(8 i + j); 8-byte types: accumulator (i, j) of the 8 x 4 tile is the register pair
+// v[8 i + 2 j : 8 i + 2 j + 1], low word first, i.e. elements (i % 2) * 8 + 2 j and + 1 of acc[i / 2].
+// frag is v64 .. v111, the fragments carried from one k-tile to the next.  Everything travels as bit patterns.
 struct AsmRegs {
   asm_v16 acc[4];
   asm_v16 frag[3];
@@ -109,7 +110,54 @@ namespace asm_loops {
 #undef CUASR_ASM_SEMIRING
 #undef CUASR_TERM2
 
+// ---- 8-byte element types: one term at a time on register pairs (there is no three-input fp64 min / max)
+// acc <- ADD(acc, MUL(q, p))
+#define CUASR_MUL_FOLD(MULOP, ADDOP, acc, t, q, p) MULOP " " t ", " q ", " p "\n" ADDOP " " acc ", " acc ", " t "\n"
+// acc <- q * p + acc with both operations rounded, the product as the left operand like the host reference
+#define CUASR_MUL_ADD(MULOP, ADDOP, acc, t, q, p) MULOP " " t ", " q ", " p "\n" ADDOP " " acc ", " t ", " acc "\n"
+
+#define CUASR_ASM_SEMIRING min_plus_f64
+#define CUASR_TERM1(...) CUASR_MUL_FOLD("v_add_f64", "v_min_f64", __VA_ARGS__)
+#include "direct64_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM1
+
+#define CUASR_ASM_SEMIRING max_plus_f64
+#define CUASR_TERM1(...) CUASR_MUL_FOLD("v_add_f64", "v_max_f64", __VA_ARGS__)
+#include "direct64_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM1
+
+#define CUASR_ASM_SEMIRING max_min_f64
+#define CUASR_TERM1(...) CUASR_MUL_FOLD("v_min_f64", "v_max_f64", __VA_ARGS__)
+#include "direct64_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM1
+
+#define CUASR_ASM_SEMIRING min_max_f64
+#define CUASR_TERM1(...) CUASR_MUL_FOLD("v_max_f64", "v_min_f64", __VA_ARGS__)
+#include "direct64_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM1
+
+#define CUASR_ASM_SEMIRING plus_times_f64
+#define CUASR_TERM1(...) CUASR_MUL_ADD("v_mul_f64", "v_add_f64", __VA_ARGS__)
+#include "direct64_asm_forms.h"
+#undef CUASR_ASM_SEMIRING
+#undef CUASR_TERM1
+
 }  // namespace asm_loops
+
+#define CUASR_ASM_SELECT64(ADD, MUL, NAME)                                                                \
+  template <> struct AsmLoop<double, ADD, MUL, true, false> { typedef asm_loops::NAME##_kx type; };      \
+  template <> struct AsmLoop<double, ADD, MUL, false, false> { typedef asm_loops::NAME##_xx type; };     \
+  template <> struct AsmLoop<double, ADD, MUL, false, true> { typedef asm_loops::NAME##_xk type; };      \
+  template <> struct AsmLoop<double, ADD, MUL, true, true> { typedef asm_loops::NAME##_kk type; };
+CUASR_ASM_SELECT64(kMinimum, kPlus, min_plus_f64)
+CUASR_ASM_SELECT64(kMaximum, kPlus, max_plus_f64)
+CUASR_ASM_SELECT64(kMaximum, kMinimum, max_min_f64)
+CUASR_ASM_SELECT64(kMinimum, kMaximum, min_max_f64)
+CUASR_ASM_SELECT64(kPlus, kMultiplies, plus_times_f64)
 
 CUASR_ASM_SELECT(float, kMinimum, kPlus, min_plus_f32)
 CUASR_ASM_SELECT(float, kMaximum, kPlus, max_plus_f32)

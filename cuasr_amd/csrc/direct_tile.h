@@ -371,8 +371,7 @@ struct DirectTile {
       static_assert(LA == 2 && LB == 1, "the generated loop moves two pieces of A and one of B per wave");
       if (nfull > 0) {
         AsmRegs r;
-        float ident_bits;
-        __builtin_memcpy(&ident_bits, &ident, 4);
+        const float ident_bits = __builtin_bit_cast(float, ident);
 #pragma unroll
         for (int v = 0; v < 4; ++v)
 #pragma unroll
@@ -406,8 +405,7 @@ struct DirectTile {
         for (int i = 0; i < 8; ++i)
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
-            const float bits = r.acc[i >> 1][(i & 1) * 8 + j];
-            __builtin_memcpy(&acc[i][j], &bits, 4);
+            acc[i][j] = __builtin_bit_cast(T, (float)r.acc[i >> 1][(i & 1) * 8 + j]);
           }
       }
     } else if constexpr (RELAXED) {
@@ -603,11 +601,11 @@ template <typename T, int ADD, int MUL> static hipError_t launch_relaxed(const P
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
-  if (a_kc && b_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(256), 0, s, p);
-  else if (a_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(256), 0, s, p);
-  else if (b_kc) hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, false, true>), grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((relaxed_srgemm_kernel<T, ADD, MUL, false, false>), grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  if (a_kc && b_kc) launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(256), 0, s, p);
+  else if (a_kc) launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(256), 0, s, p);
+  else if (b_kc) launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, false, true>), grid, dim3(256), 0, s, p);
+  else launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, false, false>), grid, dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 template <typename T, int ADD, int MUL> static hipError_t launch_direct(const Problem &p, hipStream_t s) {
@@ -622,11 +620,11 @@ template <typename T, int ADD, int MUL> static hipError_t launch_direct(const Pr
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
-  if (a_kc && b_kc) hipLaunchKernelGGL((direct_srgemm_kernel<T, ADD, MUL, true, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
-  else if (a_kc) hipLaunchKernelGGL((direct_srgemm_kernel<T, ADD, MUL, true, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
-  else if (b_kc) hipLaunchKernelGGL((direct_srgemm_kernel<T, ADD, MUL, false, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
-  else hipLaunchKernelGGL((direct_srgemm_kernel<T, ADD, MUL, false, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
-  return hipGetLastError();
+  if (a_kc && b_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, true, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+  else if (a_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, true, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+  else if (b_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, false, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+  else launch_kernel((direct_srgemm_kernel<T, ADD, MUL, false, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+  return take_launch_status();
 }
 
 }  // namespace cuasr_amd

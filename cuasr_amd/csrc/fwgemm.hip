@@ -402,15 +402,15 @@ hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   if (g.At) {
     const bool at_aligned = reinterpret_cast<uintptr_t>(g.At) % vec == 0 && g.ldat % 4 == 0;
     if (whole && aligned && at_aligned)
-      hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, true>), grid, dim3(256), 0, stream, g);
+      launch_kernel((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, true>), grid, dim3(256), 0, stream, g);
     else
-      hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, true>), grid, dim3(256), 0, stream, g);
+      launch_kernel((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, true>), grid, dim3(256), 0, stream, g);
   } else if (whole && aligned) {
-    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, false>), grid, dim3(256), 0, stream, g);
+    launch_kernel((fwgemm_tile_kernel<T, TM, TN, SN, BK, false, false>), grid, dim3(256), 0, stream, g);
   } else {
-    hipLaunchKernelGGL((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, false>), grid, dim3(256), 0, stream, g);
+    launch_kernel((fwgemm_tile_kernel<T, TM, TN, SN, BK, true, false>), grid, dim3(256), 0, stream, g);
   }
-  return hipGetLastError();
+  return take_launch_status();
 }
 
 // src (rows x cols, column-major, leading dimension ld) -> w, a column-major copy with leading
@@ -442,9 +442,9 @@ template <typename T>
 hipError_t snapshot(const void *src, int64_t ld, void *w, int64_t ldw, void *wt, int64_t ldwt, int rows, int cols,
                     hipStream_t s) {
   const dim3 grid((rows + 63) / 64, (cols + 63) / 64);
-  hipLaunchKernelGGL(snapshot_kernel<T>, grid, dim3(256), 0, s, static_cast<const T *>(src), ld, static_cast<T *>(w), ldw,
+  launch_kernel(snapshot_kernel<T>, grid, dim3(256), 0, s, static_cast<const T *>(src), ld, static_cast<T *>(w), ldw,
                      static_cast<T *>(wt), ldwt, rows, cols);
-  return hipGetLastError();
+  return take_launch_status();
 }
 
 // two copies in one launch: the first blocks0 workgroups copy (src0 -> w0), the others (src1 -> w1)
@@ -550,8 +550,8 @@ __global__ void __launch_bounds__(1024) fw_diagonal_kernel(T *d, int64_t ld, int
 
 template <typename T> hipError_t launch_naive(const FwArgs &g, hipStream_t stream) {
   dim3 grid((g.m + 63) / 64, (g.n + 3) / 4);
-  hipLaunchKernelGGL(fwgemm_naive_kernel<T>, grid, dim3(256), 0, stream, g);
-  return hipGetLastError();
+  launch_kernel(fwgemm_naive_kernel<T>, grid, dim3(256), 0, stream, g);
+  return take_launch_status();
 }
 
 int check(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, const void *dist,
@@ -671,24 +671,24 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
     int32_t *Pkk = parent + size_t(k0) + size_t(k0) * size_t(ldp);
     // 1. the diagonal block, closed by one workgroup
     if (f64)
-      hipLaunchKernelGGL(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
+      launch_kernel(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
     else
-      hipLaunchKernelGGL(fw_diagonal_kernel<float>, dim3(1), dim3(1024), 0, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
-    if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+      launch_kernel(fw_diagonal_kernel<float>, dim3(1), dim3(1024), 0, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
+    if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     // 2. snapshots of block row and block column (the products below read these, so that no
     //    workgroup sees another's updates)
     char *Drow = D + es * size_t(k0), *Dcol = D + es * size_t(k0) * size_t(ld);
     {
       const int sb0 = ((bb + 63) / 64) * ((n + 63) / 64), sb1 = ((n + 63) / 64) * ((bb + 63) / 64);
       if (f64)
-        hipLaunchKernelGGL(snapshot_pair_kernel<double>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const double *>(Drow),
+        launch_kernel(snapshot_pair_kernel<double>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const double *>(Drow),
                            reinterpret_cast<double *>(R), int64_t(FW_BLOCK), bb, n, reinterpret_cast<const double *>(Dcol),
                            reinterpret_cast<double *>(C), nn, n, bb, ld, sb0);
       else
-        hipLaunchKernelGGL(snapshot_pair_kernel<float>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const float *>(Drow),
+        launch_kernel(snapshot_pair_kernel<float>, dim3(sb0 + sb1), dim3(256), 0, s, reinterpret_cast<const float *>(Drow),
                            reinterpret_cast<float *>(R), int64_t(FW_BLOCK), bb, n, reinterpret_cast<const float *>(Dcol),
                            reinterpret_cast<float *>(C), nn, n, bb, ld, sb0);
-      if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+      if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     }
     hipError_t e = hipSuccess;
     // 3. block row <- (closed diagonal block) x (block row); block column <- (block column) x (closed
@@ -705,9 +705,9 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
       const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
                       nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK};
       const int blocks0 = ((bb + 63) / 64) * ((n + 3) / 4), blocks1 = ((n + 63) / 64) * ((bb + 3) / 4);
-      if (f64) hipLaunchKernelGGL(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
-      else hipLaunchKernelGGL(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
-      if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+      if (f64) launch_kernel(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      else launch_kernel(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     } else {
       FwExtra xr = x, xc = x;
       xr.skip_c0 = xc.skip_r0 = k0;

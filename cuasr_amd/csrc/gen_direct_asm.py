@@ -1,24 +1,30 @@
 #!/usr/bin/env python3
-"""Generates the hand-scheduled main loop of the 4-wave direct-to-LDS SRGEMM tile
-(direct_tile.h) as inline-asm text: one k-tile (16 k) of the 8 x 8 register tile per asm
-statement, for each pair of panel forms.
+"""Generates the hand-scheduled main loops of the 4-wave direct-to-LDS SRGEMM tiles
+(direct_tile.h for 4-byte, direct64_tile.h for 8-byte element types) as inline-asm text:
+one k-tile (16 k) of the register tile per asm statement, for each pair of panel forms.
 
 Why generated asm and not C++: on gfx950 a SIMD issues about one instruction every 2.1 cycles
 whatever its kind (a satisfied s_waitcnt, an s_nop or a scalar add costs as much as a v_add_f32),
-and an LDS read costs about 5.5 cycles whatever its width.  The compiler's version of this loop
-spends 1536 vector instructions per k-tile plus 96 LDS reads, 89 waits and 76 nops; this schedule
-spends the same 1536 plus 64 LDS reads (16-byte reads only), about 20 waits and no nops.
+and an LDS read costs about 5.5 cycles whatever its width.  The compiler's version of the 4-byte
+loop spends 1536 vector instructions per k-tile plus 96 LDS reads, 89 waits and 76 nops; this
+schedule spends the same 1536 plus 64 LDS reads (16-byte reads only), about 20 waits and no nops.
+For 8-byte types (4.5 cycles per fp64 instruction, the other instructions hide beneath them) the
+gain is the register count: accumulators, ONE set of fragments refilled in place and four
+temporaries fit 128 registers, i.e. 4 waves per SIMD, where the compiled loop needs 136.
 
 Register plan (128 VGPRs, 4 waves per SIMD):
-    v0   .. v63    accumulators, acc[i][j] = v(8 i + j)      (i: A index, j: B index)
+    v0   .. v63    accumulators: 4-byte acc[i][j] = v(8 i + j), 8 x 8; 8-byte acc[i][j] = v[8 i + 2 j : +1], 8 x 4
     v64  .. v111   fragments of the operand called Q, then of the operand called P
     v112 .. v115   temporaries
-  P is an x-contiguous panel ([k][X] in LDS, one 16-byte read = 4 x at one k): 16 registers hold
-    one k-pair, refilled half by half (4 x, both k) as soon as a half's last use is over.
-  Q is either k-contiguous ([k/4][X][4] in LDS, one 16-byte read = 4 k of one x): 32 registers
-    hold a k-quad, each x refilled right after its last use in the quad's second k-pair,
-    or x-contiguous like P: 16 registers, refilled by halves.
-  A k-pair is worked in two phases, one per half of P; within a phase the 8 x of Q in order.
+  A fragment register group is refilled for its next use right after its last use, so that every
+  LDS read is issued half a k-pair or more before its data is consumed.
+  4-byte types: P is an x-contiguous panel ([k][X] in LDS, one 16-byte read = 4 x at one k): 16
+    registers hold one k-pair, refilled half by half (4 x, both k).  Q is either k-contiguous
+    ([k/4][X][4], one read = 4 k of one x): 32 registers hold a k-quad, each x refilled after its
+    last use in the quad's second k-pair; or x-contiguous like P.
+  8-byte types: Q = A (8 x), P = B (4 x), each holding one k-pair: x-contiguous ([k][X], one read =
+    2 x at one k) or k-contiguous ([k/2][X][2], one read = both k of one x).
+  A k-pair is worked in two phases, one per half of P; within a phase the x of Q in order.
 
 LDS reads complete in order, so "s_waitcnt lgkmcnt(N)" leaves the N youngest in flight.  The
 generator keeps the queue of reads in flight, emits a wait only where a fragment is consumed
@@ -27,72 +33,95 @@ and checks for every vector instruction that the registers it reads hold the ope
 it means.  A statement ends with everything drained, so no read is in flight while compiler
 code runs.
 
-Output: string-literal fragments for `asm volatile(` to include; the arithmetic of two terms
-is the macro CUASR_TERM2(acc, t0, t1, q0, p0, q1, p1) that the including code defines for its
-semiring (register names as string literals), everything else is literal text.
+Output: string-literal fragments for `asm volatile(` to include.  The arithmetic is a macro the
+including code defines for its semiring (register names as string literals):
+    4-byte: CUASR_TERM2(acc, t0, t1, q0, p0, q1, p1)   acc <- add(acc, mult(q0, p0), mult(q1, p1))
+    8-byte: CUASR_TERM1(acc, t, q, p)                  acc <- add(acc, mult(q, p))
+everything else is literal text.
 """
 import os
 import sys
 
-TY, TX, BK = 32, 16, 16
-ACC0 = 0
-FRAG0 = 64
-TEMP0 = 112  # four temporaries, v112 .. v115
-WAIT_AGE = 20   # a wait also covers reads issued at least this many two-term groups ago
+BK = 16
+ACC0, FRAG0, TEMP0 = 0, 64, 112
+WAIT_AGE = 20   # a wait also covers reads issued at least this many groups of 3-4 instructions ago
 
 
 class Panel:
-    """Fragment registers and LDS reads of one operand; xt = threads along its x (8 * xt wide)."""
+    """Fragment registers and LDS reads of one operand.
+    esize 4 or 8; nx = x per thread; xt = threads along x (the panel is nx * xt wide)."""
 
-    def __init__(self, name, kc, xt, reg0, addr):
-        self.name, self.kc, self.xt, self.reg0, self.addr = name, kc, xt, reg0, addr
-        self.nregs = 32 if kc else 16
+    def __init__(self, name, kc, esize, nx, xt, reg0, addr):
+        self.name, self.kc, self.esize, self.nx, self.xt, self.reg0, self.addr = name, kc, esize, nx, xt, reg0, addr
+        self.er = esize // 4                                   # registers per element
+        self.period = 4 if (kc and esize == 4) else 2          # k a fill of one unit covers
+        self.nregs = nx * self.period * self.er
+        self.X = nx * xt
+
+    # a unit = what one refill replaces: one x of a k-contiguous panel, 4 (2) x of an x-contiguous one
+    def units(self):
+        return range(self.nx) if self.kc else range(self.nx * self.esize // 16)
+
+    def unit_of(self, x):
+        return x if self.kc else x // (16 // self.esize)
 
     def reg(self, x, k):
         if self.kc:
-            return self.reg0 + x * 4 + (k & 3)
-        return self.reg0 + ((k & 1) * 2 + (x >> 2)) * 4 + (x & 3)
+            return self.reg0 + (x * self.period + k % self.period) * self.er
+        per = 16 // self.esize                                  # x per read
+        return self.reg0 + ((k & 1) * (self.nx // per) + x // per) * 4 + (x % per) * self.er
 
     def reads_for(self, unit, k_first):
-        """LDS reads that fill `unit` with the data starting at tile-relative k_first (< 32: the
-        next tile's k is 16 + k, read through the already advanced address, i.e. offset k - 16).
-        unit: x (0..7) of a k-contiguous panel -> one read of 4 k; half (0, 1) of an x-contiguous
-        one -> two reads (k_first, k_first + 1) of 4 x."""
+        """[(asm text, {register: (operand, x, k)})] filling `unit` with the period starting at the
+        tile-relative k_first (>= 16: the next tile, read through the already advanced address)."""
         out = []
+        k = k_first % BK
         if self.kc:
-            k = k_first % BK
-            off = ((k >> 2) * 8 * self.xt + unit * self.xt) * 16
-            r = self.reg0 + unit * 4
-            out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{self.addr}] offset:{off}",
-                        {r + e: (self.name, unit, k_first + e) for e in range(4)}))
+            r = self.reg(unit, k_first)
+            off = ((k // self.period) * self.X + unit * self.xt) * 16
+            fills = {}
+            for e in range(self.period):
+                for w in range(self.er):
+                    fills[r + e * self.er + w] = (self.name, unit, k_first + e)
+            out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{self.addr}] offset:{off}", fills))
         else:
+            per = 16 // self.esize
             for s in range(2):
-                k = (k_first + s) % BK
-                off = (k * 8 * self.xt + unit * 4 * self.xt) * 4
-                r = self.reg0 + (((k_first + s) & 1) * 2 + unit) * 4
-                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{self.addr}] offset:{off}",
-                            {r + e: (self.name, unit * 4 + e, k_first + s) for e in range(4)}))
+                r = self.reg(unit * per, k_first + s)
+                off = ((k + s) * self.X + unit * per * self.xt) * self.esize
+                fills = {}
+                for e in range(per):
+                    for w in range(self.er):
+                        fills[r + e * self.er + w] = (self.name, unit * per + e, k_first + s)
+                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{self.addr}] offset:{off}", fills))
         return out
 
 
 class Body:
-    def __init__(self, a_kc, b_kc):
-        assert not (a_kc and b_kc), "two k-quad operands do not fit 128 registers"
-        # Q = the operand held per k-quad if there is one, else A; P = the other
-        q_is_a = a_kc or not b_kc
-        qa, pa = ("a_addr", "b_addr") if q_is_a else ("b_addr", "a_addr")
-        self.Q = Panel("A" if q_is_a else "B", a_kc if q_is_a else b_kc, TY if q_is_a else TX, FRAG0, qa)
-        self.P = Panel("B" if q_is_a else "A", False, TX if q_is_a else TY, FRAG0 + self.Q.nregs, pa)
+    def __init__(self, esize, a_kc, b_kc):
+        self.esize = esize
+        if esize == 4:
+            assert not (a_kc and b_kc), "two k-quad operands do not fit 128 registers"
+            ty, tx = 32, 16
+            q_is_a = a_kc or not b_kc          # Q = the operand held per k-quad if there is one, else A
+            nq = np_ = 8
+        else:
+            ty, tx = 16, 32
+            q_is_a = True
+            nq, np_ = 8, 4
         self.q_is_a = q_is_a
-        self.temp0 = TEMP0
-        assert self.P.reg0 + self.P.nregs <= TEMP0
-        self.ntemps = 4
+        qa, pa = ("a_addr", "b_addr") if q_is_a else ("b_addr", "a_addr")
+        self.Q = Panel("A" if q_is_a else "B", a_kc if q_is_a else b_kc, esize, nq, ty if q_is_a else tx, FRAG0, qa)
+        self.P = Panel("B" if q_is_a else "A", b_kc if q_is_a else a_kc, esize, np_, tx if q_is_a else ty,
+                       FRAG0 + self.Q.nregs, pa)
+        assert self.P.period == 2 and self.P.reg0 + self.P.nregs <= TEMP0
+        self.a_kc, self.b_kc = a_kc, b_kc
         self.lines = []
         self.content = {}     # register -> (operand, x, k) it holds or is being filled with
         self.inflight = []    # [(registers, group count at issue)] oldest first
-        self.groups = 0       # two-term groups emitted so far (the clock of WAIT_AGE)
+        self.groups = 0       # groups emitted so far (the clock of WAIT_AGE)
         self.tcount = 0
-        self.stats = {"valu_groups": 0, "lds": 0, "waits": 0, "other": 0}
+        self.stats = {"groups": 0, "lds": 0, "waits": 0, "other": 0}
 
     # ---- emission
     def emit(self, text, kind="other"):
@@ -123,89 +152,130 @@ class Body:
         self.emit(text, "waits")
         self.inflight = []
 
-    def term2(self, i, j, k0):
-        """acc[i][j] <- add(acc, mult(a[i][k0], b[k0][j]), mult(a[i][k0 + 1], b[k0 + 1][j]))"""
+    def vname(self, r):
+        return f"v{r}" if self.esize == 4 else f"v[{r}:{r + 1}]"
+
+    def operands(self, i, j, k):
         qx, px = (i, j) if self.q_is_a else (j, i)
-        regs = []
-        for k in (k0, k0 + 1):
-            rq, rp = self.Q.reg(qx, k), self.P.reg(px, k)
-            assert self.content.get(rq) == (self.Q.name, qx, k), (rq, self.content.get(rq), qx, k)
-            assert self.content.get(rp) == (self.P.name, px, k), (rp, self.content.get(rp), px, k)
-            regs += [rq, rp]
-        self.require(set(regs))
-        t0 = self.temp0 + self.tcount % self.ntemps
-        t1 = self.temp0 + (self.tcount + 1) % self.ntemps
-        self.tcount += 2
-        acc = ACC0 + i * 8 + j
-        self.lines.append(f'CUASR_TERM2("v{acc}", "v{t0}", "v{t1}", "v{regs[0]}", "v{regs[1]}", "v{regs[2]}", "v{regs[3]}")')
+        rq, rp = self.Q.reg(qx, k), self.P.reg(px, k)
+        for w in range(self.Q.er):
+            assert self.content.get(rq + w) == (self.Q.name, qx, k), (rq, self.content.get(rq + w), qx, k)
+            assert self.content.get(rp + w) == (self.P.name, px, k), (rp, self.content.get(rp + w), px, k)
+        return rq, rp
+
+    def term(self, i, j, k0):
+        """4-byte: acc[i][j] <- add(acc, mult(a[i][k0], b[k0][j]), mult(a[i][k0 + 1], b[k0 + 1][j]))
+        8-byte: the two terms one after the other."""
+        if self.esize == 4:
+            q0, p0 = self.operands(i, j, k0)
+            q1, p1 = self.operands(i, j, k0 + 1)
+            self.require({q0, p0, q1, p1})
+            t0 = TEMP0 + self.tcount % 4
+            t1 = TEMP0 + (self.tcount + 1) % 4
+            self.tcount += 2
+            acc = ACC0 + i * 8 + j
+            self.lines.append(f'CUASR_TERM2("v{acc}", "v{t0}", "v{t1}", "v{q0}", "v{p0}", "v{q1}", "v{p1}")')
+        else:
+            acc = ACC0 + (i * 4 + j) * 2
+            for k in (k0, k0 + 1):
+                q, p = self.operands(i, j, k)
+                self.require({q, q + 1, p, p + 1})
+                t = TEMP0 + (self.tcount % 2) * 2
+                self.tcount += 1
+                self.lines.append(f'CUASR_TERM1("{self.vname(acc)}", "{self.vname(t)}", "{self.vname(q)}", "{self.vname(p)}")')
         self.groups += 1
-        self.stats["valu_groups"] += 1
+        self.stats["groups"] += 1
+
+    # ---- global -> LDS: this wave's pieces (1 KiB each) of the tile two ahead
+    def fetch(self):
+        e = self.emit
+        e("s_cmp_lt_i32 %[fetch], 1")
+        e("s_cbranch_scc1 .Lcuasr_nofetch_%=")
+        e("s_mov_b32 %[m0_save], m0")   # M0 is the compiler's own for its LDS-bound loads: hand it back unchanged
+        if self.esize == 4:
+            # two pieces of the A panel, one of the B panel; lane offsets come ready-made
+            e("s_mov_b32 m0, %[m0_a]")
+            e("s_nop 0")
+            e("global_load_lds_dwordx4 %[off_a0], %[base_a]")
+            e("s_add_u32 m0, m0, 0x400")
+            e("s_nop 0")
+            e("global_load_lds_dwordx4 %[off_a1], %[base_a]")
+            e("s_mov_b32 m0, %[m0_b]")
+            e("s_nop 0")
+            e("global_load_lds_dwordx4 %[off_b0], %[base_b]")
+        else:
+            # two pieces of each panel (128 x 16 doubles = 16 KiB = 2 pieces for each of 8 waves).
+            # Piece q of a wave is LDS positions (2 wave + q) * 64 + lane (16 bytes each):
+            #   x-contiguous (64 positions per k): the same x, k = 2 wave + q -> the base moves on by one k
+            #   k-contiguous (128 positions per k-pair): x = 64 q + lane, same k-pair -> a second lane offset
+            for name, kc in (("a", self.a_kc), ("b", self.b_kc)):
+                e(f"s_mov_b32 m0, %[m0_{name}]")
+                e("s_nop 0")
+                e(f"global_load_lds_dwordx4 %[off_{name}0], %[base_{name}]")
+                e("s_add_u32 m0, m0, 0x400")
+                e("s_nop 0")
+                e(f"global_load_lds_dwordx4 %[off_{name}1], %[base_{name}]")
+        e("s_mov_b32 m0, %[m0_save]")
+        e(".Lcuasr_nofetch_%=:")
 
     # ---- the bodies
+    def resident_after_prime(self):
+        for unit in self.Q.units():
+            for _, fills in self.Q.reads_for(unit, 0):
+                self.content.update(fills)
+        for unit in self.P.units():
+            for _, fills in self.P.reads_for(unit, 0):
+                self.content.update(fills)
+
     def prime(self):
         """Fragments of the first k-quad / k-pair of the first tile."""
-        for unit in range(8 if self.Q.kc else 2):
+        for unit in self.Q.units():
             self.issue(self.Q, unit, 0)
-        for half in range(2):
-            self.issue(self.P, half, 0)
+        for unit in self.P.units():
+            self.issue(self.P, unit, 0)
         self.drain()
         return self.lines
 
     def tile(self):
         # state on entry = state after prime() or after a previous tile(): everything resident, nothing in flight
-        for unit in range(8 if self.Q.kc else 2):
-            for fills in [f for _, f in self.Q.reads_for(unit, 0)]:
-                self.content.update(fills)
-        for half in range(2):
-            for fills in [f for _, f in self.P.reads_for(half, 0)]:
-                self.content.update(fills)
+        self.resident_after_prime()
         entry = dict(self.content)
-
-        # global -> LDS for the tile two ahead (skipped when there is none): each wave moves two
-        # 1 KiB pieces of the A panel and one of the B panel; M0 = LDS address of the wave's piece
-        self.emit("s_cmp_lt_i32 %[fetch], 1")
-        self.emit("s_cbranch_scc1 .Lcuasr_nofetch_%=")
-        self.emit("s_mov_b32 %[m0_save], m0")   # M0 is the compiler's own for its LDS-bound loads: hand it back unchanged
-        self.emit("s_mov_b32 m0, %[m0_a]")
-        self.emit("s_nop 0")
-        self.emit("global_load_lds_dwordx4 %[off_a0], %[base_a]")
-        self.emit("s_add_u32 m0, m0, 0x400")
-        self.emit("s_nop 0")
-        self.emit("global_load_lds_dwordx4 %[off_a1], %[base_a]")
-        self.emit("s_mov_b32 m0, %[m0_b]")
-        self.emit("s_nop 0")
-        self.emit("global_load_lds_dwordx4 %[off_b0], %[base_b]")
-        self.emit("s_mov_b32 m0, %[m0_save]")
-        self.emit(".Lcuasr_nofetch_%=:")
-
+        three_stages = self.esize == 4
+        if three_stages:
+            # three LDS stages: the stage of the tile two ahead was handed back by the previous tile's barrier
+            self.fetch()
         nkp = BK // 2
+        P, Q = self.P, self.Q
+        p_units = list(P.units())
         for kp in range(nkp):
             k0 = 2 * kp
-            second = (kp & 1) == 1          # second k-pair of its k-quad
             last = kp == nkp - 1
             nk0 = k0 + 2                    # the next k-pair (>= 16: in the next tile)
+            q_ends = (k0 + 2) % Q.period == 0       # Q's residency ends with this k-pair
             for half in range(2):
                 if half == 1 and last:
                     # every read of this stage has returned and this wave's part of the next tile
                     # has landed; after the barrier that holds for the whole workgroup, and the
-                    # stage two ahead may be overwritten.  The refills from here on read the next stage.
+                    # stage is free to be overwritten.  The refills from here on read the next stage.
                     self.drain("s_waitcnt vmcnt(0) lgkmcnt(0)")
                     self.emit("s_barrier")
                     self.emit("v_add_u32 %[a_addr], %[a_step], %[a_addr]")
                     self.emit("v_add_u32 %[b_addr], %[b_step], %[b_addr]")
+                    if not three_stages:
+                        self.fetch()         # two stages: the one just handed back takes the tile two ahead
                 if half == 1:
-                    self.issue(self.P, 0, nk0)   # half 0 of P is free: refill it for the next k-pair
-                for qx in range(8):
-                    for px in range(4 * half, 4 * half + 4):
+                    for u in p_units[:len(p_units) // 2]:
+                        self.issue(P, u, nk0)       # half 0 of P is free: refill it for the next k-pair
+                for qx in range(Q.nx):
+                    for px in range(P.nx // 2 * half, P.nx // 2 * (half + 1)):
                         i, j = (qx, px) if self.q_is_a else (px, qx)
-                        self.term2(i, j, k0)
-                    if half == 1:
-                        if self.Q.kc:
-                            if second:
-                                self.issue(self.Q, qx, (k0 + 2))   # next k-quad of this x
-                        elif qx & 3 == 3:
-                            self.issue(self.Q, qx >> 2, nk0)
-            self.issue(self.P, 1, nk0)
+                        self.term(i, j, k0)
+                    if half == 1 and q_ends:
+                        u = Q.unit_of(qx)
+                        if qx == max(x for x in range(Q.nx) if Q.unit_of(x) == u):   # the unit's last x is done
+                            self.issue(Q, u, k0 + 2)
+            for u in p_units[len(p_units) // 2:]:
+                self.issue(P, u, nk0)
         self.drain()
         # the registers now hold the next tile's first fragments: same state as on entry
         shifted = {r: (o, x, k - BK) for r, (o, x, k) in self.content.items()}
@@ -215,21 +285,23 @@ class Body:
     def text(self, lines):
         out = []
         for ln in lines:
-            out.append(ln if ln.startswith("CUASR_TERM2") else '"' + ln + '\\n"')
+            out.append(ln if ln.startswith("CUASR_TERM") else '"' + ln + '\\n"')
         return "\n".join(out) + "\n"
 
 
-VARIANTS = {"kx": (True, False), "xx": (False, False), "xk": (False, True)}
+# name -> (element size, A k-contiguous, B k-contiguous)
+VARIANTS = {"kx": (4, True, False), "xx": (4, False, False), "xk": (4, False, True),
+            "d_kx": (8, True, False), "d_xx": (8, False, False), "d_xk": (8, False, True), "d_kk": (8, True, True)}
 
 
 def generate(out_dir):
     os.makedirs(out_dir, exist_ok=True)
     report = []
-    for name, (a_kc, b_kc) in VARIANTS.items():
-        b = Body(a_kc, b_kc)
+    for name, (esize, a_kc, b_kc) in VARIANTS.items():
+        b = Body(esize, a_kc, b_kc)
         with open(os.path.join(out_dir, f"direct_asm_{name}_prime.inc"), "w") as f:
             f.write(b.text(b.prime()))
-        b = Body(a_kc, b_kc)
+        b = Body(esize, a_kc, b_kc)
         with open(os.path.join(out_dir, f"direct_asm_{name}_tile.inc"), "w") as f:
             f.write(b.text(b.tile()))
         report.append((name, dict(b.stats)))

@@ -234,8 +234,8 @@ template <bool IS_MIN> static hipError_t launch(const Problem &p, hipStream_t s)
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
-  hipLaunchKernelGGL(tropical_mfma_kernel<IS_MIN>, grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  launch_kernel(tropical_mfma_kernel<IS_MIN>, grid, dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 }  // namespace tropical

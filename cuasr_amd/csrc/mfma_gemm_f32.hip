@@ -321,10 +321,10 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   // the 128 x 256 tile when its workgroups fill >= 7/8 of whole rounds of 512 (two per compute unit)
   const long long rounds = (wide * slices + 511) / 512;
   if (wide * slices * 8 >= rounds * 512 * 7)
-    hipLaunchKernelGGL(gemm_mfma_kernel<2>, dim3((unsigned)wide, (unsigned)slices), dim3(256), 0, s, p);
+    launch_kernel(gemm_mfma_kernel<2>, dim3((unsigned)wide, (unsigned)slices), dim3(256), 0, s, p);
   else
-    hipLaunchKernelGGL(gemm_mfma_kernel<1>, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
-  return hipGetLastError();
+    launch_kernel(gemm_mfma_kernel<1>, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 }  // namespace gemm_mfma

@@ -268,8 +268,8 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
-  hipLaunchKernelGGL(gemm_mfma_f64_kernel, grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  launch_kernel(gemm_mfma_f64_kernel, grid, dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 }  // namespace gemm_mfma_f64

@@ -44,8 +44,8 @@ __global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
 template <typename T> static hipError_t launch_naive(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   dim3 grid((p.n + 15) / 16, (p.m + 15) / 16, p.workspace ? p.slices : 1);
-  hipLaunchKernelGGL(naive_srgemm_kernel<T>, grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+  launch_kernel(naive_srgemm_kernel<T>, grid, dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 launch_fn find_naive(int dtype) {
@@ -195,8 +195,8 @@ template <typename T, bool SERIAL, int V, bool VOUT> static void launch_one(cons
   constexpr int U = V > 1 ? 1 : 8;      // the 16-byte path is the large-output one
   constexpr bool STREAM = V > 1;
   // (the serial form's chain of run-time operators, not memory, bounds it: 65 - 67 us at any depth)
-  if (SERIAL) hipLaunchKernelGGL((reduce_serial_kernel<T, V, VOUT, (V > 1 ? 2 : 8), STREAM>), grid, dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((reduce_splitk_kernel<T, V, VOUT, U, STREAM>), grid, dim3(256), 0, s, p);
+  if (SERIAL) launch_kernel((reduce_serial_kernel<T, V, VOUT, (V > 1 ? 2 : 8), STREAM>), grid, dim3(256), 0, s, p);
+  else launch_kernel((reduce_splitk_kernel<T, V, VOUT, U, STREAM>), grid, dim3(256), 0, s, p);
 }
 
 template <typename T, bool SERIAL> static hipError_t launch_reduce(const Problem &p, hipStream_t s) {
@@ -214,7 +214,7 @@ template <typename T, bool SERIAL> static hipError_t launch_reduce(const Problem
     const long long work = (long long)p.m * p.n;
     launch_one<T, SERIAL, 1, false>(p, dim3((unsigned)((work + 255) / 256)), s);
   }
-  return hipGetLastError();
+  return take_launch_status();
 }
 
 launch_fn find_reduce(int dtype) {

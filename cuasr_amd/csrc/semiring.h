@@ -11,7 +11,9 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <tuple>
 #include <type_traits>
+#include <utility>
 
 #include "../../include/cuasr_amd.h"
 
@@ -154,6 +156,30 @@ template <typename T> __device__ __forceinline__ EpilogueScalars<T> resolve_scal
 }
 
 typedef hipError_t (*launch_fn)(const Problem &, hipStream_t);
+
+// Kernel launches report the launch call's own status.  (hipGetLastError() after a launch would also
+// return -- and clear -- an error some earlier call of the CALLER left behind on this thread, e.g. the
+// hipErrorNotReady of a stream query: a good launch would read as a failure and the caller's error be lost.)
+// launch_kernel records the first failure of the calling thread; take_launch_status returns and clears it.
+inline thread_local hipError_t launch_status_ = hipSuccess;
+template <typename... P, size_t... I>
+inline hipError_t launch_packed_(const void *kernel, dim3 grid, dim3 block, size_t shmem, hipStream_t s, std::tuple<P...> &params,
+                                 std::index_sequence<I...>) {
+  void *ptrs[] = {static_cast<void *>(&std::get<I>(params))...};
+  return hipLaunchKernel(kernel, grid, block, ptrs, shmem, s);
+}
+template <typename... P, typename... A>
+inline void launch_kernel(void (*kernel)(P...), dim3 grid, dim3 block, size_t shmem, hipStream_t s, A &&...args) {
+  static_assert(sizeof...(P) == sizeof...(A), "one argument per kernel parameter");
+  std::tuple<P...> params{static_cast<P>(args)...};
+  const hipError_t e = launch_packed_(reinterpret_cast<const void *>(kernel), grid, block, shmem, s, params, std::index_sequence_for<P...>{});
+  if (e != hipSuccess && launch_status_ == hipSuccess) launch_status_ = e;
+}
+inline hipError_t take_launch_status() {
+  const hipError_t e = launch_status_;
+  launch_status_ = hipSuccess;
+  return e;
+}
 
 // kernel-family lookups, one definition per translation unit that owns them
 launch_fn find_naive(int dtype);

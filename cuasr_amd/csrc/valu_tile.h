@@ -615,9 +615,9 @@ template <typename T> static bool vector_possible(const Problem &p) {
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, int G>
 static void launch_ksplit(const Problem &p, dim3 grid, hipStream_t s) {
   if (vector_exact<T>(p))
-    hipLaunchKernelGGL((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, false, G>), grid, dim3(256 * G), 0, s, p);
+    launch_kernel((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, false, G>), grid, dim3(256 * G), 0, s, p);
   else
-    hipLaunchKernelGGL((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, true, G>), grid, dim3(256 * G), 0, s, p);
+    launch_kernel((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, true, G>), grid, dim3(256 * G), 0, s, p);
 }
 
 // KSPLIT: this tile may share its k range out inside the workgroup when the launch is small.
@@ -636,21 +636,21 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
     if (vector_possible<T>(p) && k_range >= 8LL * BK) {
       if (groups <= 256) {
         launch_ksplit<T, ADD, MUL, TM, TN, BK, 4>(p, grid, s);
-        return hipGetLastError();
+        return take_launch_status();
       }
       if (groups <= 512) {
         launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, grid, s);
-        return hipGetLastError();
+        return take_launch_status();
       }
     }
   }
   if (vector_exact<T>(p))
-    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, false>), grid, dim3(256), 0, s, p);
+    launch_kernel((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, false>), grid, dim3(256), 0, s, p);
   else if (vector_possible<T>(p))
-    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, true>), grid, dim3(256), 0, s, p);
+    launch_kernel((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, true, true>), grid, dim3(256), 0, s, p);
   else
-    hipLaunchKernelGGL((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, false, false>), grid, dim3(256), 0, s, p);
-  return hipGetLastError();
+    launch_kernel((valu_srgemm_kernel<T, ADD, MUL, TM, TN, BK, false, false>), grid, dim3(256), 0, s, p);
+  return take_launch_status();
 }
 
 // The chip holds 1024 full-size workgroups at a time (four per compute unit),
@@ -677,7 +677,7 @@ static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
     const long long k_range = p.workspace ? p.k_per_slice : p.k;
     if (groups >= 192 && groups <= 256 && k_range >= 8LL * BK && vector_possible<T>(p) && p.m > 0 && p.n > 0) {
       launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / (p.workspace ? p.slices : 1)), p.workspace ? p.slices : 1), s);
-      return hipGetLastError();
+      return take_launch_status();
     }
   }
   if (groups * 100 < rounds * 1024 * (long long)(CUASR_AMD_FULL_TILE_FILL_PERCENT))

@@ -225,3 +225,31 @@ def test_reduction_kernel_on_its_own(oracle, lib):
     assert lib.cuasr_amd_reduce_splitk(ctypes.byref(desc), ctypes.c_void_p(ws.data_ptr()), stream) == 0
     torch.cuda.synchronize()
     assert_same_bits(to_host(d2, "f32"), np.minimum(parts.min(axis=0), C), "hand-made partial tiles")
+
+
+def test_a_callers_pending_error_does_not_fail_a_good_launch(oracle, lib):
+    """A launch reports its own status: an error an earlier runtime call of the caller left on this thread
+    (here hipErrorNotReady from querying a busy stream) must not make a good launch read as a failure."""
+    import ctypes
+    import torch
+    import cuasr_amd
+    hip = ctypes.CDLL("libamdhip64.so")
+    hip.hipStreamQuery.argtypes = [ctypes.c_void_p]
+    A, B, C = _inputs(256, 256, 512)
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    dD = to_device(np.zeros_like(C))
+    big = torch.rand(8192, 8192, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    hip.hipGetLastError()                      # start clean
+    pending = 0
+    for _ in range(20):                        # keep the stream busy, then ask whether it is done
+        torch.mm(big, big)
+        pending = hip.hipStreamQuery(ctypes.c_void_p(stream))
+        if pending != 0:
+            break
+    if pending == 0:
+        pytest.skip("the stream never reported hipErrorNotReady")
+    for kernel in ("direct", "valu", "naive"):
+        cuasr_amd.srgemm("minimum", "plus", dA, dB, dC, dD, 0.0, 0.0, float("inf"), 0.0, kernel=kernel)   # raises on any status but success
+    torch.cuda.synchronize()
+    assert_same_bits(to_host(dD, "f32"), oracle.srgemm("minimum", "plus", A, B, C, 0.0, 0.0, np.inf), "after a pending error")
