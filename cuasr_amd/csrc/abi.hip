@@ -132,18 +132,19 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d) {
   p.alpha_ptr = d->alpha_ptr; p.beta_ptr = d->beta_ptr;
   p.add_op = d->add_op; p.mult_op = d->mult_op;
   p.slices = 1; p.k_per_slice = d->k; p.workspace = nullptr;
+  p.batch = 1; p.batch_a = p.batch_b = p.batch_c = p.batch_d = 0;
   return p;
 }
 
 enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4 };
 
-static int pick_family(const cuasr_amd_srgemm_desc *d) {
+static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
   // plus-times is the one semiring a matrix instruction computes as is
   // (its tile is 128 x 128: below 128 tiles half the compute units and more stand idle, and the
   // vector-ALU tiles, which are smaller, are faster -- 1024^3: 31 against 22 TFLOP/s)
   if (d->add_op == kPlus && d->mult_op == kMultiplies && mfma_usable(d)) {
-    const long long mfma_tiles = (long long)((d->m + 127) / 128) * ((d->n + 127) / 128) * d->split_k_slices;
+    const long long mfma_tiles = (long long)((d->m + 127) / 128) * ((d->n + 127) / 128) * d->split_k_slices * batch;
     if (mfma_tiles >= 128 || !find_valu(d->dtype, d->add_op, d->mult_op)) return kMfma;
   }
   // On gfx950 the fp32 matrix instructions and the vector ALU share one
@@ -159,7 +160,7 @@ static int pick_family(const cuasr_amd_srgemm_desc *d) {
   const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
   const int tile_n = 128;
   const long long slots = 512;
-  const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + tile_n - 1) / tile_n) * d->split_k_slices;
+  const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + tile_n - 1) / tile_n) * d->split_k_slices * batch;
   const long long rounds = (direct_groups + slots - 1) / slots;
   const bool fills = direct_groups * 8 >= rounds * slots * 7;  // >= 7/8 of its rounds
   const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;
@@ -292,9 +293,9 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   return fn(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
 
-// A batch as a sequence of launches on the stream (each validated like a single call): right for
-// matrices large enough to fill the chip; a batch of many small products would want the batch index
-// in the grid instead.
+// A strided batch.  The tile kernels take the product index from the grid (blockIdx.z), so a batch of
+// small products is one launch that fills the chip; the matrix-core and the naive kernels, and batches
+// beyond the grid's 65535, are sequences of launches.
 int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a, int64_t stride_b,
                              int64_t stride_c, int64_t stride_d, void *stream) {
   if (!desc || batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0 || stride_d < 0)
@@ -305,7 +306,29 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
   const bool col = desc->layout_c == CUASR_AMD_COLUMN_MAJOR;
   const int64_t outer = col ? desc->n : desc->m, inner = col ? desc->m : desc->n;
   if (batch > 1 && outer > 0 && inner > 0 && stride_d < (outer - 1) * desc->ldd + inner) return CUASR_AMD_ERROR_INVALID_PROBLEM;
+  if (batch == 0) return CUASR_AMD_SUCCESS;
   const int64_t es = int64_t(elem_size(desc->dtype));
+  const int family = pick_family(desc, batch);
+  if ((family == kValu || family == kDirect) && batch > 1) {
+    const launch_fn fn = family_fn(family, desc);
+    if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+    Problem p = canonical(desc);
+    // a column-major output runs as the transposed problem: the roles of A and B swap, and so do their strides
+    p.batch_a = col ? stride_b : stride_a;
+    p.batch_b = col ? stride_a : stride_b;
+    p.batch_c = stride_c;
+    p.batch_d = stride_d;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    for (int first = 0; first < batch; first += 65535) {
+      p.batch = batch - first < 65535 ? batch - first : 65535;
+      if (fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+      p.A = static_cast<const char *>(p.A) + es * p.batch_a * p.batch;
+      p.B = static_cast<const char *>(p.B) + es * p.batch_b * p.batch;
+      if (p.C) p.C = static_cast<const char *>(p.C) + es * p.batch_c * p.batch;
+      p.D = static_cast<char *>(p.D) + es * p.batch_d * p.batch;
+    }
+    return CUASR_AMD_SUCCESS;
+  }
   for (int i = 0; i < batch; ++i) {
     cuasr_amd_srgemm_desc one = *desc;
     if (one.A) one.A = static_cast<const char *>(desc->A) + es * stride_a * i;

@@ -252,6 +252,7 @@ template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) void direct64_srgemm_kernel(Problem p) {
   using Tile = Direct64Tile<T, ADD, MUL, A_KC, B_KC>;
   __shared__ typename Tile::Smem sm;
+  select_batch<T>(p);
   Tile::run(p, sm);
 }
 
@@ -283,7 +284,7 @@ template <typename T, int ADD, int MUL> static hipError_t launch_direct64(const 
   if (!direct64_ok(p)) return hipErrorNotSupported;
   const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
   if (a_kc && b_kc) launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(512), 0, s, p);
   else if (a_kc) launch_kernel((direct64_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(512), 0, s, p);

@@ -551,6 +551,7 @@ template <typename T, int ADD, int MUL, bool A_KC, bool B_KC, int TY, int TX>
 __global__ __launch_bounds__(TY *TX) __attribute__((amdgpu_waves_per_eu(4, 4))) void direct_srgemm_kernel(Problem p) {
   using Tile = DirectTile<T, ADD, MUL, A_KC, B_KC, TY, TX>;
   __shared__ typename Tile::Smem sm;
+  select_batch<T>(p);
   Tile::run(p, sm);
 }
 
@@ -558,6 +559,7 @@ template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void relaxed_srgemm_kernel(Problem p) {
   using Tile = DirectTile<T, ADD, MUL, A_KC, B_KC, 16, 16, 32, true>;
   __shared__ typename Tile::Smem sm;
+  select_batch<T>(p);
   Tile::run(p, sm);
 }
 
@@ -599,7 +601,7 @@ template <typename T, int ADD, int MUL> static hipError_t launch_relaxed(const P
   if (!direct_ok(p)) return hipErrorNotSupported;
   const long long tiles = (long long)((p.m + 127) / 128) * ((p.n + 127) / 128);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
   if (a_kc && b_kc) launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, true, true>), grid, dim3(256), 0, s, p);
   else if (a_kc) launch_kernel((relaxed_srgemm_kernel<T, ADD, MUL, true, false>), grid, dim3(256), 0, s, p);
@@ -618,7 +620,7 @@ template <typename T, int ADD, int MUL> static hipError_t launch_direct(const Pr
   if (!direct_ok(p)) return hipErrorNotSupported;
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch);
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
   if (a_kc && b_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, true, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
   else if (a_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, true, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);

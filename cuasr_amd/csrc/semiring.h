@@ -136,7 +136,22 @@ struct Problem {
   // partial accumulators go to workspace[z][m][n] (row-major, ld = n)
   int slices, k_per_slice;
   void *workspace;
+  // strided batch (tile kernels only): product blockIdx.z works on A, B, C, D moved on by z times
+  // these element strides; batch = 1 for a single product
+  int batch;
+  long long batch_a, batch_b, batch_c, batch_d;
 };
+
+// the operands of product blockIdx.z of a strided batch
+template <typename T> __device__ __forceinline__ void select_batch(Problem &p) {
+  if (p.batch > 1) {
+    const long long z = blockIdx.z;
+    p.A = reinterpret_cast<const T *>(p.A) + z * p.batch_a;
+    p.B = reinterpret_cast<const T *>(p.B) + z * p.batch_b;
+    if (p.C) p.C = reinterpret_cast<const T *>(p.C) + z * p.batch_c;
+    p.D = reinterpret_cast<T *>(p.D) + z * p.batch_d;
+  }
+}
 
 // Epilogue scalars resolved on the device (alpha/beta may live in device memory).
 template <typename T> struct EpilogueScalars {

@@ -537,6 +537,7 @@ template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool VEC, bool C
 __global__ __launch_bounds__(256) WAVES_ATTR void valu_srgemm_kernel(Problem p) {
   using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC, CAREFUL>;
   __shared__ typename Tile::Smem sm;
+  select_batch<T>(p);
   Tile::run(p, sm);
 }
 
@@ -557,6 +558,7 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   static_assert(order_free<T, ADD>::value, "a floating-point sum depends on the grouping of its terms");
   static_assert(G * sizeof(typename Tile::Smem) >= (G - 1) * sizeof(S) * TM * TN * 256, "the groups' accumulators must fit the panel space");
   __shared__ typename Tile::Smem sm[G];
+  select_batch<T>(p);
   const int g = threadIdx.x >> 8, tid = threadIdx.x & 255;
   int m0, n0, kb, ke;
   Tile::tile_and_range(p, m0, n0, kb, ke);
@@ -627,11 +629,11 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
+  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch);
   if constexpr (KSPLIT && order_free<T, ADD>::value) {
     // 256 compute units: up to 256 workgroups get four groups (1024 threads, four waves per SIMD),
     // up to 512 two; each group wants a few k-tiles of its own to be worth the fold at the end
-    const long long groups = tiles * grid.y;
+    const long long groups = tiles * grid.y * grid.z;
     const long long k_range = p.workspace ? p.k_per_slice : p.k;
     if (vector_possible<T>(p) && k_range >= 8LL * BK) {
       if (groups <= 256) {
@@ -668,7 +670,7 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, int TM_SMALL, int TN_SMALL, int BK_SMALL = BK>
 static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
-  const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1);
+  const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1) * p.batch;
   const long long rounds = (groups + 1023) / 1024;
   if constexpr (order_free<T, ADD>::value) {
     // 192 .. 256 full-size workgroups (2048^2: exactly 256) are one per compute unit for most of the
@@ -676,7 +678,7 @@ static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
     // at the rate it has on large problems, which the quarter-size tile does not reach
     const long long k_range = p.workspace ? p.k_per_slice : p.k;
     if (groups >= 192 && groups <= 256 && k_range >= 8LL * BK && vector_possible<T>(p) && p.m > 0 && p.n > 0) {
-      launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / (p.workspace ? p.slices : 1)), p.workspace ? p.slices : 1), s);
+      launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / (p.workspace ? p.slices : 1) / p.batch), p.workspace ? p.slices : 1, p.batch), s);
       return take_launch_status();
     }
   }

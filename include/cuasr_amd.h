@@ -158,9 +158,12 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream);
  * i * stride_d ELEMENTS (the reference only names batched operation as an aim,
  * README.md:11, and has no such call).  Stride 0 shares an operand between all
  * products; the outputs must lie at least one matrix apart, strides must not be
- * negative (CUASR_AMD_ERROR_INVALID_PROBLEM otherwise).  The products are
- * launched one after the other on the stream, each chosen and validated like a
- * single cuasr_amd_srgemm; the first failure is returned. */
+ * negative (CUASR_AMD_ERROR_INVALID_PROBLEM otherwise).  The kernel family is
+ * chosen once, for the whole batch (what fills the chip is the batch, not one
+ * product); on the vector-ALU tiles the product index is part of the grid, so a
+ * batch of many small products is a single launch; the matrix-core and naive
+ * kernels run the products one after the other on the stream.  Each product's
+ * result is that of a single cuasr_amd_srgemm on its operands. */
 int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a,
                              int64_t stride_b, int64_t stride_c, int64_t stride_d, void *stream);
 

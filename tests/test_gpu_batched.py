@@ -51,3 +51,57 @@ def test_batched_empty_batch_and_column_major(oracle):
                              np.zeros((m, n), np.float32, order="F"), 0.0, np.inf, np.inf)
         assert_same_bits(np.ascontiguousarray(got[i]), np.ascontiguousarray(want), f"product {i}")
     cuasr_amd.srgemm_batched("minimum", "plus", dA[:0], dB[:0], dD[:0], dD[:0], 0.0, inf, inf, 0.0)   # nothing to do
+
+
+@pytest.mark.parametrize("kernel", ["auto", "valu", "direct", "naive"])
+def test_many_small_products_in_one_launch(oracle, kernel):
+    """1024 products of 64 x 64 x 64: on the tile kernels the product index is part of the grid.  Every
+    product against the oracle, operands of the batch at strides larger than a matrix."""
+    import torch
+    batch, m, n, k = 1024, 64, 64, 64
+    rng = np.random.default_rng(5)
+    A = rng.random((batch, m + 4, k)).astype(np.float32)                 # row-major slices, 4 rows of padding between them
+    B = rng.random((batch, k, n)).astype(np.float32)
+    C = rng.random((batch, m, n)).astype(np.float32)
+    dA = torch.from_numpy(A).cuda()
+    A = A[:, :m, :]
+    dB, dC = torch.from_numpy(B).cuda(), torch.from_numpy(C).cuda()
+    dD = torch.zeros(batch, m, n, device="cuda")
+    cuasr_amd.srgemm_batched("minimum", "plus", dA[:, :m, :], dB, dC, dD, 0.0, 0.0, float("inf"), 0.0, kernel=kernel)
+    got = dD.cpu().numpy()
+    for i in range(0, batch, 1 if kernel == "auto" else 37):
+        want = oracle.srgemm("minimum", "plus", np.ascontiguousarray(A[i]), B[i], C[i], 0.0, 0.0, np.inf)
+        assert_same_bits(got[i], want, f"{kernel} product {i}")
+
+
+def test_batched_column_major_outputs_and_doubles(oracle):
+    """Column-major outputs run as the transposed problem: the batch strides of A and B swap with the operands."""
+    import torch
+    batch, m, n, k = 70, 96, 40, 130
+    rng = np.random.default_rng(8)
+    A = rng.random((batch, k, m))            # slice i transposed = column-major m x k
+    B = rng.random((batch, n, k))            # slice i transposed = column-major k x n
+    C = rng.random((batch, n, m))
+    dA, dB, dC = (torch.from_numpy(x).cuda().transpose(1, 2) for x in (A, B, C))
+    dD = torch.zeros(batch, n, m, dtype=torch.float64, device="cuda").transpose(1, 2)
+    cuasr_amd.srgemm_batched("maximum", "plus", dA, dB, dC, dD, 0.0, 0.0, float("-inf"), 0.0)
+    got = dD.cpu().numpy()
+    for i in range(batch):
+        want = oracle.srgemm("maximum", "plus", np.asfortranarray(A[i].T), np.asfortranarray(B[i].T), np.asfortranarray(C[i].T),
+                             0.0, 0.0, -np.inf)
+        assert_same_bits(np.ascontiguousarray(got[i]), np.ascontiguousarray(want), f"product {i}")
+
+
+def test_batch_larger_than_one_grid(oracle):
+    """More products than the grid's third dimension holds (65535): several launches, same results."""
+    import torch
+    batch, m, n, k = 65540, 8, 4, 8
+    rng = np.random.default_rng(9)
+    A = rng.integers(0, 50, (batch, m, k)).astype(np.float32)
+    B = rng.integers(0, 50, (batch, k, n)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    dD = torch.zeros(batch, m, n, device="cuda")
+    inf = float("inf")
+    cuasr_amd.srgemm_batched("minimum", "plus", dA, dB, dD, dD, 0.0, inf, inf, 0.0)
+    want = (A[:, :, :, None] + B[:, None, :, :]).min(axis=2)            # min-plus of every product, exact in fp32
+    assert_same_bits(dD.cpu().numpy(), want, "65540 products")
