@@ -103,6 +103,9 @@ def load():
         lib.cuasr_amd_apsp_blocked.restype = ctypes.c_int
         lib.cuasr_amd_apsp_blocked.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
                                                ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+        lib.cuasr_amd_apsp_blocked_panels.restype = ctypes.c_int
+        lib.cuasr_amd_apsp_blocked_panels.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
+                                                      ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
         lib.cuasr_amd_apsp_squaring.restype = ctypes.c_int
         lib.cuasr_amd_apsp_squaring.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p,
                                                 ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
@@ -391,7 +394,10 @@ def apsp_blocked_workspace_bytes(n, dtype):
     return int(load().cuasr_amd_apsp_blocked_workspace_bytes(DTYPES[dtype], n))
 
 
-def apsp_blocked(dist, parent, workspace, stream=None):
+PANELS = {"auto": 0, "paired": 1, "tiled": 2}
+
+
+def apsp_blocked(dist, parent, workspace, stream=None, panels="auto"):
     """All-pairs shortest paths by blocked Floyd-Warshall with predecessor
     tracking, in place on the n x n column-major ``dist`` and int32 ``parent``;
     ``workspace`` is a device tensor of at least
@@ -400,7 +406,11 @@ def apsp_blocked(dist, parent, workspace, stream=None):
     pd, ld = _column_major(dist, "dist")
     pp, ldp = _column_major(parent, "parent")
     ws = ctypes.c_void_p(workspace.data_ptr()) if workspace is not None else None
-    st = load().cuasr_amd_apsp_blocked(DTYPES[_torch_dtype_name(dist)], n, pd, ld, pp, ldp, ws, _stream_handle(stream))
+    if panels == "auto":
+        st = load().cuasr_amd_apsp_blocked(DTYPES[_torch_dtype_name(dist)], n, pd, ld, pp, ldp, ws, _stream_handle(stream))
+    else:
+        st = load().cuasr_amd_apsp_blocked_panels(DTYPES[_torch_dtype_name(dist)], n, pd, ld, pp, ldp, ws, PANELS[panels],
+                                                  _stream_handle(stream))
     if st != SUCCESS:
         raise CuasrError(st, "cuasr_amd_apsp_blocked")
     return dist, parent

@@ -651,6 +651,13 @@ extern "C" size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n) {
 
 extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
                                       void *workspace, void *stream) {
+  return cuasr_amd_apsp_blocked_panels(dtype, n, dist, ld, parent, ldp, workspace, CUASR_AMD_PANELS_AUTO, stream);
+}
+
+extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
+                                             void *workspace, int panels, void *stream) {
+  if (panels != CUASR_AMD_PANELS_AUTO && panels != CUASR_AMD_PANELS_PAIRED && panels != CUASR_AMD_PANELS_TILED)
+    return CUASR_AMD_ERROR_INVALID_PROBLEM;
   const int64_t nn = (int64_t(n) + 3) & ~int64_t(3);
   const int st = check(dtype, n, n, n, workspace, nn > 0 ? nn : 1, workspace, nn > 0 ? nn : 1, dist, ld, parent, ldp,
                        CUASR_AMD_KERNEL_AUTO);
@@ -697,7 +704,10 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
     FwExtra x;
     x.k_base = k0;
     int r;
-    if ((int64_t(n) + 127) / 128 < 128) {
+    // below 128 tiles per panel product the two share one launch of the one-thread-per-element kernel;
+    // from n = 16257 on each fills the chip on the tiled kernel
+    const bool paired = panels == CUASR_AMD_PANELS_AUTO ? (int64_t(n) + 127) / 128 < 128 : panels == CUASR_AMD_PANELS_PAIRED;
+    if (paired) {
       const FwArgs g0{bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp,
                       nullptr, 0, k0, 0, 0, k0, k0 + bb, nullptr, 0};
       // (the column product also writes the updated column's k-contiguous image for step 4; the rows
@@ -713,10 +723,10 @@ extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, 
       xr.skip_c0 = xc.skip_r0 = k0;
       xr.skip_c1 = xc.skip_r1 = k0 + bb;
       r = fwgemm_run(dtype, bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp, xr,
-                     CUASR_AMD_KERNEL_AUTO, stream);
+                     CUASR_AMD_KERNEL_VALU, stream);
       if (r != CUASR_AMD_SUCCESS) return r;
       r = fwgemm_run(dtype, n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp, xc,
-                     CUASR_AMD_KERNEL_AUTO, stream);
+                     CUASR_AMD_KERNEL_VALU, stream);
       if (r != CUASR_AMD_SUCCESS) return r;
       e = f64 ? snapshot<double>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s) : snapshot<float>(Dcol, ld, nullptr, 0, Ct, FW_BLOCK, n, bb, s);
       if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;

@@ -282,6 +282,18 @@ size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n);
 int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, int32_t *parent,
                            int64_t ldp, void *workspace, void *stream);
 
+/* The same with the choice of how a block step updates its block row and block column made by the
+ * caller: CUASR_AMD_PANELS_AUTO (what cuasr_amd_apsp_blocked does: PAIRED below n = 16257, TILED from
+ * there on, where each panel product fills the chip on its own), CUASR_AMD_PANELS_PAIRED (both products
+ * in one launch of the one-thread-per-element kernel) or CUASR_AMD_PANELS_TILED (two launches of the
+ * tiled kernel and a transposing copy of the updated block column).  Results do not depend on it.
+ * CUASR_AMD_ERROR_INVALID_PROBLEM for any other value. */
+#define CUASR_AMD_PANELS_AUTO 0
+#define CUASR_AMD_PANELS_PAIRED 1
+#define CUASR_AMD_PANELS_TILED 2
+int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64_t ld, int32_t *parent,
+                                  int64_t ldp, void *workspace, int panels, void *stream);
+
 /* Name of the kernel family AUTO would choose for this descriptor
  * ("naive", "valu", "valu_direct", "mfma"; "valu_direct+valu" when a block of the output runs on
  * the direct-to-LDS tile and the strips around it on the staged one), or NULL if the descriptor

@@ -210,6 +210,35 @@ def test_apsp_blocked_floyd_warshall(oracle, n, pad, dtype):
     _check_paths(W, dist, parent, n)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("n,pad", [(100, 0), (384, 0), (513, 1), (700, 4), (1475, 1)])
+def test_apsp_blocked_with_tiled_panels(oracle, n, pad, dtype):
+    """The way a block step updates its block row and column from n = 16257 on (two launches of the tiled
+    kernel with the diagonal block skipped, then a transposing copy of the column), forced at sizes the
+    oracle can run: dist and parent bit-identical to the oracle and to the paired form."""
+    import torch
+    rng = np.random.default_rng(177 + n)
+    W = np.where(rng.random((n, n)) < max(0.02, 3.0 / n), rng.random((n, n)) * 9 + 0.5, np.inf).astype(dtype)   # sums round
+    np.fill_diagonal(W, 0)
+    host = np.full((n + pad, n), 7.0, dtype=dtype, order="F")
+    host[:n] = W
+    name = "f32" if dtype == np.float32 else "f64"
+    results = {}
+    for panels in ("tiled", "paired"):
+        dD = to_device(host)
+        dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+        ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, name), dtype=torch.uint8, device="cuda")
+        cuasr_amd.apsp_blocked(dD[:n], dP, ws, panels=panels)
+        got = dD.cpu().numpy()
+        assert (got[n:] == 7.0).all()
+        results[panels] = (np.ascontiguousarray(got[:n]), dP.cpu().numpy())
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(want_d, want_p, 128)
+    for panels, (dist, parent) in results.items():
+        assert_same_bits(dist, np.ascontiguousarray(want_d), f"dist, {panels} panels")
+        assert np.array_equal(parent, want_p), panels
+
+
 def test_apsp_blocked_on_rounding_weights_matches_the_oracle_bit_for_bit(oracle):
     """Real-valued weights: sums round, so the result depends on the order of additions; the
     device and the oracle use the same order.  Against repeated squaring only closeness holds."""
