@@ -76,6 +76,14 @@ def build_cpp_tests():
                            "-I", os.path.join(root, "include"), "-I", os.path.join(root, "oracle", "include"),
                            src, "-L", LIB_DIR, "-lcuasr_amd", "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
                            "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,$ORIGIN/../../cuasr_amd/lib", "-o", out])
+    # the functor path of the operator templates needs hipcc: its kernel is built in the user's translation unit
+    src2 = os.path.join(root, "tests", "cpp", "test_user_functor.hip")
+    out2 = os.path.join(root, "tests", "cpp", "test_user_functor")
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                           "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
+                           "-I", os.path.join(root, "include"), "-I", os.path.join(root, "oracle", "include"),
+                           src2, "-L", LIB_DIR, "-lcuasr_amd", "-Wl,-rpath," + LIB_DIR,
+                           "-Wl,-rpath,$ORIGIN/../../cuasr_amd/lib", "-o", out2], stderr=subprocess.DEVNULL)
     return out
 
 

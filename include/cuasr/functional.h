@@ -16,9 +16,11 @@
 // constants are true infinities (what shortest-path data with unreachable
 // pairs needs).
 //
-// The device kernels are not instantiated from these functors; a functor type
-// maps to an operator tag of the C ABI through cuasr::op_tag<Functor>, which
-// user code specialises for its own functor types (see binary_xor below).
+// The library's tuned kernels are not instantiated from these functors; a functor
+// type maps to an operator tag of the C ABI through cuasr::op_tag<Functor>, which
+// user code can specialise for its own functor types (see binary_xor below).  A
+// functor type that is none of these operators gets a kernel built from its
+// operator() (cuasr/gemm/kernel/functor_srgemm.h), as in the reference.
 #pragma once
 #include <limits>
 
@@ -26,7 +28,11 @@
 
 namespace cuasr {
 
-template <typename F> struct op_tag;  // { static int const value = CUASR_AMD_OP_...; }
+/// Which operator of the C ABI a functor type is.  Specialise it for a functor of your own that computes one
+/// of those operators (as binary_xor below); a functor type without a specialisation counts as "none of
+/// them" (value < 0): device::Srgemm then builds its kernel from the functor's operator() itself, which
+/// needs the translation unit to be compiled by hipcc (cuasr/gemm/kernel/functor_srgemm.h).
+template <typename F> struct op_tag { static int const value = -1; };
 
 namespace detail {
 template <typename T> constexpr T highest() { return std::numeric_limits<T>::max(); }
@@ -39,11 +45,17 @@ template <typename T> constexpr T neg_inf() {
 }
 }  // namespace detail
 
+#if defined(__HIPCC__)
+#define CUASR_HOST_DEVICE __host__ __device__
+#else
+#define CUASR_HOST_DEVICE
+#endif
+
 #define CUASR_AMD_FUNCTOR(NAME, IDENT, ANNIH, EXPR)                               \
   template <typename T, int N = 1> struct NAME {                                  \
     static constexpr T Identity = IDENT;                                          \
     static constexpr T Annihilator = ANNIH;                                       \
-    constexpr T operator()(T lhs, T const &rhs) const { return EXPR; }            \
+    CUASR_HOST_DEVICE constexpr T operator()(T lhs, T const &rhs) const { return EXPR; } \
   };                                                                              \
   template <typename T, int N> constexpr T NAME<T, N>::Identity;                  \
   template <typename T, int N> constexpr T NAME<T, N>::Annihilator;

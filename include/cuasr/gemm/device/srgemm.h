@@ -18,6 +18,9 @@
 #include <type_traits>
 
 #include "default_srgemm_configuration.h"
+#if defined(__HIPCC__)
+#include "../kernel/functor_srgemm.h"
+#endif
 
 namespace cuasr {
 namespace gemm {
@@ -76,7 +79,11 @@ template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, 
           typename ThreadblockSwizzle_ = threadblock::GemmIdentityThreadblockSwizzle<>,
           int Stages = DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_,
                                                     AdditionOp_, MultiplicationOp_, ArchTag_>::kStages,
-          int AlignmentA = 1, int AlignmentB = 1, bool SplitKSerial = false>
+          int AlignmentA = DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_,
+                                                        AdditionOp_, MultiplicationOp_, ArchTag_>::kAlignmentA,
+          int AlignmentB = DefaultSemiRingConfiguration<ElementA_, ElementB_, ElementC_, ElementAccumulator_, OperatorClass_,
+                                                        AdditionOp_, MultiplicationOp_, ArchTag_>::kAlignmentB,
+          bool SplitKSerial = false>
 class Srgemm {
  public:
   using ElementA = ElementA_;
@@ -104,6 +111,10 @@ class Srgemm {
   static int const kAlignmentB = AlignmentB;
   static int const kAlignmentC = EpilogueOutputOp::kCount;
   static bool const kSplitKSerial = SplitKSerial;
+  /// true when AdditionOp or MultiplicationOp is none of the library's operators (no cuasr::op_tag
+  /// specialisation): the kernel is then built from the functors' operator() in this translation unit
+  /// (cuasr/gemm/kernel/functor_srgemm.h), which needs hipcc; split-K is not offered for such functors
+  static bool const kUserFunctors = op_tag<AdditionOp>::value < 0 || op_tag<MultiplicationOp>::value < 0;
 
   static_assert(std::is_same<ElementA, ElementC>::value && std::is_same<ElementB, ElementC>::value &&
                     std::is_same<ElementAccumulator, ElementC>::value,
@@ -133,6 +144,20 @@ class Srgemm {
   static Status can_implement(Arguments const &args) {
     if (!kSplitKSerial && args.split_k_slices > 1) return Status::kErrorInvalidProblem;
     if (args.split_k_slices < 1) return Status::kErrorInvalidProblem;
+    if constexpr (kUserFunctors) {
+      if (args.split_k_slices > 1) return Status::kErrorNotSupported;
+      const long long m = args.problem_size.m(), n = args.problem_size.n(), k = args.problem_size.k();
+      if (m < 0 || n < 0 || k < 0) return Status::kErrorInvalidProblem;
+      auto ld_ok = [](long long ld, bool column_major, long long rows, long long cols) { return ld >= (column_major ? rows : cols); };
+      if (m > 0 && k > 0 && !ld_ok(args.ref_A.stride(0), LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, k)) return Status::kErrorInvalidProblem;
+      if (n > 0 && k > 0 && !ld_ok(args.ref_B.stride(0), LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, k, n)) return Status::kErrorInvalidProblem;
+      if (m > 0 && n > 0) {
+        if (!args.ref_D.data() || !ld_ok(args.ref_D.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
+        if (args.ref_C.data() && !ld_ok(args.ref_C.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
+        if (k > 0 && (!args.ref_A.data() || !args.ref_B.data())) return Status::kErrorInvalidProblem;
+      }
+      return Status::kSuccess;
+    }
     cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
     d.split_k_slices = 1;  // the slice count is checked above; the rest is the plain problem's check
     return static_cast<Status>(cuasr_amd_srgemm_can_implement(&d));
@@ -156,7 +181,8 @@ class Srgemm {
     Status s = can_implement(args);
     if (s != Status::kSuccess) return s;
     if (kSplitKSerial && args.split_k_slices > 1 && !workspace) return Status::kErrorWorkspaceNull;
-    desc_ = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
+    args_ = args;
+    if constexpr (!kUserFunctors) desc_ = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
     workspace_ = workspace;
     ready_ = true;
     return Status::kSuccess;
@@ -166,6 +192,11 @@ class Srgemm {
   Status update(Arguments const &args, void *workspace = nullptr) {
     if (!ready_) return Status::kErrorInternal;
     if (kSplitKSerial && args.split_k_slices > 1 && !workspace) return Status::kErrorWorkspaceNull;
+    args_.ref_A = args.ref_A;
+    args_.ref_B = args.ref_B;
+    args_.ref_C = args.ref_C;
+    args_.ref_D = args.ref_D;
+    args_.epilogue = args.epilogue;
     desc_.A = args.ref_A.data();
     desc_.B = args.ref_B.data();
     desc_.C = args.ref_C.data();
@@ -180,6 +211,39 @@ class Srgemm {
 
   Status run(hipStream_t stream = nullptr) {
     if (!ready_) return Status::kErrorInternal;
+    if constexpr (kUserFunctors) {
+#if defined(__HIPCC__)
+      kernel::FunctorSrgemmParams<ElementC> p;
+      p.m = args_.problem_size.m();
+      p.n = args_.problem_size.n();
+      p.k = args_.problem_size.k();
+      auto strides = [](long long ld, bool column_major, long long &s_row, long long &s_col) {
+        s_row = column_major ? 1 : ld;
+        s_col = column_major ? ld : 1;
+      };
+      p.A = args_.ref_A.data();
+      strides(args_.ref_A.stride(0), LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sa_m, p.sa_k);
+      p.B = args_.ref_B.data();
+      strides(args_.ref_B.stride(0), LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sb_k, p.sb_n);
+      p.C = args_.ref_C.data();
+      strides(args_.ref_C.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sc_m, p.sc_n);
+      p.D = args_.ref_D.data();
+      strides(args_.ref_D.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sd_m, p.sd_n);
+      p.alpha = args_.epilogue.alpha;
+      p.beta = args_.epilogue.beta;
+      p.alpha_ptr = static_cast<ElementC const *>(args_.epilogue.alpha_ptr);
+      p.beta_ptr = static_cast<ElementC const *>(args_.epilogue.beta_ptr);
+      return kernel::launch_functor_srgemm<AdditionOp, MultiplicationOp, ElementC>(p, stream) == hipSuccess ? Status::kSuccess
+                                                                                                           : Status::kErrorInternal;
+#else
+      static_assert(!kUserFunctors,
+                    "cuasr::gemm::device::Srgemm: AdditionOp / MultiplicationOp is not one of the library's operators "
+                    "(plus, multiplies, minimum, maximum, binary_and, binary_or, binary_xor, bitwise_and, bitwise_or; "
+                    "no cuasr::op_tag specialisation), so the kernel has to be built from the functor itself: compile "
+                    "this translation unit with hipcc, or specialise cuasr::op_tag for the functor if it is one of them");
+      return Status::kErrorNotSupported;
+#endif
+    }
     if (kSplitKSerial && desc_.split_k_slices > 1)
       return static_cast<Status>(cuasr_amd_srgemm_splitk_serial(&desc_, workspace_, stream));
     return static_cast<Status>(cuasr_amd_srgemm(&desc_, stream));
@@ -193,6 +257,7 @@ class Srgemm {
   }
 
  private:
+  Arguments args_;
   cuasr_amd_srgemm_desc desc_;
   void *workspace_;
   bool ready_;

@@ -50,6 +50,12 @@ template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, 
                                                     AdditionOp_, MultiplicationOp_, ArchTag_>::kStages,
           int kAlignmentA = 1, int kAlignmentB = 1>
 class SrgemmSplitKParallel {
+  static_assert(op_tag<AdditionOp_>::value >= 0 && op_tag<MultiplicationOp_>::value >= 0,
+                "cuasr::gemm::device::SrgemmSplitKParallel: split-K is offered for the library's operators only (plus, "
+                "multiplies, minimum, maximum, binary_and, binary_or, binary_xor, bitwise_and, bitwise_or); a functor that "
+                "computes one of them can say so by specialising cuasr::op_tag; any other functor runs through "
+                "cuasr::gemm::device::Srgemm, which builds its kernel from the functor");
+
  public:
   using ElementA = ElementA_;
   using LayoutA = LayoutA_;

@@ -1,0 +1,137 @@
+// device::Srgemm with functors that are none of the library's operators: the kernel is built from the
+// functors' operator() (as the reference does for every functor,
+// examples/01_userdefined_semiring/userdefined_semiring.cu:56-99), and must reproduce the host reference
+// SRGEMM bit for bit -- also for an "add" that is not associative, because every output element is
+// accumulated in ascending k like the host loop.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <random>
+#include <vector>
+
+#include "cuasr/gemm/device/srgemm.h"
+#include "cuasr/reference/srgemm/host_srgemm.h"
+
+#define HIP_CHECK(x)                                                                                   \
+  do {                                                                                                 \
+    hipError_t e_ = (x);                                                                               \
+    if (e_ != hipSuccess) {                                                                            \
+      std::printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__);               \
+      std::exit(2);                                                                                    \
+    }                                                                                                  \
+  } while (0)
+
+static int g_run = 0, g_fail = 0;
+static void check(bool ok, const char *what) {
+  ++g_run;
+  if (!ok) ++g_fail;
+  std::printf("%s %s\n", ok ? "PASS" : "FAIL", what);
+}
+
+// a bounded "plus": path lengths saturate at a cap (shortest paths with a horizon)
+template <typename T, int N = 1> struct saturating_plus {
+  static constexpr T Identity = static_cast<T>(0);
+  static constexpr T Annihilator = static_cast<T>(1000);
+  __host__ __device__ T operator()(T lhs, T const &rhs) const {
+    const T s = lhs + rhs;
+    return s > static_cast<T>(1000) ? static_cast<T>(1000) : s;
+  }
+};
+template <typename T, int N> constexpr T saturating_plus<T, N>::Identity;
+template <typename T, int N> constexpr T saturating_plus<T, N>::Annihilator;
+
+// keeps the operand of larger magnitude (ties: the right one): not commutative on ties, order matters
+template <typename T, int N = 1> struct abs_max {
+  static constexpr T Identity = static_cast<T>(0);
+  static constexpr T Annihilator = static_cast<T>(0);
+  __host__ __device__ T operator()(T lhs, T const &rhs) const { return (lhs < 0 ? -lhs : lhs) > (rhs < 0 ? -rhs : rhs) ? lhs : rhs; }
+};
+template <typename T, int N> constexpr T abs_max<T, N>::Identity;
+template <typename T, int N> constexpr T abs_max<T, N>::Annihilator;
+
+// a decayed sum: not associative, rounds at every step
+template <typename T, int N = 1> struct leaky_plus {
+  static constexpr T Identity = static_cast<T>(0);
+  static constexpr T Annihilator = static_cast<T>(0);
+  __host__ __device__ T operator()(T lhs, T const &rhs) const { return lhs + static_cast<T>(0.75) * rhs; }
+};
+template <typename T, int N> constexpr T leaky_plus<T, N>::Identity;
+template <typename T, int N> constexpr T leaky_plus<T, N>::Annihilator;
+
+template <typename Add, typename Mul, typename T, typename LA, typename LB, typename LC>
+static void run_case(int m, int n, int k, T alpha, T beta, unsigned seed, const char *what) {
+  using Op = cuasr::gemm::device::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T>;
+  static_assert(Op::kUserFunctors, "this test is about functors the library has no operator for");
+  const bool a_col = LA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, b_col = LB::kAbiTag == CUASR_AMD_COLUMN_MAJOR,
+             c_col = LC::kAbiTag == CUASR_AMD_COLUMN_MAJOR;
+  const int lda = (a_col ? m : k) + 3, ldb = (b_col ? k : n) + 1, ldc = (c_col ? m : n) + 2;
+  std::vector<T> A((size_t)lda * (a_col ? k : m)), B((size_t)ldb * (b_col ? n : k)), C((size_t)ldc * (c_col ? n : m)), D(C.size()), R(C.size());
+  std::mt19937 rng(seed);
+  std::uniform_int_distribution<int> dist(-40, 40);
+  for (auto &v : A) v = static_cast<T>(dist(rng)) / static_cast<T>(std::is_integral<T>::value ? 1 : 8);
+  for (auto &v : B) v = static_cast<T>(dist(rng)) / static_cast<T>(std::is_integral<T>::value ? 1 : 8);
+  for (auto &v : C) v = static_cast<T>(dist(rng)) / static_cast<T>(std::is_integral<T>::value ? 1 : 8);
+  D.assign(D.size(), static_cast<T>(-77));
+  R = D;
+  T *dA, *dB, *dC, *dD;
+  HIP_CHECK(hipMalloc(&dA, A.size() * sizeof(T)));
+  HIP_CHECK(hipMalloc(&dB, B.size() * sizeof(T)));
+  HIP_CHECK(hipMalloc(&dC, C.size() * sizeof(T)));
+  HIP_CHECK(hipMalloc(&dD, D.size() * sizeof(T)));
+  HIP_CHECK(hipMemcpy(dA, A.data(), A.size() * sizeof(T), hipMemcpyHostToDevice));
+  HIP_CHECK(hipMemcpy(dB, B.data(), B.size() * sizeof(T), hipMemcpyHostToDevice));
+  HIP_CHECK(hipMemcpy(dC, C.data(), C.size() * sizeof(T), hipMemcpyHostToDevice));
+  HIP_CHECK(hipMemcpy(dD, D.data(), D.size() * sizeof(T), hipMemcpyHostToDevice));
+  typename Op::Arguments args({m, n, k}, {dA, lda}, {dB, ldb}, {dC, ldc}, {dD, ldc}, {alpha, beta});
+  Op op;
+  const cuasr::Status st = op(args);
+  HIP_CHECK(hipDeviceSynchronize());
+  HIP_CHECK(hipMemcpy(D.data(), dD, D.size() * sizeof(T), hipMemcpyDeviceToHost));
+  cuasr::reference::host::Srgemm<Add, Mul, T, LA, T, LB, T, LC, T, T> ref;
+  ref({m, n, k}, alpha, {A.data(), lda}, {B.data(), ldb}, beta, {C.data(), ldc}, {R.data(), ldc}, Add::Identity);
+  char name[256];
+  std::snprintf(name, sizeof name, "%s %dx%dx%d", what, m, n, k);
+  check(st == cuasr::Status::kSuccess && std::memcmp(D.data(), R.data(), D.size() * sizeof(T)) == 0, name);
+  HIP_CHECK(hipFree(dA));
+  HIP_CHECK(hipFree(dB));
+  HIP_CHECK(hipFree(dC));
+  HIP_CHECK(hipFree(dD));
+}
+
+int main() {
+  int count = 0;
+  if (hipGetDeviceCount(&count) != hipSuccess || count == 0) {
+    std::printf("no GPU\n");
+    return 1;
+  }
+  using Col = cuasr::layout::ColumnMajor;
+  using Row = cuasr::layout::RowMajor;
+  const int shapes[][3] = {{64, 64, 64}, {1, 1, 1}, {65, 63, 17}, {200, 130, 301}, {7, 300, 33}, {509, 510, 23}};
+  for (auto &s : shapes) {
+    // library add, user mult: bounded shortest paths on integers
+    run_case<cuasr::minimum<int32_t>, saturating_plus<int32_t>, int32_t, Col, Col, Col>(s[0], s[1], s[2], 0, 0, 11, "min / saturating-plus i32 ccc");
+    run_case<cuasr::minimum<int32_t>, saturating_plus<int32_t>, int32_t, Row, Col, Row>(s[0], s[1], s[2], 5, 1000, 12, "min / saturating-plus i32 rcr, beta = annihilator");
+    // user add (order-dependent on ties), library mult
+    run_case<abs_max<float>, cuasr::multiplies<float>, float, Col, Row, Col>(s[0], s[1], s[2], 1.0f, 1.0f, 13, "abs-max / times f32 crc");
+    run_case<abs_max<float>, cuasr::multiplies<float>, float, Row, Row, Row>(s[0], s[1], s[2], -2.0f, 0.5f, 14, "abs-max / times f32 rrr");
+    // both user-defined, a non-associative add in double: only the host's own order gives these bits
+    run_case<leaky_plus<double>, saturating_plus<double>, double, Col, Col, Row>(s[0], s[1], s[2], 1.5, 0.5, 15, "leaky-plus / saturating-plus f64 ccr");
+  }
+  // the run-time checks that do not depend on the functors
+  {
+    using Op = cuasr::gemm::device::Srgemm<abs_max<float>, cuasr::multiplies<float>, float, Col, float, Col, float, Col, float>;
+    float *d = nullptr;
+    HIP_CHECK(hipMalloc(&d, 64 * 64 * 4));
+    typename Op::Arguments bad_ld({64, 64, 64}, {d, 10}, {d, 64}, {d, 64}, {d, 64}, {1.0f, 1.0f});
+    check(Op::can_implement(bad_ld) == cuasr::Status::kErrorInvalidProblem, "leading dimension smaller than the extent is refused");
+    typename Op::Arguments split({64, 64, 64}, {d, 64}, {d, 64}, {d, 64}, {d, 64}, {1.0f, 1.0f}, 4);
+    check(Op::can_implement(split) == cuasr::Status::kErrorInvalidProblem, "split_k_slices > 1 is refused (device/srgemm.h:198-200)");
+    Op op;
+    check(op.run() == cuasr::Status::kErrorInternal, "run before initialize is refused");
+    HIP_CHECK(hipFree(d));
+  }
+  std::printf("%d checks, %d failed\n", g_run, g_fail);
+  return g_fail ? 1 : 0;
+}

@@ -222,3 +222,33 @@ def test_inputs_are_reproducible():
     assert np.all(np.diag(g) == 0) and np.isinf(g).mean() > 0.8
     w = inputs.words32(3, 64, 64)
     assert w.dtype == np.uint32 and 0.4 < np.unpackbits(np.ascontiguousarray(w).view(np.uint8)).mean() < 0.6
+
+
+def test_user_functor_without_hipcc_is_a_readable_compile_error(tmp_path):
+    """A functor that is none of the library's operators needs its kernel built from the functor: with a
+    host-only compiler device::Srgemm::run must stop the build with a message that says what to do."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    src = tmp_path / "user.cpp"
+    src.write_text("""
+#include "cuasr/gemm/device/srgemm.h"
+template <typename T, int N = 1> struct my_op {
+  static constexpr T Identity = 0, Annihilator = 0;
+  T operator()(T l, T const &r) const { return l + 2 * r; }
+};
+int main() {
+  using L = cuasr::layout::ColumnMajor;
+  cuasr::gemm::device::Srgemm<my_op<float>, cuasr::plus<float>, float, L, float, L, float, L, float> op;
+  return (int)op.run();
+}
+""")
+    cmd = ["g++", "-std=c++17", "-fsyntax-only", "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include",
+           "-I", os.path.join(root, "include"), str(src)]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "compile this translation unit with hipcc" in r.stderr
+    # the same program with library functors compiles with the host compiler alone
+    src.write_text(src.read_text().replace("my_op<float>", "cuasr::minimum<float>"))
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]

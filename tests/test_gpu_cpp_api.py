@@ -21,3 +21,17 @@ def test_cpp_operator_api(lib):
     print(r.stderr[-2000:])
     assert r.returncode == 0, r.stdout[-4000:]
     assert "0 failed" in r.stdout
+
+
+def test_cpp_user_defined_functors(lib):
+    """tests/cpp/test_user_functor.hip: device::Srgemm with functors the library has no operator for (the
+    kernel is built from the functors, in a translation unit compiled by hipcc) against the host reference."""
+    binary = os.path.join(HERE, "cpp", "test_user_functor")
+    if not os.path.exists(binary):
+        from cuasr_amd import build
+        build.build_cpp_tests()
+    r = subprocess.run([binary], capture_output=True, text=True, timeout=600)
+    print(r.stdout[-4000:])
+    print(r.stderr[-2000:])
+    assert r.returncode == 0, r.stdout[-4000:]
+    assert "0 failed" in r.stdout
