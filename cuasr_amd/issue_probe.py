@@ -1,0 +1,168 @@
+"""Instruction-issue probe for gfx950: the measurements the hand-scheduled main loops
+(csrc/gen_direct_asm.py) are designed around, and the ceiling they are judged against.
+
+    python -m cuasr_amd.issue_probe --build      # writes and compiles cuasr_amd/lib/issue_probe (hipcc, no GPU needed)
+    cuasr_amd/lib/issue_probe [iterations]       # runs it on the GPU, prints one line per loop
+
+Every loop is one inline-asm block of the fp32 min-plus inner loop of an 8 x 8 register tile (64
+groups of add, add, min3 = 128 terms per lane) or a variation of it, run by 256-thread workgroups,
+1 to 4 per compute unit (= 1 to 4 waves per SIMD), with nothing else in the loop:
+    add / min3 / min / fma / fmac alone   what one instruction kind issues at
+    mix                                   the min-plus group itself: the ceiling of any min-plus kernel
+    mix + SGPR operand                    a fragment broadcast through scalar registers
+    mix + N LDS reads (4 / 8 / 16 bytes)  what fetching the fragments costs (results not consumed)
+    mix + N waits / nops / scalar adds    what an instruction that does no arithmetic costs
+    fp64 add / max / mix (+ the same)     the same questions for 8-byte elements
+Times are HIP events around the second of two launches; the clock is read inside the kernel
+(shader cycle counter against the 100 MHz wall clock), so cycle figures are per measured clock.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+OUT = os.path.join(HERE, "lib", "issue_probe")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+ACC = list(range(32, 96))
+A0, A1 = list(range(96, 104)), list(range(104, 112))
+B0, B1 = list(range(112, 120)), list(range(120, 128))
+T = list(range(24, 32))
+
+
+def mix(sgpr_b=False):
+    groups, t = [], 0
+    for i in range(8):
+        for j in range(8):
+            t0, t1 = T[t % 8], T[(t + 1) % 8]
+            t += 2
+            b0 = f"s{16 + j}" if sgpr_b else f"v{B0[j]}"
+            b1 = f"s{24 + j}" if sgpr_b else f"v{B1[j]}"
+            acc = ACC[i * 8 + j]
+            groups.append([f"v_add_f32 v{t0}, {b0}, v{A0[i]}", f"v_add_f32 v{t1}, {b1}, v{A1[i]}",
+                           f"v_min3_f32 v{acc}, v{acc}, v{t0}, v{t1}"])
+    return groups
+
+
+def sprinkle(groups, n, make):
+    """n extra instructions spread evenly over the groups"""
+    lines, every, c = [], (len(groups) // n if n else 10 ** 9), 0
+    for gi, grp in enumerate(groups):
+        if n and gi % every == 0 and c < n:
+            lines.append(make(c))
+            c += 1
+        lines += grp
+    return lines
+
+
+def only(template, n=192):
+    return [template.format(t=T[x % 8], acc=ACC[x % 64], a=A0[(x // 8) % 8], b=B0[x % 8], s=16 + x % 8) for x in range(n)]
+
+
+def lds_read(width):
+    regs = {32: list(range(4, 20)), 64: list(range(4, 20, 2)), 128: [4, 8, 12, 16]}[width]
+    name = {32: lambda r: f"v{r}", 64: lambda r: f"v[{r}:{r + 1}]", 128: lambda r: f"v[{r}:{r + 3}]"}[width]
+    return lambda c: f"ds_read_b{width} {name(regs[c % len(regs)])}, %0 offset:{(c * 1024) % 32768}"
+
+
+def f64_mix():
+    acc = [32 + 2 * i for i in range(32)]
+    a = [96 + 2 * i for i in range(8)]
+    b = [112 + 2 * i for i in range(4)]
+    t = [16 + 2 * i for i in range(4)]
+    r = lambda x: f"v[{x}:{x + 1}]"
+    return [[f"v_add_f64 {r(t[(i * 4 + j) % 4])}, {r(a[i])}, {r(b[j])}",
+             f"v_max_f64 {r(acc[i * 4 + j])}, {r(acc[i * 4 + j])}, {r(t[(i * 4 + j) % 4])}"] for i in range(8) for j in range(4)]
+
+
+def kernels():
+    k = {}  # name -> (lines, instructions counted, terms per lane, "f32" | "f64")
+    flat = lambda g: [ln for grp in g for ln in grp]
+    k["add_f32"] = (only("v_add_f32 v{t}, v{b}, v{a}"), 192, 0, "f32")
+    k["add_f32_sgpr_operand"] = (only("v_add_f32 v{t}, s{s}, v{a}"), 192, 0, "f32")
+    k["min3_f32"] = (only("v_min3_f32 v{acc}, v{acc}, v{b}, v{a}"), 192, 0, "f32")
+    k["min_f32"] = (only("v_min_f32 v{acc}, v{acc}, v{b}"), 192, 0, "f32")
+    k["fma_f32_vop3"] = (only("v_fma_f32 v{acc}, v{b}, v{a}, v{acc}"), 192, 0, "f32")
+    k["fmac_f32_vop2"] = (only("v_fmac_f32 v{acc}, v{b}, v{a}"), 192, 0, "f32")
+    k["bitop3_b32"] = (only("v_bitop3_b32 v{acc}, v{b}, v{a}, v{acc} bitop3:0x6a"), 192, 0, "f32")
+    k["mix"] = (flat(mix()), 192, 128, "f32")
+    k["mix_sgpr_b"] = (flat(mix(True)), 192, 128, "f32")
+    for n in (4, 8, 16):
+        for w in (64, 128):
+            k[f"mix_lds{n}_b{w}"] = (sprinkle(mix(), n, lds_read(w)), 192, 128, "f32")
+    for n in (16, 64):
+        k[f"mix_waitcnt{n}"] = (sprinkle(mix(), n, lambda c: "s_waitcnt lgkmcnt(0)"), 192, 128, "f32")
+        k[f"mix_nop{n}"] = (sprinkle(mix(), n, lambda c: "s_nop 0"), 192, 128, "f32")
+        k[f"mix_salu{n}"] = (sprinkle(mix(), n, lambda c: "s_add_u32 s20, s20, 1"), 192, 128, "f32")
+    g64 = f64_mix()
+    k["add_f64"] = ([g[0] for g in g64] * 2, 64, 0, "f64")
+    k["max_f64"] = ([g[1] for g in g64] * 2, 64, 0, "f64")
+    k["mix_f64"] = (flat(g64), 64, 32, "f64")
+    k["mix_f64_lds6_b128"] = (sprinkle(g64, 6, lds_read(128)), 64, 32, "f64")
+    k["mix_f64_waitcnt8"] = (sprinkle(g64, 8, lambda c: "s_waitcnt lgkmcnt(0)"), 64, 32, "f64")
+    k["mix_f64_nop32"] = (sprinkle(g64, 32, lambda c: "s_nop 0"), 64, 32, "f64")
+    return k
+
+
+def source():
+    clob = ",".join(f'"v{r}"' for r in range(4, 128)) + "," + ",".join(f'"s{r}"' for r in range(16, 32)) + ',"scc"'
+    out = ["// written by cuasr_amd/issue_probe.py", "#include <hip/hip_runtime.h>", "#include <cstdio>", "#include <cstdlib>",
+           '#define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)']
+    ks = kernels()
+    for name, (lines, _, _, _) in ks.items():
+        body = "\\n".join(lines + ["s_waitcnt lgkmcnt(0)"])
+        out.append(f'''__global__ __launch_bounds__(256) void k_{name}(unsigned long long *out, int iters) {{
+  __shared__ float lds[9216];
+  for (int i = threadIdx.x; i < 9216; i += 256) lds[i] = i;
+  __syncthreads();
+  const unsigned addr = (unsigned)(size_t)(__attribute__((address_space(3))) float *)&lds[0] + (threadIdx.x & 63) * 16;
+  const unsigned long long c0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {{
+    asm volatile("{body}" :: "v"(addr) : {clob});
+  }}
+  const unsigned long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
+  if (threadIdx.x == 0) {{ out[2 * blockIdx.x] = c1 - c0; out[2 * blockIdx.x + 1] = w1 - w0; }}
+}}''')
+    out.append('''int main(int argc, char **argv) {
+  setvbuf(stdout, NULL, _IONBF, 0);
+  hipDeviceProp_t prop; CK(hipGetDeviceProperties(&prop, 0));
+  unsigned long long *out, *h = (unsigned long long *)malloc(16 * 8192);
+  CK(hipMalloc(&out, 16 * 8192));
+  hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+  const int iters = argc > 1 ? atoi(argv[1]) : 20000;
+  printf("%s, %d compute units; %d iterations per launch\\n", prop.name, prop.multiProcessorCount, iters);
+  for (int bpc : {1, 2, 3, 4}) {
+    const int blocks = prop.multiProcessorCount * bpc;
+    auto run = [&](auto kern, const char *name, double ninstr, double terms, double ops_per_term) {
+      hipLaunchKernelGGL(kern, blocks, 256, 0, 0, out, iters); CK(hipDeviceSynchronize());
+      CK(hipEventRecord(e0)); hipLaunchKernelGGL(kern, blocks, 256, 0, 0, out, iters); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+      float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+      CK(hipMemcpy(h, out, 16 * blocks, hipMemcpyDeviceToHost));
+      double cyc = 0, wall = 0; for (int b = 0; b < blocks; ++b) { cyc += h[2 * b]; wall += h[2 * b + 1]; }
+      const double ghz = cyc / (wall * 10.0);   // the wall clock ticks at 100 MHz
+      printf("waves/SIMD %d  %-22s %8.3f ms  %.2f GHz  %5.2f cycles per counted instruction and SIMD", bpc, name, ms, ghz,
+             ms * 1e-3 * ghz * 1e9 / (ninstr * iters * bpc));
+      if (terms > 0) printf("  %6.1f TOPS", ops_per_term * terms * iters * 256.0 * blocks / ms / 1e9);
+      printf("\\n");
+    };''')
+    for name, (_, ninstr, terms, _) in ks.items():
+        out.append(f'    run(k_{name}, "{name}", {ninstr}, {terms}, 2.0);')
+    out.append("  }\n  return 0;\n}")
+    return "\n".join(out)
+
+
+def build():
+    os.makedirs(os.path.dirname(OUT), exist_ok=True)
+    os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    src = os.path.join(HERE, "build", "issue_probe.hip")
+    with open(src, "w") as f:
+        f.write(source())
+    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O3", "-w", "-o", OUT, src])
+    return OUT
+
+
+if __name__ == "__main__":
+    if "--build" in sys.argv:
+        print(build())
+    else:
+        print(__doc__)
