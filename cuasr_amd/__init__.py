@@ -22,7 +22,7 @@ OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
        "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
 DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3}
 COLUMN_MAJOR, ROW_MAJOR = 0, 1
-KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3, "direct": 4}
+KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3, "direct": 4, "streamk": 5}
 STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
                 "kErrorInvalidLayout", "kErrorInvalidProblem", "kErrorNotSupported",
                 "kErrorWorkspaceNull", "kErrorInternal", "kErrorArchMismatch",

@@ -18,6 +18,9 @@ launch_fn find_direct_f32(int, int);
 launch_fn find_direct_i32(int, int);
 launch_fn find_direct_u32(int, int);
 launch_fn find_direct_f64(int, int);
+streamk_fn find_streamk_f32(int, int);
+streamk_fn find_streamk_i32(int, int);
+streamk_fn find_streamk_u32(int, int);
 bool direct_can_run(const Problem &);
 bool direct64_can_run(const Problem &);
 bool mfma_f32_can_run(const Problem &);
@@ -39,6 +42,15 @@ launch_fn find_direct(int dtype, int add_op, int mult_op) {
     case CUASR_AMD_I32: return find_direct_i32(add_op, mult_op);
     case CUASR_AMD_U32: return find_direct_u32(add_op, mult_op);
     case CUASR_AMD_F64: return find_direct_f64(add_op, mult_op);
+    default: return nullptr;
+  }
+}
+
+streamk_fn find_streamk(int dtype, int add_op, int mult_op) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return find_streamk_f32(add_op, mult_op);
+    case CUASR_AMD_I32: return find_streamk_i32(add_op, mult_op);
+    case CUASR_AMD_U32: return find_streamk_u32(add_op, mult_op);
     default: return nullptr;
   }
 }
@@ -75,6 +87,28 @@ static bool direct_usable(const cuasr_amd_srgemm_desc *d) {
   return d->dtype == CUASR_AMD_F64 ? direct64_can_run(canonical(d)) : direct_can_run(canonical(d));
 }
 
+// The stream-K form of the direct tile: exact only for an add that does not depend on the order or grouping of
+// its terms, with alpha = the multiplicative identity given by value, on the panel forms that have a hand-scheduled loop.
+static bool streamk_usable(const cuasr_amd_srgemm_desc *d) {
+  if (!find_streamk(d->dtype, d->add_op, d->mult_op) || !direct_usable(d)) return false;
+  const Problem c = canonical(d);
+  if (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) return false;  // both k-contiguous: no such loop
+  if (d->alpha_ptr) return false;
+  const uint64_t mask = elem_size(d->dtype) == 8 ? ~0ull : 0xffffffffull;
+  return ((d->alpha.bits ^ d->mult_identity.bits) & mask) == 0;
+}
+
+// ... and worth it: the plain tiles would leave a good part of their last round of 512 places empty, and every
+// workgroup's share of the k-tiles is long enough to carry a tile's prologue and fold
+static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
+  if (batch != 1 || d->split_k_slices != 1 || !streamk_usable(d)) return false;
+  const Problem c = canonical(d);
+  const long long tiles = (long long)((c.m + 255) / 256) * ((c.n + 127) / 128), ktiles = (c.k + 15) / 16;
+  const long long rounds = (tiles + 511) / 512;
+  if (tiles * 10 >= rounds * 512 * 9) return false;   // >= 90 % of the places filled: nothing to gain
+  return tiles >= 64 && tiles * ktiles >= 512 * 48;
+}
+
 static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (!d) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_U32) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
@@ -87,7 +121,7 @@ static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (d->m < 0 || d->n < 0 || d->k < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->reserved != 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (splitk ? d->split_k_slices < 1 : d->split_k_slices != 1) return CUASR_AMD_ERROR_INVALID_PROBLEM;
-  if (d->kernel < CUASR_AMD_KERNEL_AUTO || d->kernel > CUASR_AMD_KERNEL_VALU_DIRECT) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->kernel < CUASR_AMD_KERNEL_AUTO || d->kernel > CUASR_AMD_KERNEL_VALU_STREAMK) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   auto min_ld = [](int layout, int rows, int cols) { return (long long)(layout == CUASR_AMD_COLUMN_MAJOR ? rows : cols); };
   if (d->m > 0 && d->k > 0 && d->lda < min_ld(d->layout_a, d->m, d->k)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->n > 0 && d->k > 0 && d->ldb < min_ld(d->layout_b, d->k, d->n)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
@@ -105,6 +139,7 @@ static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
     return CUASR_AMD_ERROR_NOT_SUPPORTED;
   if (d->kernel == CUASR_AMD_KERNEL_MFMA && !mfma_usable(d)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   if (d->kernel == CUASR_AMD_KERNEL_VALU_DIRECT && !direct_usable(d)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+  if (d->kernel == CUASR_AMD_KERNEL_VALU_STREAMK && (d->split_k_slices != 1 || !streamk_usable(d))) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   return CUASR_AMD_SUCCESS;
 }
 
@@ -136,7 +171,7 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d) {
   return p;
 }
 
-enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4 };
+enum Family { kNaive = 1, kValu = 2, kMfma = 3, kDirect = 4, kStreamK = 5 };
 
 static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   if (d->kernel != CUASR_AMD_KERNEL_AUTO) return d->kernel;
@@ -171,6 +206,7 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   // panel forms (two k-quad operands do not fit 128 registers) and its 2-wave variant is slower than the
   // staged tile (4096^3 min-plus: 70.4 against 72.9 TOPS)
   const bool both_kc = !f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
+  if (streamk_preferred(d, batch)) return kStreamK;
   if (direct_usable(d) && ((fills && !((both_kc || masked) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
@@ -225,6 +261,20 @@ static Problem sub_problem(const Problem &p, size_t es, int r0, int c0, int rows
   return q;
 }
 
+// compute units of the current device (asked once per device)
+static int compute_units(void) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<int> table[kMaxDevices];
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 0;
+  int n = table[dev].load(std::memory_order_relaxed);
+  if (n <= 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+    table[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 static launch_fn family_fn(int family, const cuasr_amd_srgemm_desc *d) {
   switch (family) {
     case kMfma: return find_mfma(d->dtype, d->add_op, d->mult_op);
@@ -266,6 +316,7 @@ const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc) {
   switch (pick_family(desc)) {
     case kMfma: return "mfma";
     case kDirect: return "valu_direct";
+    case kStreamK: return "valu_streamk";
     case kValu: return direct_block(desc, canonical(desc)).rows ? "valu_direct+valu" : "valu";  // a block + two strips
     default: return "naive";
   }
@@ -276,9 +327,19 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   if (st != CUASR_AMD_SUCCESS) return st;
   const Problem p = canonical(desc);
   const int family = pick_family(desc);
-  const launch_fn fn = family_fn(family, desc);
+  const launch_fn fn = family == kStreamK ? find_direct(desc->dtype, desc->add_op, desc->mult_op) : family_fn(family, desc);
   if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (family == kStreamK) {
+    // the source term into D, then the product folded into it by two workgroups per compute unit
+    const prepare_fold_fn prepare = find_prepare_fold(desc->dtype);
+    const streamk_fn run = find_streamk(desc->dtype, desc->add_op, desc->mult_op);
+    const int groups = 2 * compute_units();
+    if (!prepare || !run || groups <= 0) return CUASR_AMD_ERROR_NOT_SUPPORTED;
+    const long long tiles = (long long)((p.m + 255) / 256) * ((p.n + 127) / 128);  // the direct tile is 256 x 128
+    if (prepare(p, 256, 128, tiles / groups * groups, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    return run(p, groups, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+  }
   if (family == kValu) {
     const Block b = direct_block(desc, p);
     const launch_fn direct = b.rows ? find_direct(desc->dtype, desc->add_op, desc->mult_op) : nullptr;
@@ -371,6 +432,7 @@ static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *
   // operands only, so a workspace that is element-aligned but not 16-byte aligned is sorted out here:
   // AUTO goes on to the staged family (or the naive kernel), a forced direct tile is refused.
   int family = pick_family(desc);
+  if (family == kStreamK) family = kDirect;  // (one slice through the split-K entry points: the plain tile)
   if (family == kDirect && !(desc->dtype == CUASR_AMD_F64 ? direct64_can_run(p) : direct_can_run(p))) {
     if (desc->kernel != CUASR_AMD_KERNEL_AUTO) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
     family = find_valu(desc->dtype, desc->add_op, desc->mult_op) ? kValu : kNaive;

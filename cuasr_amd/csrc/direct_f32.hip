@@ -18,4 +18,14 @@ launch_fn find_direct_f32(int add_op, int mult_op) {
 
 bool direct_can_run(const Problem &p) { return direct_ok(p); }
 
+// the semirings whose stream-K form is exact: the add neither depends on the order or grouping of its
+// terms nor has to be distributed over (alpha is the multiplicative identity there)
+streamk_fn find_streamk_f32(int add_op, int mult_op) {
+  if (add_op == kMinimum && mult_op == kPlus) return launch_direct_streamk<float, kMinimum, kPlus>;
+  if (add_op == kMaximum && mult_op == kPlus) return launch_direct_streamk<float, kMaximum, kPlus>;
+  if (add_op == kMaximum && mult_op == kMinimum) return launch_direct_streamk<float, kMaximum, kMinimum>;
+  if (add_op == kMinimum && mult_op == kMaximum) return launch_direct_streamk<float, kMinimum, kMaximum>;
+  return nullptr;
+}
+
 }  // namespace cuasr_amd

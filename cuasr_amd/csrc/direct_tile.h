@@ -290,21 +290,61 @@ struct DirectTile {
     (relaxed_kpair<KP>(acc, a, b, a_addr, b_addr), ...);
   }
 
+  // what a workgroup does with the accumulators of a segment (one output tile, a range of k)
+  enum : int {
+    kEpilogue = 0,    // the whole product: D = add(mult(alpha, acc), mult(beta, C)); or a split-K slice: raw partials to the workspace
+    kFoldOwned = 1,   // D already holds mult(beta, C) (or the identity): D = add(acc, D); this workgroup alone works on the tile
+    kFoldShared = 2   // the same, but other workgroups fold other ranges of k into the same tile: one atomic fold per element
+  };
+
   static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
-    const int tid = threadIdx.x, tx = tid % TX, ty = tid / TX, lane = tid & 63, wave = tid >> 6;
     const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
     int bm, bn;
     tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
-    const int m0 = bm * BM, n0 = bn * BN;
-    const T *A = reinterpret_cast<const T *>(p.A);
-    const T *B = reinterpret_cast<const T *>(p.B);
-    const T ident = scalar_as<T>(p.add_identity);
-
     int kb = 0, ke = p.k;
     if (p.workspace) {
       kb = blockIdx.y * p.k_per_slice;
       ke = min(p.k, kb + p.k_per_slice);
     }
+    segment(p, sm, bm * BM, bn * BN, kb, ke, kEpilogue);
+  }
+
+  // add(v, *addr) into *addr, atomically at device scope and without waiting for an answer.  The adds of the
+  // semirings that run in this form all have a native atomic: xor / or on words; minimum and maximum of
+  // floats through the integer atomics (a float without sign bit orders like its bits as a signed integer, one
+  // with sign bit the other way round like its bits as an unsigned integer, and every float of the second kind is
+  // below every float of the first both as a number and as a signed integer / above as an unsigned one).
+  static __device__ __forceinline__ void atomic_fold(T *addr, T v) {
+    const int bits = __builtin_bit_cast(int, v);
+    int *si = reinterpret_cast<int *>(addr);
+    unsigned *ui = reinterpret_cast<unsigned *>(addr);
+    if constexpr (ADD == kBitXor) {
+      __hip_atomic_fetch_xor(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (ADD == kBitOr) {
+      __hip_atomic_fetch_or(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (ADD == kMinimum && is_fp<T>::value) {
+      if (bits >= 0) __hip_atomic_fetch_min(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_fetch_max(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if constexpr (ADD == kMaximum && is_fp<T>::value) {
+      if (bits >= 0) __hip_atomic_fetch_max(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_fetch_min(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      // any other add: a compare-and-swap loop (no semiring that is launched in this form gets here)
+      unsigned old = __hip_atomic_load(ui, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      while (true) {
+        const unsigned want = __builtin_bit_cast(unsigned, fold_epilogue<ADD, MUL>(v, __builtin_bit_cast(T, old)));
+        if (want == old) break;
+        if (__hip_atomic_compare_exchange_strong(ui, &old, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+      }
+    }
+  }
+
+  static __device__ __forceinline__ void segment(const Problem &p, Smem &sm, const int m0, const int n0, const int kb, const int ke,
+                                                 const int mode) {
+    const int tid = threadIdx.x, tx = tid % TX, ty = tid / TX, lane = tid & 63, wave = tid >> 6;
+    const T *A = reinterpret_cast<const T *>(p.A);
+    const T *B = reinterpret_cast<const T *>(p.B);
+    const T ident = scalar_as<T>(p.add_identity);
 
     // each wave moves 2 x 1 KiB of the A panel and 2 x 1 KiB of the B panel per k-tile
     const char *base_a = reinterpret_cast<const char *>(A + (long long)m0 * p.sa_m + (long long)kb * p.sa_k);
@@ -487,6 +527,26 @@ struct DirectTile {
       }
     }
 
+    if (mode != kEpilogue) {
+      // ---- fold into D, which already holds the source term (alpha is the multiplicative identity here)
+      T *D = reinterpret_cast<T *>(p.D);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int row = m0 + own<A_KC, TY>(i, ty);
+        if ((unsigned)row < (unsigned)p.m) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int col = n0 + own<B_KC, TX>(j, tx);
+            if ((unsigned)col < (unsigned)p.n) {
+              T *at = D + (long long)row * p.ldd + col;
+              if (mode == kFoldShared) atomic_fold(at, acc[i][j]);
+              else *at = fold_epilogue<ADD, MUL>(acc[i][j], *at);
+            }
+          }
+        }
+      }
+      return;
+    }
     // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or raw partials
     T *out;
     long long ld_out;
@@ -553,6 +613,46 @@ __global__ __launch_bounds__(TY *TX) __attribute__((amdgpu_waves_per_eu(4, 4))) 
   __shared__ typename Tile::Smem sm;
   select_batch<T>(p);
   Tile::run(p, sm);
+}
+
+// The same tile with the work of the last, partly filled round shared out evenly ("stream-K").  With G
+// workgroups (two per compute unit) and T output tiles, the first floor(T / G) * G tiles are whole tiles as in
+// the plain kernel, workgroup w taking tiles w, w + G, ...; the remaining R < G tiles are R x k-tiles units of work
+// in tile-major order, of which workgroup w takes units [w * total / G, (w + 1) * total / G) -- a run of k-tiles
+// that may end one output tile and begin the next.  For outputs whose tiles do not fill whole rounds of the chip
+// (3072^2 is 288 tiles for 512 places, 5120^2 is 800) every workgroup then still has the same amount of work.
+// The ranges of k of a shared tile meet in D: a launch before this one writes the source term into those tiles
+// (prepare_fold_kernel), a workgroup that happens to have such a tile to itself folds its accumulators into it
+// with plain loads and stores, the others with one atomic per element.  Only for adds whose result does not
+// depend on the order or grouping of the terms, and with alpha = the multiplicative identity (so that nothing
+// has to distribute over the add).
+template <typename T, int ADD, int MUL, bool A_KC, bool B_KC, int TY, int TX>
+__global__ __launch_bounds__(TY *TX) __attribute__((amdgpu_waves_per_eu(4, 4))) void direct_streamk_kernel(Problem p) {
+  using Tile = DirectTile<T, ADD, MUL, A_KC, B_KC, TY, TX>;
+  __shared__ typename Tile::Smem sm;
+  const int tiles_m = (p.m + Tile::BM - 1) / Tile::BM, tiles_n = (p.n + Tile::BN - 1) / Tile::BN;
+  const long long tiles = (long long)tiles_m * tiles_n, whole = tiles / gridDim.x * gridDim.x;
+  bool first = true;
+  int bm, bn;
+  for (long long tile = blockIdx.x; tile < whole; tile += gridDim.x) {
+    streamk_tile_coords(tile, tiles_m, tiles_n, bm, bn);
+    if (!first) __syncthreads();  // every wave is done with the LDS panels of the previous tile
+    first = false;
+    Tile::segment(p, sm, bm * Tile::BM, bn * Tile::BN, 0, p.k, Tile::kEpilogue);
+  }
+  const long long ktiles = (p.k + Tile::BK - 1) / Tile::BK, total = (tiles - whole) * ktiles;
+  long long u = total * blockIdx.x / gridDim.x;
+  const long long end = total * (blockIdx.x + 1) / gridDim.x;
+  while (u < end) {
+    const long long r = u / ktiles;
+    const int kt0 = (int)(u - r * ktiles), kt1 = (int)(end - r * ktiles < ktiles ? end - r * ktiles : ktiles);
+    streamk_tile_coords(whole + r, tiles_m, tiles_n, bm, bn);
+    if (!first) __syncthreads();
+    first = false;
+    Tile::segment(p, sm, bm * Tile::BM, bn * Tile::BN, kt0 * Tile::BK, min(p.k, kt1 * Tile::BK),
+                  (kt0 == 0 && kt1 == ktiles) ? Tile::kFoldOwned : Tile::kFoldShared);
+    u += kt1 - kt0;
+  }
 }
 
 template <typename T, int ADD, int MUL, bool A_KC, bool B_KC>
@@ -627,6 +727,25 @@ template <typename T, int ADD, int MUL> static hipError_t launch_direct(const Pr
   else if (b_kc) launch_kernel((direct_srgemm_kernel<T, ADD, MUL, false, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
   else launch_kernel((direct_srgemm_kernel<T, ADD, MUL, false, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
   return take_launch_status();
+}
+
+// stream-K form of the direct tile (see direct_streamk_kernel); `groups` workgroups, normally two per compute unit.
+// The tiles from floor(tiles / groups) * groups on must already hold the source term (prepare_fold_kernel with this
+// tile's extents, CUASR_AMD_DIRECT_TY * 8 x CUASR_AMD_DIRECT_TX * 8).
+template <typename T, int ADD, int MUL> static hipError_t launch_direct_streamk(const Problem &p, int groups, hipStream_t s) {
+  constexpr int TY = CUASR_AMD_DIRECT_TY, TX = CUASR_AMD_DIRECT_TX;
+  if (p.m == 0 || p.n == 0 || p.k == 0) return hipSuccess;
+  if (!direct_ok(p) || direct_prefers_relaxed(p) || p.workspace || p.batch != 1 || groups < 1) return hipErrorNotSupported;
+  if constexpr (std::is_void<typename AsmLoop<T, ADD, MUL, false, false>::type>::value) {
+    return hipErrorNotSupported;
+  } else {
+    const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
+    dim3 grid((unsigned)groups);
+    if (a_kc) launch_kernel((direct_streamk_kernel<T, ADD, MUL, true, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+    else if (b_kc) launch_kernel((direct_streamk_kernel<T, ADD, MUL, false, true, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+    else launch_kernel((direct_streamk_kernel<T, ADD, MUL, false, false, TY, TX>), grid, dim3(TY * TX), 0, s, p);
+    return take_launch_status();
+  }
 }
 
 }  // namespace cuasr_amd

@@ -16,4 +16,12 @@ launch_fn find_direct_u32(int add_op, int mult_op) {
   return nullptr;
 }
 
+// the semirings whose stream-K form is exact: the add neither depends on the order or grouping of its
+// terms nor has to be distributed over (alpha is the multiplicative identity there)
+streamk_fn find_streamk_u32(int add_op, int mult_op) {
+  if (add_op == kBitXor && mult_op == kBitAnd) return launch_direct_streamk<uint32_t, kBitXor, kBitAnd>;
+  if (add_op == kBitOr && mult_op == kBitAnd) return launch_direct_streamk<uint32_t, kBitOr, kBitAnd>;
+  return nullptr;
+}
+
 }  // namespace cuasr_amd

@@ -217,6 +217,42 @@ template <typename T, bool SERIAL> static hipError_t launch_reduce(const Problem
   return take_launch_status();
 }
 
+// ------------------------------------------------------------ source term for the stream-K tiles
+// D <- mult(beta, C) where the source is needed, else the additive identity, on the output tiles (bm x bn) from
+// `first` on in the stream-K tile order: what the workgroups that share those tiles fold their ranges of k into
+// (the epilogue's add then has nothing left to do).  One workgroup per tile.  D may be C.
+template <typename T> __global__ __launch_bounds__(256) void prepare_fold_kernel(Problem p, int bm, int bn, long long first) {
+  const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
+  const int tiles_m = (p.m + bm - 1) / bm, tiles_n = (p.n + bn - 1) / bn;
+  int tm, tn;
+  streamk_tile_coords(first + blockIdx.x, tiles_m, tiles_n, tm, tn);
+  const int m0 = tm * bm, n0 = tn * bn;
+  for (int idx = threadIdx.x; idx < bm * bn; idx += 256) {
+    const int row = m0 + idx / bn, col = n0 + idx % bn;
+    if (row < p.m && col < p.n) {
+      T v = e.ident;
+      if (e.source_needed) v = apply_op<T>(p.mult_op, e.beta, reinterpret_cast<const T *>(p.C)[(long long)row * p.ldc + col]);
+      reinterpret_cast<T *>(p.D)[(long long)row * p.ldd + col] = v;
+    }
+  }
+}
+
+template <typename T> static hipError_t launch_prepare_fold(const Problem &p, int bm, int bn, long long first, hipStream_t s) {
+  const long long tiles = (long long)((p.m + bm - 1) / bm) * ((p.n + bn - 1) / bn);
+  if (tiles <= first) return hipSuccess;
+  launch_kernel(prepare_fold_kernel<T>, dim3((unsigned)(tiles - first)), dim3(256), 0, s, p, bm, bn, first);
+  return take_launch_status();
+}
+
+prepare_fold_fn find_prepare_fold(int dtype) {
+  switch (dtype) {
+    case CUASR_AMD_F32: return launch_prepare_fold<float>;
+    case CUASR_AMD_I32: return launch_prepare_fold<int32_t>;
+    case CUASR_AMD_U32: return launch_prepare_fold<uint32_t>;
+    default: return nullptr;
+  }
+}
+
 launch_fn find_reduce(int dtype) {
   switch (dtype) {
     case CUASR_AMD_F32: return launch_reduce<float, false>;

@@ -170,6 +170,15 @@ template <typename T> __device__ __forceinline__ EpilogueScalars<T> resolve_scal
   return e;
 }
 
+// Tile order of the stream-K launches (the kernel and the launch that prepares D must agree on it): down
+// the columns of a band of 8 tile rows, so that workgroups with neighbouring ids share panels.
+__host__ __device__ __forceinline__ void streamk_tile_coords(long long tile, int tiles_m, int tiles_n, int &bm, int &bn) {
+  const int band = (int)(tile / (8LL * tiles_n)), in_band = (int)(tile - (long long)band * 8 * tiles_n);
+  const int rows = tiles_m - band * 8 < 8 ? tiles_m - band * 8 : 8;
+  bm = band * 8 + in_band % rows;
+  bn = in_band / rows;
+}
+
 typedef hipError_t (*launch_fn)(const Problem &, hipStream_t);
 
 // Kernel launches report the launch call's own status.  (hipGetLastError() after a launch would also
@@ -202,5 +211,10 @@ launch_fn find_valu(int dtype, int add_op, int mult_op);
 launch_fn find_mfma(int dtype, int add_op, int mult_op);
 launch_fn find_reduce(int dtype);
 launch_fn find_reduce_serial(int dtype);
+// the stream-K form of the direct tile: (problem, workgroups, stream), and the launch before it that writes the
+// source term into the output tiles the workgroups share: (problem, tile rows, tile columns, first shared tile, stream)
+typedef hipError_t (*streamk_fn)(const Problem &, int, hipStream_t);
+typedef hipError_t (*prepare_fold_fn)(const Problem &, int, int, long long, hipStream_t);
+prepare_fold_fn find_prepare_fold(int dtype);
 
 }  // namespace cuasr_amd

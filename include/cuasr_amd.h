@@ -88,8 +88,14 @@ typedef enum cuasr_amd_kernel {
   CUASR_AMD_KERNEL_NAIVE = 1, /* one thread per output element               */
   CUASR_AMD_KERNEL_VALU = 2,  /* LDS-staged, register-blocked vector-ALU tile */
   CUASR_AMD_KERNEL_MFMA = 3,  /* matrix-core assisted tile                    */
-  CUASR_AMD_KERNEL_VALU_DIRECT = 4 /* vector-ALU tile fed by direct-to-LDS loads;
-                                      needs 16-byte aligned, vector-sized operands */
+  CUASR_AMD_KERNEL_VALU_DIRECT = 4, /* vector-ALU tile fed by direct-to-LDS loads;
+                                       needs 16-byte aligned, vector-sized operands */
+  CUASR_AMD_KERNEL_VALU_STREAMK = 5 /* the same tile with the k-tiles of all output tiles shared out evenly over
+                                       two workgroups per compute unit, for outputs whose tiles do not fill
+                                       whole rounds of the chip; 4-byte min/max-plus, max-min, min-max, xor-and,
+                                       or-and with alpha = the multiplicative identity given by value; not for
+                                       split-K or batches.  Two launches: D <- the source term, then the product
+                                       folded into D (D may alias C as always) */
 } cuasr_amd_kernel;
 
 /* One element of the problem's type; read through the member `dtype` names. */
@@ -295,7 +301,7 @@ int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64_t ld, int3
                                   int64_t ldp, void *workspace, int panels, void *stream);
 
 /* Name of the kernel family AUTO would choose for this descriptor
- * ("naive", "valu", "valu_direct", "mfma"; "valu_direct+valu" when a block of the output runs on
+ * ("naive", "valu", "valu_direct", "valu_streamk", "mfma"; "valu_direct+valu" when a block of the output runs on
  * the direct-to-LDS tile and the strips around it on the staged one), or NULL if the descriptor
  * is invalid. */
 const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc);

@@ -300,3 +300,53 @@ def test_large_output_in_two_regions(oracle, lib, case):
     la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
     for beta_one in (True, False):
         run(oracle, add, mult, dtype, m, n, k, la, lb, lc, "auto", beta_one)
+
+
+STREAMK_SEMIRINGS = [("minimum", "plus", "f32"), ("maximum", "plus", "f32"), ("maximum", "minimum", "f32"),
+                     ("minimum", "maximum", "f32"), ("bit_xor", "bit_and", "u32"), ("bit_or", "bit_and", "i32")]
+
+
+@pytest.mark.parametrize("sr", STREAMK_SEMIRINGS)
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "crr", "ccr", "rrc"])
+def test_streamk_direct_tile(oracle, lib, sr, layouts):
+    """The direct tile with the k-tiles of all output tiles shared out over the workgroups: ranges of k of one
+    tile meet in D (plain fold for a workgroup that has a tile to itself, atomic folds otherwise).  Shapes of
+    one tile, of a few tiles with far more workgroups than tiles (every tile split many ways), ragged edges and
+    a ragged last k-tile; beta = zero (D starts from the identity) and beta = one (from the source)."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for shape in [(128, 128, 64), (256, 384, 100), (516, 260, 52), (132, 388, 1028), (768, 640, 4096)]:
+        for beta_one in (False, True):
+            run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "streamk", beta_one)
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus", "f32"), ("bit_xor", "bit_and", "u32")])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc"])
+def test_streamk_more_tiles_than_workgroups(oracle, lib, sr, layouts):
+    """561 and 1100 tiles for 512 workgroups: whole tiles first (one and two per workgroup), the rest shared."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for shape in [(4352, 4224, 48), (5632, 6400, 36)]:
+        run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "streamk", True)
+
+
+def test_streamk_is_what_auto_picks_for_half_filled_rounds(oracle, lib):
+    """3072 x 3072 is 288 tiles for 512 places; AUTO takes the stream-K form there, and not for 4096^2 (512 tiles), a
+    pair of k-contiguous operands, a short k, or an alpha that is not the multiplicative identity."""
+    import ctypes
+    import cuasr_amd
+    from cuasr_amd import COLUMN_MAJOR, ROW_MAJOR, MatRef
+
+    def chosen(m, n, k, la=COLUMN_MAJOR, lb=COLUMN_MAJOR, alpha=0.0, add="minimum", mult="plus"):
+        A = MatRef(0x10000, m if la == COLUMN_MAJOR else k, la, m, k)
+        B = MatRef(0x10000, k if lb == COLUMN_MAJOR else n, lb, k, n)
+        C = MatRef(0x10000, m, COLUMN_MAJOR, m, n)
+        d = cuasr_amd.make_desc(add, mult, "f32", A, B, C, C, alpha, 0.0, float("inf"), 0.0)
+        return lib.cuasr_amd_selected_kernel(ctypes.byref(d))
+    assert chosen(3072, 3072, 3072) == b"valu_streamk"
+    assert chosen(5120, 5120, 5120) == b"valu_streamk"
+    assert chosen(4096, 4096, 4096) == b"valu_direct"
+    assert chosen(3072, 3072, 64) != b"valu_streamk"
+    assert chosen(3072, 3072, 3072, alpha=1.0) != b"valu_streamk"
+    assert chosen(3072, 3072, 3072, la=ROW_MAJOR, lb=COLUMN_MAJOR) != b"valu_streamk"   # both operands k-contiguous: no such loop
+    assert chosen(3072, 3072, 3072, la=COLUMN_MAJOR, lb=ROW_MAJOR) == b"valu_streamk"
+    assert chosen(3072, 3072, 3072, add="plus", mult="multiplies") != b"valu_streamk"
+    run(oracle, "minimum", "plus", "f32", 3072, 3072, 1024, "col", "col", "col", "auto", True)
