@@ -308,7 +308,170 @@ def generate(out_dir):
     return report
 
 
+# ---------------------------------------------------------------------------------------------
+# plus-times on the matrix cores (mfma_direct_f32.hip): v_mfma_f32_32x32x2_f32, direct-to-LDS panels
+#
+#   workgroup 256 threads = 4 waves (2 x 2), output tile 128 x 256, wave tile 64 x 128 = 2 x 4 blocks of 32 x 32
+#   v0   .. v127   accumulators, block (bm, bn) in v[16 (4 bm + bn) : +15]
+#   v128 .. v143   A fragments: buffer u, block bm, four registers = the four steps of a period of 8 k
+#   v144 .. v175   B fragments: buffer u, block bn, four registers
+# The instruction takes k from lanes 0..31 and another k from lanes 32..63; WHICH two k a step multiplies is
+# free as long as A and B agree, so a period of 8 k is walked as (k, k + 4) for k = 0..3: lanes 0..31 hold the
+# first k-quad of the period, lanes 32..63 the second.  A k-contiguous panel ([k/4][X][4] in LDS) then delivers a
+# block's four steps with ONE 16-byte read per lane and no bank conflict; an x-contiguous panel ([k][X]) with
+# four 4-byte reads of 32 + 32 consecutive floats.  Fragments are double-buffered by period; the reads for the
+# next period are issued after the first eight matrix instructions of this one, so a register is overwritten
+# 500 cycles and more after the last instruction that read it was issued.
+class MfmaBody(Body):
+    def __init__(self, a_kc, b_kc):
+        self.a_kc, self.b_kc = a_kc, b_kc
+        self.lines, self.inflight, self.groups = [], [], 0
+        self.stats = {"groups": 0, "lds": 0, "waits": 0, "other": 0}
+        self.content = {}
+
+    @staticmethod
+    def frag(operand, u, blk, s):
+        return (128 + (u * 2 + blk) * 4 + s) if operand == "A" else (144 + (u * 4 + blk) * 4 + s)
+
+    def reads(self, period):
+        """[(asm text, {register: content})]: LDS reads of the fragments of absolute period `period` (0, 1 of this
+        tile; 2 = the next tile's first, through the already advanced addresses) into buffer period % 2."""
+        u, P, out = period % 2, period % 2, []
+        for operand, kc, X, nblk, addr in (("A", self.a_kc, 128, 2, "a_addr"), ("B", self.b_kc, 256, 4, "b_addr")):
+            for blk in range(nblk):
+                r = self.frag(operand, u, blk, 0)
+                if kc:
+                    out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}] offset:{(2 * P * X + blk * 32) * 16}",
+                                {r + s: (operand, blk, period, s) for s in range(4)}))
+                else:
+                    for s in range(4):
+                        out.append((f"ds_read_b32 v{r + s}, %[{addr}] offset:{((8 * P + s) * X + blk * 32) * 4}",
+                                    {r + s: (operand, blk, period, s)}))
+        return out
+
+    def read(self, item):
+        text, fills = item
+        self.emit(text, "lds")
+        self.content.update(fills)
+        self.inflight.append((set(fills), self.groups))
+
+    def mfma(self, period, s, bm, bn):
+        u = period % 2
+        ra, rb = self.frag("A", u, bm, s), self.frag("B", u, bn, s)
+        assert self.content.get(ra) == ("A", bm, period, s) and self.content.get(rb) == ("B", bn, period, s)
+        self.require_exact({ra, rb})
+        acc = 16 * (4 * bm + bn)
+        self.lines.append(f'"v_mfma_f32_32x32x2_f32 v[{acc}:{acc + 15}], v{ra}, v{rb}, v[{acc}:{acc + 15}]\\n"')
+        self.groups += 1
+        self.stats["groups"] += 1
+
+    def require_exact(self, regs):
+        last = max((i for i, (rs, _) in enumerate(self.inflight) if rs & regs), default=None)
+        if last is None:
+            return
+        left = len(self.inflight) - 1 - last
+        assert left <= 15
+        self.emit(f"s_waitcnt lgkmcnt({left})", "waits")
+        self.inflight = self.inflight[last + 1:]
+
+    def period(self, period, aux, first, last):
+        """The 32 matrix instructions of a period of 8 k, with the callables of `aux` spread evenly behind
+        instructions first .. last of them (counted from 0)."""
+        order = [(s, bm, bn) for s in range(4) for bn in range(4) for bm in range(2)]
+        behind = {}
+        for i, item in enumerate(aux):
+            slot = first + (i * (last - first + 1)) // len(aux)
+            behind.setdefault(slot, []).append(item)
+        for i, (s, bm, bn) in enumerate(order):
+            self.mfma(period, s, bm, bn)
+            for item in behind.get(i, []):
+                item()
+
+    def prime(self):
+        for item in self.reads(0):
+            self.read(item)
+        self.drain()
+        return self.lines
+
+    def dma_chunk(self, index):
+        """One 1 KiB piece of the tile two ahead, global -> LDS (skipped when there is no such tile): pieces 0, 1
+        of the A panel, 2..5 of the B panel.  M0 holds the LDS address of the piece."""
+        e = self.emit
+        name, base, m0, h = ("a", "base_a", "m0_a", index) if index < 2 else ("b", "base_b", "m0_b", index - 2)
+        e("s_cmp_lt_i32 %[fetch], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_%=")
+        e(f"s_add_u32 m0, %[{m0}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[{base}]")
+        e(f".Lcuasr_nofetch{index}_%=:")
+
+    def tile(self):
+        e = self.emit
+        for operand, nblk in (("A", 2), ("B", 4)):
+            for blk in range(nblk):
+                for s in range(4):
+                    self.content[self.frag(operand, 0, blk, s)] = (operand, blk, 0, s)
+        entry = dict(self.content)
+        e("s_mov_b32 %[m0_save], m0")
+        # period 0 (buffer 0).  Behind its matrix instructions, a few at a time: the six loads of the tile two
+        # ahead and the LDS reads of period 1 (same stage) -- everything but the matrix instructions is spread so
+        # that the matrix pipe never waits for a run of other instructions, and the last eight matrix instructions
+        # (500 cycles) cover the latency of the last read
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(6)]
+        rd = [(lambda it=it: self.read(it)) for it in self.reads(1)]
+        # interleave the two kinds
+        mixed, q = [], 0
+        for i, r in enumerate(rd):
+            while q < 6 and q * len(rd) <= i * 6:
+                mixed.append(aux[q])
+                q += 1
+            mixed.append(r)
+        mixed += aux[q:]
+        self.period(0, mixed, 1, 23)
+        e("s_mov_b32 m0, %[m0_save]")
+        # every read of this stage has returned; this wave's part of the next tile has landed (its six loads are
+        # older than the six of the tile two ahead, if those were issued); after the barrier both hold for the
+        # workgroup, and the reads from here on go to the next stage
+        e("s_cmp_lt_i32 %[fetch], 1")
+        e("s_cbranch_scc1 .Lcuasr_all_%=")
+        e("s_waitcnt vmcnt(6) lgkmcnt(0)")
+        e("s_branch .Lcuasr_join_%=")
+        e(".Lcuasr_all_%=:")
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        e(".Lcuasr_join_%=:")
+        self.inflight = []
+        e("s_barrier")
+        e("v_add_u32 %[a_addr], %[a_step], %[a_addr]")
+        e("v_add_u32 %[b_addr], %[b_step], %[b_addr]")
+        self.period(1, [(lambda it=it: self.read(it)) for it in self.reads(2)], 1, 23)
+        self.drain()
+        shifted = {r: (o, b, p - 2, s) for r, (o, b, p, s) in self.content.items() if p >= 2}
+        assert shifted == entry, "tile body does not reproduce its entry state"
+        return self.lines
+
+    def text(self, lines):
+        return "\n".join(ln if ln.startswith('"v_mfma') else '"' + ln + '\\n"' for ln in lines) + "\n"
+
+
+MFMA_VARIANTS = {"m_kx": (True, False), "m_xx": (False, False), "m_xk": (False, True), "m_kk": (True, True)}
+
+
+def generate_mfma(out_dir):
+    os.makedirs(out_dir, exist_ok=True)
+    report = []
+    for name, (a_kc, b_kc) in MFMA_VARIANTS.items():
+        b = MfmaBody(a_kc, b_kc)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_prime.inc"), "w") as f:
+            f.write(b.text(b.prime()))
+        b = MfmaBody(a_kc, b_kc)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_tile.inc"), "w") as f:
+            f.write(b.text(b.tile()))
+        report.append((name, dict(b.stats)))
+    return report
+
+
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
-    for name, stats in generate(sys.argv[1] if len(sys.argv) > 1 else os.path.join(here, "gen")):
+    out = sys.argv[1] if len(sys.argv) > 1 else os.path.join(here, "gen")
+    for name, stats in generate(out) + generate_mfma(out):
         print(name, stats)

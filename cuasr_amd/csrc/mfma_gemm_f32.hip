@@ -24,6 +24,10 @@
 #include "mfma_common.h"
 
 namespace cuasr_amd {
+
+bool mfma_direct_f32_can_run(const Problem &);                // mfma_direct_f32.hip
+hipError_t mfma_direct_f32_launch(const Problem &, hipStream_t);
+
 namespace gemm_mfma {
 
 using namespace mfma_panel;
@@ -320,9 +324,11 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   // the 128 x 256 tile when its workgroups fill >= 7/8 of whole rounds of 512 (two per compute unit)
   const long long rounds = (wide * slices + 511) / 512;
-  if (wide * slices * 8 >= rounds * 512 * 7)
+  if (wide * slices * 8 >= rounds * 512 * 7) {
+    // whole k-tiles and loadable straight into LDS: the hand-scheduled form of the same tile
+    if (mfma_direct_f32_can_run(p)) return mfma_direct_f32_launch(p, s);
     launch_kernel(gemm_mfma_kernel<2>, dim3((unsigned)wide, (unsigned)slices), dim3(256), 0, s, p);
-  else
+  } else
     launch_kernel(gemm_mfma_kernel<1>, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
   return take_launch_status();
 }
