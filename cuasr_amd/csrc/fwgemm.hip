@@ -41,6 +41,10 @@ struct FwArgs {
   // one-thread-per-element kernel only: every output it computes is also stored transposed,
   // out_t[col + row * ld_out_t] (the k-contiguous image a later product's lookups read)
   void *out_t; int64_t ld_out_t;
+  // tile kernel, blocked Floyd-Warshall only: the diagonal block that starts at (ahead0, ahead0) and has
+  // ahead_bb (> 0) rows is updated by the launch's first workgroup, which then closes it (fw_close_256):
+  // the next block step finds its diagonal block done
+  int ahead0, ahead_bb;
 };
 
 // cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
@@ -121,7 +125,7 @@ template <> struct vec4_of<double> { typedef double type __attribute__((ext_vect
 // GUARD = true : any extents and alignment; out-of-range operands read as
 //                +infinity, whose products never improve anything.
 template <typename T, int TM, int TN, int SN, int BK, bool GUARD, bool HAS_AT>
-__global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
+__device__ __forceinline__ void fwgemm_tile_body(const FwArgs &g, const int block_x, const int block_y) {
   typedef typename vec4_of<T>::type V4;
   constexpr int BM = 16 * TM, BN = 16 * TN, PAD = 4;
   constexpr int NA = BM * BK / 4 / 256, NB = BN * BK / 4 / 256;
@@ -133,7 +137,7 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   const T *B = static_cast<const T *>(g.B);
   const int tid = threadIdx.x & 255;
   const int tx = tid & 15, ty = tid >> 4;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
+  const int m0 = block_x * BM, n0 = block_y * BN;
   // (the host only passes ranges whose ends fall on tile boundaries or beyond the matrix)
   if ((m0 < g.skip_r1 && m0 + BM > g.skip_r0) || (n0 < g.skip_c1 && n0 + BN > g.skip_c0)) return;
   const T inf = std::numeric_limits<T>::infinity();
@@ -391,6 +395,209 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   }
 }
 
+constexpr int FW_BLOCK = 128;  // vertices per block step of the blocked Floyd-Warshall
+
+// Floyd-Warshall inside one diagonal block of bb <= FW_BLOCK rows, by one workgroup of 256 threads that
+// holds the block in registers, an 8 x 8 patch per thread: the same element-by-element sequence as
+// fw_diagonal_kernel below (k ascending, d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent =
+// k_base + k), for a caller that has only 256 threads: the tile kernel's first workgroup.
+//
+// Four instructions per element and step (add, compare, two selects), 64 elements per thread: a step is
+// 256 vector instructions per wave, which one wave per SIMD issues in about 1100 cycles -- and everything
+// else a step needs (publishing row and column k + 1 to LDS, the barrier, reading them back) would add
+// its full latency to that, because the steps depend on each other.  So a step is done in two parts:
+//   A. the patch's row and column (k + 1) & 7 -- every thread's, since which thread owns row / column
+//      k + 1 is only known at run time -- then the owners publish them, then the barrier;
+//   B. the reads of row / column k + 1 are issued, and the other 49 elements of step k are done while
+//      they are on their way.
+// relax4 / relax3: compare (strictly: -0 must not replace +0), select distance and parent, for four
+// (three) elements at a time.  Written out as instructions for two reasons.  Nothing reads the parents
+// before the end, and left alone the optimiser postpones their selects over a whole unrolled round of
+// steps and keeps 512 comparison results instead, which do not fit the scalar registers.  And a select
+// that directly follows its comparison waits for the mask: with three other instructions in between a
+// block took 100 us instead of 131.
+__device__ __forceinline__ void relax4(float &x0, float &x1, float &x2, float &x3, int32_t &p0, int32_t &p1, int32_t &p2,
+                                       int32_t &p3, float c0, float c1, float c2, float c3, int32_t kv) {
+  unsigned long long m0, m1, m2, m3;
+  asm volatile(
+      "v_cmp_lt_f32 %[m0], %[c0], %[x0]\n\tv_cmp_lt_f32 %[m1], %[c1], %[x1]\n\t"
+      "v_cmp_lt_f32 %[m2], %[c2], %[x2]\n\tv_cmp_lt_f32 %[m3], %[c3], %[x3]\n\t"
+      "v_cndmask_b32 %[x0], %[x0], %[c0], %[m0]\n\tv_cndmask_b32 %[x1], %[x1], %[c1], %[m1]\n\t"
+      "v_cndmask_b32 %[x2], %[x2], %[c2], %[m2]\n\tv_cndmask_b32 %[x3], %[x3], %[c3], %[m3]\n\t"
+      "v_cndmask_b32 %[p0], %[p0], %[kv], %[m0]\n\tv_cndmask_b32 %[p1], %[p1], %[kv], %[m1]\n\t"
+      "v_cndmask_b32 %[p2], %[p2], %[kv], %[m2]\n\tv_cndmask_b32 %[p3], %[p3], %[kv], %[m3]"
+      : [x0] "+v"(x0), [x1] "+v"(x1), [x2] "+v"(x2), [x3] "+v"(x3), [p0] "+v"(p0), [p1] "+v"(p1), [p2] "+v"(p2),
+        [p3] "+v"(p3), [m0] "=&s"(m0), [m1] "=&s"(m1), [m2] "=&s"(m2), [m3] "=&s"(m3)
+      : [c0] "v"(c0), [c1] "v"(c1), [c2] "v"(c2), [c3] "v"(c3), [kv] "v"(kv));
+}
+__device__ __forceinline__ void relax3(float &x0, float &x1, float &x2, int32_t &p0, int32_t &p1, int32_t &p2, float c0,
+                                       float c1, float c2, int32_t kv) {
+  unsigned long long m0, m1, m2;
+  asm volatile(
+      "v_cmp_lt_f32 %[m0], %[c0], %[x0]\n\tv_cmp_lt_f32 %[m1], %[c1], %[x1]\n\tv_cmp_lt_f32 %[m2], %[c2], %[x2]\n\t"
+      "v_cndmask_b32 %[x0], %[x0], %[c0], %[m0]\n\tv_cndmask_b32 %[x1], %[x1], %[c1], %[m1]\n\t"
+      "v_cndmask_b32 %[x2], %[x2], %[c2], %[m2]\n\t"
+      "v_cndmask_b32 %[p0], %[p0], %[kv], %[m0]\n\tv_cndmask_b32 %[p1], %[p1], %[kv], %[m1]\n\t"
+      "v_cndmask_b32 %[p2], %[p2], %[kv], %[m2]"
+      : [x0] "+v"(x0), [x1] "+v"(x1), [x2] "+v"(x2), [p0] "+v"(p0), [p1] "+v"(p1), [p2] "+v"(p2), [m0] "=&s"(m0),
+        [m1] "=&s"(m1), [m2] "=&s"(m2)
+      : [c0] "v"(c0), [c1] "v"(c1), [c2] "v"(c2), [kv] "v"(kv));
+}
+
+__device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *parent, int64_t ldp, int bb, int k_base) {
+  typedef vec4_of<float>::type V4;
+  __shared__ __attribute__((aligned(32))) float colbuf[2][FW_BLOCK];  // d[i][k] for the step that reads this buffer
+  __shared__ __attribute__((aligned(32))) float rowbuf[2][FW_BLOCK];  // d[k][j]
+  const int tid = threadIdx.x & 255, ti = tid & 15, tj = tid >> 4;  // rows 8 ti .. 8 ti + 7, columns 8 tj .. 8 tj + 7
+  const float inf = std::numeric_limits<float>::infinity();
+  float cur[8][8];  // [row in patch][column in patch]
+  int32_t par[8][8];
+  // (loads from clamped addresses, then a select: a branch per element would keep 64 lane masks alive)
+#pragma unroll
+  for (int b = 0; b < 8; ++b)
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const int i = 8 * ti + a, j = 8 * tj + b;
+      const float v = d[min(i, bb - 1) + int64_t(min(j, bb - 1)) * ld];
+      cur[a][b] = (i < bb && j < bb) ? v : inf;
+      par[a][b] = -1;
+    }
+  // S = kn & 7, the row / column of the patch that is published, is a compile-time constant (the step
+  // loop is unrolled by eight): indexed by a run-time value the patch would live in scratch memory
+  auto publish = [&](int kn, int buf, auto sc) {
+    constexpr int S = decltype(sc)::value;
+    if ((kn >> 3) == ti) {  // my patch holds row kn
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        V4 v;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) v[b] = cur[S][4 * h + b];
+        *reinterpret_cast<V4 *>(&rowbuf[buf][8 * tj + 4 * h]) = v;
+      }
+    }
+    if ((kn >> 3) == tj) {  // my patch holds column kn
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        V4 v;
+#pragma unroll
+        for (int a = 0; a < 4; ++a) v[a] = cur[4 * h + a][S];
+        *reinterpret_cast<V4 *>(&colbuf[buf][8 * ti + 4 * h]) = v;
+      }
+    }
+  };
+  float ci[8], rj[8];  // column k at my rows, row k at my columns, for the step in hand
+  auto fetch = [&](float (&c)[8], float (&r)[8], int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const V4 cv = *reinterpret_cast<const V4 *>(&colbuf[buf][8 * ti + 4 * h]);
+      const V4 rv = *reinterpret_cast<const V4 *>(&rowbuf[buf][8 * tj + 4 * h]);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        c[4 * h + x] = cv[x];
+        r[4 * h + x] = rv[x];
+      }
+    }
+  };
+  auto step = [&](int k, auto uc) {
+    constexpr int U = decltype(uc)::value;  // k & 7
+    constexpr int N = (U + 1) & 7;          // the row and the column of the patch that step k + 1 may need
+    constexpr int O[7] = {N > 0 ? 0 : 1, N > 1 ? 1 : 2, N > 2 ? 2 : 3, N > 3 ? 3 : 4, N > 4 ? 4 : 5, N > 5 ? 5 : 6, N > 6 ? 6 : 7};
+    const int buf = U & 1;
+    int32_t kv = k_base + k;
+    asm volatile("" : "+v"(kv));  // one register for the step, not a constant folded into every select
+    // A. row N, then column N of the other rows
+    relax4(cur[N][0], cur[N][1], cur[N][2], cur[N][3], par[N][0], par[N][1], par[N][2], par[N][3], ci[N] + rj[0],
+           ci[N] + rj[1], ci[N] + rj[2], ci[N] + rj[3], kv);
+    relax4(cur[N][4], cur[N][5], cur[N][6], cur[N][7], par[N][4], par[N][5], par[N][6], par[N][7], ci[N] + rj[4],
+           ci[N] + rj[5], ci[N] + rj[6], ci[N] + rj[7], kv);
+    relax4(cur[O[0]][N], cur[O[1]][N], cur[O[2]][N], cur[O[3]][N], par[O[0]][N], par[O[1]][N], par[O[2]][N], par[O[3]][N],
+           ci[O[0]] + rj[N], ci[O[1]] + rj[N], ci[O[2]] + rj[N], ci[O[3]] + rj[N], kv);
+    relax3(cur[O[4]][N], cur[O[5]][N], cur[O[6]][N], par[O[4]][N], par[O[5]][N], par[O[6]][N], ci[O[4]] + rj[N],
+           ci[O[5]] + rj[N], ci[O[6]] + rj[N], kv);
+    // into the other pair of buffers: nobody reads it before the barrier, and nobody is still reading it
+    // from the step before (everybody has passed that step's barrier, and waited for its reads in part A)
+    publish(k + 1, buf ^ 1, std::integral_constant<int, N>{});
+    __syncthreads();
+    float cn[8], rn[8];
+    fetch(cn, rn, buf ^ 1);
+    // B. the rest of step k, under the latency of those reads
+#pragma unroll
+    for (int i = 0; i < 7; ++i) {
+      const int a = O[i];
+      relax4(cur[a][O[0]], cur[a][O[1]], cur[a][O[2]], cur[a][O[3]], par[a][O[0]], par[a][O[1]], par[a][O[2]], par[a][O[3]],
+             ci[a] + rj[O[0]], ci[a] + rj[O[1]], ci[a] + rj[O[2]], ci[a] + rj[O[3]], kv);
+      relax3(cur[a][O[4]], cur[a][O[5]], cur[a][O[6]], par[a][O[4]], par[a][O[5]], par[a][O[6]], ci[a] + rj[O[4]],
+             ci[a] + rj[O[5]], ci[a] + rj[O[6]], kv);
+    }
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      ci[x] = cn[x];
+      rj[x] = rn[x];
+    }
+  };
+  publish(0, 0, std::integral_constant<int, 0>{});
+  __syncthreads();
+  fetch(ci, rj, 0);
+  // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
+  // +infinity and improve nothing
+#pragma unroll 1
+  for (int k8 = 0; k8 < bb; k8 += 8) {
+    step(k8 + 0, std::integral_constant<int, 0>{});
+    step(k8 + 1, std::integral_constant<int, 1>{});
+    step(k8 + 2, std::integral_constant<int, 2>{});
+    step(k8 + 3, std::integral_constant<int, 3>{});
+    step(k8 + 4, std::integral_constant<int, 4>{});
+    step(k8 + 5, std::integral_constant<int, 5>{});
+    step(k8 + 6, std::integral_constant<int, 6>{});
+    step(k8 + 7, std::integral_constant<int, 7>{});
+  }
+  // (elements of the padding never improve: their parent is still -1)
+#pragma unroll
+  for (int b = 0; b < 8; ++b)
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const int i = 8 * ti + a, j = 8 * tj + b;
+      if (par[a][b] >= 0) {
+        d[i + int64_t(j) * ld] = cur[a][b];
+        parent[i + int64_t(j) * ldp] = par[a][b];
+      }
+    }
+}
+
+// The tile kernel.  Grid (tiles along m, tiles along n); with g.ahead_bb > 0 the grid has one more row,
+// whose first workgroup -- the first one the launch starts -- takes the tile that is the next diagonal
+// block and then closes that block, while the workgroups of the other rows do the remaining tiles as
+// ever.  Only where a tile is a whole diagonal block (4-byte elements; the host asks for nothing else).
+template <typename T, int TM, int TN, int SN, int BK, bool GUARD, bool HAS_AT>
+__global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
+  constexpr int BM = 16 * TM, BN = 16 * TN;
+  constexpr bool CAN_CLOSE = BM == FW_BLOCK && BN == FW_BLOCK && std::is_same<T, float>::value;
+  int bx = blockIdx.x, by = blockIdx.y;
+  bool ahead = false;
+  if constexpr (CAN_CLOSE) {
+    if (g.ahead_bb > 0) {
+      if (by == 0) {
+        if (bx != 0) return;
+        ahead = true;
+        bx = by = g.ahead0 / FW_BLOCK;
+      } else {
+        by -= 1;
+        if (by * BN == g.ahead0 && bx * BM == g.ahead0) return;  // the first workgroup's
+      }
+    }
+  }
+  fwgemm_tile_body<T, TM, TN, SN, BK, GUARD, HAS_AT>(g, bx, by);
+  if constexpr (CAN_CLOSE) {
+    if (ahead) {
+      // this workgroup's own stores, read back by other threads of it
+      __threadfence();
+      __syncthreads();
+      fw_close_256(static_cast<float *>(g.dist) + g.ahead0 + int64_t(g.ahead0) * g.ldc, g.ldc,
+                      g.parent + g.ahead0 + int64_t(g.ahead0) * g.ldp, g.ldp, g.ahead_bb, g.ahead0);
+    }
+  }
+}
+
 template <typename T, int TM, int TN, int SN, int BK>
 hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
@@ -398,7 +605,8 @@ hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   const size_t vec = 4 * sizeof(T);
   const bool aligned = reinterpret_cast<uintptr_t>(g.A) % vec == 0 && reinterpret_cast<uintptr_t>(g.B) % vec == 0 &&
                        g.lda % 4 == 0 && g.ldb % 4 == 0;
-  dim3 grid((g.m + BM - 1) / BM, (g.n + BN - 1) / BN);
+  if (g.ahead_bb > 0 && (BM != FW_BLOCK || BN != FW_BLOCK)) return hipErrorInvalidValue;
+  dim3 grid((g.m + BM - 1) / BM, (g.n + BN - 1) / BN + (g.ahead_bb > 0 ? 1 : 0));
   if (g.At) {
     const bool at_aligned = reinterpret_cast<uintptr_t>(g.At) % vec == 0 && g.ldat % 4 == 0;
     if (whole && aligned && at_aligned)
@@ -471,7 +679,6 @@ __global__ void __launch_bounds__(256) snapshot_pair_kernel(const T *src0, T *w0
 // only, and they do not change during step k (the block's diagonal is not negative): every step
 // reads them from two 128-element LDS buffers and publishes column k + 1 and row k + 1 into the
 // other pair, so one barrier per step is enough and a thread reads two vectors per 16 updates.
-constexpr int FW_BLOCK = 128;
 template <typename T>
 __global__ void __launch_bounds__(1024) fw_diagonal_kernel(T *d, int64_t ld, int32_t *parent, int64_t ldp, int bb, int k_base) {
   typedef typename vec4_of<T>::type V4;
@@ -580,13 +787,17 @@ namespace {
 struct FwExtra {
   const void *At = nullptr; int64_t ldat = 0;
   int k_base = 0, skip_r0 = 0, skip_r1 = 0, skip_c0 = 0, skip_c1 = 0;
+  // blocked Floyd-Warshall: let the product also close the diagonal block that starts at ahead0 (ahead_bb rows).
+  // Only the tile kernel can; *closed_ahead says whether this launch did.
+  int ahead0 = 0, ahead_bb = 0;
+  bool *closed_ahead = nullptr;
 };
 int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, void *dist,
                int64_t ldc, int32_t *parent, int64_t ldp, const FwExtra &x, int kernel, void *stream) {
   const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
   if (st != CUASR_AMD_SUCCESS || m == 0 || n == 0 || k == 0) return st;
-  const FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, x.At, x.ldat, x.k_base,
-                 x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1};
+  FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, x.At, x.ldat, x.k_base,
+           x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1, nullptr, 0, 0, 0};
   hipStream_t s = static_cast<hipStream_t>(stream);
   // a launch of a few workgroups is better spread over one thread per element
   // ... and so is one of few tiles (the tile kernel's workgroups would each run alone on a
@@ -595,6 +806,11 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
   const int64_t tiles = ((int64_t(m) + 127) / 128) * ((int64_t(n) + 127) / 128);
   const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 96;
   const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
+  if (!naive && x.ahead_bb > 0 && dtype == CUASR_AMD_F32) {  // (the 8-byte tile is half a diagonal block)
+    g.ahead0 = x.ahead0;
+    g.ahead_bb = x.ahead_bb;
+  }
+  if (x.closed_ahead) *x.closed_ahead = g.ahead_bb > 0;
   hipError_t e;
   if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 4, 16>(g, s);
   else e = naive ? launch_naive<double>(g, s) : launch_tile<double, 4, 8, 4, 16>(g, s);
@@ -672,16 +888,19 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
   char *R = static_cast<char *>(workspace);             // block row,    FW_BLOCK x n,  leading dimension FW_BLOCK
   char *C = R + es * FW_BLOCK * size_t(nn);             // block column, n x FW_BLOCK,  leading dimension nn
   char *Ct = C + es * FW_BLOCK * size_t(nn);            // updated block column with k contiguous, leading dimension FW_BLOCK
+  bool closed = false;  // this step's diagonal block was closed by the step before, beside its big product
   for (int k0 = 0; k0 < n; k0 += FW_BLOCK) {
     const int bb = n - k0 < FW_BLOCK ? n - k0 : FW_BLOCK;
     char *Dkk = D + es * (size_t(k0) + size_t(k0) * size_t(ld));
     int32_t *Pkk = parent + size_t(k0) + size_t(k0) * size_t(ldp);
     // 1. the diagonal block, closed by one workgroup
-    if (f64)
-      launch_kernel(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
-    else
-      launch_kernel(fw_diagonal_kernel<float>, dim3(1), dim3(1024), 0, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
-    if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    if (!closed) {
+      if (f64)
+        launch_kernel(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
+      else
+        launch_kernel(fw_diagonal_kernel<float>, dim3(1), dim3(1024), 0, s, reinterpret_cast<float *>(Dkk), ld, Pkk, ldp, bb, k0);
+      if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    }
     // 2. snapshots of block row and block column (the products below read these, so that no
     //    workgroup sees another's updates)
     char *Drow = D + es * size_t(k0), *Dcol = D + es * size_t(k0) * size_t(ld);
@@ -709,11 +928,11 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
     const bool paired = panels == CUASR_AMD_PANELS_AUTO ? (int64_t(n) + 127) / 128 < 128 : panels == CUASR_AMD_PANELS_PAIRED;
     if (paired) {
       const FwArgs g0{bb, n, bb, R + es * size_t(k0) * FW_BLOCK, FW_BLOCK, R, FW_BLOCK, Drow, ld, parent + k0, ldp,
-                      nullptr, 0, k0, 0, 0, k0, k0 + bb, nullptr, 0};
+                      nullptr, 0, k0, 0, 0, k0, k0 + bb, nullptr, 0, 0, 0};
       // (the column product also writes the updated column's k-contiguous image for step 4; the rows
       // of the diagonal block, which it skips, are not read there)
       const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
-                      nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK};
+                      nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK, 0, 0};
       const int blocks0 = ((bb + 63) / 64) * ((n + 3) / 4), blocks1 = ((n + 63) / 64) * ((bb + 3) / 4);
       if (f64) launch_kernel(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
       else launch_kernel(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
@@ -732,7 +951,16 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
       if (e != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     }
     // 4. everything outside block row and block column <- (block column) x (block row), read in place
-    //    (those panels are not written in this step); the column's k-contiguous image serves the lookups
+    //    (those panels are not written in this step); the column's k-contiguous image serves the lookups.
+    //    The next step's diagonal block is the first tile this product finishes, and the same workgroup
+    //    closes it right away: a block's 128 dependent steps take as long as half the product, and nothing
+    //    else of the next step can start before them.
+    closed = false;
+    if (k0 + bb < n) {
+      x.ahead0 = k0 + bb;
+      x.ahead_bb = n - x.ahead0 < FW_BLOCK ? n - x.ahead0 : FW_BLOCK;
+      x.closed_ahead = &closed;
+    }
     x.At = Ct;
     x.ldat = FW_BLOCK;
     x.skip_r0 = x.skip_c0 = k0;
