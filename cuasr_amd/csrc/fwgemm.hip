@@ -42,8 +42,8 @@ struct FwArgs {
   // out_t[col + row * ld_out_t] (the k-contiguous image a later product's lookups read)
   void *out_t; int64_t ld_out_t;
   // tile kernel, blocked Floyd-Warshall only: the diagonal block that starts at (ahead0, ahead0) and has
-  // ahead_bb (> 0) rows is updated by the launch's first workgroup, which then closes it (fw_close_256):
-  // the next block step finds its diagonal block done
+  // ahead_bb (> 0) rows is the next block step's and has had this step's update already: the launch's
+  // first workgroup closes it (fw_close_256) while the others do the product, which leaves that tile alone
   int ahead0, ahead_bb;
 };
 
@@ -565,37 +565,29 @@ __device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *pare
 }
 
 // The tile kernel.  Grid (tiles along m, tiles along n); with g.ahead_bb > 0 the grid has one more row,
-// whose first workgroup -- the first one the launch starts -- takes the tile that is the next diagonal
-// block and then closes that block, while the workgroups of the other rows do the remaining tiles as
-// ever.  Only where a tile is a whole diagonal block (4-byte elements; the host asks for nothing else).
+// whose first workgroup -- the first one the launch starts -- closes the next block step's diagonal
+// block while the workgroups of the other rows do the product's tiles, all but that block.  The block's
+// 128 dependent steps take about as long as the whole product and nothing else of the next block step can
+// start before them; here they cost one of the launch's 512 places.  Only where a tile is a whole
+// diagonal block (4-byte elements; the host asks for nothing else).
 template <typename T, int TM, int TN, int SN, int BK, bool GUARD, bool HAS_AT>
 __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
   constexpr bool CAN_CLOSE = BM == FW_BLOCK && BN == FW_BLOCK && std::is_same<T, float>::value;
   int bx = blockIdx.x, by = blockIdx.y;
-  bool ahead = false;
   if constexpr (CAN_CLOSE) {
     if (g.ahead_bb > 0) {
       if (by == 0) {
-        if (bx != 0) return;
-        ahead = true;
-        bx = by = g.ahead0 / FW_BLOCK;
-      } else {
-        by -= 1;
-        if (by * BN == g.ahead0 && bx * BM == g.ahead0) return;  // the first workgroup's
+        if (bx == 0)
+          fw_close_256(static_cast<float *>(g.dist) + g.ahead0 + int64_t(g.ahead0) * g.ldc, g.ldc,
+                       g.parent + g.ahead0 + int64_t(g.ahead0) * g.ldp, g.ldp, g.ahead_bb, g.ahead0);
+        return;
       }
+      by -= 1;
+      if (by * BN == g.ahead0 && bx * BM == g.ahead0) return;
     }
   }
   fwgemm_tile_body<T, TM, TN, SN, BK, GUARD, HAS_AT>(g, bx, by);
-  if constexpr (CAN_CLOSE) {
-    if (ahead) {
-      // this workgroup's own stores, read back by other threads of it
-      __threadfence();
-      __syncthreads();
-      fw_close_256(static_cast<float *>(g.dist) + g.ahead0 + int64_t(g.ahead0) * g.ldc, g.ldc,
-                      g.parent + g.ahead0 + int64_t(g.ahead0) * g.ldp, g.ldp, g.ahead_bb, g.ahead0);
-    }
-  }
 }
 
 template <typename T, int TM, int TN, int SN, int BK>
@@ -787,11 +779,20 @@ namespace {
 struct FwExtra {
   const void *At = nullptr; int64_t ldat = 0;
   int k_base = 0, skip_r0 = 0, skip_r1 = 0, skip_c0 = 0, skip_c1 = 0;
-  // blocked Floyd-Warshall: let the product also close the diagonal block that starts at ahead0 (ahead_bb rows).
-  // Only the tile kernel can; *closed_ahead says whether this launch did.
+  // blocked Floyd-Warshall: let the launch also close the diagonal block that starts at ahead0 (ahead_bb rows),
+  // which the product then leaves alone.  Only the tile kernel can; *closed_ahead says whether this launch did.
   int ahead0 = 0, ahead_bb = 0;
   bool *closed_ahead = nullptr;
 };
+// one-thread-per-element kernel or tiles: a launch of a few workgroups is better spread over one thread per
+// element, and so is one of few tiles (the tile kernel's workgroups would each run alone on a compute
+// unit): measured on square problems, the two kernels meet at about 100 tiles (1024^3: 193 against 270 us,
+// 1280^3: 356 against 334, 1408^3: 466 against 366)
+bool takes_naive_kernel(int m, int n, int kernel) {
+  const int64_t tiles = ((int64_t(m) + 127) / 128) * ((int64_t(n) + 127) / 128);
+  const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 96;
+  return kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
+}
 int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const void *B, int64_t ldb, void *dist,
                int64_t ldc, int32_t *parent, int64_t ldp, const FwExtra &x, int kernel, void *stream) {
   const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
@@ -799,13 +800,7 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
   FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, x.At, x.ldat, x.k_base,
            x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1, nullptr, 0, 0, 0};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // a launch of a few workgroups is better spread over one thread per element
-  // ... and so is one of few tiles (the tile kernel's workgroups would each run alone on a
-  // compute unit): measured on square problems, the two kernels meet at about 100 tiles
-  // (1024^3: 193 against 270 us, 1280^3: 356 against 334, 1408^3: 466 against 366)
-  const int64_t tiles = ((int64_t(m) + 127) / 128) * ((int64_t(n) + 127) / 128);
-  const bool tiny = int64_t(m) * n < 64 * 64 || tiles < 96;
-  const bool naive = kernel == CUASR_AMD_KERNEL_NAIVE || (kernel == CUASR_AMD_KERNEL_AUTO && tiny);
+  const bool naive = takes_naive_kernel(m, n, kernel);
   if (!naive && x.ahead_bb > 0 && dtype == CUASR_AMD_F32) {  // (the 8-byte tile is half a diagonal block)
     g.ahead0 = x.ahead0;
     g.ahead_bb = x.ahead_bb;
@@ -888,7 +883,7 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
   char *R = static_cast<char *>(workspace);             // block row,    FW_BLOCK x n,  leading dimension FW_BLOCK
   char *C = R + es * FW_BLOCK * size_t(nn);             // block column, n x FW_BLOCK,  leading dimension nn
   char *Ct = C + es * FW_BLOCK * size_t(nn);            // updated block column with k contiguous, leading dimension FW_BLOCK
-  bool closed = false;  // this step's diagonal block was closed by the step before, beside its big product
+  bool closed = false;  // this step's diagonal block was closed during the step before, beside its big product
   for (int k0 = 0; k0 < n; k0 += FW_BLOCK) {
     const int bb = n - k0 < FW_BLOCK ? n - k0 : FW_BLOCK;
     char *Dkk = D + es * (size_t(k0) + size_t(k0) * size_t(ld));
@@ -952,9 +947,8 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
     }
     // 4. everything outside block row and block column <- (block column) x (block row), read in place
     //    (those panels are not written in this step); the column's k-contiguous image serves the lookups.
-    //    The next step's diagonal block is the first tile this product finishes, and the same workgroup
-    //    closes it right away: a block's 128 dependent steps take as long as half the product, and nothing
-    //    else of the next step can start before them.
+    //    The next step's diagonal block gets its update first, so that the product's launch can close it
+    //    at the same time (fwgemm_tile_kernel).
     closed = false;
     if (k0 + bb < n) {
       x.ahead0 = k0 + bb;
@@ -965,6 +959,19 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
     x.ldat = FW_BLOCK;
     x.skip_r0 = x.skip_c0 = k0;
     x.skip_r1 = x.skip_c1 = k0 + bb;
+    if (x.ahead_bb > 0 && !f64 && !takes_naive_kernel(n, n, CUASR_AMD_KERNEL_AUTO)) {
+      // this step's update of that block, by a launch of its own (64 workgroups, a few microseconds): the
+      // closure can then start with the big product instead of after one of its tiles
+      const int a0 = x.ahead0, abb = x.ahead_bb;
+      FwExtra xa;
+      xa.k_base = k0;
+      r = fwgemm_run(dtype, abb, abb, bb, Dcol + es * size_t(a0), ld, Drow + es * size_t(a0) * size_t(ld), ld,
+                     D + es * (size_t(a0) + size_t(a0) * size_t(ld)), ld, parent + size_t(a0) + size_t(a0) * size_t(ldp), ldp,
+                     xa, CUASR_AMD_KERNEL_AUTO, stream);
+      if (r != CUASR_AMD_SUCCESS) return r;
+    } else {
+      x.ahead_bb = 0;
+    }
     r = fwgemm_run(dtype, n, n, bb, Dcol, ld, Drow, ld, dist, ld, parent, ldp, x, CUASR_AMD_KERNEL_AUTO, stream);
     if (r != CUASR_AMD_SUCCESS) return r;
   }
