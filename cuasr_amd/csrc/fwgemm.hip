@@ -38,7 +38,7 @@ struct FwArgs {
   const void *At; int64_t ldat;
   int k_base;                               // recorded parents are k_base + k
   int skip_r0, skip_r1, skip_c0, skip_c1;   // outputs in these rows or these columns are left alone
-  // one-thread-per-element kernel only: every output it computes is also stored transposed,
+  // one-thread-per-element and row-by-four-columns kernels only: every output they compute is also stored transposed,
   // out_t[col + row * ld_out_t] (the k-contiguous image a later product's lookups read)
   void *out_t; int64_t ld_out_t;
   // tile kernel, blocked Floyd-Warshall only: the diagonal block that starts at (ahead0, ahead0) and has
@@ -100,24 +100,141 @@ __global__ void __launch_bounds__(256) fwgemm_naive_kernel(FwArgs g) {
   fwgemm_naive_block<T>(g, blockIdx.x, blockIdx.y);
 }
 
+template <typename T> struct vec4_of;
+template <> struct vec4_of<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct vec4_of<double> { typedef double type __attribute__((ext_vector_type(4))); };
+
+// One thread per output row and four columns, for products too small for the tile kernel but on the
+// critical path (the block row and the block column of a blocked Floyd-Warshall step): a workgroup of 256
+// threads covers 64 rows x 16 columns.  Same order-free form as the tile kernel: per chunk of 16 k a plain
+// min-plus (a 3-input minimum per two products), and "chunk minimum < running minimum" (strict) moves the
+// running minimum.  A chunk in which any of the wave's 64 rows improved is resolved on the spot, from the
+// operands still in registers: the first k whose product equals the chunk minimum (the same single addition
+// of the same operands, so equality is exact) is the parent, and that product, sign of zero included, the
+// distance.  (Looking the chunk up after the loop, as the tile kernel does, costs a gather of 16 cache lines
+// per lane and column here: 27 us for the two panels at n = 4096.)  A's 16 values of a chunk serve four
+// columns.  The one-thread-per-element scan spends four instructions per term, two of which read a mask, and reads each A
+// value once per output column: 29 us.
+template <typename T> __device__ __forceinline__ void fwgemm_rowcols_block(const FwArgs &g, int bx, int by) {
+  constexpr int CK = 16, NC = 4;
+  const int row_of_lane = bx * 64 + (threadIdx.x & 63);
+  const int col0 = __builtin_amdgcn_readfirstlane(by * 16 + (threadIdx.x >> 6) * NC);
+  if (col0 >= g.n) return;  // (the whole wave)
+  // every lane stays to the end, because every lane fetches one of the chunk's B values for the wave: rows
+  // beyond the matrix or in the skipped range are computed on a clamped row and never stored
+  const bool row_live = row_of_lane < g.m && !(row_of_lane >= g.skip_r0 && row_of_lane < g.skip_r1);
+  const int row = row_of_lane < g.m ? row_of_lane : g.m - 1;
+  const T inf = std::numeric_limits<T>::infinity();
+  const int64_t lda = g.lda;
+  // columns beyond the matrix or in the skipped range: computed on a clamped column, never stored
+  int64_t out[NC];
+  bool live[NC];
+  T curr[NC];
+  int32_t par[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int cc = col0 + c, cl = cc < g.n ? cc : g.n - 1;
+    live[c] = row_live && cc < g.n && !(cc >= g.skip_c0 && cc < g.skip_c1);
+    out[c] = cl;
+    curr[c] = static_cast<const T *>(g.dist)[row + int64_t(cl) * g.ldc];
+    par[c] = -1;
+  }
+  // one chunk of CK k-values; FULL: all of them exist (the ragged last chunk takes +infinity for the others,
+  // which neither improves anything nor equals a minimum that did)
+  // B's 4 x 16 values of a chunk: one load per lane (lane = column, k), handed round through a piece of LDS that
+  // belongs to the wave (no barrier: a wave's LDS accesses complete in order) and read back as broadcasts.
+  // Through scalar loads instead, every chunk and column waited for a scalar-cache miss, and every add read
+  // a scalar register, which costs it a second issue slot.
+  __shared__ T bstage[4][2][NC * CK];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const T *blane = static_cast<const T *>(g.B) + int64_t(min(col0 + (lane >> 4), g.n - 1)) * g.ldb;
+  const T *ap = static_cast<const T *>(g.A) + row;
+  auto load = [&](T (&av)[CK], T &bl, int k0, auto full) {
+    constexpr bool FULL = decltype(full)::value;
+    bl = blane[FULL ? k0 + (lane & 15) : min(k0 + (lane & 15), g.k - 1)];
+#pragma unroll
+    for (int u = 0; u < CK; ++u) {
+      if constexpr (FULL) av[u] = *ap;
+      else av[u] = k0 + u < g.k ? *ap : inf;
+      if (FULL || k0 + u + 1 < g.k) ap += lda;
+    }
+  };
+  auto compute = [&](const T (&av)[CK], T bl, int k0, int buf) {
+    typedef typename vec4_of<T>::type V4;
+    bstage[wave][buf][lane] = bl;
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      T bv[CK];
+#pragma unroll
+      for (int q = 0; q < CK / 4; ++q) {
+        const V4 v = *reinterpret_cast<const V4 *>(&bstage[wave][buf][c * CK + q * 4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) bv[q * 4 + e] = v[e];
+      }
+      T prod[CK], best = inf;
+#pragma unroll
+      for (int u = 0; u < CK; ++u) prod[u] = av[u] + bv[u];
+#pragma unroll
+      for (int u = 0; u < CK; u += 2) best = hw_min<T>(hw_min<T>(best, prod[u]), prod[u + 1]);
+      const bool lower = best < curr[c];
+      if (__builtin_amdgcn_ballot_w64(lower)) {  // the same for the whole wave
+        int first = 0;
+#pragma unroll
+        for (int u = CK - 1; u >= 0; --u) first = prod[u] == best ? u : first;
+        T value = best;
+        // a minimum of zero: the hardware's may carry the other sign than the first product that equals it
+        if (__builtin_amdgcn_ballot_w64(lower && best == T(0))) {
+#pragma unroll
+          for (int u = CK - 1; u >= 0; --u) value = pick(prod[u] == best, prod[u], value);
+        }
+        curr[c] = lower ? value : curr[c];
+        par[c] = lower ? g.k_base + k0 + first : par[c];
+      }
+    }
+  };
+  // the next chunk's A values are requested before this chunk is worked on: a wave has eight chunks and a
+  // compute unit sixteen such waves, too few to hide a memory round trip per chunk behind each other
+  const int nfull = g.k / CK;
+  T av[2][CK], bl[2];
+  if (nfull > 0) load(av[0], bl[0], 0, std::true_type{});
+  for (int ch = 0; ch < nfull; ch += 2) {
+    if (ch + 1 < nfull) load(av[1], bl[1], (ch + 1) * CK, std::true_type{});
+    compute(av[0], bl[0], ch * CK, 0);
+    if (ch + 1 < nfull) {
+      if (ch + 2 < nfull) load(av[0], bl[0], (ch + 2) * CK, std::true_type{});
+      compute(av[1], bl[1], (ch + 1) * CK, 1);
+    }
+  }
+  if (nfull * CK < g.k) {
+    load(av[0], bl[0], nfull * CK, std::false_type{});
+    compute(av[0], bl[0], nfull * CK, 0);
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    if (!live[c]) continue;
+    if (par[c] >= 0) {
+      static_cast<T *>(g.dist)[row + out[c] * g.ldc] = curr[c];
+      g.parent[row + out[c] * g.ldp] = par[c];
+    }
+    if (g.out_t) static_cast<T *>(g.out_t)[out[c] + int64_t(row) * g.ld_out_t] = curr[c];
+  }
+}
+
 // two independent products in one launch (the block row and the block column of a blocked
 // Floyd-Warshall step, each too small to fill the chip): the first blocks0 workgroups work on
 // g0, the others on g1
 template <typename T>
-__global__ void __launch_bounds__(256) fwgemm_naive_pair_kernel(FwArgs g0, FwArgs g1, int blocks0) {
+__global__ void __launch_bounds__(256) fwgemm_pair_kernel(FwArgs g0, FwArgs g1, int blocks0) {
   const int b = blockIdx.x;
   if (b < blocks0) {
     const int gx = (g0.m + 63) / 64;
-    fwgemm_naive_block<T>(g0, b % gx, b / gx);
+    fwgemm_rowcols_block<T>(g0, b % gx, b / gx);
   } else {
     const int gx = (g1.m + 63) / 64;
-    fwgemm_naive_block<T>(g1, (b - blocks0) % gx, (b - blocks0) / gx);
+    fwgemm_rowcols_block<T>(g1, (b - blocks0) % gx, (b - blocks0) / gx);
   }
 }
 
-template <typename T> struct vec4_of;
-template <> struct vec4_of<float> { typedef float type __attribute__((ext_vector_type(4))); };
-template <> struct vec4_of<double> { typedef double type __attribute__((ext_vector_type(4))); };
 
 // 256 threads as 16 x 16; each owns TM x TN outputs in groups of four rows /
 // columns that lie 64 apart, so a workgroup covers (16 TM) x (16 TN).
@@ -928,9 +1045,9 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
       // of the diagonal block, which it skips, are not read there)
       const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
                       nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK, 0, 0};
-      const int blocks0 = ((bb + 63) / 64) * ((n + 3) / 4), blocks1 = ((n + 63) / 64) * ((bb + 3) / 4);
-      if (f64) launch_kernel(fwgemm_naive_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
-      else launch_kernel(fwgemm_naive_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      const int blocks0 = ((bb + 63) / 64) * ((n + 15) / 16), blocks1 = ((n + 63) / 64) * ((bb + 15) / 16);
+      if (f64) launch_kernel(fwgemm_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      else launch_kernel(fwgemm_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
       if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     } else {
       FwExtra xr = x, xc = x;
