@@ -470,8 +470,130 @@ def generate_mfma(out_dir):
     return report
 
 
+
+# ---------------------------------------------------------------------------------------------
+# plus-times for double on the matrix cores (mfma_direct_f64.hip): v_mfma_f64_16x16x4_f64
+#
+#   workgroup 256 threads = 4 waves (2 x 2), output tile 128 x 128, wave tile 64 x 64 = 4 x 4 blocks of 16 x 16
+#   v0   .. v127   accumulators, block (bm, bn) in v[8 (4 bm + bn) : +7] (four doubles per lane)
+#   v128 .. v159   A fragments: buffer u, block bm, two doubles = the two steps of a period of 8 k
+#   v160 .. v191   B fragments: buffer u, block bn
+# The instruction takes four k, one from each group of 16 lanes; a period of 8 k is walked as the k-pairs
+# (2 g, 2 g + 1) of lane group g: step s multiplies k = 2 g + s.  A k-contiguous panel ([k/2][X][2] in LDS) then
+# delivers a block's two steps with one 16-byte read per lane, an x-contiguous one ([k][X]) with two 8-byte reads.
+# Two LDS stages: the loads of the tile two ahead are issued after the barrier in the middle of a tile, which
+# is where the stage they go to has been read for the last time.
+class Mfma64Body(MfmaBody):
+    @staticmethod
+    def frag(operand, u, blk, s):
+        return (128 if operand == "A" else 160) + (u * 4 + blk) * 4 + 2 * s
+
+    def reads(self, period):
+        u, P, out = period % 2, period % 2, []
+        for operand, kc, addr in (("A", self.a_kc, "a_addr"), ("B", self.b_kc, "b_addr")):
+            X = 128
+            for blk in range(4):
+                r = self.frag(operand, u, blk, 0)
+                if kc:
+                    fills = {}
+                    for s in range(2):
+                        fills[r + 2 * s] = fills[r + 2 * s + 1] = (operand, blk, period, s)
+                    out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}] offset:{(4 * P * X + blk * 16) * 16}", fills))
+                else:
+                    for s in range(2):
+                        out.append((f"ds_read_b64 v[{r + 2 * s}:{r + 2 * s + 1}], %[{addr}] offset:{((8 * P + s) * X + blk * 16) * 8}",
+                                    {r + 2 * s: (operand, blk, period, s), r + 2 * s + 1: (operand, blk, period, s)}))
+        return out
+
+    def mfma(self, period, s, bm, bn):
+        u = period % 2
+        ra, rb = self.frag("A", u, bm, s), self.frag("B", u, bn, s)
+        for r, want in ((ra, ("A", bm, period, s)), (rb, ("B", bn, period, s))):
+            assert self.content.get(r) == want and self.content.get(r + 1) == want
+        self.require_exact({ra, ra + 1, rb, rb + 1})
+        acc = 8 * (4 * bm + bn)
+        self.lines.append(f'"v_mfma_f64_16x16x4_f64 v[{acc}:{acc + 7}], v[{ra}:{ra + 1}], v[{rb}:{rb + 1}], v[{acc}:{acc + 7}]\\n"')
+        self.groups += 1
+        self.stats["groups"] += 1
+
+    def period(self, period, aux, first, last):
+        order = [(s, bm, bn) for s in range(2) for bn in range(4) for bm in range(4)]
+        behind = {}
+        for i, item in enumerate(aux):
+            slot = first + (i * (last - first + 1)) // len(aux)
+            behind.setdefault(slot, []).append(item)
+        for i, (s, bm, bn) in enumerate(order):
+            self.mfma(period, s, bm, bn)
+            for item in behind.get(i, []):
+                item()
+
+    def dma_chunk(self, index):
+        """One 1 KiB piece of the tile two ahead: pieces 0..3 of the A panel, 4..7 of the B panel."""
+        e = self.emit
+        name, base, m0, h = ("a", "base_a", "m0_a", index) if index < 4 else ("b", "base_b", "m0_b", index - 4)
+        e("s_cmp_lt_i32 %[fetch], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_%=")
+        e(f"s_add_u32 m0, %[{m0}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[{base}]")
+        e(f".Lcuasr_nofetch{index}_%=:")
+
+    def tile(self):
+        e = self.emit
+        for operand in ("A", "B"):
+            for blk in range(4):
+                for s in range(2):
+                    r = self.frag(operand, 0, blk, s)
+                    self.content[r] = self.content[r + 1] = (operand, blk, 0, s)
+        entry = dict(self.content)
+        # period 0 (buffer 0), the LDS reads of period 1 (same stage) behind its matrix instructions
+        self.period(0, [(lambda it=it: self.read(it)) for it in self.reads(1)], 1, 22)
+        # every read of this stage has returned and this wave's part of the next tile has landed (no younger load
+        # is in flight: those of the tile two ahead are issued below); after the barrier both hold for the workgroup
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        self.inflight = []
+        e("s_barrier")
+        e("v_add_u32 %[a_addr], %[a_step], %[a_addr]")
+        e("v_add_u32 %[b_addr], %[b_step], %[b_addr]")
+        e("s_mov_b32 %[m0_save], m0")
+        # period 1 (buffer 1): the next tile's first fragments and the eight loads of the tile two ahead, into the
+        # stage this tile has just left
+        rd = [(lambda it=it: self.read(it)) for it in self.reads(2)]
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(8)]
+        mixed, q = [], 0
+        for i, r in enumerate(rd):
+            while q < 8 and q * len(rd) <= i * 8:
+                mixed.append(aux[q])
+                q += 1
+            mixed.append(r)
+        mixed += aux[q:]
+        self.period(1, mixed, 0, 22)
+        e("s_mov_b32 m0, %[m0_save]")
+        self.drain()
+        shifted = {r: (o, b, p - 2, s) for r, (o, b, p, s) in self.content.items() if p >= 2}
+        assert shifted == entry, "tile body does not reproduce its entry state"
+        return self.lines
+
+
+MFMA64_VARIANTS = {"md_kx": (True, False), "md_xx": (False, False), "md_xk": (False, True), "md_kk": (True, True)}
+
+
+def generate_mfma64(out_dir):
+    os.makedirs(out_dir, exist_ok=True)
+    report = []
+    for name, (a_kc, b_kc) in MFMA64_VARIANTS.items():
+        b = Mfma64Body(a_kc, b_kc)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_prime.inc"), "w") as f:
+            f.write(b.text(b.prime()))
+        b = Mfma64Body(a_kc, b_kc)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_tile.inc"), "w") as f:
+            f.write(b.text(b.tile()))
+        report.append((name, dict(b.stats)))
+    return report
+
+
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
     out = sys.argv[1] if len(sys.argv) > 1 else os.path.join(here, "gen")
-    for name, stats in generate(out) + generate_mfma(out):
+    for name, stats in generate(out) + generate_mfma(out) + generate_mfma64(out):
         print(name, stats)

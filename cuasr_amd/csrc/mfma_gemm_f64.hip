@@ -20,6 +20,10 @@
 #include "semiring.h"
 
 namespace cuasr_amd {
+
+bool mfma_direct_f64_can_run(const Problem &);                // mfma_direct_f64.hip
+hipError_t mfma_direct_f64_launch(const Problem &, hipStream_t);
+
 namespace gemm_mfma_f64 {
 
 typedef double v2d __attribute__((ext_vector_type(2)));
@@ -267,6 +271,10 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   if (!can_run(p)) return hipErrorNotSupported;
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  // whole k-tiles, loadable straight into LDS, and outputs that fill their rounds of 512 workgroups at least to
+  // 7/8: the hand-scheduled form of the same tile
+  const long long groups = tiles * (p.workspace ? p.slices : 1), rounds = (groups + 511) / 512;
+  if (groups * 8 >= rounds * 512 * 7 && mfma_direct_f64_can_run(p)) return mfma_direct_f64_launch(p, s);
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
   launch_kernel(gemm_mfma_f64_kernel, grid, dim3(256), 0, s, p);
   return take_launch_status();

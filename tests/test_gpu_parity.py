@@ -198,6 +198,21 @@ def test_plus_times_mfma_f64_small_integers(oracle, lib, shape, layouts):
         run(oracle, "plus", "multiplies", "f64", *shape, la, lb, lc, "mfma", beta_one)
 
 
+@pytest.mark.parametrize("shape", [(3584, 2048, 16), (3586, 2046, 48), (3586, 2046, 160), (3584, 2048, 32)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_plus_times_mfma_f64_hand_scheduled(oracle, lib, shape, layouts):
+    """Outputs that fill a round of 128 x 128 tiles with k a multiple of 16 take the hand-scheduled fp64
+    matrix-core loop (one, two, three and ten k-tiles; ragged edges in m and n); small integers, so the
+    host reference's bits are the answer."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    run(oracle, "plus", "multiplies", "f64", *shape, la, lb, lc, "mfma", shape[2] == 48)
+
+
+def test_plus_times_mfma_f64_hand_scheduled_splitk(oracle, lib):
+    run(oracle, "plus", "multiplies", "f64", 1024, 1024, 512, "row", "col", "row", "mfma", True, splitk=8)
+    run(oracle, "plus", "multiplies", "f64", 1024, 1024, 1024, "col", "row", "col", "mfma", False, splitk=8)
+
+
 def test_plus_times_mfma_f64_splitk(oracle, lib):
     run(oracle, "plus", "multiplies", "f64", 128, 128, 1000, "row", "col", "row", "mfma", True, splitk=8)
     run(oracle, "plus", "multiplies", "f64", 100, 60, 332, "col", "col", "col", "mfma", True, splitk=3)
