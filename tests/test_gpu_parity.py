@@ -149,6 +149,25 @@ def test_direct_tile(oracle, lib, sr, shape, layouts):
         run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "direct", beta_one)
 
 
+@pytest.mark.parametrize("sr", [("bit_xor", "bit_and", "u32"), ("bit_or", "bit_and", "u32"), ("bit_xor", "bit_and", "i32")])
+@pytest.mark.parametrize("shape", [(256, 128, 16), (256, 128, 32), (260, 132, 48), (516, 388, 160), (1024, 1024, 1024), (12, 8, 64)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"])
+def test_direct_tile_on_words(oracle, lib, sr, shape, layouts):
+    """xor-and / or-and on 32-bit words with k a multiple of 16 on the direct-to-LDS tile: one, two, three and
+    many k-tiles (every depth of its three-stage prologue), ragged edges in m and n, an output smaller than a
+    tile, every layout combination."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    if shape[0] >= 1024 and layouts not in ("ccc", "rcr", "crr", "rrr"):
+        pytest.skip("large shape: four layout combinations are enough")
+    for beta_one in (False, True):
+        run(oracle, sr[0], sr[1], sr[2], *shape, la, lb, lc, "direct", beta_one)
+
+
+def test_direct_tile_on_words_splitk(oracle, lib):
+    run(oracle, "bit_xor", "bit_and", "u32", 260, 132, 512, "col", "col", "col", "direct", True, splitk=4)
+    run(oracle, "bit_or", "bit_and", "u32", 256, 256, 1024, "row", "row", "row", "direct", False, splitk=8)
+
+
 @pytest.mark.parametrize("slices", [1, 3, 8])
 def test_splitk_direct(oracle, lib, slices):
     run(oracle, "minimum", "plus", "f32", 128, 128, 1000, "row", "col", "row", "direct", False, splitk=slices)
