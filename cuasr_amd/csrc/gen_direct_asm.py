@@ -323,21 +323,21 @@ def generate(out_dir):
 # next period are issued after the first eight matrix instructions of this one, so a register is overwritten
 # 500 cycles and more after the last instruction that read it was issued.
 class MfmaBody(Body):
-    def __init__(self, a_kc, b_kc):
+    def __init__(self, a_kc, b_kc, nbn=4):
         self.a_kc, self.b_kc = a_kc, b_kc
+        self.nbn = nbn   # 32-column blocks per wave: 4 (output tile 128 x 256) or 2 (128 x 128, accumulators v0 .. v63)
         self.lines, self.inflight, self.groups = [], [], 0
         self.stats = {"groups": 0, "lds": 0, "waits": 0, "other": 0}
         self.content = {}
 
-    @staticmethod
-    def frag(operand, u, blk, s):
-        return (128 + (u * 2 + blk) * 4 + s) if operand == "A" else (144 + (u * 4 + blk) * 4 + s)
+    def frag(self, operand, u, blk, s):
+        return (128 + (u * 2 + blk) * 4 + s) if operand == "A" else (144 + (u * self.nbn + blk) * 4 + s)
 
     def reads(self, period):
         """[(asm text, {register: content})]: LDS reads of the fragments of absolute period `period` (0, 1 of this
         tile; 2 = the next tile's first, through the already advanced addresses) into buffer period % 2."""
         u, P, out = period % 2, period % 2, []
-        for operand, kc, X, nblk, addr in (("A", self.a_kc, 128, 2, "a_addr"), ("B", self.b_kc, 256, 4, "b_addr")):
+        for operand, kc, X, nblk, addr in (("A", self.a_kc, 128, 2, "a_addr"), ("B", self.b_kc, 64 * self.nbn, self.nbn, "b_addr")):
             for blk in range(nblk):
                 r = self.frag(operand, u, blk, 0)
                 if kc:
@@ -360,7 +360,7 @@ class MfmaBody(Body):
         ra, rb = self.frag("A", u, bm, s), self.frag("B", u, bn, s)
         assert self.content.get(ra) == ("A", bm, period, s) and self.content.get(rb) == ("B", bn, period, s)
         self.require_exact({ra, rb})
-        acc = 16 * (4 * bm + bn)
+        acc = 16 * (self.nbn * bm + bn)
         self.lines.append(f'"v_mfma_f32_32x32x2_f32 v[{acc}:{acc + 15}], v{ra}, v{rb}, v[{acc}:{acc + 15}]\\n"')
         self.groups += 1
         self.stats["groups"] += 1
@@ -377,7 +377,7 @@ class MfmaBody(Body):
     def period(self, period, aux, first, last):
         """The 32 matrix instructions of a period of 8 k, with the callables of `aux` spread evenly behind
         instructions first .. last of them (counted from 0)."""
-        order = [(s, bm, bn) for s in range(4) for bn in range(4) for bm in range(2)]
+        order = [(s, bm, bn) for s in range(4) for bn in range(self.nbn) for bm in range(2)]
         behind = {}
         for i, item in enumerate(aux):
             slot = first + (i * (last - first + 1)) // len(aux)
@@ -407,7 +407,7 @@ class MfmaBody(Body):
 
     def tile(self):
         e = self.emit
-        for operand, nblk in (("A", 2), ("B", 4)):
+        for operand, nblk in (("A", 2), ("B", self.nbn)):
             for blk in range(nblk):
                 for s in range(4):
                     self.content[self.frag(operand, 0, blk, s)] = (operand, blk, 0, s)
@@ -417,24 +417,26 @@ class MfmaBody(Body):
         # ahead and the LDS reads of period 1 (same stage) -- everything but the matrix instructions is spread so
         # that the matrix pipe never waits for a run of other instructions, and the last eight matrix instructions
         # (500 cycles) cover the latency of the last read
-        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(6)]
+        nld = 2 + self.nbn                       # this wave's loads per k-tile
+        last = 8 * self.nbn - 9                  # the last eight matrix instructions of a period cover the latency
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(nld)]
         rd = [(lambda it=it: self.read(it)) for it in self.reads(1)]
         # interleave the two kinds
         mixed, q = [], 0
         for i, r in enumerate(rd):
-            while q < 6 and q * len(rd) <= i * 6:
+            while q < nld and q * len(rd) <= i * nld:
                 mixed.append(aux[q])
                 q += 1
             mixed.append(r)
         mixed += aux[q:]
-        self.period(0, mixed, 1, 23)
+        self.period(0, mixed, 1, last)
         e("s_mov_b32 m0, %[m0_save]")
         # every read of this stage has returned; this wave's part of the next tile has landed (its six loads are
         # older than the six of the tile two ahead, if those were issued); after the barrier both hold for the
         # workgroup, and the reads from here on go to the next stage
         e("s_cmp_lt_i32 %[fetch], 1")
         e("s_cbranch_scc1 .Lcuasr_all_%=")
-        e("s_waitcnt vmcnt(6) lgkmcnt(0)")
+        e(f"s_waitcnt vmcnt({nld}) lgkmcnt(0)")
         e("s_branch .Lcuasr_join_%=")
         e(".Lcuasr_all_%=:")
         e("s_waitcnt vmcnt(0) lgkmcnt(0)")
@@ -443,7 +445,7 @@ class MfmaBody(Body):
         e("s_barrier")
         e("v_add_u32 %[a_addr], %[a_step], %[a_addr]")
         e("v_add_u32 %[b_addr], %[b_step], %[b_addr]")
-        self.period(1, [(lambda it=it: self.read(it)) for it in self.reads(2)], 1, 23)
+        self.period(1, [(lambda it=it: self.read(it)) for it in self.reads(2)], 1, last)
         self.drain()
         shifted = {r: (o, b, p - 2, s) for r, (o, b, p, s) in self.content.items() if p >= 2}
         assert shifted == entry, "tile body does not reproduce its entry state"
@@ -453,22 +455,22 @@ class MfmaBody(Body):
         return "\n".join(ln if ln.startswith('"v_mfma') else '"' + ln + '\\n"' for ln in lines) + "\n"
 
 
-MFMA_VARIANTS = {"m_kx": (True, False), "m_xx": (False, False), "m_xk": (False, True), "m_kk": (True, True)}
+MFMA_VARIANTS = {"m_kx": (True, False, 4), "m_xx": (False, False, 4), "m_xk": (False, True, 4), "m_kk": (True, True, 4),
+                 "m2_kx": (True, False, 2), "m2_xx": (False, False, 2), "m2_xk": (False, True, 2), "m2_kk": (True, True, 2)}
 
 
 def generate_mfma(out_dir):
     os.makedirs(out_dir, exist_ok=True)
     report = []
-    for name, (a_kc, b_kc) in MFMA_VARIANTS.items():
-        b = MfmaBody(a_kc, b_kc)
+    for name, (a_kc, b_kc, nbn) in MFMA_VARIANTS.items():
+        b = MfmaBody(a_kc, b_kc, nbn)
         with open(os.path.join(out_dir, f"mfma_asm_{name}_prime.inc"), "w") as f:
             f.write(b.text(b.prime()))
-        b = MfmaBody(a_kc, b_kc)
+        b = MfmaBody(a_kc, b_kc, nbn)
         with open(os.path.join(out_dir, f"mfma_asm_{name}_tile.inc"), "w") as f:
             f.write(b.text(b.tile()))
         report.append((name, dict(b.stats)))
     return report
-
 
 
 # ---------------------------------------------------------------------------------------------

@@ -197,6 +197,15 @@ def test_plus_times_mfma_hand_scheduled(oracle, lib, shape, layouts):
     run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", shape[2] == 48)
 
 
+@pytest.mark.parametrize("shape", [(2048, 2048, 16), (2052, 2044, 48), (1156, 1284, 160), (2048, 2048, 32)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
+def test_plus_times_mfma_hand_scheduled_narrow_tile(oracle, lib, shape, layouts):
+    """Outputs whose 128 x 256 tiles would leave most of a round empty take the 128 x 128 form of the
+    hand-scheduled loop; same cases as for the wide one."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", shape[2] == 48)
+
+
 def test_plus_times_mfma_hand_scheduled_splitk(oracle, lib):
     run(oracle, "plus", "multiplies", "f32", 1024, 1024, 512, "row", "col", "row", "mfma", True, splitk=16)
     run(oracle, "plus", "multiplies", "f32", 1024, 1024, 1024, "col", "row", "col", "mfma", False, splitk=16)
