@@ -25,6 +25,8 @@ bool direct_can_run(const Problem &);
 bool direct64_can_run(const Problem &);
 bool mfma_f32_can_run(const Problem &);
 bool mfma_f64_can_run(const Problem &);
+bool mfma_direct_f32_can_run(const Problem &);
+bool mfma_direct_f64_can_run(const Problem &);
 
 launch_fn find_valu(int dtype, int add_op, int mult_op) {
   switch (dtype) {
@@ -354,9 +356,10 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream) {
   return fn(p, s) == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
 }
 
-// A strided batch.  The tile kernels take the product index from the grid (blockIdx.z), so a batch of
-// small products is one launch that fills the chip; the matrix-core and the naive kernels, and batches
-// beyond the grid's 65535, are sequences of launches.
+// A strided batch.  The tile kernels -- the vector-ALU ones and the hand-scheduled matrix-core ones -- take the
+// product index from the grid (blockIdx.z), so a batch of small products is one launch that fills the chip; the
+// compiled matrix-core kernels (ragged k, unaligned products) and the naive kernel, and batches beyond the
+// grid's 65535, are sequences of launches.
 int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a, int64_t stride_b,
                              int64_t stride_c, int64_t stride_d, void *stream) {
   if (!desc || batch < 0 || stride_a < 0 || stride_b < 0 || stride_c < 0 || stride_d < 0)
@@ -370,7 +373,17 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
   if (batch == 0) return CUASR_AMD_SUCCESS;
   const int64_t es = int64_t(elem_size(desc->dtype));
   const int family = pick_family(desc, batch);
-  if ((family == kValu || family == kDirect) && batch > 1) {
+  bool in_grid = (family == kValu || family == kDirect) && batch > 1;
+  if (family == kMfma && batch > 1 && desc->add_op == kPlus && desc->mult_op == kMultiplies) {
+    // the hand-scheduled matrix-core tiles take a batch in the grid too; the compiled ones (ragged k, unaligned
+    // products) do not: ask with the first launch's problem
+    Problem probe = canonical(desc);
+    probe.batch = batch < 65535 ? batch : 65535;
+    probe.batch_a = col ? stride_b : stride_a;
+    probe.batch_b = col ? stride_a : stride_b;
+    in_grid = desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
+  }
+  if (in_grid) {
     const launch_fn fn = family_fn(family, desc);
     if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;
     Problem p = canonical(desc);

@@ -198,6 +198,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, NBN == 4
   constexpr int BN = 64 * NBN, WN = 32 * NBN;
   constexpr unsigned B_STAGE = BK * BN * 4;
   __shared__ Smem<NBN> sm;
+  select_batch<float>(p);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -320,6 +321,7 @@ static bool can_run(const Problem &p) {
   if (!mfma_panel::can_run(p)) return false;
   if (p.k % BK) return false;
   if (p.workspace && p.k_per_slice % BK) return false;
+  if (p.batch > 1 && (p.workspace || p.batch_a % 4 || p.batch_b % 4)) return false;  // every product 16-byte aligned
   const long long lim = 1LL << 30;  // elements
   if (p.sa_m * (long long)BM >= lim || p.sa_k * (long long)BK >= lim || p.sb_n * 256LL >= lim || p.sb_k * (long long)BK >= lim)
     return false;
@@ -335,7 +337,7 @@ static hipError_t launch(const Problem &p, bool wide, hipStream_t s) {
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   const bool a_kc = p.sa_m != 1, b_kc = p.sb_n != 1;
   auto go = [&](auto kernel) {
-    launch_kernel(kernel, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
+    launch_kernel(kernel, dim3((unsigned)tiles, (unsigned)slices, (unsigned)(p.batch > 1 ? p.batch : 1)), dim3(256), 0, s, p);
     return take_launch_status();
   };
   if (wide) {

@@ -141,6 +141,7 @@ __device__ __forceinline__ void Loop<true, true>::tile(CUASR_MFMA64_TILE_ARGS) {
 template <bool A_KC, bool B_KC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_direct_f64_kernel(Problem p) {
   __shared__ Smem sm;
+  select_batch<double>(p);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_m = (p.m + BM - 1) / BM, tiles_n = (p.n + BN - 1) / BN;
@@ -264,6 +265,7 @@ static bool can_run(const Problem &p) {
   if (b_xc ? (p.n % 2 || p.sb_k % 2) : (p.sb_k != 1 || p.sb_n % 2)) return false;
   if (p.k % BK) return false;
   if (p.workspace && p.k_per_slice % BK) return false;
+  if (p.batch > 1 && (p.workspace || p.batch_a % 2 || p.batch_b % 2)) return false;  // every product 16-byte aligned
   const long long lim = 1LL << 29;  // elements
   if (p.sa_m * (long long)BM >= lim || p.sa_k * (long long)BK >= lim || p.sb_n * (long long)BN >= lim || p.sb_k * (long long)BK >= lim)
     return false;
@@ -277,7 +279,7 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   const bool a_kc = p.sa_m != 1, b_kc = p.sb_n != 1;
   auto go = [&](auto kernel) {
-    launch_kernel(kernel, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
+    launch_kernel(kernel, dim3((unsigned)tiles, (unsigned)slices, (unsigned)(p.batch > 1 ? p.batch : 1)), dim3(256), 0, s, p);
     return take_launch_status();
   };
   if (a_kc) return b_kc ? go(gemm_mfma_direct_f64_kernel<true, true>) : go(gemm_mfma_direct_f64_kernel<true, false>);

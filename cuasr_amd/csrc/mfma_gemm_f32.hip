@@ -327,10 +327,12 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   // times, and the tile that wastes less of its last such round wins (2048^3: 132 against 71 TFLOP/s for the narrow
   // tile, 5120^3: 133 against 117, 6144^3: 150 against 136); where both fill theirs (4096^3: 149.1 and 149.8) the
   // wide one, which moves a quarter less data per flop.
+  const long long batch = p.batch > 1 ? p.batch : 1;
   if (mfma_direct_f32_can_run(p)) {
     auto fill = [](long long groups) { return (double)groups / (256.0 * (double)((groups + 255) / 256)); };
-    return mfma_direct_f32_launch(p, fill(wide * slices) >= 0.995 * fill(tiles * slices), s);
+    return mfma_direct_f32_launch(p, fill(wide * slices * batch) >= 0.995 * fill(tiles * slices * batch), s);
   }
+  if (batch > 1) return hipErrorNotSupported;  // the compiled kernels take one product per launch
   // the 128 x 256 tile when its workgroups fill >= 7/8 of whole rounds of 512 (two per compute unit)
   const long long rounds = (wide * slices + 511) / 512;
   if (wide * slices * 8 >= rounds * 512 * 7)

@@ -274,6 +274,7 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   // whole k-tiles, loadable straight into LDS: the hand-scheduled form of the same tile (faster at every size
   // measured, also where a round of workgroups is mostly empty: 2048^3 71.9 against 54.8 TFLOP/s)
   if (mfma_direct_f64_can_run(p)) return mfma_direct_f64_launch(p, s);
+  if (p.batch > 1) return hipErrorNotSupported;  // the compiled kernel takes one product per launch
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
   launch_kernel(gemm_mfma_f64_kernel, grid, dim3(256), 0, s, p);
   return take_launch_status();

@@ -166,10 +166,12 @@ int cuasr_amd_srgemm(const cuasr_amd_srgemm_desc *desc, void *stream);
  * products; the outputs must lie at least one matrix apart, strides must not be
  * negative (CUASR_AMD_ERROR_INVALID_PROBLEM otherwise).  The kernel family is
  * chosen once, for the whole batch (what fills the chip is the batch, not one
- * product); on the vector-ALU tiles the product index is part of the grid, so a
- * batch of many small products is a single launch; the matrix-core and naive
- * kernels run the products one after the other on the stream.  Each product's
- * result is that of a single cuasr_amd_srgemm on its operands. */
+ * product); on the vector-ALU tiles, and on the matrix-core tiles for products
+ * whose k is a multiple of 16 and whose operands (batch strides included) are
+ * 16-byte aligned, the product index is part of the grid, so a batch of many
+ * small products is a single launch; the other matrix-core kernels and the
+ * naive kernel run the products one after the other on the stream.  Each
+ * product's result is that of a single cuasr_amd_srgemm on its operands. */
 int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a,
                              int64_t stride_b, int64_t stride_c, int64_t stride_d, void *stream);
 

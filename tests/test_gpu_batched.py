@@ -105,3 +105,37 @@ def test_batch_larger_than_one_grid(oracle):
     cuasr_amd.srgemm_batched("minimum", "plus", dA, dB, dD, dD, 0.0, inf, inf, 0.0)
     want = (A[:, :, :, None] + B[:, None, :, :]).min(axis=2)            # min-plus of every product, exact in fp32
     assert_same_bits(dD.cpu().numpy(), want, "65540 products")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kernel", ["auto", "mfma"])
+def test_plus_times_batch_on_the_matrix_cores(oracle, dtype, kernel):
+    """A batch of plus-times products large enough for the matrix cores: the hand-scheduled tiles take the
+    product index from the grid.  Small integers, so the sums are exact in any order; row-major products with
+    padding rows between them, one B shared by the whole batch, and a column-major batch."""
+    import torch
+    batch, m, n, k = 12, 512, 384, 160
+    rng = np.random.default_rng(23)
+    A = rng.integers(-4, 5, (batch, m + 4, k)).astype(dtype)
+    B = rng.integers(-4, 5, (k, n)).astype(dtype)
+    C = rng.integers(-9, 9, (batch, m, n)).astype(dtype)
+    dA = torch.from_numpy(A).cuda()
+    dB = torch.from_numpy(B).cuda().unsqueeze(0).expand(batch, k, n)
+    dC = torch.from_numpy(C).cuda()
+    dD = torch.zeros(batch, m, n, dtype=dA.dtype, device="cuda")
+    cuasr_amd.srgemm_batched("plus", "multiplies", dA[:, :m, :], dB, dC, dD, 1.0, 1.0, 0.0, 1.0, kernel=kernel)
+    got = dD.cpu().numpy()
+    for i in range(batch):
+        want = oracle.srgemm("plus", "multiplies", np.ascontiguousarray(A[i, :m]), B, C[i], 1.0, 1.0, 0.0)
+        assert_same_bits(got[i], want, f"{kernel} product {i}")
+    # column-major products (the transposed problem: A and B swap, and so do their batch strides)
+    At = rng.integers(-4, 5, (batch, k, m)).astype(dtype)              # slices are column-major m x k
+    Bt = rng.integers(-4, 5, (batch, n, k)).astype(dtype)
+    dAt, dBt = torch.from_numpy(At).cuda().transpose(1, 2), torch.from_numpy(Bt).cuda().transpose(1, 2)
+    dDt = torch.zeros(batch, n, m, dtype=dAt.dtype, device="cuda").transpose(1, 2)
+    cuasr_amd.srgemm_batched("plus", "multiplies", dAt, dBt, dDt, dDt, 1.0, 0.0, 0.0, 1.0, kernel=kernel)
+    got = dDt.cpu().numpy()
+    for i in range(0, batch, 5):
+        want = oracle.srgemm("plus", "multiplies", np.asfortranarray(At[i].T), np.asfortranarray(Bt[i].T),
+                             np.zeros((m, n), dtype, order="F"), 1.0, 0.0, 0.0)
+        assert_same_bits(np.ascontiguousarray(got[i]), np.ascontiguousarray(want), f"{kernel} column-major product {i}")
