@@ -18,6 +18,7 @@
 //     stored distance is that product, which keeps the sign of a zero as the
 //     sequential scan would.
 // Operands must be free of NaN and of -infinity (+infinity marks "no edge").
+#include "direct_tile.h"
 #include "semiring.h"
 
 #include <limits>
@@ -707,6 +708,185 @@ __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   fwgemm_tile_body<T, TM, TN, SN, BK, GUARD, HAS_AT>(g, bx, by);
 }
 
+// ---- the predecessor-tracking product on the hand-scheduled direct-to-LDS tile (direct_tile.h, direct_asm.h)
+//
+// For whole, aligned fp32 problems with the k-contiguous image of A at hand.  Column-major dist = A (x) B is the
+// row-major transposed problem dist^T = B^T (x) A^T, so the tile's "A" panel is B (k-contiguous) and its "B" panel
+// is A (x-contiguous): the generated loop's kx form, 512 threads, 256 columns x 128 rows of dist per workgroup, the
+// loop's accumulators being the running minima themselves (they start from dist).  What the loop cannot do is
+// remember WHEN a minimum improved, and its 128 registers leave no room for that; so this kernel runs it with
+// 256 registers (two waves per SIMD) and keeps, beside it, a copy of the accumulators as they were two k-tiles
+// ago and a 16-bit chunk index per element: after every second k-tile "accumulator < copy" (strict) records
+// the chunk of 32 k, four instructions per element and 32 k against the 48 of the terms themselves.  The
+// epilogue is the tile kernel's: improved elements are queued in LDS and looked up, 32 values of A's row (from
+// the k-contiguous image) and 32 of B's column each, first k whose sum equals the minimum.
+constexpr int FWD_CHUNK = 32;
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) fwgemm_direct_kernel(FwArgs g) {
+  typedef DirectTile<float, kMinimum, kPlus, true, false, 32, 16> Tile;
+  typedef AsmLoop<float, kMinimum, kPlus, true, false>::type Loop;
+  typedef vec4_of<float>::type V4;
+  constexpr int BC = 256, BR = 128, BK = 16, STAGES = 3;   // dist columns and rows per workgroup
+  __shared__ Tile::Smem sm;
+  const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16, lane = tid & 63, wave = tid >> 6;
+  int bc, br;
+  Tile::tile_coords(blockIdx.x, g.n / BC, g.m / BR, bc, br);
+  const int n0 = bc * BC, m0 = br * BR;
+  const float *A = static_cast<const float *>(g.A);
+  const float *B = static_cast<const float *>(g.B);
+  float *dist = static_cast<float *>(g.dist);
+  // output (i, j) of the thread: dist column n0 + 32 i + ty, dist row m0 + 64 (j / 4) + 4 tx + j % 4
+  auto col_of = [&](int i) { return n0 + 32 * i + ty; };
+  auto row_of = [&](int j) { return m0 + 64 * (j >> 2) + 4 * tx + (j & 3); };
+
+  AsmRegs r;
+  // element e = 8 i + j: the loop's accumulator is v(e); its value before the chunk in hand run[e / 16][e % 16] =
+  // v(128 + e); its chunk index 16 bits of chunk[e / 32][(e / 2) % 16] = v(192 + e / 2), 0xffff = never improved
+  asm_v16 run[4], chunk[2];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const V4 v = *reinterpret_cast<const V4 *>(dist + row_of(4 * h) + int64_t(col_of(i)) * g.ldc);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        run[i >> 1][(i & 1) * 8 + 4 * h + e] = v[e];
+        r.acc[i >> 1][(i & 1) * 8 + 4 * h + e] = v[e];
+      }
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 2; ++v) chunk[v] = asm_v16(__builtin_bit_cast(float, 0xffffffffu));
+#pragma unroll
+  for (int v = 0; v < 3; ++v) r.frag[v] = asm_v16(0.0f);
+
+  // global -> LDS: the tile's "A" panel is B's 256 columns (k-contiguous, two pieces per wave and k-tile), its
+  // "B" panel A's 128 rows (x-contiguous, one piece per wave)
+  const char *base_a = reinterpret_cast<const char *>(B + int64_t(n0) * g.ldb);
+  const char *base_b = reinterpret_cast<const char *>(A + m0);
+  const long long a_next = (long long)BK * 4, b_next = (long long)BK * g.lda * 4;
+  const unsigned b_kbytes = (unsigned)g.lda * 4u;
+  const unsigned off_a0 = Tile::tile_offset<true, BC>((wave * 2 + 0) * 64 + lane, Tile::x_offset<true, BC>((wave * 2 + 0) * 64 + lane, g.ldb, n0, g.n), 4u, BK);
+  const unsigned off_a1 = Tile::tile_offset<true, BC>((wave * 2 + 1) * 64 + lane, Tile::x_offset<true, BC>((wave * 2 + 1) * 64 + lane, g.ldb, n0, g.n), 4u, BK);
+  const unsigned off_b0 = Tile::tile_offset<false, BR>(wave * 64 + lane, Tile::x_offset<false, BR>(wave * 64 + lane, 1, m0, g.m), b_kbytes, BK);
+  auto fetch = [&](int stage) {
+    Tile::dma16(reinterpret_cast<const float *>(base_a + off_a0), &sm.a[stage][(wave * 2 + 0) * 256]);
+    Tile::dma16(reinterpret_cast<const float *>(base_a + off_a1), &sm.a[stage][(wave * 2 + 1) * 256]);
+    Tile::dma16(reinterpret_cast<const float *>(base_b + off_b0), &sm.b[stage][wave * 256]);
+    base_a += a_next;
+    base_b += b_next;
+  };
+  const int ntiles = g.k / BK;   // the host sends whole pairs of k-tiles only
+  fetch(0);
+  __syncthreads();
+  fetch(1);  // from here base_a / base_b point at tile 2
+  const unsigned m0_a0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) float *)&sm.a[0][(wave * 2) * 256]);
+  const unsigned m0_b0 = __builtin_amdgcn_readfirstlane((unsigned)(size_t)(__attribute__((address_space(3))) float *)&sm.b[0][wave * 256]);
+  constexpr unsigned A_STAGE = BK * BC * 4, B_STAGE = BK * BR * 4;
+  unsigned a_addr = (unsigned)(size_t)(__attribute__((address_space(3))) float *)&sm.a[0][0] + ty * 16;
+  unsigned b_addr = (unsigned)(size_t)(__attribute__((address_space(3))) float *)&sm.b[0][0] + tx * 16;
+  Loop::prime(r, a_addr, b_addr);
+  int stage = 0;
+  auto one_tile = [&](int t) {
+    const int next = stage + 1 == STAGES ? 0 : stage + 1, stage2 = next + 1 == STAGES ? 0 : next + 1;
+    Loop::tile(r, a_addr, b_addr, (unsigned)((next - stage) * (int)A_STAGE), (unsigned)((next - stage) * (int)B_STAGE),
+               ntiles - (t + 2), m0_a0 + stage2 * A_STAGE, m0_b0 + stage2 * B_STAGE, off_a0, off_a1, off_b0, base_a, base_b);
+    base_a += a_next;
+    base_b += b_next;
+    stage = next;
+  };
+#pragma unroll 1
+  for (int t = 0; t < ntiles; t += 2) {   // a chunk of 32 k: two k-tiles, then the bookkeeping (no branch around it)
+    one_tile(t);
+    one_tile(t + 1);
+    // the bookkeeping (gen/fwgemm_merge.inc, written by gen_direct_asm.py): a cheap test whether any of the
+    // wave's elements changed in this chunk, and only then, per element, "now < before" => chunk index, before = now
+    const uint32_t c = (uint32_t)(t >> 1);
+    asm volatile(
+#include "gen/fwgemm_merge.inc"
+        : "+{v[0:15]}"(r.acc[0]), "+{v[16:31]}"(r.acc[1]), "+{v[32:47]}"(r.acc[2]), "+{v[48:63]}"(r.acc[3]),
+          "+{v[128:143]}"(run[0]), "+{v[144:159]}"(run[1]), "+{v[160:175]}"(run[2]), "+{v[176:191]}"(run[3]),
+          "+{v[192:207]}"(chunk[0]), "+{v[208:223]}"(chunk[1])
+        : [chunk] "v"(c)
+        : "v224", "vcc");
+  }
+
+  // ---- improved elements: the first k of the recorded chunk whose sum equals the minimum.  One canonical row i
+  // (one dist column per thread) of the lanes' outputs at a time into a queue in LDS (the panels are done with),
+  // which all 512 threads then work off, one element per thread and turn.
+  constexpr int CAP = 512 * 8;
+  static_assert(sizeof(Tile::Smem) >= 3 * CAP * sizeof(int), "the queue must fit in the panels");
+  __shared__ int q_count;
+  int *q_pos = reinterpret_cast<int *>(&sm.a[0][0]);   // row | column << 8, inside the tile
+  int *q_ch = q_pos + CAP;
+  float *q_want = reinterpret_cast<float *>(q_ch + CAP);
+  const float *At = static_cast<const float *>(g.At);
+  int tx2 = tx, ty2 = ty;
+  asm volatile("" : "+v"(tx2), "+v"(ty2));
+#pragma unroll 1
+  for (int i = 0; i < 8; ++i) {
+    __syncthreads();  // everybody is done with the panels / with the queue of the row before
+    if (tid == 0) q_count = 0;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // (i is a run-time value here: the registers are read through a select chain over the 8 rows)
+      uint32_t w = 0;
+      float want = 0.f;
+#pragma unroll
+      for (int ii = 0; ii < 8; ++ii)
+        if (ii == i) {
+          w = __builtin_bit_cast(uint32_t, (float)chunk[ii >> 2][(ii & 3) * 4 + (j >> 1)]);
+          want = run[ii >> 1][(ii & 1) * 8 + j];
+        }
+      const uint32_t ch = (j & 1) ? w >> 16 : w & 0xffffu;
+      if (ch != 0xffffu) {
+        const int slot = atomicAdd(&q_count, 1);
+        q_pos[slot] = (64 * (j >> 2) + 4 * tx2 + (j & 3)) | ((32 * i + ty2) << 8);
+        q_ch[slot] = (int)ch;
+        q_want[slot] = want;
+      }
+    }
+    __syncthreads();
+    const int count = q_count;
+    for (int e = tid; e < count; e += 512) {
+      const int pos = q_pos[e], row = m0 + (pos & 255), col = n0 + (pos >> 8), k0 = q_ch[e] * FWD_CHUNK;
+      const float want = q_want[e];
+      const V4 *ap = reinterpret_cast<const V4 *>(At + k0 + int64_t(row) * g.ldat);
+      const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(col) * g.ldb);
+      V4 pa[FWD_CHUNK / 4], pb[FWD_CHUNK / 4];
+#pragma unroll
+      for (int q = 0; q < FWD_CHUNK / 4; ++q) {
+        pa[q] = ap[q];
+        pb[q] = bp[q];
+      }
+      float value = want;
+      int first = 0;
+#pragma unroll
+      for (int kk = FWD_CHUNK - 1; kk >= 0; --kk) {
+        const float prod = pa[kk >> 2][kk & 3] + pb[kk >> 2][kk & 3];
+        const bool hit = prod == want;
+        first = hit ? kk : first;
+        value = pick(hit, prod, value);
+      }
+      dist[row + int64_t(col) * g.ldc] = value;
+      g.parent[row + int64_t(col) * g.ldp] = g.k_base + k0 + first;
+    }
+  }
+}
+
+// whole tiles of 128 rows x 256 columns, k in whole chunks, every operand (and the k-contiguous image of A)
+// 16-byte aligned with leading dimensions that are multiples of 4, no rows / columns to skip, chunk indices in 16 bits
+bool fwgemm_direct_ok(const FwArgs &g) {
+  auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  if (g.m <= 0 || g.n <= 0 || g.k < 2 * FWD_CHUNK || g.m % 128 || g.n % 256 || g.k % FWD_CHUNK || g.k / FWD_CHUNK >= 0xffff) return false;
+  if (!g.At || !al(g.A) || !al(g.B) || !al(g.dist) || !al(g.At)) return false;
+  if (g.lda % 4 || g.ldb % 4 || g.ldc % 4 || g.ldat % 4) return false;
+  if (g.skip_r1 > g.skip_r0 || g.skip_c1 > g.skip_c0 || g.ahead_bb > 0 || g.out_t) return false;
+  // 32-bit byte offsets inside a tile
+  if (int64_t(g.ldb) * 256 * 4 >= (int64_t(1) << 31) || int64_t(g.lda) * 16 * 4 >= (int64_t(1) << 31)) return false;
+  return int64_t(g.m / 128) * (g.n / 256) <= 0x7fffffff;
+}
+
 template <typename T, int TM, int TN, int SN, int BK>
 hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
@@ -924,6 +1104,10 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
   }
   if (x.closed_ahead) *x.closed_ahead = g.ahead_bb > 0;
   hipError_t e;
+  if (dtype == CUASR_AMD_F32 && !naive && kernel == CUASR_AMD_KERNEL_AUTO && fwgemm_direct_ok(g)) {
+    launch_kernel(fwgemm_direct_kernel, dim3((unsigned)(int64_t(g.m / 128) * (g.n / 256))), dim3(512), 0, s, g);
+    return take_launch_status() == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;
+  }
   if (dtype == CUASR_AMD_F32) e = naive ? launch_naive<float>(g, s) : launch_tile<float, 8, 8, 4, 16>(g, s);
   else e = naive ? launch_naive<double>(g, s) : launch_tile<double, 4, 8, 4, 16>(g, s);
   return e == hipSuccess ? CUASR_AMD_SUCCESS : CUASR_AMD_ERROR_INTERNAL;

@@ -594,8 +594,40 @@ def generate_mfma64(out_dir):
     return report
 
 
+
+# ---------------------------------------------------------------------------------------------
+# The bookkeeping of the predecessor-tracking product on the direct tile (fwgemm.hip, fwgemm_direct_kernel):
+# after a chunk of k the loop's 64 accumulators (v0 .. v63) are compared with their values before it
+# (v128 .. v191); where one is lower, the chunk's index goes into that element's 16 bits of v192 .. v223 and
+# the copy is brought up to date.  First a cheap test whether ANY of the wave's elements changed at all -- one
+# three-input bit operation per element, diff |= now ^ before -- because once the distances have settled
+# almost no chunk changes anything.  Fixed registers throughout, so the compiler has nothing to allocate
+# around the loop's statements (as C++, the rare path's temporaries pushed the loop's fragments out to
+# scratch memory at every check).
+def generate_fwgemm_merge(out_dir):
+    os.makedirs(out_dir, exist_ok=True)
+    lines = ["v_mov_b32 v224, 0"]
+    for e in range(64):
+        lines.append(f"v_bitop3_b32 v224, v{e}, v{128 + e}, v224 bitop3:0xbe")
+    lines += ["v_cmp_ne_u32 vcc, 0, v224", "s_cbranch_vccz .Lcuasr_same_%="]
+    # (the wait between a comparison and its select is deliberate: with the copy of the element before in its place
+    # the product ran 4 % slower over a shortest-path job; and the two halves of a chunk word are written four
+    # instructions apart, more than the one wait state a write of part of a register wants before it is read again)
+    for e in range(64):
+        w, half = 192 + e // 2, e & 1
+        lines += [f"v_cmp_lt_f32 vcc, v{e}, v{128 + e}",
+                  "s_nop 1",
+                  f"v_cndmask_b32_sdwa v{w}, v{w}, %[chunk], vcc dst_sel:WORD_{half} dst_unused:UNUSED_PRESERVE "
+                  f"src0_sel:WORD_{half} src1_sel:WORD_0",
+                  f"v_mov_b32 v{128 + e}, v{e}"]
+    lines.append(".Lcuasr_same_%=:")
+    with open(os.path.join(out_dir, "fwgemm_merge.inc"), "w") as f:
+        f.write("\n".join('"' + ln + '\\n"' for ln in lines) + "\n")
+    return [("fwgemm_merge", {"lines": len(lines)})]
+
+
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
     out = sys.argv[1] if len(sys.argv) > 1 else os.path.join(here, "gen")
-    for name, stats in generate(out) + generate_mfma(out) + generate_mfma64(out):
+    for name, stats in generate(out) + generate_mfma(out) + generate_mfma64(out) + generate_fwgemm_merge(out):
         print(name, stats)

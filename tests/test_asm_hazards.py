@@ -13,7 +13,7 @@ import pytest
 import asm_inflight
 from cuasr_amd import build as B
 
-FILES = ["direct_f32.hip", "direct_i32.hip", "direct_u32.hip", "direct_f64.hip", "mfma_direct_f32.hip", "mfma_direct_f64.hip"]
+FILES = ["direct_f32.hip", "direct_i32.hip", "direct_u32.hip", "direct_f64.hip", "mfma_direct_f32.hip", "mfma_direct_f64.hip", "fwgemm.hip"]
 
 
 def _listing(src, out_dir):
@@ -112,7 +112,7 @@ def test_no_instruction_touches_a_register_an_asm_lds_read_is_filling(tmp_path):
         texts = list(ex.map(lambda s: _listing(s, str(tmp_path)), FILES))
     kernels = 0
     for src, text in zip(FILES, texts):
-        res = asm_inflight.check_listing(text, "gemm_mfma_direct" if src.startswith("mfma") else "srgemm_kernel")
+        res = asm_inflight.check_listing(text, "gemm_mfma_direct" if src.startswith("mfma") else "fwgemm_direct_kernel" if src.startswith("fwgemm") else "srgemm_kernel")
         assert res, f"{src}: no kernels found in the listing"
         kernels += len(res)
         bad = {k: v[:3] for k, v in res.items() if v}
