@@ -296,6 +296,28 @@ def test_apsp_squaring_two_steps_on_the_tiled_kernel(oracle, n, dtype):
     assert np.array_equal(dP.cpu().numpy(), want_p)
 
 
+@pytest.mark.parametrize("n,squarings", [(1280, 3), (2048, 1)])
+def test_apsp_squaring_on_the_direct_tile(oracle, n, squarings):
+    """Whole tiles of 128 x 256 with k in whole chunks of 32 (fp32) take the predecessor-tracking product on the
+    hand-scheduled direct-to-LDS tile: real-valued weights (sums round, ties are rare) and a share of exact zeros
+    (ties with the diagonal), dist and parent bit for bit after every squaring."""
+    import torch
+    rng = np.random.default_rng(900 + n)
+    W = np.where(rng.random((n, n)) < 0.02, rng.random((n, n)) * 7 + 0.25, np.inf).astype(np.float32)
+    W[rng.random((n, n)) < 0.002] = 0.0
+    np.fill_diagonal(W, 0)
+    dD = to_device(np.asfortranarray(W))
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    ws = torch.empty(cuasr_amd.apsp_workspace_bytes(n, "f32"), dtype=torch.uint8, device="cuda")
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    for s in range(squarings):
+        cuasr_amd.apsp_squaring(dD, dP, ws, iterations=1)
+        snap = want_d.copy(order="F")
+        oracle.fwgemm(snap, snap, want_d, want_p)
+        assert_same_bits(np.ascontiguousarray(dD.cpu().numpy()), np.ascontiguousarray(want_d), f"dist after squaring {s + 1}")
+        assert np.array_equal(dP.cpu().numpy(), want_p), f"parent after squaring {s + 1}"
+
+
 def test_apsp_4096_blocked_and_squaring_agree():
     """Full size, integer weights (every order of additions exact): blocked Floyd-Warshall and
     repeated squaring are different algorithms and must find the same distances; both parent
