@@ -20,7 +20,7 @@ HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "cuasr_amd.h")
 # enums of include/cuasr_amd.h
 OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
        "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
-DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3}
+DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3, "f16": 4}
 COLUMN_MAJOR, ROW_MAJOR = 0, 1
 KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3, "direct": 4, "streamk": 5}
 STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
@@ -29,12 +29,12 @@ STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
                 "kErrorInsufficientDriver", "kErrorMemoryAllocation", "kInvalid"]
 SUCCESS = 0
 
-_NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}
+_NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16}
 
 
 class Scalar(ctypes.Union):
     _fields_ = [("f32", ctypes.c_float), ("f64", ctypes.c_double), ("i32", ctypes.c_int32),
-                ("u32", ctypes.c_uint32), ("bits", ctypes.c_uint64)]
+                ("u32", ctypes.c_uint32), ("f16", ctypes.c_uint16), ("bits", ctypes.c_uint64)]
 
 
 class SrgemmDesc(ctypes.Structure):
@@ -162,6 +162,8 @@ def _set_scalar(s, value, dtype):
         s.f64 = float(value)
     elif dtype == "i32":
         s.i32 = int(value)
+    elif dtype == "f16":
+        s.f16 = int(np.array([value], dtype=np.float16).view(np.uint16)[0])   # the binary16 bit pattern
     else:
         s.u32 = int(value) & 0xFFFFFFFF
 
@@ -189,7 +191,7 @@ class MatRef:
 def _torch_dtype_name(t):
     import torch
     return {torch.float32: "f32", torch.float64: "f64", torch.int32: "i32",
-            getattr(torch, "uint32", None): "u32"}[t.dtype]
+            getattr(torch, "uint32", None): "u32", torch.float16: "f16"}[t.dtype]
 
 
 def make_desc(add_op, mult_op, dtype, A, B, C, D, alpha, beta, add_identity, mult_identity,

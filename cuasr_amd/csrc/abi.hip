@@ -12,6 +12,7 @@ launch_fn find_valu_f32(int, int);
 launch_fn find_valu_f64(int, int);
 launch_fn find_valu_i32(int, int);
 launch_fn find_valu_u32(int, int);
+launch_fn find_valu_f16(int, int);
 launch_fn find_mfma_f32(int, int);
 launch_fn find_mfma_f64(int, int);
 launch_fn find_direct_f32(int, int);
@@ -34,6 +35,7 @@ launch_fn find_valu(int dtype, int add_op, int mult_op) {
     case CUASR_AMD_F64: return find_valu_f64(add_op, mult_op);
     case CUASR_AMD_I32: return find_valu_i32(add_op, mult_op);
     case CUASR_AMD_U32: return find_valu_u32(add_op, mult_op);
+    case CUASR_AMD_F16: return find_valu_f16(add_op, mult_op);
     default: return nullptr;
   }
 }
@@ -63,7 +65,7 @@ launch_fn find_mfma(int dtype, int add_op, int mult_op) {
   return nullptr;
 }
 
-static size_t elem_size(int dtype) { return dtype == CUASR_AMD_F64 ? 8 : 4; }
+static size_t elem_size(int dtype) { return dtype == CUASR_AMD_F64 ? 8 : dtype == CUASR_AMD_F16 ? 2 : 4; }
 
 static bool is_bitwise(int op) { return op == kBitAnd || op == kBitOr || op == kBitXor; }
 
@@ -113,12 +115,12 @@ static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
 
 static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (!d) return CUASR_AMD_ERROR_INVALID_PROBLEM;
-  if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_U32) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
+  if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_F16) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
   const int layouts[3] = {d->layout_a, d->layout_b, d->layout_c};
   for (int l : layouts)
     if (l != CUASR_AMD_COLUMN_MAJOR && l != CUASR_AMD_ROW_MAJOR) return CUASR_AMD_ERROR_INVALID_LAYOUT;
   if (!valid_add(d->add_op) || !valid_mult(d->mult_op)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
-  const bool fp = d->dtype == CUASR_AMD_F32 || d->dtype == CUASR_AMD_F64;
+  const bool fp = d->dtype == CUASR_AMD_F32 || d->dtype == CUASR_AMD_F64 || d->dtype == CUASR_AMD_F16;
   if (fp && (is_bitwise(d->add_op) || is_bitwise(d->mult_op))) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   if (d->m < 0 || d->n < 0 || d->k < 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (d->reserved != 0) return CUASR_AMD_ERROR_INVALID_PROBLEM;
@@ -417,7 +419,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
 
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
   if (!desc || desc->m < 0 || desc->n < 0 || desc->split_k_slices < 1) return 0;
-  if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_U32) return 0;
+  if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_F16) return 0;
   return elem_size(desc->dtype) * size_t(desc->m) * size_t(desc->n) * size_t(desc->split_k_slices);
 }
 

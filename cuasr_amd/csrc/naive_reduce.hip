@@ -54,6 +54,7 @@ launch_fn find_naive(int dtype) {
     case CUASR_AMD_F64: return launch_naive<double>;
     case CUASR_AMD_I32: return launch_naive<int32_t>;
     case CUASR_AMD_U32: return launch_naive<uint32_t>;
+    case CUASR_AMD_F16: return launch_naive<half_t>;
     default: return nullptr;
   }
 }
@@ -259,6 +260,7 @@ launch_fn find_reduce(int dtype) {
     case CUASR_AMD_F64: return launch_reduce<double, false>;
     case CUASR_AMD_I32: return launch_reduce<int32_t, false>;
     case CUASR_AMD_U32: return launch_reduce<uint32_t, false>;
+    case CUASR_AMD_F16: return launch_reduce<half_t, false>;
     default: return nullptr;
   }
 }
@@ -269,6 +271,7 @@ launch_fn find_reduce_serial(int dtype) {
     case CUASR_AMD_F64: return launch_reduce<double, true>;
     case CUASR_AMD_I32: return launch_reduce<int32_t, true>;
     case CUASR_AMD_U32: return launch_reduce<uint32_t, true>;
+    case CUASR_AMD_F16: return launch_reduce<half_t, true>;
     default: return nullptr;
   }
 }

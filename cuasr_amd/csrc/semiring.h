@@ -22,7 +22,10 @@ namespace cuasr_amd {
 enum : int { kPlus = 0, kMultiplies = 1, kMinimum = 2, kMaximum = 3, kLogicalAnd = 4,
              kLogicalOr = 5, kBitAnd = 6, kBitOr = 7, kBitXor = 8 };
 
+typedef _Float16 half_t;  // IEEE binary16; arithmetic on it rounds every result to binary16
+
 template <typename T> struct is_fp : std::integral_constant<bool, std::is_floating_point<T>::value> {};
+template <> struct is_fp<half_t> : std::true_type {};
 
 template <typename T> __device__ __forceinline__ T hw_min(T l, T r) { return r < l ? r : l; }
 template <typename T> __device__ __forceinline__ T hw_max(T l, T r) { return l < r ? r : l; }
@@ -118,6 +121,9 @@ template <> __host__ __device__ __forceinline__ float scalar_as<float>(const cua
 template <> __host__ __device__ __forceinline__ double scalar_as<double>(const cuasr_amd_scalar &s) { return s.f64; }
 template <> __host__ __device__ __forceinline__ int32_t scalar_as<int32_t>(const cuasr_amd_scalar &s) { return s.i32; }
 template <> __host__ __device__ __forceinline__ uint32_t scalar_as<uint32_t>(const cuasr_amd_scalar &s) { return s.u32; }
+template <> __host__ __device__ __forceinline__ half_t scalar_as<half_t>(const cuasr_amd_scalar &s) {
+  return __builtin_bit_cast(half_t, s.f16);
+}
 
 // The problem in kernel form.  The host has already turned a column-major C
 // into the transposed problem (C^T = B^T (x) A^T, as the reference does in

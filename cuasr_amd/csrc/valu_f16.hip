@@ -1,0 +1,284 @@
+// Vector-ALU tile for element type binary16 (half precision), two output columns per register.
+//
+// The reference names half precision as an aim only (README.md:11); its templates, instantiated
+// with a half type for every element, would round each operator's result to binary16
+// (arch/srmma.h:65-92: d = add(c, mult(a, b)) in ElementC).  So does this tile: every term is one
+// packed add (or max, min, mul) and every fold one packed min / max / add on two binary16 values.
+//
+// What gfx950 gives for it (cuasr_amd/issue_probe.py, "mix_f16"): a packed binary16 instruction
+// issues every 4.2 cycles per SIMD, twice as long as a 4-byte one, so two terms per instruction buy
+// no rate by themselves (99.6 against 97 TOPS for the bare loops) -- but LDS reads, waits and address
+// arithmetic issue beneath the 4-cycle instructions for free, two waves per SIMD already reach that
+// rate, and the operands are half as many bytes.  Hence a plain compiled loop, staged through
+// registers, which can also transpose on the way to LDS: one kernel serves every layout.
+//
+// Tile: 256 threads, 128 rows x 256 columns x 32 k.  A thread holds 8 rows x 16 columns (two groups
+// of 8 consecutive columns, 128 apart) as 64 registers of two columns each.  LDS: A panel [k][128],
+// B panel [k][256], both with the output direction contiguous, two stages.  Per k a thread reads one
+// 16-byte vector of A (its 8 rows; the instruction's half-word selects broadcast one of them) and two
+// of B, and issues 64 packed adds + 32 three-input packed minima for 128 terms.
+#include "semiring.h"
+
+namespace cuasr_amd {
+namespace half_tile {
+
+typedef half_t h2 __attribute__((ext_vector_type(2)));
+typedef half_t h8 __attribute__((ext_vector_type(8)));
+
+constexpr int BM = 128, BN = 256, BK = 32, THREADS = 256;
+
+struct Smem {
+  half_t a[2][BK][BM];
+  half_t b[2][BK][BN];
+};
+
+template <int OP> __device__ __forceinline__ h2 pk(h2 l, h2 r) {
+  if constexpr (OP == kPlus) return l + r;
+  else if constexpr (OP == kMultiplies) return l * r;
+  else if constexpr (OP == kMinimum) return __builtin_elementwise_min(l, r);
+  else return __builtin_elementwise_max(l, r);
+}
+
+// acc <- add(acc, mult(a0, b0), mult(a1, b1)), the two terms in this order
+template <int ADD, int MUL> __device__ __forceinline__ void two_terms(h2 &acc, h2 a0, h2 b0, h2 a1, h2 b1) {
+  const h2 t0 = pk<MUL>(a0, b0), t1 = pk<MUL>(a1, b1);
+  // the three-input forms (v_pk_minimum3_f16 / v_pk_maximum3_f16) differ from min / max only on NaN
+  if constexpr (ADD == kMinimum) acc = __builtin_elementwise_minimum(__builtin_elementwise_minimum(acc, t0), t1);
+  else if constexpr (ADD == kMaximum) acc = __builtin_elementwise_maximum(__builtin_elementwise_maximum(acc, t0), t1);
+  else acc = pk<ADD>(pk<ADD>(acc, t0), t1);
+}
+template <int ADD, int MUL> __device__ __forceinline__ void one_term(h2 &acc, h2 a, h2 b) {
+  acc = pk<ADD>(acc, pk<MUL>(a, b));
+}
+
+__device__ __forceinline__ h2 both(half_t v) { return h2{v, v}; }
+__device__ __forceinline__ h2 pair_of(const h8 &v, int j) { return h2{v[2 * j], v[2 * j + 1]}; }
+
+// One operand's share of a k-tile on its way from memory to LDS.  The panel is X wide (X = BM for A, BN
+// for B); a chunk is 8 elements: of one k and 8 consecutive x when x is the contiguous direction in
+// memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
+template <int X, bool KC, bool GUARD> struct Stager {
+  static constexpr int CHUNKS = X * BK / 8 / THREADS;
+  h8 r[CHUNKS];
+
+  // chunk c -> (x, k) of its first element, tile-relative
+  static __device__ __forceinline__ void where(int c, int &x, int &k) {
+    if constexpr (KC) { k = (c % (BK / 8)) * 8; x = c / (BK / 8); }
+    else { x = (c % (X / 8)) * 8; k = c / (X / 8); }
+  }
+
+  // base: the operand's element (x = 0, k = 0); sx, sk: element strides; x0, k0: the tile's origin;
+  // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored)
+  __device__ __forceinline__ void load(const half_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn) {
+#pragma unroll
+    for (int q = 0; q < CHUNKS; ++q) {
+      int x, k;
+      where(threadIdx.x + q * THREADS, x, k);
+      const half_t *src = base + (long long)(x0 + x) * sx + (long long)(k0 + k) * sk;
+      if constexpr (!GUARD) {
+        r[q] = *reinterpret_cast<const h8 *>(src);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int xe = x0 + x + (KC ? 0 : e), ke = k0 + k + (KC ? e : 0);
+          r[q][e] = (xe < xn && ke < kn) ? src[(KC ? sk : sx) * e] : half_t(0);
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(half_t (*panel)[X]) const {
+#pragma unroll
+    for (int q = 0; q < CHUNKS; ++q) {
+      int x, k;
+      where(threadIdx.x + q * THREADS, x, k);
+      if constexpr (KC) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) panel[k + e][x] = r[q][e];
+      } else {
+        *reinterpret_cast<h8 *>(&panel[k][x]) = r[q];
+      }
+    }
+  }
+};
+
+template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void half_tile_kernel(Problem p) {
+  __shared__ __attribute__((aligned(16))) Smem sm;
+  select_batch<half_t>(p);
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+  int kb = 0, ke = p.k;
+  if (p.workspace) {
+    kb = blockIdx.y * p.k_per_slice;
+    ke = min(p.k, kb + p.k_per_slice);
+  }
+  const half_t *A = reinterpret_cast<const half_t *>(p.A), *B = reinterpret_cast<const half_t *>(p.B);
+  const half_t ident = scalar_as<half_t>(p.add_identity);
+
+  h2 acc[8][8];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = both(ident);
+
+  Stager<BM, A_KC, GUARD> sa;
+  Stager<BN, B_KC, GUARD> sb;
+  const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
+  if (tiles_k > 0) {
+    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke);
+    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke);
+    sa.store(sm.a[0]);
+    sb.store(sm.b[0]);
+  }
+  __syncthreads();
+  for (int t = 0; t < tiles_k; ++t) {
+    const int s = t & 1, k0 = kb + t * BK;
+    if (t + 1 < tiles_k) {
+      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke);
+      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke);
+    }
+    const half_t(*pa)[BM] = sm.a[s];
+    const half_t(*pb)[BN] = sm.b[s];
+    if (!GUARD || ke - k0 >= BK) {
+#pragma unroll 2
+      for (int kk = 0; kk < BK; kk += 2) {
+        const h8 a0 = *reinterpret_cast<const h8 *>(&pa[kk][ty * 8]), a1 = *reinterpret_cast<const h8 *>(&pa[kk + 1][ty * 8]);
+        const h8 b00 = *reinterpret_cast<const h8 *>(&pb[kk][tx * 8]), b01 = *reinterpret_cast<const h8 *>(&pb[kk][128 + tx * 8]);
+        const h8 b10 = *reinterpret_cast<const h8 *>(&pb[kk + 1][tx * 8]), b11 = *reinterpret_cast<const h8 *>(&pb[kk + 1][128 + tx * 8]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            two_terms<ADD, MUL>(acc[i][j], both(a0[i]), pair_of(b00, j), both(a1[i]), pair_of(b10, j));
+            two_terms<ADD, MUL>(acc[i][4 + j], both(a0[i]), pair_of(b01, j), both(a1[i]), pair_of(b11, j));
+          }
+      }
+    } else {
+      for (int kk = 0; kk < ke - k0; ++kk) {  // the ragged last k-tile
+        const h8 a0 = *reinterpret_cast<const h8 *>(&pa[kk][ty * 8]);
+        const h8 b00 = *reinterpret_cast<const h8 *>(&pb[kk][tx * 8]), b01 = *reinterpret_cast<const h8 *>(&pb[kk][128 + tx * 8]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            one_term<ADD, MUL>(acc[i][j], both(a0[i]), pair_of(b00, j));
+            one_term<ADD, MUL>(acc[i][4 + j], both(a0[i]), pair_of(b01, j));
+          }
+      }
+    }
+    if (t + 1 < tiles_k) {
+      sa.store(sm.a[s ^ 1]);
+      sb.store(sm.b[s ^ 1]);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or the raw accumulators of a k-slice
+  const EpilogueScalars<half_t> e = resolve_scalars<half_t>(p, MUL);
+  half_t *ws = p.workspace ? reinterpret_cast<half_t *>(p.workspace) + (long long)blockIdx.y * p.m * p.n : nullptr;
+  const half_t *C = reinterpret_cast<const half_t *>(p.C);
+  half_t *D = reinterpret_cast<half_t *>(p.D);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int row = m0 + ty * 8 + i;
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int col = n0 + g * 128 + tx * 8;
+      h8 v;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[2 * j] = acc[i][g * 4 + j][0];
+        v[2 * j + 1] = acc[i][g * 4 + j][1];
+      }
+      if (ws) {
+        if constexpr (!GUARD) {
+          *reinterpret_cast<h8 *>(ws + (long long)row * p.n + col) = v;
+        } else {
+#pragma unroll
+          for (int x = 0; x < 8; ++x)
+            if ((unsigned)row < (unsigned)p.m && (unsigned)(col + x) < (unsigned)p.n) ws[(long long)row * p.n + col + x] = v[x];
+        }
+        continue;
+      }
+      h8 c;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) c[x] = e.ident;
+      if (e.source_needed) {
+        if constexpr (!GUARD) {
+          c = *reinterpret_cast<const h8 *>(C + (long long)row * p.ldc + col);
+        } else {
+#pragma unroll
+          for (int x = 0; x < 8; ++x)
+            if ((unsigned)row < (unsigned)p.m && (unsigned)(col + x) < (unsigned)p.n) c[x] = C[(long long)row * p.ldc + col + x];
+        }
+      }
+      h8 out;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        out[x] = Op<MUL>::apply(e.alpha, v[x]);
+        if (e.source_needed) out[x] = fold_epilogue<ADD, MUL>(out[x], Op<MUL>::apply(e.beta, c[x]));
+      }
+      if constexpr (!GUARD) {
+        *reinterpret_cast<h8 *>(D + (long long)row * p.ldd + col) = out;
+      } else {
+#pragma unroll
+        for (int x = 0; x < 8; ++x)
+          if ((unsigned)row < (unsigned)p.m && (unsigned)(col + x) < (unsigned)p.n) D[(long long)row * p.ldd + col + x] = out[x];
+      }
+    }
+  }
+}
+
+// whole tiles, whole 16-byte vectors at 16-byte boundaries everywhere: the unguarded kernel
+static bool exact(const Problem &p, bool a_kc, bool b_kc) {
+  auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  if (p.m % BM || p.n % BN || p.k % BK || p.k == 0) return false;
+  if (p.workspace && (p.k_per_slice % BK || !al16(p.workspace))) return false;
+  if ((a_kc ? p.sa_m : p.sa_k) % 8 || (b_kc ? p.sb_n : p.sb_k) % 8) return false;
+  if (!al16(p.A) || !al16(p.B) || !al16(p.D) || p.ldd % 8) return false;
+  if (p.C && (!al16(p.C) || p.ldc % 8)) return false;
+  if (p.batch > 1 && (p.batch_a % 8 || p.batch_b % 8 || p.batch_c % 8 || p.batch_d % 8)) return false;
+  return true;
+}
+
+template <int ADD, int MUL> static hipError_t launch(const Problem &p, hipStream_t s) {
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  // one direction of each operand is contiguous (the C ABI produces nothing else)
+  if ((p.sa_m != 1 && p.sa_k != 1) || (p.sb_n != 1 && p.sb_k != 1)) return hipErrorNotSupported;
+  const bool a_kc = p.sa_m != 1, b_kc = p.sb_n != 1;
+  const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(THREADS);
+  const bool fast = exact(p, a_kc, b_kc);
+#define CUASR_HALF_LAUNCH(AK, BK_, G) launch_kernel((half_tile_kernel<ADD, MUL, AK, BK_, G>), grid, block, 0, s, p)
+  if (fast) {
+    if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true, false); else CUASR_HALF_LAUNCH(true, false, false); }
+    else { if (b_kc) CUASR_HALF_LAUNCH(false, true, false); else CUASR_HALF_LAUNCH(false, false, false); }
+  } else {
+    if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true, true); else CUASR_HALF_LAUNCH(true, false, true); }
+    else { if (b_kc) CUASR_HALF_LAUNCH(false, true, true); else CUASR_HALF_LAUNCH(false, false, true); }
+  }
+#undef CUASR_HALF_LAUNCH
+  return take_launch_status();
+}
+
+}  // namespace half_tile
+
+// The semirings whose operators are each one packed instruction with nothing to watch: sums, minima and
+// maxima of data free of -0 never produce -0 (products do: min-times and max-times stay on the naive kernel,
+// as do the logical pairs).
+launch_fn find_valu_f16(int add_op, int mult_op) {
+#define PAIR(ADD, MUL) \
+  if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL>;
+  PAIR(kMinimum, kPlus)
+  PAIR(kMaximum, kPlus)
+  PAIR(kMinimum, kMaximum)
+  PAIR(kMaximum, kMinimum)
+  PAIR(kPlus, kMultiplies)
+#undef PAIR
+  return nullptr;
+}
+
+}  // namespace cuasr_amd

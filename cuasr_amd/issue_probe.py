@@ -12,6 +12,7 @@ groups of add, add, min3 = 128 terms per lane) or a variation of it, run by 256-
     mix + SGPR operand                    a fragment broadcast through scalar registers
     mix + N LDS reads (4 / 8 / 16 bytes)  what fetching the fragments costs (results not consumed)
     mix + N waits / nops / scalar adds    what an instruction that does no arithmetic costs
+    packed fp16 add / min / minimum3 / mix the same for two fp16 terms per instruction
     fp64 add / max / mix (+ the same)     the same questions for 8-byte elements
 Times are HIP events around the second of two launches; the clock is read inside the kernel
 (shader cycle counter against the 100 MHz wall clock), so cycle figures are per measured clock.
@@ -41,6 +42,21 @@ def mix(sgpr_b=False):
             acc = ACC[i * 8 + j]
             groups.append([f"v_add_f32 v{t0}, {b0}, v{A0[i]}", f"v_add_f32 v{t1}, {b1}, v{A1[i]}",
                            f"v_min3_f32 v{acc}, v{acc}, v{t0}, v{t1}"])
+    return groups
+
+
+def mix_f16():
+    """min-plus on packed fp16: acc[i][j] holds two columns; row i's fragment word holds two k (or two
+    rows), picked by op_sel; 256 terms per lane in 192 instructions"""
+    groups, t = [], 0
+    for i in range(8):
+        for j in range(8):
+            t0, t1 = T[t % 8], T[(t + 1) % 8]
+            t += 2
+            acc = ACC[i * 8 + j]
+            groups.append([f"v_pk_add_f16 v{t0}, v{A0[i]}, v{B0[j]} op_sel_hi:[0,1]",
+                           f"v_pk_add_f16 v{t1}, v{A0[i]}, v{B1[j]} op_sel:[1,0] op_sel_hi:[1,1]",
+                           f"v_pk_minimum3_f16 v{acc}, v{acc}, v{t0}, v{t1}"])
     return groups
 
 
@@ -85,6 +101,16 @@ def kernels():
     k["fma_f32_vop3"] = (only("v_fma_f32 v{acc}, v{b}, v{a}, v{acc}"), 192, 0, "f32")
     k["fmac_f32_vop2"] = (only("v_fmac_f32 v{acc}, v{b}, v{a}"), 192, 0, "f32")
     k["bitop3_b32"] = (only("v_bitop3_b32 v{acc}, v{b}, v{a}, v{acc} bitop3:0x6a"), 192, 0, "f32")
+    # packed fp16: two terms per instruction and lane; the fragment of one operand is broadcast by the
+    # instruction's own half-word selects
+    k["pk_add_f16"] = (only("v_pk_add_f16 v{t}, v{b}, v{a}"), 192, 0, "f32")
+    k["pk_add_f16_broadcast"] = (only("v_pk_add_f16 v{t}, v{b}, v{a} op_sel:[1,0] op_sel_hi:[1,1]"), 192, 0, "f32")
+    k["pk_min_f16"] = (only("v_pk_min_f16 v{acc}, v{acc}, v{b}"), 192, 0, "f32")
+    k["pk_minimum3_f16"] = (only("v_pk_minimum3_f16 v{acc}, v{acc}, v{b}, v{a}"), 192, 0, "f32")
+    k["pk_mul_f16"] = (only("v_pk_mul_f16 v{t}, v{b}, v{a}"), 192, 0, "f32")
+    k["mix_f16"] = (flat(mix_f16()), 192, 256, "f32")
+    for n in (6, 12):
+        k[f"mix_f16_lds{n}_b128"] = (sprinkle(mix_f16(), n, lds_read(128)), 192, 256, "f32")
     k["mix"] = (flat(mix()), 192, 128, "f32")
     k["mix_sgpr_b"] = (flat(mix(True)), 192, 128, "f32")
     for n in (4, 8, 16):

@@ -73,7 +73,11 @@ typedef enum cuasr_amd_dtype {
   CUASR_AMD_F32 = 0,
   CUASR_AMD_F64 = 1,
   CUASR_AMD_I32 = 2,
-  CUASR_AMD_U32 = 3
+  CUASR_AMD_U32 = 3,
+  /* IEEE binary16 in A, B, C, D, the scalars and the accumulator: every operator rounds its result to
+   * binary16, as the reference's templates do when they are instantiated with cutlass::half_t for all
+   * element types (the reference names half precision as an aim only, README.md:11) */
+  CUASR_AMD_F16 = 4
 } cuasr_amd_dtype;
 
 typedef enum cuasr_amd_layout {
@@ -104,6 +108,7 @@ typedef union cuasr_amd_scalar {
   double f64;
   int32_t i32;
   uint32_t u32;
+  uint16_t f16;  /* the bit pattern of an IEEE binary16 value (C has no portable type for it) */
   uint64_t bits;
 } cuasr_amd_scalar;
 

@@ -18,7 +18,7 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
        "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
 DTYPES = {np.dtype(np.float32): 0, np.dtype(np.float64): 1,
-          np.dtype(np.int32): 2, np.dtype(np.uint32): 3}
+          np.dtype(np.int32): 2, np.dtype(np.uint32): 3, np.dtype(np.float16): 4}
 COLUMN_MAJOR, ROW_MAJOR = 0, 1
 
 _lib = None

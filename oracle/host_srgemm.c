@@ -61,7 +61,7 @@
 enum { OP_PLUS = 0, OP_MULTIPLIES = 1, OP_MINIMUM = 2, OP_MAXIMUM = 3,
        OP_LOGICAL_AND = 4, OP_LOGICAL_OR = 5, OP_BIT_AND = 6, OP_BIT_OR = 7,
        OP_BIT_XOR = 8 };
-enum { DT_F32 = 0, DT_F64 = 1, DT_I32 = 2, DT_U32 = 3 };
+enum { DT_F32 = 0, DT_F64 = 1, DT_I32 = 2, DT_U32 = 3, DT_F16 = 4 };
 enum { LAYOUT_COLUMN_MAJOR = 0, LAYOUT_ROW_MAJOR = 1 };
 
 #define BLK 32
@@ -76,6 +76,72 @@ enum { LAYOUT_COLUMN_MAJOR = 0, LAYOUT_ROW_MAJOR = 1 };
 #define F_BIT_AND(l, r)     ((l) & (r))
 #define F_BIT_OR(l, r)      ((l) | (r))
 #define F_BIT_XOR(l, r)     ((l) ^ (r))
+#define F_NE(l, r)          ((l) != (r))
+
+/*
+ * IEEE binary16, held as its bit pattern (gcc 11 on x86-64 has no _Float16).  The reference has no
+ * half-precision kernels (README.md:11 names them as an aim); what its templates would compute with a
+ * half type for every element (arch/srmma.h:65-92, functional.h:46-49, :89-92, :132, :172) is each
+ * operator's exact result rounded once to binary16, ties to even.  Here: widen both operands to
+ * binary32 (exact), operate in binary32, round to binary16.  That is the correctly rounded binary16
+ * result: a product of two 11-bit significands is exact in 24 bits, and for a sum the binary32
+ * rounding in between is harmless because 24 >= 2 * 11 + 2 (the classic double-rounding bound).
+ * Comparisons are made on the widened values, so -0 == +0 and the operand returned is the reference's.
+ */
+typedef uint16_t h16;
+
+static inline float h2f(h16 h) {
+  const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu, bits;
+  if (e == 0) {
+    if (m == 0) {
+      bits = sign;                                   /* zero */
+    } else {                                         /* subnormal: value m * 2^-24 */
+      int shift = 0;
+      while (!(m & 0x400u)) { m <<= 1; ++shift; }
+      bits = sign | ((uint32_t)(113 - shift) << 23) | ((m & 0x3ffu) << 13);
+    }
+  } else if (e == 31) {
+    bits = sign | 0x7f800000u | (m << 13);           /* infinity, NaN */
+  } else {
+    bits = sign | ((e + 112) << 23) | (m << 13);
+  }
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+
+static inline h16 f2h(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x >= 0x7f800000u) return (h16)(sign | 0x7c00u | (x > 0x7f800000u ? 0x200u : 0)); /* inf / NaN */
+  if (x >= 0x477ff000u) return (h16)(sign | 0x7c00u);   /* >= 65520 rounds to infinity */
+  if (x < 0x33000001u) return (h16)sign;                /* <= 2^-25 rounds to zero (the tie goes to even = 0) */
+  const int e = (int)(x >> 23) - 127;                   /* unbiased exponent, -25 .. 15 */
+  uint32_t m = (x & 0x7fffffu) | 0x800000u;             /* 24-bit significand */
+  int drop;                                             /* low bits of m that binary16 cannot hold */
+  uint32_t base;
+  if (e >= -14) { drop = 13; base = (uint32_t)(e + 15) << 10; m &= 0x7fffffu; }   /* normal */
+  else { drop = 13 + (-14 - e); base = 0; }                                       /* subnormal: keep the leading 1 */
+  const uint32_t kept = m >> drop, rest = m & ((1u << drop) - 1u), half = 1u << (drop - 1);
+  uint32_t r = base + kept;                             /* a carry out of the significand bumps the exponent */
+  if (rest > half || (rest == half && (kept & 1u))) ++r;
+  return (h16)(sign | r);
+}
+
+/* entry points for the tests that pin the two conversions */
+float oracle_half_to_float(uint16_t h) { return h2f(h); }
+uint16_t oracle_float_to_half(float f) { return f2h(f); }
+
+#define H_PLUS(l, r)        f2h(h2f(l) + h2f(r))
+#define H_MULTIPLIES(l, r)  f2h(h2f(l) * h2f(r))
+#define H_MINIMUM(l, r)     (h2f(r) < h2f(l) ? (r) : (l))
+#define H_MAXIMUM(l, r)     (h2f(l) < h2f(r) ? (r) : (l))
+#define H_LOGICAL_AND(l, r) ((h16)((h2f(l) != 0.0f && h2f(r) != 0.0f) ? 0x3c00u : 0u))
+#define H_LOGICAL_OR(l, r)  ((h16)((h2f(l) != 0.0f || h2f(r) != 0.0f) ? 0x3c00u : 0u))
+#define H_NE(l, r)          (h2f(l) != h2f(r))
 
 #if defined(__x86_64__) && defined(__GNUC__) && !defined(ORACLE_NO_CLONES)
 #define CLONES __attribute__((target_clones("avx512f", "avx2", "default")))
@@ -105,7 +171,7 @@ typedef struct {
  * i loop vectorises; per element the order of operations is exactly
  * accum = add(mult(a, b), accum) for k ascending.
  */
-#define DEFINE_KERNEL(NAME, T, ADD, MUL)                                        \
+#define DEFINE_KERNEL(NAME, T, ADD, MUL, NE)                                      \
   CLONES static void NAME(const job_t *jb) {                                    \
     const int M = jb->m, N = jb->n;                                             \
     const T *A = (const T *)jb->A, *B = (const T *)jb->B;                       \
@@ -170,7 +236,7 @@ typedef struct {
             int need = 1;                                                       \
             if (jb->skip_source_if_unneeded) {                                  \
               const T one = *(const T *)jb->mult_identity;                      \
-              need = (ident != (T)MUL(beta, one));                              \
+              need = NE(ident, (T)MUL(beta, one));                              \
             }                                                                   \
             for (int j = 0; j < nc; ++j)                                        \
               for (int i = 0; i < mr; ++i) {                                    \
@@ -216,8 +282,11 @@ typedef struct {
   }
 
 #define DEFINE_PAIR(T, TN, ADDN, MULN)                                          \
-  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, F_##ADDN, F_##MULN)              \
+  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, F_##ADDN, F_##MULN, F_NE)        \
   DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, F_##ADDN, F_##MULN)
+#define DEFINE_HALF_PAIR(T, TN, ADDN, MULN)                                     \
+  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, H_##ADDN, H_##MULN, H_NE)        \
+  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, H_##ADDN, H_##MULN)
 
 /* add-ops x mult-ops available to floating types */
 #define FOR_FLOAT_PAIRS(X, T, TN)                                               \
@@ -246,6 +315,7 @@ FOR_FLOAT_PAIRS(DEFINE_PAIR, int32_t, i32)
 FOR_INT_EXTRA_PAIRS(DEFINE_PAIR, int32_t, i32)
 FOR_FLOAT_PAIRS(DEFINE_PAIR, uint32_t, u32)
 FOR_INT_EXTRA_PAIRS(DEFINE_PAIR, uint32_t, u32)
+FOR_FLOAT_PAIRS(DEFINE_HALF_PAIR, h16, f16)
 
 typedef void (*kernel_fn)(const job_t *);
 
@@ -263,12 +333,13 @@ static kernel_fn lookup(int dtype, int add_op, int mult_op, int naive) {
   case DT_U32:
     FOR_FLOAT_PAIRS(LOOKUP_ROW, uint32_t, u32)
     FOR_INT_EXTRA_PAIRS(LOOKUP_ROW, uint32_t, u32) break;
+  case DT_F16: FOR_FLOAT_PAIRS(LOOKUP_ROW, h16, f16) break;
   default: break;
   }
   return 0;
 }
 
-static size_t dtype_size(int dtype) { return dtype == DT_F64 ? 8 : 4; }
+static size_t dtype_size(int dtype) { return dtype == DT_F64 ? 8 : dtype == DT_F16 ? 2 : 4; }
 
 static void set_strides(job_t *jb, int layout_a, int64_t lda, int layout_b,
                         int64_t ldb, int layout_c, int64_t ldc, int64_t ldd) {

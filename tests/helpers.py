@@ -2,7 +2,7 @@
 keeps the matrix layout, and the bit-exact comparison."""
 import numpy as np
 
-NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}
+NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16}
 
 
 def to_device(a):
@@ -37,7 +37,7 @@ def assert_same_bits(got, want, what=""):
         return
     g = np.ascontiguousarray(got)
     w = np.ascontiguousarray(want)
-    ui = {4: np.uint32, 8: np.uint64}[g.itemsize]
+    ui = {2: np.uint16, 4: np.uint32, 8: np.uint64}[g.itemsize]
     bad = np.argwhere(g.view(ui) != w.view(ui))
     i = tuple(bad[0])
     raise AssertionError(f"{what}: {len(bad)} of {g.size} elements differ; first at {i}: "

@@ -1,0 +1,158 @@
+"""Half precision (binary16 in every operand and the accumulator) against the CPU oracle, bit for bit,
+through the C ABI: the packed vector-ALU tile in both its forms (whole tiles of aligned operands, and
+guarded), every layout, the naive kernel for the pairs the tile does not take, split-K, batches, views."""
+import numpy as np
+import pytest
+
+from helpers import assert_same_bits, order_of, to_device
+
+pytestmark = pytest.mark.gpu
+
+TILE_PAIRS = [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"), ("plus", "multiplies")]
+OTHER_PAIRS = [("minimum", "multiplies"), ("maximum", "multiplies"), ("logical_or", "logical_and")]
+LAYOUTS = ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"]
+
+
+def operands(add, mult, m, n, k, la, lb, lc, seed=1):
+    """Values whose sums and products do not fit binary16 exactly, so that every operator's rounding counts."""
+    from cuasr_amd import inputs
+    lo, hi = (-1.0, 1.0) if mult == "multiplies" else (0.5, 100.0)
+    A = inputs.uniform(seed, m, k, lo, hi, np.float16, order_of(la))
+    B = inputs.uniform(seed + 1, k, n, lo, hi, np.float16, order_of(lb))
+    C = inputs.uniform(seed + 2, m, n, lo, hi, np.float16, order_of(lc))
+    if mult == "logical_and":
+        A[A < 30] = 0
+        B[B < 30] = 0
+    return A, B, C
+
+
+def scalars(add, mult, beta_one):
+    import cuasr_amd
+    ident = cuasr_amd.op_identity(add, "f16", True)
+    one = cuasr_amd.op_identity(mult, "f16", True)
+    zero = cuasr_amd.op_annihilator(mult, "f16", True)
+    if add == "maximum" and mult == "plus":
+        zero = ident  # the max-semiring zero, not plus::Annihilator
+    return ident, one, (one if beta_one else zero)
+
+
+def check(oracle, add, mult, m, n, k, layouts, kernel, beta_one=True, seed=1, splitk=0, alpha=None, beta=None):
+    import torch
+    import cuasr_amd
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    A, B, C = operands(add, mult, m, n, k, la, lb, lc, seed)
+    ident, one, b = scalars(add, mult, beta_one)
+    alpha = one if alpha is None else np.float16(alpha)
+    beta = b if beta is None else np.float16(beta)
+    want = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident)   # (split-K runs order-free adds only: the slices cannot matter)
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    dD = to_device(np.zeros_like(C))
+    print(f"half {add}-{mult} {m}x{n}x{k} {layouts} {kernel} beta_one={beta_one} splitk={splitk}", flush=True)
+    if splitk:
+        ws = torch.empty(cuasr_amd.splitk_workspace_bytes(m, n, splitk, "f16") // 2 + 8, dtype=torch.float16, device="cuda")
+        cuasr_amd.srgemm_splitk(add, mult, dA, dB, dC, dD, splitk, ws, alpha, beta, ident, one, dtype="f16", kernel=kernel)
+    else:
+        cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, alpha, beta, ident, one, dtype="f16", kernel=kernel)
+    torch.cuda.synchronize()
+    assert_same_bits(dD.cpu().numpy(), want, f"{add}-{mult} f16 {m}x{n}x{k} {layouts} {kernel}")
+
+
+@pytest.mark.parametrize("sr", TILE_PAIRS)
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_packed_tile(oracle, lib, sr, layouts):
+    # whole tiles (the unguarded kernel), ragged everything, single element, tall and thin
+    for shape in [(128, 256, 32), (256, 512, 96), (100, 300, 45), (1, 1, 1), (130, 258, 33), (64, 8, 200)]:
+        for beta_one in (False, True):
+            check(oracle, *sr, *shape, layouts, "valu", beta_one)
+
+
+def test_selected_family(lib):
+    import cuasr_amd
+    dA = to_device(np.zeros((128, 64), np.float16))
+    dB = to_device(np.zeros((64, 256), np.float16))
+    dD = to_device(np.zeros((128, 256), np.float16))
+    for (add, mult), name in [(("minimum", "plus"), b"valu"), (("plus", "multiplies"), b"valu"), (("minimum", "multiplies"), b"naive")]:
+        ident, one, zero = scalars(add, mult, False)
+        desc = cuasr_amd.make_desc(add, mult, "f16", dA, dB, dD, dD, one, zero, ident, one)
+        assert lib.cuasr_amd_selected_kernel(desc) == name
+    # bitwise operators are not defined on floating point
+    desc = cuasr_amd.make_desc("bit_xor", "bit_and", "f16", dA, dB, dD, dD, 0, 0, 0, 1)
+    assert lib.cuasr_amd_srgemm_can_implement(desc) == 5
+
+
+@pytest.mark.parametrize("sr", TILE_PAIRS + OTHER_PAIRS)
+@pytest.mark.parametrize("kernel", ["auto", "naive"])
+def test_every_pair(oracle, lib, sr, kernel):
+    for layouts in ("ccc", "rcr"):
+        check(oracle, *sr, 70, 90, 33, layouts, kernel)
+        check(oracle, *sr, 128, 256, 64, layouts, kernel, beta_one=False)
+
+
+def test_scaled_epilogue(oracle, lib):
+    # alpha and beta that are neither identity nor annihilator: both products are rounded before the add
+    check(oracle, "plus", "multiplies", 128, 256, 64, "ccc", "valu", alpha=1.5, beta=-0.75)
+    check(oracle, "plus", "multiplies", 90, 70, 50, "rcr", "valu", alpha=0.3, beta=2.5)
+    check(oracle, "minimum", "plus", 128, 256, 64, "ccc", "valu", alpha=3.25, beta=0.125)
+    check(oracle, "maximum", "minimum", 130, 100, 64, "crc", "valu", alpha=40.0, beta=60.0)
+
+
+@pytest.mark.parametrize("slices", [1, 3, 8])
+@pytest.mark.parametrize("kernel", ["auto", "naive"])
+def test_splitk(oracle, lib, slices, kernel):
+    for shape, layouts in [((256, 256, 1024), "ccc"), ((100, 60, 1000), "rcr"), ((128, 256, 96), "crc")]:
+        check(oracle, "minimum", "plus", *shape, layouts, kernel, splitk=slices)
+        check(oracle, "maximum", "minimum", *shape, layouts, kernel, splitk=slices, beta_one=False)
+
+
+def test_apsp_shaped_1024(oracle, lib):
+    for layouts in ("ccc", "rcr", "crr"):
+        check(oracle, "minimum", "plus", 1024, 1024, 1024, layouts, "auto")
+    check(oracle, "plus", "multiplies", 512, 512, 512, "ccc", "auto")
+
+
+def test_views_at_odd_offsets(oracle, lib):
+    """Operands inside larger allocations, two bytes off every vector boundary: the guarded kernel."""
+    import torch
+    import cuasr_amd
+    m, n, k = 131, 257, 67
+    for layouts in ("ccc", "rcr"):
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        A, B, C = operands("minimum", "plus", m + 3, n + 3, k + 3, la, lb, lc, seed=9)   # each three larger than its view
+        ident, one, _ = scalars("minimum", "plus", True)
+        a, b, c = A[1:1 + m, 1:1 + k], B[1:1 + k, 1:1 + n], C[1:1 + m, 1:1 + n]
+        want = oracle.srgemm("minimum", "plus", a, b, c, one, one, ident)
+        dA, dB, dC = to_device(A), to_device(B), to_device(C)
+        dD = to_device(np.full_like(C, 7))
+        cuasr_amd.srgemm("minimum", "plus", dA[1:1 + m, 1:1 + k], dB[1:1 + k, 1:1 + n], dC[1:1 + m, 1:1 + n], dD[1:1 + m, 1:1 + n],
+                         one, one, ident, one, dtype="f16")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        assert_same_bits(got[1:1 + m, 1:1 + n], want, f"view {layouts}")
+        frame = got.copy()
+        frame[1:1 + m, 1:1 + n] = 7
+        assert (frame == 7).all(), "wrote outside the view"
+
+
+def test_batch_in_the_grid(oracle, lib):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    for (m, n, k, batch) in [(64, 64, 64, 9), (128, 256, 64, 3), (50, 30, 70, 4)]:
+        A = inputs.uniform(3, batch * m, k, 0.5, 100.0, np.float16, "C").reshape(batch, m, k)
+        B = inputs.uniform(4, batch * k, n, 0.5, 100.0, np.float16, "C").reshape(batch, k, n)
+        C = inputs.uniform(5, batch * m, n, 0.5, 100.0, np.float16, "C").reshape(batch, m, n)
+        ident, one, _ = scalars("minimum", "plus", True)
+        dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), torch.from_numpy(C).cuda()
+        dD = torch.zeros_like(dC)
+        cuasr_amd.srgemm_batched("minimum", "plus", dA, dB, dC, dD, one, one, ident, one, dtype="f16")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        for i in range(batch):
+            want = oracle.srgemm("minimum", "plus", A[i], B[i], C[i], one, one, ident)
+            assert_same_bits(got[i], want, f"batch product {i} of {m}x{n}x{k}")
+
+
+def test_no_terms(oracle, lib):
+    # k = 0: the accumulator is the additive identity and only the epilogue runs
+    check(oracle, "minimum", "plus", 40, 50, 0, "ccc", "auto")
+    check(oracle, "plus", "multiplies", 128, 256, 0, "rcr", "valu")
