@@ -281,9 +281,12 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         # benchmark matrix (bench/device/harness.h:157-181 counts 2 * N^3 / t the same way)
         n = args.size or 4096
         add, mult, dt = args.add, args.mult, args.dtype
-        npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32}[dt]
+        npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16}[dt]
         la, lb, lc = ["F" if c == "c" else "C" for c in args.layouts]
-        if dt in ("f32", "f64"):
+        if dt == "f16" and mult != "multiplies":
+            # distances of a few units: sums stay well inside binary16's range and still round
+            A, B, C = (inputs.uniform(701 + i, n, n, 0.5, 100.0, npd, o) for i, o in enumerate((la, lb, lc)))
+        elif dt in ("f32", "f64", "f16"):
             A, B, C = (inputs.uniform(701 + i, n, n, -1.0, 1.0, npd, o) for i, o in enumerate((la, lb, lc)))
         elif dt == "u32":
             A, B, C = (inputs.words32(701 + i, n, n, o) for i, o in enumerate((la, lb, lc)))
@@ -293,7 +296,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         one = cuasr_amd.op_identity(mult, dt, True)
         up = lambda X: (col_major if X.flags.f_contiguous else row_major)(X.view(np.int32) if dt == "u32" else X)
         dA, dB, dC = up(A), up(B), up(C)
-        tdt = {"f32": torch.float32, "f64": torch.float64, "i32": torch.int32, "u32": torch.int32}[dt]
+        tdt = {"f32": torch.float32, "f64": torch.float64, "i32": torch.int32, "u32": torch.int32, "f16": torch.float16}[dt]
         dD = torch.empty(n, n, dtype=tdt, device=dev)
         dD = dD.t() if lc == "F" else dD
 
@@ -441,7 +444,7 @@ def main():
                              "srgemm", "fwgemm", "apsp_blocked"])
     ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
     ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32"], help="workload srgemm")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32", "f16"], help="workload srgemm")
     ap.add_argument("--layouts", default="ccc", help="workload srgemm: layouts of A, B, C (c = column-major, r = row-major)")
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")
