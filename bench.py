@@ -414,6 +414,19 @@ def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
     del wl
     torch.cuda.empty_cache()
 
+    # Half precision (the reference names it as an aim, README.md:11): min-plus on binary16, 4096^3, column-major;
+    # the first 64 rows against the oracle, which rounds every sum to binary16 as the device does
+    wl = build_workload(ns(workload="srgemm", add="minimum", mult="plus", dtype="f16", layouts="ccc", size=4096), np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    want = oracle.srgemm(add, mult, rows_of(A, 64), B, rows_of(C, 64), alpha, beta, ident)
+    got = wl["result"]()[:64]
+    out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(np.asfortranarray(got).tobytes() == np.asfortranarray(want).tobytes()),
+                     checked="first 64 rows of the output",
+                     note="packed binary16 instructions issue at half the rate of 4-byte ones: two terms per instruction, the same vector peak"))
+    del wl
+    torch.cuda.empty_cache()
+
     # All-pairs shortest paths with predecessors on top of SRGEMM (README.md:338-342 of the reference,
     # cpu_fwgemm_naive): a whole job at n = 4096 by blocked Floyd-Warshall, counted as 2 n^3 operations, and the
     # same kind of graph at n = 1024 against the oracle's blocked iteration, dist and parent bit for bit

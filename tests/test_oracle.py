@@ -72,7 +72,7 @@ FLOAT_PAIRS = [("plus", "multiplies"), ("minimum", "plus"), ("maximum", "plus"),
 INT_PAIRS = FLOAT_PAIRS + [("bit_xor", "bit_and"), ("bit_xor", "logical_and"), ("bit_or", "bit_and")]
 
 
-@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.uint32])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64, np.int32, np.uint32, np.float16])
 @pytest.mark.parametrize("shape", [(1, 1, 1), (7, 6, 5), (17, 27, 17), (33, 34, 3)])
 def test_against_literal_loop(oracle, dtype, shape):
     m, n, k = shape
@@ -87,6 +87,70 @@ def test_against_literal_loop(oracle, dtype, shape):
             for naive in (False, True):
                 got = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident, naive=naive)
                 assert bits(got) == bits(np.asarray(want, order=lc)), (add, mult, la, lb, lc, naive)
+
+
+def test_binary16_conversions_match_numpy(oracle):
+    """The oracle holds binary16 as bit patterns and converts by hand (its compiler has no half type):
+    every one of the 65536 patterns widens as numpy's float16 does, and narrowing rounds to nearest even
+    on random binary32 values, on every midpoint between neighbouring binary16 values and on the values
+    next to each midpoint (where a wrong tie rule or a dropped sticky bit shows)."""
+    import ctypes
+    lib = oracle.lib()
+    lib.oracle_half_to_float.restype, lib.oracle_half_to_float.argtypes = ctypes.c_float, [ctypes.c_uint16]
+    lib.oracle_float_to_half.restype, lib.oracle_float_to_half.argtypes = ctypes.c_uint16, [ctypes.c_float]
+    every = np.arange(65536, dtype=np.uint16)
+    want = every.view(np.float16).astype(np.float32)
+    got = np.array([lib.oracle_half_to_float(int(h)) for h in every], dtype=np.float32)
+    finite = ~np.isnan(want)
+    assert np.array_equal(got.view(np.uint32)[finite], want.view(np.uint32)[finite]) and np.isnan(got[~finite]).all()
+    halves = np.arange(0, 0x7c01, dtype=np.uint16).view(np.float16).astype(np.float64)   # 0 .. 65504, then inf
+    halves[-1] = 65536.0                                                                  # the value binary16 would hold next
+    mids = ((halves[:-1] + halves[1:]) / 2).astype(np.float32)                            # exact in binary32
+    near = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(1e9))])
+    rnd = inputs.splitmix64(11, 60000).astype(np.uint32).view(np.float32)
+    f = np.concatenate([near, -near, rnd, np.array([0.0, -0.0, np.inf, -np.inf, 65504.0, 65519.99, 65520.0, 1e30], np.float32)])
+    f = f[~np.isnan(f)]
+    with np.errstate(over="ignore"):
+        want = f.astype(np.float16).view(np.uint16)
+    got = np.array([lib.oracle_float_to_half(float(x)) for x in f], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("pair", FLOAT_PAIRS)
+def test_binary16_every_operator_rounds_once(oracle, pair):
+    """Values whose sums and products do not fit binary16: the oracle against the literal loop on numpy
+    float16 scalars (numpy rounds each float16 operation once, to nearest even), both oracle loops."""
+    add, mult = pair
+    m, n, k = 9, 10, 37
+    lo, hi = (-2.0, 2.0) if mult == "multiplies" else (-300.0, 300.0)
+    A = inputs.uniform(21, m, k, lo, hi, np.float16, "F")
+    B = inputs.uniform(22, k, n, lo, hi, np.float16, "C")
+    C = inputs.uniform(23, m, n, lo, hi, np.float16, "F")
+    A[0, :5] = np.float16(6e-5) * np.arange(5, dtype=np.float16)      # subnormal operands and results
+    B[:5, 0] = np.float16(3e-4)
+    for alpha, beta, ident in [(1.0, 0.0, 0.0), (0.7, 1.3, np.inf), (1.0, 1.0, -np.inf), (3.0, 0.25, 65504.0)]:
+        want = literal_srgemm(add, mult, A, B, C, np.float16(alpha), np.float16(beta), np.float16(ident))
+        for naive in (False, True):
+            got = oracle.srgemm(add, mult, A, B, C, np.float16(alpha), np.float16(beta), np.float16(ident), naive=naive)
+            nan = np.isnan(want)      # (inf - inf in max-plus with a -inf identity: any NaN will do)
+            assert np.array_equal(np.isnan(got), nan)
+            assert bits(np.where(nan, 0, got)) == bits(np.where(nan, 0, np.asarray(want, order="F"))), (add, mult, alpha, beta, ident, naive)
+
+
+def test_binary16_shortest_paths_on_small_integers(oracle):
+    """Integer weights whose path sums stay below 2048 are exact in binary16: repeated min-plus squaring
+    in half precision gives Floyd-Warshall's distances."""
+    n = 60
+    rng = np.random.default_rng(5)
+    W = np.where(rng.random((n, n)) < 0.2, rng.integers(1, 9, (n, n)), np.inf)
+    np.fill_diagonal(W, 0)
+    want = floyd_warshall(W.copy())
+    assert want[np.isfinite(want)].max() < 2048
+    D = np.asfortranarray(W.astype(np.float16))
+    inf = np.float16(np.inf)
+    for _ in range(6):
+        D = oracle.srgemm("minimum", "plus", D, D, D, np.float16(0), np.float16(0), inf)
+    assert np.array_equal(D.astype(np.float64), want)
 
 
 def test_blocked_equals_naive_on_ragged_and_submatrix(oracle):
