@@ -20,7 +20,7 @@ HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "cuasr_amd.h")
 # enums of include/cuasr_amd.h
 OPS = {"plus": 0, "multiplies": 1, "minimum": 2, "maximum": 3, "logical_and": 4,
        "logical_or": 5, "bit_and": 6, "bit_or": 7, "bit_xor": 8}
-DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3, "f16": 4}
+DTYPES = {"f32": 0, "f64": 1, "i32": 2, "u32": 3, "f16": 4, "i8": 5}
 COLUMN_MAJOR, ROW_MAJOR = 0, 1
 KERNELS = {"auto": 0, "naive": 1, "valu": 2, "mfma": 3, "direct": 4, "streamk": 5}
 STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
@@ -29,7 +29,8 @@ STATUS_NAMES = ["kSuccess", "kErrorMisalignedOperand", "kErrorInvalidDataType",
                 "kErrorInsufficientDriver", "kErrorMemoryAllocation", "kInvalid"]
 SUCCESS = 0
 
-_NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16}
+_NP_OF = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16,
+          "i8": np.int32}   # (int8 operands: the scalars, C and D are int32)
 
 
 class Scalar(ctypes.Union):
@@ -160,7 +161,7 @@ def _set_scalar(s, value, dtype):
         s.f32 = float(value)
     elif dtype == "f64":
         s.f64 = float(value)
-    elif dtype == "i32":
+    elif dtype in ("i32", "i8"):
         s.i32 = int(value)
     elif dtype == "f16":
         s.f16 = int(np.array([value], dtype=np.float16).view(np.uint16)[0])   # the binary16 bit pattern

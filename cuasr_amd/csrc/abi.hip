@@ -15,6 +15,7 @@ launch_fn find_valu_u32(int, int);
 launch_fn find_valu_f16(int, int);
 launch_fn find_mfma_f32(int, int);
 launch_fn find_mfma_f64(int, int);
+launch_fn find_mfma_i8(int, int);
 launch_fn find_direct_f32(int, int);
 launch_fn find_direct_i32(int, int);
 launch_fn find_direct_u32(int, int);
@@ -62,10 +63,13 @@ streamk_fn find_streamk(int dtype, int add_op, int mult_op) {
 launch_fn find_mfma(int dtype, int add_op, int mult_op) {
   if (dtype == CUASR_AMD_F32) return find_mfma_f32(add_op, mult_op);
   if (dtype == CUASR_AMD_F64) return find_mfma_f64(add_op, mult_op);
+  if (dtype == CUASR_AMD_I8) return find_mfma_i8(add_op, mult_op);
   return nullptr;
 }
 
+// bytes per element of C, D, the scalars and the workspace; and of A and B (int8 operands meet int32 everything else)
 static size_t elem_size(int dtype) { return dtype == CUASR_AMD_F64 ? 8 : dtype == CUASR_AMD_F16 ? 2 : 4; }
+static size_t operand_size(int dtype) { return dtype == CUASR_AMD_I8 ? 1 : elem_size(dtype); }
 
 static bool is_bitwise(int op) { return op == kBitAnd || op == kBitOr || op == kBitXor; }
 
@@ -82,6 +86,7 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d);
 // the matrix-core tiles use 16-byte loads and so need aligned, vector-sized operands
 static bool mfma_usable(const cuasr_amd_srgemm_desc *d) {
   if (!find_mfma(d->dtype, d->add_op, d->mult_op)) return false;
+  if (d->dtype == CUASR_AMD_I8) return true;  // its kernel has a guarded form for every extent and alignment
   return d->dtype == CUASR_AMD_F64 ? mfma_f64_can_run(canonical(d)) : mfma_f32_can_run(canonical(d));
 }
 
@@ -115,7 +120,7 @@ static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
 
 static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
   if (!d) return CUASR_AMD_ERROR_INVALID_PROBLEM;
-  if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_F16) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
+  if (d->dtype < CUASR_AMD_F32 || d->dtype > CUASR_AMD_I8) return CUASR_AMD_ERROR_INVALID_DATA_TYPE;
   const int layouts[3] = {d->layout_a, d->layout_b, d->layout_c};
   for (int l : layouts)
     if (l != CUASR_AMD_COLUMN_MAJOR && l != CUASR_AMD_ROW_MAJOR) return CUASR_AMD_ERROR_INVALID_LAYOUT;
@@ -135,10 +140,11 @@ static int validate(const cuasr_amd_srgemm_desc *d, bool splitk) {
     if (!d->D) return CUASR_AMD_ERROR_INVALID_PROBLEM;
     if (d->k > 0 && (!d->A || !d->B)) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   }
-  const size_t es = elem_size(d->dtype);
-  const void *ptrs[6] = {d->A, d->B, d->C, d->D, d->alpha_ptr, d->beta_ptr};
+  const size_t es = elem_size(d->dtype), os = operand_size(d->dtype);
+  const void *ptrs[4] = {d->C, d->D, d->alpha_ptr, d->beta_ptr};
   for (const void *q : ptrs)
     if (reinterpret_cast<uintptr_t>(q) % es) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
+  if (reinterpret_cast<uintptr_t>(d->A) % os || reinterpret_cast<uintptr_t>(d->B) % os) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;
   if (d->kernel == CUASR_AMD_KERNEL_VALU && !find_valu(d->dtype, d->add_op, d->mult_op))
     return CUASR_AMD_ERROR_NOT_SUPPORTED;
   if (d->kernel == CUASR_AMD_KERNEL_MFMA && !mfma_usable(d)) return CUASR_AMD_ERROR_NOT_SUPPORTED;
@@ -373,7 +379,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
   const int64_t outer = col ? desc->n : desc->m, inner = col ? desc->m : desc->n;
   if (batch > 1 && outer > 0 && inner > 0 && stride_d < (outer - 1) * desc->ldd + inner) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (batch == 0) return CUASR_AMD_SUCCESS;
-  const int64_t es = int64_t(elem_size(desc->dtype));
+  const int64_t es = int64_t(elem_size(desc->dtype)), os = int64_t(operand_size(desc->dtype));
   const int family = pick_family(desc, batch);
   bool in_grid = (family == kValu || family == kDirect) && batch > 1;
   if (family == kMfma && batch > 1 && desc->add_op == kPlus && desc->mult_op == kMultiplies) {
@@ -383,7 +389,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
     probe.batch = batch < 65535 ? batch : 65535;
     probe.batch_a = col ? stride_b : stride_a;
     probe.batch_b = col ? stride_a : stride_b;
-    in_grid = desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
+    in_grid = desc->dtype == CUASR_AMD_I8 ? true : desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
   }
   if (in_grid) {
     const launch_fn fn = family_fn(family, desc);
@@ -398,8 +404,8 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
     for (int first = 0; first < batch; first += 65535) {
       p.batch = batch - first < 65535 ? batch - first : 65535;
       if (fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
-      p.A = static_cast<const char *>(p.A) + es * p.batch_a * p.batch;
-      p.B = static_cast<const char *>(p.B) + es * p.batch_b * p.batch;
+      p.A = static_cast<const char *>(p.A) + os * p.batch_a * p.batch;
+      p.B = static_cast<const char *>(p.B) + os * p.batch_b * p.batch;
       if (p.C) p.C = static_cast<const char *>(p.C) + es * p.batch_c * p.batch;
       p.D = static_cast<char *>(p.D) + es * p.batch_d * p.batch;
     }
@@ -407,8 +413,8 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
   }
   for (int i = 0; i < batch; ++i) {
     cuasr_amd_srgemm_desc one = *desc;
-    if (one.A) one.A = static_cast<const char *>(desc->A) + es * stride_a * i;
-    if (one.B) one.B = static_cast<const char *>(desc->B) + es * stride_b * i;
+    if (one.A) one.A = static_cast<const char *>(desc->A) + os * stride_a * i;
+    if (one.B) one.B = static_cast<const char *>(desc->B) + os * stride_b * i;
     if (one.C) one.C = static_cast<const char *>(desc->C) + es * stride_c * i;
     if (one.D) one.D = static_cast<char *>(desc->D) + es * stride_d * i;
     const int r = cuasr_amd_srgemm(&one, stream);
@@ -419,7 +425,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
 
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
   if (!desc || desc->m < 0 || desc->n < 0 || desc->split_k_slices < 1) return 0;
-  if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_F16) return 0;
+  if (desc->dtype < CUASR_AMD_F32 || desc->dtype > CUASR_AMD_I8) return 0;
   return elem_size(desc->dtype) * size_t(desc->m) * size_t(desc->n) * size_t(desc->split_k_slices);
 }
 

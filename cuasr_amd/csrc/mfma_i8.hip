@@ -1,0 +1,225 @@
+// Plus-times on int8 operands with int32 accumulation, on the matrix cores.
+//
+// The reference carries threadblock cores for int8 operands built around the 4-way byte dot product
+// (include/cuasr/gemm/threadblock/default_srmma_core_simt.h:733-1381: ElementA = ElementB = int8_t,
+// InstructionShape 1 x 1 x 4), but never instantiates them.  On gfx950 the instruction for that job is
+// v_mfma_i32_32x32x32_i8: a wave multiplies a 32 x 32 (rows x k) block of A by a 32 x 32 block of B, every lane
+// supplying 16 consecutive k of one row (column).  Integer sums wrap modulo 2^32 whatever their order, so the
+// result is bit-identical to the k-ascending reference loop.
+//
+// Tile: 256 threads (2 x 2 waves), 128 x 128 x 64; a wave holds 2 x 2 blocks of 32 x 32 (64 accumulator
+// registers).  LDS holds both panels k-contiguous, [x][64 k + 16 bytes of padding] (the padding makes the 16-byte
+// fragment reads of 32 consecutive rows conflict-free), two stages.  Operands are staged through registers, which
+// is where an operand whose rows (columns) are contiguous in memory gets transposed: a thread loads 16 x at 4
+// consecutive k (four 16-byte loads), turns them with byte permutes into 16 words of 4 k each and writes those.
+#include "semiring.h"
+
+namespace cuasr_amd {
+namespace mfma_i8 {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 128, BN = 128, BK = 64, THREADS = 256, PITCH = BK + 16;
+
+struct Smem {
+  int8_t a[2][BM][PITCH];
+  int8_t b[2][BN][PITCH];
+};
+
+// One operand's share of a k-tile (128 x, 64 k) on its way from memory to LDS.
+//   KC (k contiguous in memory): 512 chunks of 16 k of one x, two per thread, written as they are.
+//   otherwise (x contiguous):    128 units of 16 x by 4 k, one per thread of the half of the workgroup
+//                                `first_thread` names; four 16-byte loads, transposed in registers.
+// GUARD: bytes beyond the extents read as zero (a zero factor adds nothing to a sum of products).
+template <bool KC, bool GUARD> struct Stager {
+  v4i r[KC ? 2 : 4];
+
+  static __device__ __forceinline__ v4i fetch(const int8_t *src, long long step, int first, int count, int limit, bool live) {
+    // 16 bytes from src, src + step, ...; byte e is element first + e of a run that ends at `limit`
+    if constexpr (!GUARD) {
+      return *reinterpret_cast<const v4i *>(src);
+    } else {
+      v4i v = {0, 0, 0, 0};
+      if (live) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int byte = (first + e < limit) ? (int)(unsigned char)src[step * e] : 0;
+          v[e / 4] |= byte << (8 * (e % 4));
+        }
+      }
+      return v;
+    }
+  }
+
+  __device__ __forceinline__ void load(const int8_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn, int first_thread) {
+    if constexpr (KC) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int c = threadIdx.x + q * THREADS, k = (c % 4) * 16, x = c / 4;
+        r[q] = fetch(base + (long long)(x0 + x) * sx + (k0 + k), 1, k0 + k, 16, kn, x0 + x < xn);
+      }
+    } else {
+      const int u = (int)threadIdx.x - first_thread;
+      if (u >= 0 && u < 128) {
+        const int x = (u % 8) * 16, k = (u / 8) * 4;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+          r[kk] = fetch(base + (x0 + x) + (long long)(k0 + k + kk) * sk, 1, x0 + x, 16, xn, k0 + k + kk < kn);
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(int8_t (*panel)[PITCH], int first_thread) const {
+    if constexpr (KC) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        const int c = threadIdx.x + q * THREADS, k = (c % 4) * 16, x = c / 4;
+        *reinterpret_cast<v4i *>(&panel[x][k]) = r[q];
+      }
+    } else {
+      const int u = (int)threadIdx.x - first_thread;
+      if (u >= 0 && u < 128) {
+        const int x = (u % 8) * 16, k = (u / 8) * 4;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          // words d of the four loads hold x = 4d .. 4d+3 at k, k+1, k+2, k+3: a 4 x 4 byte transpose
+          const unsigned a = r[0][d], b = r[1][d], c = r[2][d], e = r[3][d];
+          const unsigned ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602);
+          const unsigned ce_lo = __builtin_amdgcn_perm(e, c, 0x05010400), ce_hi = __builtin_amdgcn_perm(e, c, 0x07030602);
+          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 0][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x05040100);
+          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 1][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x07060302);
+          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 2][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x05040100);
+          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 3][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x07060302);
+        }
+      }
+    }
+  }
+};
+
+template <bool A_KC, bool B_KC, bool GUARD>
+__global__ __launch_bounds__(THREADS) void mfma_i8_kernel(Problem p) {
+  __shared__ __attribute__((aligned(16))) Smem sm;
+  select_batch<int32_t, int8_t>(p);
+  const int tiles_n = (p.n + BN - 1) / BN;
+  const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
+  const int l32 = lane & 31, half = lane >> 5;
+  int kb = 0, ke = p.k;
+  if (p.workspace) {
+    kb = blockIdx.y * p.k_per_slice;
+    ke = min(p.k, kb + p.k_per_slice);
+  }
+  const int8_t *A = reinterpret_cast<const int8_t *>(p.A), *B = reinterpret_cast<const int8_t *>(p.B);
+
+  v16i acc[2][2];
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[bi][bj][e] = 0;
+
+  // when both operands need the transpose, the two halves of the workgroup take one each
+  constexpr int A_FIRST = 0, B_FIRST = A_KC ? 0 : 128;
+  Stager<A_KC, GUARD> sa;
+  Stager<B_KC, GUARD> sb;
+  const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
+  if (tiles_k > 0) {
+    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke, A_FIRST);
+    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke, B_FIRST);
+    sa.store(sm.a[0], A_FIRST);
+    sb.store(sm.b[0], B_FIRST);
+  }
+  __syncthreads();
+  for (int t = 0; t < tiles_k; ++t) {
+    const int s = t & 1, k0 = kb + t * BK;
+    if (t + 1 < tiles_k) {
+      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke, A_FIRST);
+      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke, B_FIRST);
+    }
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks) {
+      v4i a[2], b[2];
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) a[bi] = *reinterpret_cast<const v4i *>(&sm.a[s][wm * 64 + bi * 32 + l32][ks * 32 + half * 16]);
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) b[bj] = *reinterpret_cast<const v4i *>(&sm.b[s][wn * 64 + bj * 32 + l32][ks * 32 + half * 16]);
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
+    }
+    if (t + 1 < tiles_k) {
+      sa.store(sm.a[s ^ 1], A_FIRST);
+      sb.store(sm.b[s ^ 1], B_FIRST);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue.  Register e of lane l in block (bi, bj): row 8*(e/4) + 4*(l/32) + e%4, column l%32.
+  const EpilogueScalars<int32_t> sc = resolve_scalars<int32_t>(p, kMultiplies);
+  int32_t *ws = p.workspace ? reinterpret_cast<int32_t *>(p.workspace) + (long long)blockIdx.y * p.m * p.n : nullptr;
+  const int32_t *C = reinterpret_cast<const int32_t *>(p.C);
+  int32_t *D = reinterpret_cast<int32_t *>(p.D);
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+      const int col = n0 + wn * 64 + bj * 32 + l32;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+        if (GUARD && !((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) continue;
+        const int32_t v = acc[bi][bj][e];
+        if (ws) {
+          ws[(long long)row * p.n + col] = v;
+        } else {
+          // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
+          uint32_t out = (uint32_t)sc.alpha * (uint32_t)v;
+          if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)C[(long long)row * p.ldc + col];
+          D[(long long)row * p.ldd + col] = (int32_t)out;
+        }
+      }
+    }
+}
+
+// whole tiles of 16-byte aligned operands: the unguarded kernel
+static bool exact(const Problem &p, bool a_kc, bool b_kc) {
+  auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  if (p.m % BM || p.n % BN || p.k % BK || p.k == 0) return false;
+  if (p.workspace && p.k_per_slice % BK) return false;
+  if ((a_kc ? p.sa_m : p.sa_k) % 16 || (b_kc ? p.sb_n : p.sb_k) % 16) return false;
+  if (!al16(p.A) || !al16(p.B)) return false;
+  if (p.batch > 1 && (p.batch_a % 16 || p.batch_b % 16)) return false;
+  return true;
+}
+
+static hipError_t launch(const Problem &p, hipStream_t s) {
+  if (p.m == 0 || p.n == 0) return hipSuccess;
+  if ((p.sa_m != 1 && p.sa_k != 1) || (p.sb_n != 1 && p.sb_k != 1)) return hipErrorNotSupported;
+  // (an operand with both strides 1 is a single row or column: either form reads it correctly)
+  const bool a_kc = p.sa_k == 1, b_kc = p.sb_k == 1;
+  const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(THREADS);
+  const bool fast = exact(p, a_kc, b_kc);
+#define CUASR_I8_LAUNCH(AK, BK_, G) launch_kernel((mfma_i8_kernel<AK, BK_, G>), grid, block, 0, s, p)
+  if (fast) {
+    if (a_kc) { if (b_kc) CUASR_I8_LAUNCH(true, true, false); else CUASR_I8_LAUNCH(true, false, false); }
+    else { if (b_kc) CUASR_I8_LAUNCH(false, true, false); else CUASR_I8_LAUNCH(false, false, false); }
+  } else {
+    if (a_kc) { if (b_kc) CUASR_I8_LAUNCH(true, true, true); else CUASR_I8_LAUNCH(true, false, true); }
+    else { if (b_kc) CUASR_I8_LAUNCH(false, true, true); else CUASR_I8_LAUNCH(false, false, true); }
+  }
+#undef CUASR_I8_LAUNCH
+  return take_launch_status();
+}
+
+}  // namespace mfma_i8
+
+launch_fn find_mfma_i8(int add_op, int mult_op) {
+  return (add_op == kPlus && mult_op == kMultiplies) ? mfma_i8::launch : nullptr;
+}
+
+}  // namespace cuasr_amd

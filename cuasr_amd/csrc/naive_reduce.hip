@@ -10,15 +10,16 @@
 namespace cuasr_amd {
 
 // ---------------------------------------------------------------- naive SRGEMM
-template <typename T>
+// TI: the type A and B are stored in (int8 operands are widened to the int32 everything else is in)
+template <typename T, typename TI = T>
 __global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
   const int j = blockIdx.x * 16 + (threadIdx.x & 15);
   const int i = blockIdx.y * 16 + (threadIdx.x >> 4);
   const int z = blockIdx.z;
   if (i >= p.m || j >= p.n) return;
   const EpilogueScalars<T> e = resolve_scalars<T>(p, p.mult_op);
-  const T *A = reinterpret_cast<const T *>(p.A) + (long long)i * p.sa_m;
-  const T *B = reinterpret_cast<const T *>(p.B) + (long long)j * p.sb_n;
+  const TI *A = reinterpret_cast<const TI *>(p.A) + (long long)i * p.sa_m;
+  const TI *B = reinterpret_cast<const TI *>(p.B) + (long long)j * p.sb_n;
   int k0 = 0, k1 = p.k;
   if (p.workspace) {
     k0 = z * p.k_per_slice;
@@ -26,7 +27,7 @@ __global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
   }
   T acc = e.ident;
   for (int kk = k0; kk < k1; ++kk) {
-    const T prod = apply_op<T>(p.mult_op, A[(long long)kk * p.sa_k], B[(long long)kk * p.sb_k]);
+    const T prod = apply_op<T>(p.mult_op, T(A[(long long)kk * p.sa_k]), T(B[(long long)kk * p.sb_k]));
     acc = apply_op<T>(p.add_op, prod, acc);  // host reference order: add(prod, acc)
   }
   if (p.workspace) {
@@ -41,10 +42,10 @@ __global__ __launch_bounds__(256) void naive_srgemm_kernel(Problem p) {
   reinterpret_cast<T *>(p.D)[(long long)i * p.ldd + j] = out;
 }
 
-template <typename T> static hipError_t launch_naive(const Problem &p, hipStream_t s) {
+template <typename T, typename TI = T> static hipError_t launch_naive(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   dim3 grid((p.n + 15) / 16, (p.m + 15) / 16, p.workspace ? p.slices : 1);
-  launch_kernel(naive_srgemm_kernel<T>, grid, dim3(256), 0, s, p);
+  launch_kernel((naive_srgemm_kernel<T, TI>), grid, dim3(256), 0, s, p);
   return take_launch_status();
 }
 
@@ -55,6 +56,7 @@ launch_fn find_naive(int dtype) {
     case CUASR_AMD_I32: return launch_naive<int32_t>;
     case CUASR_AMD_U32: return launch_naive<uint32_t>;
     case CUASR_AMD_F16: return launch_naive<half_t>;
+    case CUASR_AMD_I8: return (launch_naive<int32_t, int8_t>);
     default: return nullptr;
   }
 }
@@ -261,6 +263,7 @@ launch_fn find_reduce(int dtype) {
     case CUASR_AMD_I32: return launch_reduce<int32_t, false>;
     case CUASR_AMD_U32: return launch_reduce<uint32_t, false>;
     case CUASR_AMD_F16: return launch_reduce<half_t, false>;
+    case CUASR_AMD_I8: return launch_reduce<int32_t, false>;   // (the partial products are int32)
     default: return nullptr;
   }
 }
@@ -272,6 +275,7 @@ launch_fn find_reduce_serial(int dtype) {
     case CUASR_AMD_I32: return launch_reduce<int32_t, true>;
     case CUASR_AMD_U32: return launch_reduce<uint32_t, true>;
     case CUASR_AMD_F16: return launch_reduce<half_t, true>;
+    case CUASR_AMD_I8: return launch_reduce<int32_t, true>;
     default: return nullptr;
   }
 }

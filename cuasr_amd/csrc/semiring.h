@@ -149,11 +149,11 @@ struct Problem {
 };
 
 // the operands of product blockIdx.z of a strided batch
-template <typename T> __device__ __forceinline__ void select_batch(Problem &p) {
+template <typename T, typename TI = T> __device__ __forceinline__ void select_batch(Problem &p) {
   if (p.batch > 1) {
     const long long z = blockIdx.z;
-    p.A = reinterpret_cast<const T *>(p.A) + z * p.batch_a;
-    p.B = reinterpret_cast<const T *>(p.B) + z * p.batch_b;
+    p.A = reinterpret_cast<const TI *>(p.A) + z * p.batch_a;
+    p.B = reinterpret_cast<const TI *>(p.B) + z * p.batch_b;
     if (p.C) p.C = reinterpret_cast<const T *>(p.C) + z * p.batch_c;
     p.D = reinterpret_cast<T *>(p.D) + z * p.batch_d;
   }

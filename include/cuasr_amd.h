@@ -77,7 +77,12 @@ typedef enum cuasr_amd_dtype {
   /* IEEE binary16 in A, B, C, D, the scalars and the accumulator: every operator rounds its result to
    * binary16, as the reference's templates do when they are instantiated with cutlass::half_t for all
    * element types (the reference names half precision as an aim only, README.md:11) */
-  CUASR_AMD_F16 = 4
+  CUASR_AMD_F16 = 4,
+  /* A and B hold int8; C, D, the scalars and the accumulator are int32 -- the element types of the reference's
+   * dp4a cores (include/cuasr/gemm/threadblock/default_srmma_core_simt.h:747-757: ElementA = ElementB = int8_t,
+   * ElementC a parameter; they are never instantiated there).  Every operator acts on the values widened to
+   * int32; lda / ldb count int8 elements, ldc / ldd int32 elements */
+  CUASR_AMD_I8 = 5
 } cuasr_amd_dtype;
 
 typedef enum cuasr_amd_layout {

@@ -67,6 +67,15 @@ def mat_ref(a):
     return a.ctypes.data_as(ctypes.c_void_p), int(ld), layout
 
 
+def _element_types(A, B, C):
+    """(dtype of C, D and the scalars; the oracle's type code).  int8 operands go with int32 everything else."""
+    if A.dtype == np.int8:
+        assert B.dtype == np.int8 and C.dtype == np.int32
+        return np.dtype(np.int32), 5
+    assert B.dtype == A.dtype and C.dtype == A.dtype
+    return A.dtype, DTYPES[A.dtype]
+
+
 def _scalar(v, dtype):
     return np.array([v], dtype=dtype)
 
@@ -85,8 +94,7 @@ def srgemm(add_op, mult_op, A, B, C, alpha, beta, add_identity, out=None,
     A is m x k, B is k x n, C is m x n; each row- or column-major (taken from
     the strides).  D gets C's layout.  Returns D.
     """
-    dt = A.dtype
-    assert B.dtype == dt and C.dtype == dt
+    dt, code = _element_types(A, B, C)
     m, k = A.shape
     k2, n = B.shape
     assert k2 == k and C.shape == (m, n)
@@ -98,7 +106,7 @@ def srgemm(add_op, mult_op, A, B, C, alpha, beta, add_identity, out=None,
     assert ld_layout == lc or m == 1 or n == 1
     al, be, ident = _scalar(alpha, dt), _scalar(beta, dt), _scalar(add_identity, dt)
     rc = lib().oracle_srgemm(
-        DTYPES[dt], OPS[add_op], OPS[mult_op], m, n, k,
+        code, OPS[add_op], OPS[mult_op], m, n, k,
         al.ctypes.data_as(ctypes.c_void_p), pa, ctypes.c_int64(lda), la,
         pb, ctypes.c_int64(ldb), lb, be.ctypes.data_as(ctypes.c_void_p),
         pc, ctypes.c_int64(ldc), pd, ctypes.c_int64(ldd), lc,
@@ -111,7 +119,7 @@ def srgemm(add_op, mult_op, A, B, C, alpha, beta, add_identity, out=None,
 def srgemm_splitk(add_op, mult_op, A, B, C, alpha, beta, add_identity,
                   mult_identity, slices, tbk=8, out=None, nthreads=0):
     """CPU model of the two-kernel parallel split-K (partials, then reduce)."""
-    dt = A.dtype
+    dt, code = _element_types(A, B, C)
     m, k = A.shape
     _, n = B.shape
     D = out if out is not None else empty_like_layout(C)
@@ -122,7 +130,7 @@ def srgemm_splitk(add_op, mult_op, A, B, C, alpha, beta, add_identity,
     al, be = _scalar(alpha, dt), _scalar(beta, dt)
     ident, one = _scalar(add_identity, dt), _scalar(mult_identity, dt)
     rc = lib().oracle_srgemm_splitk(
-        DTYPES[dt], OPS[add_op], OPS[mult_op], m, n, k,
+        code, OPS[add_op], OPS[mult_op], m, n, k,
         al.ctypes.data_as(ctypes.c_void_p), pa, ctypes.c_int64(lda), la,
         pb, ctypes.c_int64(ldb), lb, be.ctypes.data_as(ctypes.c_void_p),
         pc, ctypes.c_int64(ldc), pd, ctypes.c_int64(ldd), lc,
@@ -136,7 +144,7 @@ def srgemm_splitk(add_op, mult_op, A, B, C, alpha, beta, add_identity,
 def srgemm_splitk_serial(add_op, mult_op, A, B, C, alpha, beta, add_identity,
                          mult_identity, slices, tbk=8, out=None, nthreads=0):
     """CPU model of the serial split-K: the slices' epilogues chained through D."""
-    dt = A.dtype
+    dt, code = _element_types(A, B, C)
     m, k = A.shape
     _, n = B.shape
     D = out if out is not None else empty_like_layout(C)
@@ -147,7 +155,7 @@ def srgemm_splitk_serial(add_op, mult_op, A, B, C, alpha, beta, add_identity,
     al, be = _scalar(alpha, dt), _scalar(beta, dt)
     ident, one = _scalar(add_identity, dt), _scalar(mult_identity, dt)
     rc = lib().oracle_srgemm_splitk_serial(
-        DTYPES[dt], OPS[add_op], OPS[mult_op], m, n, k,
+        code, OPS[add_op], OPS[mult_op], m, n, k,
         al.ctypes.data_as(ctypes.c_void_p), pa, ctypes.c_int64(lda), la,
         pb, ctypes.c_int64(ldb), lb, be.ctypes.data_as(ctypes.c_void_p),
         pc, ctypes.c_int64(ldc), pd, ctypes.c_int64(ldd), lc,

@@ -61,7 +61,7 @@
 enum { OP_PLUS = 0, OP_MULTIPLIES = 1, OP_MINIMUM = 2, OP_MAXIMUM = 3,
        OP_LOGICAL_AND = 4, OP_LOGICAL_OR = 5, OP_BIT_AND = 6, OP_BIT_OR = 7,
        OP_BIT_XOR = 8 };
-enum { DT_F32 = 0, DT_F64 = 1, DT_I32 = 2, DT_U32 = 3, DT_F16 = 4 };
+enum { DT_F32 = 0, DT_F64 = 1, DT_I32 = 2, DT_U32 = 3, DT_F16 = 4, DT_I8 = 5 };
 enum { LAYOUT_COLUMN_MAJOR = 0, LAYOUT_ROW_MAJOR = 1 };
 
 #define BLK 32
@@ -171,10 +171,10 @@ typedef struct {
  * i loop vectorises; per element the order of operations is exactly
  * accum = add(mult(a, b), accum) for k ascending.
  */
-#define DEFINE_KERNEL(NAME, T, ADD, MUL, NE)                                      \
+#define DEFINE_KERNEL(NAME, T, TI, ADD, MUL, NE)                                  \
   CLONES static void NAME(const job_t *jb) {                                    \
     const int M = jb->m, N = jb->n;                                             \
-    const T *A = (const T *)jb->A, *B = (const T *)jb->B;                       \
+    const TI *A = (const TI *)jb->A, *B = (const TI *)jb->B;                    \
     const T *C = (const T *)jb->C;                                              \
     T *D = (T *)jb->D;                                                          \
     const T alpha = *(const T *)jb->alpha, beta = *(const T *)jb->beta;         \
@@ -198,11 +198,11 @@ typedef struct {
             for (int kk = 0; kk < KK; ++kk) {                                   \
               for (int i = 0; i < BLK; ++i)                                     \
                 Ap[(size_t)kk * BLK + i] = i < mr                               \
-                  ? A[(int64_t)(r0 + i) * jb->sa_m + (int64_t)(k0 + kk) * jb->sa_k] \
+                  ? (T)A[(int64_t)(r0 + i) * jb->sa_m + (int64_t)(k0 + kk) * jb->sa_k] \
                   : ident;                                                      \
               for (int j = 0; j < BLK; ++j)                                     \
                 Bp[(size_t)kk * BLK + j] = j < nc                               \
-                  ? B[(int64_t)(k0 + kk) * jb->sb_k + (int64_t)(c0 + j) * jb->sb_n] \
+                  ? (T)B[(int64_t)(k0 + kk) * jb->sb_k + (int64_t)(c0 + j) * jb->sb_n] \
                   : ident;                                                      \
             }                                                                   \
             for (int jq = 0; jq < BLK; jq += 4) {                               \
@@ -258,9 +258,9 @@ typedef struct {
 
 /* the literal triple loop, no blocking, no packing: an independent second
  * implementation used to cross-check the blocked one */
-#define DEFINE_NAIVE(NAME, T, ADD, MUL)                                         \
+#define DEFINE_NAIVE(NAME, T, TI, ADD, MUL)                                     \
   static void NAME(const job_t *jb) {                                           \
-    const T *A = (const T *)jb->A, *B = (const T *)jb->B;                       \
+    const TI *A = (const TI *)jb->A, *B = (const TI *)jb->B;                    \
     const T *C = (const T *)jb->C;                                              \
     T *D = (T *)jb->D;                                                          \
     const T alpha = *(const T *)jb->alpha, beta = *(const T *)jb->beta;         \
@@ -269,8 +269,8 @@ typedef struct {
       for (int col = 0; col < jb->n; ++col) {                                   \
         T accum = ident;                                                        \
         for (int kk = 0; kk < jb->k; ++kk) {                                    \
-          const T a = A[(int64_t)row * jb->sa_m + (int64_t)kk * jb->sa_k];      \
-          const T b = B[(int64_t)kk * jb->sb_k + (int64_t)col * jb->sb_n];      \
+          const T a = (T)A[(int64_t)row * jb->sa_m + (int64_t)kk * jb->sa_k];   \
+          const T b = (T)B[(int64_t)kk * jb->sb_k + (int64_t)col * jb->sb_n];   \
           const T prod = MUL(a, b);                                             \
           accum = ADD(prod, accum);                                             \
         }                                                                       \
@@ -282,11 +282,16 @@ typedef struct {
   }
 
 #define DEFINE_PAIR(T, TN, ADDN, MULN)                                          \
-  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, F_##ADDN, F_##MULN, F_NE)        \
-  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, F_##ADDN, F_##MULN)
+  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, T, F_##ADDN, F_##MULN, F_NE)     \
+  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, T, F_##ADDN, F_##MULN)
 #define DEFINE_HALF_PAIR(T, TN, ADDN, MULN)                                     \
-  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, H_##ADDN, H_##MULN, H_NE)        \
-  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, H_##ADDN, H_##MULN)
+  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, T, H_##ADDN, H_##MULN, H_NE)     \
+  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, T, H_##ADDN, H_##MULN)
+/* int8 operands, everything else int32: the element types of the reference's dp4a cores
+ * (include/cuasr/gemm/threadblock/default_srmma_core_simt.h:747-757); a and b are widened first */
+#define DEFINE_BYTE_PAIR(T, TN, ADDN, MULN)                                     \
+  DEFINE_KERNEL(blk_##TN##_##ADDN##_##MULN, T, int8_t, F_##ADDN, F_##MULN, F_NE) \
+  DEFINE_NAIVE(nv_##TN##_##ADDN##_##MULN, T, int8_t, F_##ADDN, F_##MULN)
 
 /* add-ops x mult-ops available to floating types */
 #define FOR_FLOAT_PAIRS(X, T, TN)                                               \
@@ -316,6 +321,8 @@ FOR_INT_EXTRA_PAIRS(DEFINE_PAIR, int32_t, i32)
 FOR_FLOAT_PAIRS(DEFINE_PAIR, uint32_t, u32)
 FOR_INT_EXTRA_PAIRS(DEFINE_PAIR, uint32_t, u32)
 FOR_FLOAT_PAIRS(DEFINE_HALF_PAIR, h16, f16)
+FOR_FLOAT_PAIRS(DEFINE_BYTE_PAIR, int32_t, i8)
+FOR_INT_EXTRA_PAIRS(DEFINE_BYTE_PAIR, int32_t, i8)
 
 typedef void (*kernel_fn)(const job_t *);
 
@@ -334,6 +341,9 @@ static kernel_fn lookup(int dtype, int add_op, int mult_op, int naive) {
     FOR_FLOAT_PAIRS(LOOKUP_ROW, uint32_t, u32)
     FOR_INT_EXTRA_PAIRS(LOOKUP_ROW, uint32_t, u32) break;
   case DT_F16: FOR_FLOAT_PAIRS(LOOKUP_ROW, h16, f16) break;
+  case DT_I8:
+    FOR_FLOAT_PAIRS(LOOKUP_ROW, int32_t, i8)
+    FOR_INT_EXTRA_PAIRS(LOOKUP_ROW, int32_t, i8) break;
   default: break;
   }
   return 0;

@@ -1,0 +1,116 @@
+"""int8 operands with int32 accumulation (the element types of the reference's dp4a cores) against the CPU
+oracle, bit for bit, through the C ABI: plus-times on the matrix cores in every layout, aligned and ragged,
+the other operator pairs on the naive kernel, split-K, batches."""
+import numpy as np
+import pytest
+
+from helpers import assert_same_bits, order_of, to_device
+
+pytestmark = pytest.mark.gpu
+
+LAYOUTS = ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"]
+
+
+def operands(m, n, k, la, lb, lc, seed=1):
+    from cuasr_amd import inputs
+    A = inputs.integers(seed, m, k, -128, 127, np.int8, order_of(la))
+    B = inputs.integers(seed + 1, k, n, -128, 127, np.int8, order_of(lb))
+    C = inputs.integers(seed + 2, m, n, -100000, 100000, np.int32, order_of(lc))
+    return A, B, C
+
+
+def check(oracle, add, mult, m, n, k, layouts, kernel="auto", alpha=None, beta=None, splitk=0, seed=1):
+    import torch
+    import cuasr_amd
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    A, B, C = operands(m, n, k, la, lb, lc, seed)
+    ident = int(cuasr_amd.op_identity(add, "i8"))
+    one = int(cuasr_amd.op_identity(mult, "i8"))
+    alpha = one if alpha is None else alpha
+    beta = one if beta is None else beta
+    want = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident)
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    dD = to_device(np.zeros_like(C))
+    print(f"int8 {add}-{mult} {m}x{n}x{k} {layouts} {kernel} alpha={alpha} beta={beta} splitk={splitk}", flush=True)
+    if splitk:
+        ws = torch.empty(cuasr_amd.splitk_workspace_bytes(m, n, splitk, "i8") // 4 + 4, dtype=torch.int32, device="cuda")
+        cuasr_amd.srgemm_splitk(add, mult, dA, dB, dC, dD, splitk, ws, alpha, beta, ident, one, dtype="i8", kernel=kernel)
+    else:
+        cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, alpha, beta, ident, one, dtype="i8", kernel=kernel)
+    torch.cuda.synchronize()
+    assert_same_bits(dD.cpu().numpy(), want, f"{add}-{mult} i8 {m}x{n}x{k} {layouts} {kernel}")
+
+
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_plus_times_on_the_matrix_cores(oracle, lib, layouts):
+    # whole tiles of aligned operands (the unguarded kernel), then ragged / tiny / thin ones (the guarded one)
+    for shape in [(128, 128, 64), (256, 384, 192), (100, 70, 45), (1, 1, 1), (130, 258, 67), (64, 8, 200), (16, 16, 16)]:
+        check(oracle, "plus", "multiplies", *shape, layouts, "mfma")
+        check(oracle, "plus", "multiplies", *shape, layouts, "auto", alpha=3, beta=-2)
+        check(oracle, "plus", "multiplies", *shape, layouts, "auto", alpha=1, beta=0)
+
+
+def test_selected_family(lib):
+    import cuasr_amd
+    dA = to_device(np.zeros((128, 64), np.int8))
+    dB = to_device(np.zeros((64, 256), np.int8))
+    dD = to_device(np.zeros((128, 256), np.int32))
+    for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"naive"), (("bit_xor", "bit_and"), b"naive")]:
+        desc = cuasr_amd.make_desc(add, mult, "i8", dA, dB, dD, dD, 1, 0, 0, 1)
+        assert lib.cuasr_amd_selected_kernel(desc) == name
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"),
+                                ("logical_or", "logical_and"), ("bit_xor", "bit_and"), ("bit_or", "bit_and"),
+                                ("minimum", "multiplies"), ("plus", "multiplies")])
+def test_every_pair_on_widened_operands(oracle, lib, sr):
+    for layouts in ("ccc", "rcr"):
+        check(oracle, *sr, 70, 90, 33, layouts, "auto")
+        check(oracle, *sr, 70, 90, 33, layouts, "naive")
+
+
+@pytest.mark.parametrize("slices", [1, 3, 8])
+def test_splitk(oracle, lib, slices):
+    # sums of int32 wrap modulo 2^32 in any order: split-K is bit-exact for plus-times too
+    for shape, layouts in [((256, 256, 1024), "ccc"), ((100, 60, 1000), "rcr"), ((128, 128, 192), "crc")]:
+        check(oracle, "plus", "multiplies", *shape, layouts, "auto", alpha=2, beta=5, splitk=slices)
+    check(oracle, "minimum", "plus", 100, 60, 1000, "ccc", "auto", splitk=slices)
+
+
+def test_1024(oracle, lib):
+    for layouts in ("ccc", "rcr", "crr"):
+        check(oracle, "plus", "multiplies", 1024, 1024, 1024, layouts, "auto", alpha=1, beta=1)
+
+
+def test_wraparound(oracle, lib):
+    """All operands at -128 and a long k: the int32 sums wrap, the same way on both sides."""
+    import torch
+    import cuasr_amd
+    m, n, k = 128, 128, 200000
+    A = np.full((m, k), -128, np.int8)
+    B = np.full((k, n), -128, np.int8, order="F")
+    C = np.zeros((m, n), np.int32)
+    want = np.full((m, n), (16384 * k + 2 ** 31) % 2 ** 32 - 2 ** 31, np.int64).astype(np.int32)
+    dA, dB, dC = to_device(A), to_device(B), to_device(C)
+    dD = to_device(np.zeros_like(C))
+    cuasr_amd.srgemm("plus", "multiplies", dA, dB, dC, dD, 1, 0, 0, 1, dtype="i8")
+    torch.cuda.synchronize()
+    assert_same_bits(dD.cpu().numpy(), want, "wrapped sums")
+
+
+def test_batch_in_the_grid(oracle, lib):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    for (m, n, k, batch) in [(64, 64, 64, 9), (128, 128, 128, 3), (50, 30, 70, 4)]:
+        A = inputs.integers(3, batch * m, k, -128, 127, np.int8, "C").reshape(batch, m, k)
+        B = inputs.integers(4, batch * k, n, -128, 127, np.int8, "C").reshape(batch, k, n)
+        C = inputs.integers(5, batch * m, n, -1000, 1000, np.int32, "C").reshape(batch, m, n)
+        dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), torch.from_numpy(C).cuda()
+        dD = torch.zeros_like(dC)
+        cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, 1, 1, 0, 1, dtype="i8")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        for i in range(batch):
+            want = oracle.srgemm("plus", "multiplies", A[i], B[i], C[i], 1, 1, 0)
+            assert_same_bits(got[i], want, f"batch product {i} of {m}x{n}x{k}")

@@ -153,6 +153,29 @@ def test_binary16_shortest_paths_on_small_integers(oracle):
     assert np.array_equal(D.astype(np.float64), want)
 
 
+def test_int8_operands_are_widened_first(oracle):
+    """int8 A and B with int32 C, D, scalars and accumulator: every pair against numpy on int64 (no value here
+    leaves the int32 range), both loops, all layouts."""
+    rng = np.random.default_rng(3)
+    m, n, k = 19, 23, 41
+    for la, lb, lc in itertools.product("FC", repeat=3):
+        A = np.asarray(rng.integers(-128, 128, (m, k)).astype(np.int8), order=la)
+        B = np.asarray(rng.integers(-128, 128, (k, n)).astype(np.int8), order=lb)
+        C = np.asarray(rng.integers(-10 ** 6, 10 ** 6, (m, n)).astype(np.int32), order=lc)
+        a, b, c = A.astype(np.int64), B.astype(np.int64), C.astype(np.int64)
+        sums = a[:, :, None] + b[None, :, :]
+        wants = {("plus", "multiplies"): (7 * (a @ b) - 3 * c, 7, -3, 0),
+                 ("minimum", "plus"): (np.minimum(sums.min(1) + 5, c + 2), 5, 2, 2 ** 31 - 1),
+                 ("maximum", "plus"): (np.maximum(sums.max(1), c), 0, 0, -2 ** 31),
+                 ("maximum", "minimum"): (np.maximum(np.minimum(np.minimum(a[:, :, None], b[None, :, :]).max(1), 100), np.minimum(c, 50)),
+                                          100, 50, -2 ** 31),
+                 ("bit_xor", "bit_and"): (np.bitwise_xor.reduce(a[:, :, None] & b[None, :, :], axis=1) ^ c, -1, -1, 0)}
+        for (add, mult), (want, alpha, beta, ident) in wants.items():
+            for naive in (False, True):
+                got = oracle.srgemm(add, mult, A, B, C, alpha, beta, ident, naive=naive)
+                assert np.array_equal(got.astype(np.int64), want), (add, mult, la, lb, lc, naive)
+
+
 def test_blocked_equals_naive_on_ragged_and_submatrix(oracle):
     big_a = inputs.uniform(1, 140, 90)
     big_b = inputs.uniform(2, 90, 150)
