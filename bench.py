@@ -31,6 +31,7 @@ sys.path.insert(0, ROOT)
 # MI355X published peaks
 FP32_VECTOR_PEAK = 157.3   # TFLOP/s, FMA counted as 2 flops (also the fp32 matrix-core peak)
 FP64_VECTOR_PEAK = 78.6    # also the fp64 matrix-core peak
+INT8_MATRIX_PEAK = 5000.0  # TOP/s, dense int8 on the matrix cores
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel come from profiles/traffic.json, which the profiling
@@ -281,9 +282,13 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         # benchmark matrix (bench/device/harness.h:157-181 counts 2 * N^3 / t the same way)
         n = args.size or 4096
         add, mult, dt = args.add, args.mult, args.dtype
-        npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16}[dt]
+        npd = {"f32": np.float32, "f64": np.float64, "i32": np.int32, "u32": np.uint32, "f16": np.float16, "i8": np.int32}[dt]
         la, lb, lc = ["F" if c == "c" else "C" for c in args.layouts]
-        if dt == "f16" and mult != "multiplies":
+        if dt == "i8":
+            # int8 operands over their whole range, int32 C and D
+            A, B = (inputs.integers(701 + i, n, n, -128, 127, np.int8, o) for i, o in enumerate((la, lb)))
+            C = inputs.integers(703, n, n, -100000, 100000, np.int32, lc)
+        elif dt == "f16" and mult != "multiplies":
             # distances of a few units: sums stay well inside binary16's range and still round
             A, B, C = (inputs.uniform(701 + i, n, n, 0.5, 100.0, npd, o) for i, o in enumerate((la, lb, lc)))
         elif dt in ("f32", "f64", "f16"):
@@ -296,7 +301,7 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         one = cuasr_amd.op_identity(mult, dt, True)
         up = lambda X: (col_major if X.flags.f_contiguous else row_major)(X.view(np.int32) if dt == "u32" else X)
         dA, dB, dC = up(A), up(B), up(C)
-        tdt = {"f32": torch.float32, "f64": torch.float64, "i32": torch.int32, "u32": torch.int32, "f16": torch.float16}[dt]
+        tdt = {"f32": torch.float32, "f64": torch.float64, "i32": torch.int32, "u32": torch.int32, "f16": torch.float16, "i8": torch.int32}[dt]
         dD = torch.empty(n, n, dtype=tdt, device=dev)
         dD = dD.t() if lc == "F" else dD
 
@@ -304,13 +309,14 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
             cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dt, kernel=args.kernel)
 
         desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one)
-        matrix = add == "plus" and mult == "multiplies" and dt in ("f32", "f64")
+        matrix = add == "plus" and mult == "multiplies" and dt in ("f32", "f64", "i8")
         return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=desc, host=(add, mult, A, B, C, one, one, ident),
                     result=lambda: dD.cpu().numpy(),
                     metric=f"{dt} {add}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"{add}-{mult} SRGEMM {dt}, M=N=K={n}, layouts (A, B, C) = {args.layouts} "
                              "(c = column-major, r = row-major), beta = one with a seeded C",
-                    bound="mfma" if matrix else "valu", peak=FP64_VECTOR_PEAK if dt == "f64" else FP32_VECTOR_PEAK,
+                    bound="mfma" if matrix else "valu",
+                    peak=FP64_VECTOR_PEAK if dt == "f64" else INT8_MATRIX_PEAK if (dt == "i8" and matrix) else FP32_VECTOR_PEAK,
                     instr_per_term=None)
 
     raise SystemExit(f"bench.py: unknown workload {w!r}")
@@ -457,7 +463,7 @@ def main():
                              "srgemm", "fwgemm", "apsp_blocked"])
     ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
     ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
-    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32", "f16"], help="workload srgemm")
+    ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32", "f16", "i8"], help="workload srgemm")
     ap.add_argument("--layouts", default="ccc", help="workload srgemm: layouts of A, B, C (c = column-major, r = row-major)")
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")

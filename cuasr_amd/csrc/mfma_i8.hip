@@ -7,11 +7,17 @@
 // supplying 16 consecutive k of one row (column).  Integer sums wrap modulo 2^32 whatever their order, so the
 // result is bit-identical to the k-ascending reference loop.
 //
-// Tile: 256 threads (2 x 2 waves), 128 x 128 x 64; a wave holds 2 x 2 blocks of 32 x 32 (64 accumulator
-// registers).  LDS holds both panels k-contiguous, [x][64 k + 16 bytes of padding] (the padding makes the 16-byte
-// fragment reads of 32 consecutive rows conflict-free), two stages.  Operands are staged through registers, which
+// Tile: 256 threads (2 x 2 waves), 128 x 128 x 128; a wave holds 2 x 2 blocks of 32 x 32 (64 accumulator
+// registers), two workgroups per compute unit.  The instruction is so fast (32 cycles for 65536 operations) that a
+// k-tile is over in a thousand cycles, less than a trip to memory: the loads of tile t + 2 are issued before tile t
+// is worked on and stay in registers for two tiles (two register sets, the tile loop unrolled by two), while LDS
+// holds tiles t and t + 1.  LDS holds both panels k-contiguous, [x][128 k + 16 bytes of padding] (the padding makes
+// the 16-byte fragment reads of 32 consecutive rows conflict-free).  Operands are staged through registers, which
 // is where an operand whose rows (columns) are contiguous in memory gets transposed: a thread loads 16 x at 4
 // consecutive k (four 16-byte loads), turns them with byte permutes into 16 words of 4 k each and writes those.
+// Measured and not kept: a 256 x 256 tile (4 x 4 blocks per wave, 256 accumulator registers, one wave per SIMD),
+// which halves the LDS reads per instruction: 0.75 against 1.02 POP/s at 4096^3 -- one wave per SIMD of compiled
+// code has nothing to hide its own waits behind.
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -20,23 +26,26 @@ namespace mfma_i8 {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 128, BN = 128, BK = 64, THREADS = 256, PITCH = BK + 16;
+constexpr int BM = 128, BN = 128, BK = 128, THREADS = 256, PITCH = BK + 16;
+constexpr int KCH = BK / 16;  // 16-byte chunks along k
 
 struct Smem {
   int8_t a[2][BM][PITCH];
   int8_t b[2][BN][PITCH];
 };
 
-// One operand's share of a k-tile (128 x, 64 k) on its way from memory to LDS.
-//   KC (k contiguous in memory): 512 chunks of 16 k of one x, two per thread, written as they are.
-//   otherwise (x contiguous):    128 units of 16 x by 4 k, one per thread of the half of the workgroup
-//                                `first_thread` names; four 16-byte loads, transposed in registers.
+// One operand's share of a k-tile (X x, BK k) on its way from memory to LDS.
+//   KC (k contiguous in memory): chunks of 16 k of one x, written as they are.
+//   otherwise (x contiguous):    units of 16 x by 4 k; four 16-byte loads, transposed in registers.
 // GUARD: bytes beyond the extents read as zero (a zero factor adds nothing to a sum of products).
-template <bool KC, bool GUARD> struct Stager {
-  v4i r[KC ? 2 : 4];
+template <int X, bool KC, bool GUARD> struct Stager {
+  static constexpr int CHUNKS = KCH * X / THREADS;                 // KC: 16-byte chunks per thread
+  static constexpr int NUNITS = (X / 16) * (BK / 4);                // otherwise: units in the tile ...
+  static constexpr int UNITS = (NUNITS + THREADS - 1) / THREADS;    // ... and per thread
+  v4i r[KC ? CHUNKS : 4 * UNITS];
 
-  static __device__ __forceinline__ v4i fetch(const int8_t *src, long long step, int first, int count, int limit, bool live) {
-    // 16 bytes from src, src + step, ...; byte e is element first + e of a run that ends at `limit`
+  static __device__ __forceinline__ v4i fetch(const int8_t *src, int first, int limit, bool live) {
+    // 16 consecutive bytes; byte e is element first + e of a run that ends at `limit`
     if constexpr (!GUARD) {
       return *reinterpret_cast<const v4i *>(src);
     } else {
@@ -44,7 +53,7 @@ template <bool KC, bool GUARD> struct Stager {
       if (live) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          const int byte = (first + e < limit) ? (int)(unsigned char)src[step * e] : 0;
+          const int byte = (first + e < limit) ? (int)(unsigned char)src[e] : 0;
           v[e / 4] |= byte << (8 * (e % 4));
         }
       }
@@ -52,45 +61,51 @@ template <bool KC, bool GUARD> struct Stager {
     }
   }
 
-  __device__ __forceinline__ void load(const int8_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn, int first_thread) {
+  __device__ __forceinline__ void load(const int8_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn) {
     if constexpr (KC) {
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const int c = threadIdx.x + q * THREADS, k = (c % 4) * 16, x = c / 4;
-        r[q] = fetch(base + (long long)(x0 + x) * sx + (k0 + k), 1, k0 + k, 16, kn, x0 + x < xn);
+      for (int q = 0; q < CHUNKS; ++q) {
+        const int c = threadIdx.x + q * THREADS, k = (c % KCH) * 16, x = c / KCH;
+        r[q] = fetch(base + (long long)(x0 + x) * sx + (k0 + k), k0 + k, kn, x0 + x < xn);
       }
     } else {
-      const int u = (int)threadIdx.x - first_thread;
-      if (u >= 0 && u < 128) {
-        const int x = (u % 8) * 16, k = (u / 8) * 4;
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk)
-          r[kk] = fetch(base + (x0 + x) + (long long)(k0 + k + kk) * sk, 1, x0 + x, 16, xn, k0 + k + kk < kn);
+      for (int q = 0; q < UNITS; ++q) {
+        const int u = threadIdx.x + q * THREADS;
+        if (u < NUNITS) {
+          const int x = (u % (X / 16)) * 16, k = (u / (X / 16)) * 4;
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk)
+            r[4 * q + kk] = fetch(base + (x0 + x) + (long long)(k0 + k + kk) * sk, x0 + x, xn, k0 + k + kk < kn);
+        }
       }
     }
   }
 
-  __device__ __forceinline__ void store(int8_t (*panel)[PITCH], int first_thread) const {
+  __device__ __forceinline__ void store(int8_t (*panel)[PITCH]) const {
     if constexpr (KC) {
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        const int c = threadIdx.x + q * THREADS, k = (c % 4) * 16, x = c / 4;
+      for (int q = 0; q < CHUNKS; ++q) {
+        const int c = threadIdx.x + q * THREADS, k = (c % KCH) * 16, x = c / KCH;
         *reinterpret_cast<v4i *>(&panel[x][k]) = r[q];
       }
     } else {
-      const int u = (int)threadIdx.x - first_thread;
-      if (u >= 0 && u < 128) {
-        const int x = (u % 8) * 16, k = (u / 8) * 4;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          // words d of the four loads hold x = 4d .. 4d+3 at k, k+1, k+2, k+3: a 4 x 4 byte transpose
-          const unsigned a = r[0][d], b = r[1][d], c = r[2][d], e = r[3][d];
-          const unsigned ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602);
-          const unsigned ce_lo = __builtin_amdgcn_perm(e, c, 0x05010400), ce_hi = __builtin_amdgcn_perm(e, c, 0x07030602);
-          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 0][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x05040100);
-          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 1][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x07060302);
-          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 2][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x05040100);
-          *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 3][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x07060302);
+      for (int q = 0; q < UNITS; ++q) {
+        const int u = threadIdx.x + q * THREADS;
+        if (u < NUNITS) {
+          const int x = (u % (X / 16)) * 16, k = (u / (X / 16)) * 4;
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            // words d of the four loads hold x = 4d .. 4d+3 at k, k+1, k+2, k+3: a 4 x 4 byte transpose
+            const unsigned a = r[4 * q + 0][d], b = r[4 * q + 1][d], c = r[4 * q + 2][d], e = r[4 * q + 3][d];
+            const unsigned ab_lo = __builtin_amdgcn_perm(b, a, 0x05010400), ab_hi = __builtin_amdgcn_perm(b, a, 0x07030602);
+            const unsigned ce_lo = __builtin_amdgcn_perm(e, c, 0x05010400), ce_hi = __builtin_amdgcn_perm(e, c, 0x07030602);
+            *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 0][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x05040100);
+            *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 1][k]) = __builtin_amdgcn_perm(ce_lo, ab_lo, 0x07060302);
+            *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 2][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x05040100);
+            *reinterpret_cast<unsigned *>(&panel[x + 4 * d + 3][k]) = __builtin_amdgcn_perm(ce_hi, ab_hi, 0x07060302);
+          }
         }
       }
     }
@@ -98,7 +113,7 @@ template <bool KC, bool GUARD> struct Stager {
 };
 
 template <bool A_KC, bool B_KC, bool GUARD>
-__global__ __launch_bounds__(THREADS) void mfma_i8_kernel(Problem p) {
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void mfma_i8_kernel(Problem p) {
   __shared__ __attribute__((aligned(16))) Smem sm;
   select_batch<int32_t, int8_t>(p);
   const int tiles_n = (p.n + BN - 1) / BN;
@@ -120,23 +135,26 @@ __global__ __launch_bounds__(THREADS) void mfma_i8_kernel(Problem p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[bi][bj][e] = 0;
 
-  // when both operands need the transpose, the two halves of the workgroup take one each
-  constexpr int A_FIRST = 0, B_FIRST = A_KC ? 0 : 128;
-  Stager<A_KC, GUARD> sa;
-  Stager<B_KC, GUARD> sb;
+  Stager<BM, A_KC, GUARD> sa[2];
+  Stager<BN, B_KC, GUARD> sb[2];
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   if (tiles_k > 0) {
-    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke, A_FIRST);
-    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke, B_FIRST);
-    sa.store(sm.a[0], A_FIRST);
-    sb.store(sm.b[0], B_FIRST);
+    sa[1].load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke);
+    sb[1].load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke);
+    if (tiles_k > 1) {
+      sa[0].load(A, p.sa_m, p.sa_k, m0, kb + BK, p.m, ke);
+      sb[0].load(B, p.sb_n, p.sb_k, n0, kb + BK, p.n, ke);
+    }
+    sa[1].store(sm.a[0]);
+    sb[1].store(sm.b[0]);
   }
   __syncthreads();
-  for (int t = 0; t < tiles_k; ++t) {
+  // one k-tile: `la`, `lb` take the loads of tile t + 2; `ha`, `hb` hold tile t + 1, which goes to LDS afterwards
+  auto tile = [&](int t, auto &la, auto &lb, const auto &ha, const auto &hb) {
     const int s = t & 1, k0 = kb + t * BK;
-    if (t + 1 < tiles_k) {
-      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke, A_FIRST);
-      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke, B_FIRST);
+    if (t + 2 < tiles_k) {
+      la.load(A, p.sa_m, p.sa_k, m0, k0 + 2 * BK, p.m, ke);
+      lb.load(B, p.sb_n, p.sb_k, n0, k0 + 2 * BK, p.n, ke);
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 32; ++ks) {
@@ -151,10 +169,14 @@ __global__ __launch_bounds__(THREADS) void mfma_i8_kernel(Problem p) {
         for (int bj = 0; bj < 2; ++bj) acc[bi][bj] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
     }
     if (t + 1 < tiles_k) {
-      sa.store(sm.a[s ^ 1], A_FIRST);
-      sb.store(sm.b[s ^ 1], B_FIRST);
+      ha.store(sm.a[s ^ 1]);
+      hb.store(sm.b[s ^ 1]);
     }
     __syncthreads();
+  };
+  for (int t = 0; t < tiles_k; t += 2) {
+    tile(t, sa[1], sb[1], sa[0], sb[0]);
+    if (t + 1 < tiles_k) tile(t + 1, sa[0], sb[0], sa[1], sb[1]);
   }
 
   // ---- epilogue.  Register e of lane l in block (bi, bj): row 8*(e/4) + 4*(l/32) + e%4, column l%32.

@@ -82,6 +82,14 @@ def test_1024(oracle, lib):
         check(oracle, "plus", "multiplies", 1024, 1024, 1024, layouts, "auto", alpha=1, beta=1)
 
 
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_many_tiles(oracle, lib, layouts):
+    """Hundreds of tiles and several k-tiles (the prefetch runs two tiles ahead): whole tiles of aligned operands,
+    and ragged edges with an odd k (the guarded form)."""
+    check(oracle, "plus", "multiplies", 3584, 3840, 640, layouts, "auto", alpha=1, beta=1)
+    check(oracle, "plus", "multiplies", 3587, 3830, 333, layouts, "auto", alpha=-3, beta=2)
+
+
 def test_wraparound(oracle, lib):
     """All operands at -128 and a long k: the int32 sums wrap, the same way on both sides."""
     import torch
