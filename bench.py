@@ -433,6 +433,19 @@ def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
     del wl
     torch.cuda.empty_cache()
 
+    # int8 operands with int32 accumulation (the element types of the reference's dp4a cores,
+    # default_srmma_core_simt.h:747-757), plus-times on the matrix cores, 4096^3, A row-major and B column-major
+    # (both k-contiguous); the first 256 rows against the oracle
+    wl = build_workload(ns(workload="srgemm", add="plus", mult="multiplies", dtype="i8", layouts="rcr", size=4096), np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    want = oracle.srgemm(add, mult, rows_of(A, 256), B, rows_of(C, 256), int(alpha), int(beta), int(ident))
+    got = wl["result"]()[:256]
+    out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(np.ascontiguousarray(got).tobytes() == np.ascontiguousarray(want).tobytes()),
+                     checked="first 256 rows of the output"))
+    del wl
+    torch.cuda.empty_cache()
+
     # All-pairs shortest paths with predecessors on top of SRGEMM (README.md:338-342 of the reference,
     # cpu_fwgemm_naive): a whole job at n = 4096 by blocked Floyd-Warshall, counted as 2 n^3 operations, and the
     # same kind of graph at n = 1024 against the oracle's blocked iteration, dist and parent bit for bit
