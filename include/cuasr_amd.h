@@ -130,7 +130,7 @@ typedef union cuasr_amd_scalar {
 typedef struct cuasr_amd_srgemm_desc {
   int32_t add_op;          /* cuasr_amd_op */
   int32_t mult_op;         /* cuasr_amd_op */
-  int32_t dtype;           /* cuasr_amd_dtype: A, B, C, D and accumulator */
+  int32_t dtype;           /* cuasr_amd_dtype: A, B, C, D and accumulator (CUASR_AMD_I8: int8 A and B, int32 the rest) */
   int32_t layout_a;        /* cuasr_amd_layout */
   int32_t layout_b;
   int32_t layout_c;
@@ -186,7 +186,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
                              int64_t stride_b, int64_t stride_c, int64_t stride_d, void *stream);
 
 /* Bytes of device workspace the split-K call needs:
- * sizeof(element) * m * n * split_k_slices. */
+ * sizeof(element of C) * m * n * split_k_slices. */
 size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc);
 
 /* Two launches on `stream`: partial products of `split_k_slices` K-slices into

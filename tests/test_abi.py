@@ -72,6 +72,33 @@ def test_can_implement(lib):
     assert ok(d) == 4
 
 
+def test_half_and_int8_element_types(lib):
+    ok = lambda d: lib.cuasr_amd_srgemm_can_implement(ctypes.byref(d))
+    sel = lambda d: lib.cuasr_amd_selected_kernel(ctypes.byref(d))
+    # binary16: two-byte alignment everywhere, no bitwise operators, the packed tile for the tropical pairs and plus-times
+    assert ok(desc(dtype="f16", ptr=0x10002)) == 0
+    assert ok(desc(dtype="f16", ptr=0x10001)) == 1
+    assert ok(desc(dtype="f16", add="bit_xor", mult="bit_and")) == 5
+    assert ok(desc(dtype="f16", kernel="mfma")) == 5 and ok(desc(dtype="f16", kernel="direct")) == 5
+    assert sel(desc(dtype="f16")) == b"valu" and sel(desc(dtype="f16", m=63, n=1, k=5)) == b"valu"
+    assert sel(desc(dtype="f16", add="plus", mult="multiplies")) == b"valu"
+    assert sel(desc(dtype="f16", add="minimum", mult="multiplies")) == b"naive"
+    assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "f16") == 2 * 100 * 7 * 3
+    # int8 operands, int32 everything else: A and B at any byte, C and D at four; every integer pair is defined
+    d = desc(dtype="i8", add="plus", mult="multiplies")
+    assert ok(d) == 0 and sel(d) == b"mfma"
+    d.A, d.B = 0x10001, 0x10003
+    assert ok(d) == 0
+    d.D = 0x10002
+    assert ok(d) == 1
+    assert sel(desc(dtype="i8")) == b"naive" and ok(desc(dtype="i8", add="bit_xor", mult="bit_and")) == 0
+    assert ok(desc(dtype="i8", kernel="valu")) == 5
+    assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "i8") == 4 * 100 * 7 * 3
+    d = desc()
+    d.dtype = 6
+    assert ok(d) == 2
+
+
 def test_kernel_selection(lib):
     sel = lambda d: lib.cuasr_amd_selected_kernel(ctypes.byref(d))
     big = dict(m=4096, n=4096, k=4096)
