@@ -17,6 +17,8 @@
 // B panel [k][256], both with the output direction contiguous, two stages.  Per k a thread reads one
 // 16-byte vector of A (its 8 rows; the instruction's half-word selects broadcast one of them) and two
 // of B, and issues 64 packed adds + 32 three-input packed minima for 128 terms.
+// Outputs too small to give the 256 compute units two such tiles each take smaller ones of the same kernel
+// (64 x 128 and 32 x 128: 4 or 2 rows and one column group per thread, guarded form only).
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -25,11 +27,12 @@ namespace half_tile {
 typedef half_t h2 __attribute__((ext_vector_type(2)));
 typedef half_t h8 __attribute__((ext_vector_type(8)));
 
-constexpr int BM = 128, BN = 256, BK = 32, THREADS = 256;
+constexpr int BK = 32, THREADS = 256;
 
-struct Smem {
-  half_t a[2][BK][BM];
-  half_t b[2][BK][BN];
+// TR rows per thread (tile height 16 TR), NG groups of 8 columns per thread (tile width 128 NG)
+template <int TR, int NG> struct Smem {
+  half_t a[2][BK][16 * TR];
+  half_t b[2][BK][128 * NG];
 };
 
 template <int OP> __device__ __forceinline__ h2 pk(h2 l, h2 r) {
@@ -53,12 +56,13 @@ template <int ADD, int MUL> __device__ __forceinline__ void one_term(h2 &acc, h2
 
 __device__ __forceinline__ h2 both(half_t v) { return h2{v, v}; }
 __device__ __forceinline__ h2 pair_of(const h8 &v, int j) { return h2{v[2 * j], v[2 * j + 1]}; }
+template <int N> struct frag_of { typedef half_t type __attribute__((ext_vector_type(N))); };
 
 // One operand's share of a k-tile on its way from memory to LDS.  The panel is X wide (X = BM for A, BN
 // for B); a chunk is 8 elements: of one k and 8 consecutive x when x is the contiguous direction in
 // memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
 template <int X, bool KC, bool GUARD> struct Stager {
-  static constexpr int CHUNKS = X * BK / 8 / THREADS;
+  static constexpr int TOTAL = X * BK / 8, CHUNKS = (TOTAL + THREADS - 1) / THREADS;  // (a small panel leaves threads idle)
   h8 r[CHUNKS];
 
   // chunk c -> (x, k) of its first element, tile-relative
@@ -68,20 +72,28 @@ template <int X, bool KC, bool GUARD> struct Stager {
   }
 
   // base: the operand's element (x = 0, k = 0); sx, sk: element strides; x0, k0: the tile's origin;
-  // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored)
-  __device__ __forceinline__ void load(const half_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn) {
+  // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored);
+  // vec (guarded form): chunks of this operand lie at 16-byte boundaries, so one that is wholly inside the
+  // extents is read as a vector all the same
+  __device__ __forceinline__ void load(const half_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn, bool vec) {
 #pragma unroll
     for (int q = 0; q < CHUNKS; ++q) {
+      if (TOTAL % THREADS && (int)threadIdx.x + q * THREADS >= TOTAL) break;
       int x, k;
       where(threadIdx.x + q * THREADS, x, k);
       const half_t *src = base + (long long)(x0 + x) * sx + (long long)(k0 + k) * sk;
       if constexpr (!GUARD) {
         r[q] = *reinterpret_cast<const h8 *>(src);
       } else {
+        const bool whole = KC ? (x0 + x < xn && k0 + k + 8 <= kn) : (x0 + x + 8 <= xn && k0 + k < kn);
+        if (vec && whole) {
+          r[q] = *reinterpret_cast<const h8 *>(src);
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int xe = x0 + x + (KC ? 0 : e), ke = k0 + k + (KC ? e : 0);
-          r[q][e] = (xe < xn && ke < kn) ? src[(KC ? sk : sx) * e] : half_t(0);
+          for (int e = 0; e < 8; ++e) {
+            const int xe = x0 + x + (KC ? 0 : e), ke = k0 + k + (KC ? e : 0);
+            r[q][e] = (xe < xn && ke < kn) ? src[(KC ? sk : sx) * e] : half_t(0);
+          }
         }
       }
     }
@@ -90,6 +102,7 @@ template <int X, bool KC, bool GUARD> struct Stager {
   __device__ __forceinline__ void store(half_t (*panel)[X]) const {
 #pragma unroll
     for (int q = 0; q < CHUNKS; ++q) {
+      if (TOTAL % THREADS && (int)threadIdx.x + q * THREADS >= TOTAL) break;
       int x, k;
       where(threadIdx.x + q * THREADS, x, k);
       if constexpr (KC) {
@@ -102,9 +115,11 @@ template <int X, bool KC, bool GUARD> struct Stager {
   }
 };
 
-template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD>
+template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD, int TR = 8, int NG = 2>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void half_tile_kernel(Problem p) {
-  __shared__ __attribute__((aligned(16))) Smem sm;
+  constexpr int BM = 16 * TR, BN = 128 * NG;
+  typedef typename frag_of<TR>::type rows_t;
+  __shared__ __attribute__((aligned(16))) Smem<TR, NG> sm;
   select_batch<half_t>(p);
   const int tiles_n = (p.n + BN - 1) / BN;
   const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
@@ -117,18 +132,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const half_t *A = reinterpret_cast<const half_t *>(p.A), *B = reinterpret_cast<const half_t *>(p.B);
   const half_t ident = scalar_as<half_t>(p.add_identity);
 
-  h2 acc[8][8];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
+  h2 acc[TR][4 * NG];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < TR; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[i][j] = both(ident);
+    for (int j = 0; j < 4 * NG; ++j) acc[i][j] = both(ident);
 
   Stager<BM, A_KC, GUARD> sa;
   Stager<BN, B_KC, GUARD> sb;
+  // (tile origins are multiples of 8 in x; the k origin is one if the slice's is)
+  const bool vec_a = reinterpret_cast<uintptr_t>(A) % 16 == 0 && (A_KC ? p.sa_m : p.sa_k) % 8 == 0 && kb % 8 == 0;
+  const bool vec_b = reinterpret_cast<uintptr_t>(B) % 16 == 0 && (B_KC ? p.sb_n : p.sb_k) % 8 == 0 && kb % 8 == 0;
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   if (tiles_k > 0) {
-    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke);
-    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke);
+    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke, vec_a);
+    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke, vec_b);
     sa.store(sm.a[0]);
     sb.store(sm.b[0]);
   }
@@ -136,36 +154,41 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   for (int t = 0; t < tiles_k; ++t) {
     const int s = t & 1, k0 = kb + t * BK;
     if (t + 1 < tiles_k) {
-      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke);
-      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke);
+      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke, vec_a);
+      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke, vec_b);
     }
     const half_t(*pa)[BM] = sm.a[s];
     const half_t(*pb)[BN] = sm.b[s];
     if (!GUARD || ke - k0 >= BK) {
 #pragma unroll 2
       for (int kk = 0; kk < BK; kk += 2) {
-        const h8 a0 = *reinterpret_cast<const h8 *>(&pa[kk][ty * 8]), a1 = *reinterpret_cast<const h8 *>(&pa[kk + 1][ty * 8]);
-        const h8 b00 = *reinterpret_cast<const h8 *>(&pb[kk][tx * 8]), b01 = *reinterpret_cast<const h8 *>(&pb[kk][128 + tx * 8]);
-        const h8 b10 = *reinterpret_cast<const h8 *>(&pb[kk + 1][tx * 8]), b11 = *reinterpret_cast<const h8 *>(&pb[kk + 1][128 + tx * 8]);
+        const rows_t a0 = *reinterpret_cast<const rows_t *>(&pa[kk][ty * TR]), a1 = *reinterpret_cast<const rows_t *>(&pa[kk + 1][ty * TR]);
+        h8 b0[NG], b1[NG];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int g = 0; g < NG; ++g) {
+          b0[g] = *reinterpret_cast<const h8 *>(&pb[kk][g * 128 + tx * 8]);
+          b1[g] = *reinterpret_cast<const h8 *>(&pb[kk + 1][g * 128 + tx * 8]);
+        }
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            two_terms<ADD, MUL>(acc[i][j], both(a0[i]), pair_of(b00, j), both(a1[i]), pair_of(b10, j));
-            two_terms<ADD, MUL>(acc[i][4 + j], both(a0[i]), pair_of(b01, j), both(a1[i]), pair_of(b11, j));
-          }
+        for (int i = 0; i < TR; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int g = 0; g < NG; ++g)
+              two_terms<ADD, MUL>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j), both(a1[i]), pair_of(b1[g], j));
       }
     } else {
       for (int kk = 0; kk < ke - k0; ++kk) {  // the ragged last k-tile
-        const h8 a0 = *reinterpret_cast<const h8 *>(&pa[kk][ty * 8]);
-        const h8 b00 = *reinterpret_cast<const h8 *>(&pb[kk][tx * 8]), b01 = *reinterpret_cast<const h8 *>(&pb[kk][128 + tx * 8]);
+        const rows_t a0 = *reinterpret_cast<const rows_t *>(&pa[kk][ty * TR]);
+        h8 b0[NG];
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int g = 0; g < NG; ++g) b0[g] = *reinterpret_cast<const h8 *>(&pb[kk][g * 128 + tx * 8]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            one_term<ADD, MUL>(acc[i][j], both(a0[i]), pair_of(b00, j));
-            one_term<ADD, MUL>(acc[i][4 + j], both(a0[i]), pair_of(b01, j));
-          }
+        for (int i = 0; i < TR; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) one_term<ADD, MUL>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j));
       }
     }
     if (t + 1 < tiles_k) {
@@ -181,10 +204,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const half_t *C = reinterpret_cast<const half_t *>(p.C);
   half_t *D = reinterpret_cast<half_t *>(p.D);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int row = m0 + ty * 8 + i;
+  for (int i = 0; i < TR; ++i) {
+    const int row = m0 + ty * TR + i;
 #pragma unroll
-    for (int g = 0; g < 2; ++g) {
+    for (int g = 0; g < NG; ++g) {
       const int col = n0 + g * 128 + tx * 8;
       h8 v;
 #pragma unroll
@@ -234,7 +257,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 // whole tiles, whole 16-byte vectors at 16-byte boundaries everywhere: the unguarded kernel
 static bool exact(const Problem &p, bool a_kc, bool b_kc) {
   auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-  if (p.m % BM || p.n % BN || p.k % BK || p.k == 0) return false;
+  if (p.m % 128 || p.n % 256 || p.k % BK || p.k == 0) return false;
   if (p.workspace && (p.k_per_slice % BK || !al16(p.workspace))) return false;
   if ((a_kc ? p.sa_m : p.sa_k) % 8 || (b_kc ? p.sb_n : p.sb_k) % 8) return false;
   if (!al16(p.A) || !al16(p.B) || !al16(p.D) || p.ldd % 8) return false;
@@ -243,25 +266,38 @@ static bool exact(const Problem &p, bool a_kc, bool b_kc) {
   return true;
 }
 
+template <int ADD, int MUL, bool GUARD, int TR, int NG> static hipError_t launch_tile(const Problem &p, bool a_kc, bool b_kc, hipStream_t s) {
+  const long long tiles = (long long)((p.m + 16 * TR - 1) / (16 * TR)) * ((p.n + 128 * NG - 1) / (128 * NG));
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(THREADS);
+#define CUASR_HALF_LAUNCH(AK, BK_) launch_kernel((half_tile_kernel<ADD, MUL, AK, BK_, GUARD, TR, NG>), grid, block, 0, s, p)
+  if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true); else CUASR_HALF_LAUNCH(true, false); }
+  else { if (b_kc) CUASR_HALF_LAUNCH(false, true); else CUASR_HALF_LAUNCH(false, false); }
+#undef CUASR_HALF_LAUNCH
+  return take_launch_status();
+}
+
 template <int ADD, int MUL> static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   // one direction of each operand is contiguous (the C ABI produces nothing else)
   if ((p.sa_m != 1 && p.sa_k != 1) || (p.sb_n != 1 && p.sb_k != 1)) return hipErrorNotSupported;
   const bool a_kc = p.sa_m != 1, b_kc = p.sb_n != 1;
-  const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
-  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(THREADS);
-  const bool fast = exact(p, a_kc, b_kc);
-#define CUASR_HALF_LAUNCH(AK, BK_, G) launch_kernel((half_tile_kernel<ADD, MUL, AK, BK_, G>), grid, block, 0, s, p)
-  if (fast) {
-    if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true, false); else CUASR_HALF_LAUNCH(true, false, false); }
-    else { if (b_kc) CUASR_HALF_LAUNCH(false, true, false); else CUASR_HALF_LAUNCH(false, false, false); }
-  } else {
-    if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true, true); else CUASR_HALF_LAUNCH(true, false, true); }
-    else { if (b_kc) CUASR_HALF_LAUNCH(false, true, true); else CUASR_HALF_LAUNCH(false, false, true); }
+  // Which tile: a compute unit works its workgroups off at nearly the same rate whether one or several are
+  // resident (a packed instruction occupies the vector ALU for four cycles, so even one wave per SIMD keeps it
+  // 89 % busy), and the smaller tiles do less work per LDS read and per barrier (about 0.7 and 0.55 of the full
+  // tile's rate, measured at 2048^3 and 1024^3).  So the time is about (workgroups per compute unit, rounded
+  // up) x tile area / rate; take the smallest.
+  auto cost = [&](int bm, int bn, long long rate_percent) {
+    const long long groups = (long long)((p.m + bm - 1) / bm) * ((p.n + bn - 1) / bn) * (p.workspace ? p.slices : 1) * p.batch;
+    return (groups + 255) / 256 * bm * bn * 100 / rate_percent;
+  };
+  const long long full = cost(128, 256, 100), mid = cost(64, 128, 70), small = cost(32, 128, 55);
+  if (full <= mid && full <= small) {
+    if (exact(p, a_kc, b_kc)) return launch_tile<ADD, MUL, false, 8, 2>(p, a_kc, b_kc, s);
+    return launch_tile<ADD, MUL, true, 8, 2>(p, a_kc, b_kc, s);
   }
-#undef CUASR_HALF_LAUNCH
-  return take_launch_status();
+  if (mid <= small) return launch_tile<ADD, MUL, true, 4, 1>(p, a_kc, b_kc, s);
+  return launch_tile<ADD, MUL, true, 2, 1>(p, a_kc, b_kc, s);
 }
 
 }  // namespace half_tile

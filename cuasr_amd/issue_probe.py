@@ -13,6 +13,7 @@ groups of add, add, min3 = 128 terms per lane) or a variation of it, run by 256-
     mix + N LDS reads (4 / 8 / 16 bytes)  what fetching the fragments costs (results not consumed)
     mix + N waits / nops / scalar adds    what an instruction that does no arithmetic costs
     packed fp16 add / min / minimum3 / mix the same for two fp16 terms per instruction
+    SDWA byte add / min3_i32 / mix         int8 operands widened by the add's own byte selects
     fp64 add / max / mix (+ the same)     the same questions for 8-byte elements
 Times are HIP events around the second of two launches; the clock is read inside the kernel
 (shader cycle counter against the 100 MHz wall clock), so cycle figures are per measured clock.
@@ -57,6 +58,21 @@ def mix_f16():
             groups.append([f"v_pk_add_f16 v{t0}, v{A0[i]}, v{B0[j]} op_sel_hi:[0,1]",
                            f"v_pk_add_f16 v{t1}, v{A0[i]}, v{B1[j]} op_sel:[1,0] op_sel_hi:[1,1]",
                            f"v_pk_minimum3_f16 v{acc}, v{acc}, v{t0}, v{t1}"])
+    return groups
+
+
+def mix_i8():
+    """min-plus on int8 operands with int32 accumulators: a register holds 4 k of one row (column); the add picks
+    its bytes and widens them"""
+    groups, t = [], 0
+    for i in range(8):
+        for j in range(8):
+            t0, t1 = T[t % 8], T[(t + 1) % 8]
+            t += 2
+            acc = ACC[i * 8 + j]
+            groups.append([f"v_add_u32_sdwa v{t0}, sext(v{A0[i]}), sext(v{B0[j]}) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0 src1_sel:BYTE_0",
+                           f"v_add_u32_sdwa v{t1}, sext(v{A0[i]}), sext(v{B0[j]}) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:BYTE_1",
+                           f"v_min3_i32 v{acc}, v{acc}, v{t0}, v{t1}"])
     return groups
 
 
@@ -111,6 +127,10 @@ def kernels():
     k["mix_f16"] = (flat(mix_f16()), 192, 256, "f32")
     for n in (6, 12):
         k[f"mix_f16_lds{n}_b128"] = (sprinkle(mix_f16(), n, lds_read(128)), 192, 256, "f32")
+    # int8 operands, four to a register, widened by the add itself (SDWA byte selects with sign extension)
+    k["add_u32_sdwa_bytes"] = (only("v_add_u32_sdwa v{t}, sext(v{b}), sext(v{a}) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:BYTE_2"), 192, 0, "f32")
+    k["min3_i32"] = (only("v_min3_i32 v{acc}, v{acc}, v{b}, v{a}"), 192, 0, "f32")
+    k["mix_i8_sdwa"] = (flat(mix_i8()), 192, 128, "f32")
     k["mix"] = (flat(mix()), 192, 128, "f32")
     k["mix_sgpr_b"] = (flat(mix(True)), 192, 128, "f32")
     for n in (4, 8, 16):

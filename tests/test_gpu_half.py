@@ -66,6 +66,17 @@ def test_packed_tile(oracle, lib, sr, layouts):
             check(oracle, *sr, *shape, layouts, "valu", beta_one)
 
 
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_every_tile_size(oracle, lib, layouts):
+    """The kernel comes in three tile sizes, picked by how many workgroups the output gives the chip: the full
+    tile unguarded (whole tiles of aligned operands) and guarded, the 64 x 128 tile, the 32 x 128 tile."""
+    check(oracle, "minimum", "plus", 4096, 4096, 64, layouts, "valu")              # 512 full tiles, unguarded
+    check(oracle, "maximum", "minimum", 4000, 4100, 70, layouts, "valu", False)    # full tiles, ragged: guarded
+    check(oracle, "minimum", "plus", 2048, 2048, 96, layouts, "valu")              # 64 x 128 tiles
+    check(oracle, "plus", "multiplies", 1000, 2000, 50, layouts, "valu")           # 64 x 128 tiles, ragged
+    check(oracle, "maximum", "plus", 1024, 1024, 64, layouts, "valu")              # 32 x 128 tiles
+
+
 def test_selected_family(lib):
     import cuasr_amd
     dA = to_device(np.zeros((128, 64), np.float16))
