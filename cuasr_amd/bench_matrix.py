@@ -10,6 +10,13 @@ shapes are the library's business here, so the matrix is semiring x type x layou
 
 Layouts name A and B as the reference does (n = column-major, t = row-major); C and D are
 column-major.  Prints a table of TOPS (2 ops per term) and, with --json, one JSON object per case.
+
+    python -m cuasr_amd.bench_matrix --tune [...]
+
+times every case on every kernel family that accepts it as well (the reference's generator sweeps
+tile shapes per semiring for this purpose, test/device/simt_sm50.py:193-367) and lists the cases
+where the library's own choice (kernel = auto) is more than 3 % slower than the best forced
+family: the table the selection rules in csrc/abi.hip are checked against.
 """
 import argparse
 import ctypes
@@ -27,6 +34,7 @@ def main():
     ap.add_argument("--layouts", default="nn,nt,tn,tt")
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--json", default=None)
+    ap.add_argument("--tune", action="store_true", help="also time every forced kernel family; list where auto loses")
     args = ap.parse_args()
 
     import numpy as np
@@ -40,6 +48,7 @@ def main():
     sizes = [int(x) for x in args.sizes.split(",")]
     layouts = args.layouts.split(",")
     sink = open(args.json, "w") if args.json else None
+    losses = []
     # the clock takes ~100 ms of load to ramp up: keep the chip busy for a while before the first case
     warm = torch.rand(4096, 4096, device="cuda")
     t_end = torch.cuda.Event(enable_timing=True)
@@ -74,33 +83,69 @@ def main():
                     A = A0.t() if lay[0] == "n" else A0
                     B = B0.t() if lay[1] == "n" else B0
                     C, D = C0.t(), D0.t()
-                    # the descriptor is built once: at the small sizes a launch is shorter than building it
-                    desc = cuasr_amd.make_desc(add, mult, dt, A, B, C, D, one, one, ident, one, 1, args.kernel)
-                    ref, launch = ctypes.byref(desc), cuasr_amd.load().cuasr_amd_srgemm
-                    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+                    def time_family(kernel):
+                        # the descriptor is built once: at the small sizes a launch is shorter than building it
+                        desc = cuasr_amd.make_desc(add, mult, dt, A, B, C, D, one, one, ident, one, 1, kernel)
+                        ref, lib = ctypes.byref(desc), cuasr_amd.load()
+                        if lib.cuasr_amd_srgemm_can_implement(ref) != 0:
+                            return None, None
+                        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
-                    def run():
-                        if launch(ref, stream) != 0:
-                            raise RuntimeError(f"cuasr_amd_srgemm failed for {add}-{mult} {dt} {n} {lay}")
-                    for _ in range(max(3, reps // 4)):
-                        run()
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    for _ in range(reps):
-                        run()
-                    e1.record()
-                    torch.cuda.synchronize()
-                    ms = e0.elapsed_time(e1) / reps
-                    tops = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+                        def run():
+                            if lib.cuasr_amd_srgemm(ref, stream) != 0:
+                                raise RuntimeError(f"cuasr_amd_srgemm failed for {add}-{mult} {dt} {n} {lay} {kernel}")
+                        # the clock follows the kernel that ran last: give it this kernel for 25 ms before timing
+                        w0, w1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        w0.record()
+                        while True:
+                            for _ in range(max(3, reps // 4)):
+                                run()
+                            w1.record()
+                            torch.cuda.synchronize()
+                            if w0.elapsed_time(w1) > 25.0:
+                                break
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record()
+                        for _ in range(reps):
+                            run()
+                        e1.record()
+                        torch.cuda.synchronize()
+                        ms = e0.elapsed_time(e1) / reps
+                        fam = (lib.cuasr_amd_selected_kernel(desc) or b"?").decode() if kernel == "auto" else kernel
+                        return 2.0 * n ** 3 / (ms * 1e-3) / 1e12, fam
+
+                    tops, fam = time_family(args.kernel)
+                    if tops is None:
+                        raise RuntimeError(f"kernel = {args.kernel} cannot run {add}-{mult} {dt} {n} {lay}")
                     per_layout.append(tops)
+                    record = {"add": add, "mult": mult, "dtype": dt, "n": n, "layout": lay, "ms": round(2.0 * n ** 3 / tops / 1e9, 5),
+                              "tops": round(tops, 2), "kernel_family": fam}
+                    if args.tune:
+                        forced = {}
+                        for k in ("valu", "direct", "streamk", "mfma"):
+                            t, _ = time_family(k)
+                            if t is not None:
+                                forced[k] = round(t, 2)
+                        record["forced"] = forced
+                        # the first case after a change of kernel runs on a clock that is still settling:
+                        # the library's own choice is timed once more, after the others, and the better time counts
+                        again, _ = time_family(args.kernel)
+                        tops = max(tops, again)
+                        per_layout[-1] = tops
+                        record["tops"], record["ms"] = round(tops, 2), round(2.0 * n ** 3 / tops / 1e9, 5)
+                        best = max(forced, key=forced.get) if forced else None
+                        if best and forced[best] > 1.03 * tops:
+                            losses.append((forced[best] / tops, f"{add}-{mult} {dt} N={n} {lay}: auto ({fam}) {tops:.1f}, {best} {forced[best]:.1f}"))
                     if sink:
-                        fam = (cuasr_amd.load().cuasr_amd_selected_kernel(desc) or b"?").decode() if args.kernel == "auto" else args.kernel
-                        sink.write(json.dumps({"add": add, "mult": mult, "dtype": dt, "n": n, "layout": lay, "ms": round(ms, 5),
-                                               "tops": round(tops, 2), "kernel_family": fam}) + "\n")
+                        sink.write(json.dumps(record) + "\n")
                 cells.append(" ".join(f"{t:.1f}" for t in per_layout))
             print(f"| {add}-{mult} | " + " | ".join(cells) + " |", flush=True)
     if sink:
         sink.close()
+    if args.tune:
+        print(f"\ncases where kernel = auto is more than 3 % behind the best forced family: {len(losses)}")
+        for _, line in sorted(losses, reverse=True):
+            print("  " + line)
 
 
 if __name__ == "__main__":

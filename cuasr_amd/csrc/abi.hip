@@ -111,6 +111,9 @@ static bool streamk_usable(const cuasr_amd_srgemm_desc *d) {
 // workgroup's share of the k-tiles is long enough to carry a tile's prologue and fold
 static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
   if (batch != 1 || d->split_k_slices != 1 || !streamk_usable(d)) return false;
+  // min-max and max-min spend two instructions per term and their staged tile is within 5 % of the direct one:
+  // the shared tiles' fold costs more than the fuller rounds give (3072^3: 43.7 against 46.6 TOPS; 5120^3 a tie)
+  if (d->mult_op == kMinimum || d->mult_op == kMaximum) return false;
   const Problem c = canonical(d);
   const long long tiles = (long long)((c.m + 255) / 256) * ((c.n + 127) / 128), ktiles = (c.k + 15) / 16;
   const long long rounds = (tiles + 511) / 512;
@@ -204,10 +207,15 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   const bool f64 = d->dtype == CUASR_AMD_F64;  // fp64 direct tile: 128 x 128, two per compute unit like the 4-byte one
   const int tile_m = f64 ? 128 : (c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) ? 128 : 256;  // relaxed variant: 128 x 128
   const int tile_n = 128;
-  const long long slots = 512;
+  // (an fp64 instruction occupies the vector ALU for four cycles: one workgroup per compute unit already runs at
+  // nearly the full rate -- 2048^3 max-plus, 256 tiles: 30.9 TOPS against 28.8 on the staged tile -- so its rounds are
+  // of 256; from `python -m cuasr_amd.bench_matrix --tune`)
+  const long long slots = f64 ? 256 : 512;
   const long long direct_groups = (long long)((c.m + tile_m - 1) / tile_m) * ((c.n + tile_n - 1) / tile_n) * d->split_k_slices * batch;
   const long long rounds = (direct_groups + slots - 1) / slots;
-  const bool fills = direct_groups * 8 >= rounds * slots * 7;  // >= 7/8 of its rounds
+  // >= 7/8 of its rounds (fp64: 95 % -- its staged tile is within 10 % of the direct one, so a last round that
+  // is 11 % empty, 5120^2, already costs more than the direct tile gains: 28.3 against 29.5 TOPS)
+  const bool fills = f64 ? direct_groups * 100 >= rounds * slots * 95 : direct_groups * 8 >= rounds * slots * 7;
   const bool have_valu = find_valu(d->dtype, d->add_op, d->mult_op) != nullptr;
   // or-and: the staged tile turns its panels into masks on their way to LDS and spends one
   // `acc | (a & b)` per term; the direct tile cannot (its panels never pass through registers)
@@ -240,6 +248,9 @@ static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
   const int tile_n = 128;
   const long long slots = 512;
   const int tr = c.m / tile_m, tc = c.n / tile_n;  // whole tiles only
+  // fp64: the strips of a mid-sized output are short launches that cost what the block gains (3072^2: 29.0 against
+  // 30.8 TOPS on the staged tile alone; 5120^2: 30.6 against 29.5)
+  if (f64 && (long long)tr * tc < 1024) return none;
   long long best = 0;
   Block b = none;
   for (int r = 1; r <= tr; ++r) {

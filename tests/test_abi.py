@@ -111,6 +111,9 @@ def test_kernel_selection(lib):
     assert sel(desc(add="plus", mult="multiplies", m=1024, n=1024)) == b"valu"   # 64 tiles of 128 x 128 leave the chip idle
     assert sel(desc(dtype="f64")) == b"valu"
     assert sel(desc(dtype="f64", m=8192, n=8192, k=64)) == b"valu_direct"   # fp64 direct-to-LDS tile, 128 x 64
+    assert sel(desc(dtype="f64", m=2048, n=2048, k=64)) == b"valu_direct"   # 256 of them: one per compute unit is a full round for fp64
+    assert sel(desc(m=3072, n=3072, k=4096)) == b"valu_streamk"             # min-plus, half a round of tiles: stream-K ...
+    assert sel(desc(m=3072, n=3072, k=4096, mult="maximum")) == b"valu"     # ... but not for the two-instruction min-max
     assert sel(desc(dtype="f64", add="plus", mult="multiplies", m=2048, n=2048)) == b"mfma"   # fp64 matrix cores
     assert sel(desc(dtype="f64", add="plus", mult="multiplies")) == b"valu"
     assert sel(desc(add="plus", mult="bit_or", dtype="i32")) == b"naive"
