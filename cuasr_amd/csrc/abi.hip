@@ -13,6 +13,7 @@ launch_fn find_valu_f64(int, int);
 launch_fn find_valu_i32(int, int);
 launch_fn find_valu_u32(int, int);
 launch_fn find_valu_f16(int, int);
+launch_fn find_valu_i8(int, int);
 launch_fn find_mfma_f32(int, int);
 launch_fn find_mfma_f64(int, int);
 launch_fn find_mfma_i8(int, int);
@@ -37,6 +38,7 @@ launch_fn find_valu(int dtype, int add_op, int mult_op) {
     case CUASR_AMD_I32: return find_valu_i32(add_op, mult_op);
     case CUASR_AMD_U32: return find_valu_u32(add_op, mult_op);
     case CUASR_AMD_F16: return find_valu_f16(add_op, mult_op);
+    case CUASR_AMD_I8: return find_valu_i8(add_op, mult_op);
     default: return nullptr;
   }
 }

@@ -19,6 +19,12 @@
 // of B, and issues 64 packed adds + 32 three-input packed minima for 128 terms.
 // Outputs too small to give the 256 compute units two such tiles each take smaller ones of the same kernel
 // (64 x 128 and 32 x 128: 4 or 2 rows and one column group per thread, guarded form only).
+//
+// int8 operands (CUASR_AMD_I8: int8 A and B, int32 everything else) ride on the same kernel for min-plus,
+// max-plus, min-max and max-min: every int8 value, and every sum of two, is a binary16 value, so the terms and
+// their minima are exact; the operands are converted on their way to LDS, the accumulators on their way out,
+// and the epilogue (the caller's additive identity included) is integer arithmetic.  On the vector ALU that is
+// twice the rate integers get (three-input integer minima and byte-selecting adds issue at half rate).
 #include "semiring.h"
 
 namespace cuasr_amd {
@@ -57,11 +63,18 @@ template <int ADD, int MUL> __device__ __forceinline__ void one_term(h2 &acc, h2
 __device__ __forceinline__ h2 both(half_t v) { return h2{v, v}; }
 __device__ __forceinline__ h2 pair_of(const h8 &v, int j) { return h2{v[2 * j], v[2 * j + 1]}; }
 template <int N> struct frag_of { typedef half_t type __attribute__((ext_vector_type(N))); };
+// what C, D, the scalars and the workspace hold for operands of type TI; 8 of them, 8 operands
+template <typename TI> struct out_of { typedef half_t type; };
+template <> struct out_of<int8_t> { typedef int32_t type; };
+template <typename T> struct vec8 { typedef T type __attribute__((ext_vector_type(8), aligned(sizeof(T) * 8 < 16 ? sizeof(T) * 8 : 16))); };
+template <typename TI> __device__ __forceinline__ half_t to_half(TI v) { return half_t(float(v)); }
+template <> __device__ __forceinline__ half_t to_half<half_t>(half_t v) { return v; }
 
 // One operand's share of a k-tile on its way from memory to LDS.  The panel is X wide (X = BM for A, BN
 // for B); a chunk is 8 elements: of one k and 8 consecutive x when x is the contiguous direction in
 // memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
-template <int X, bool KC, bool GUARD> struct Stager {
+template <int X, bool KC, bool GUARD, typename TI> struct Stager {
+  typedef typename vec8<TI>::type raw8;
   static constexpr int TOTAL = X * BK / 8, CHUNKS = (TOTAL + THREADS - 1) / THREADS;  // (a small panel leaves threads idle)
   h8 r[CHUNKS];
 
@@ -73,26 +86,32 @@ template <int X, bool KC, bool GUARD> struct Stager {
 
   // base: the operand's element (x = 0, k = 0); sx, sk: element strides; x0, k0: the tile's origin;
   // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored);
-  // vec (guarded form): chunks of this operand lie at 16-byte boundaries, so one that is wholly inside the
+  // vec (guarded form): chunks of this operand lie at vector boundaries, so one that is wholly inside the
   // extents is read as a vector all the same
-  __device__ __forceinline__ void load(const half_t *base, long long sx, long long sk, int x0, int k0, int xn, int kn, bool vec) {
+  static __device__ __forceinline__ h8 widen(const raw8 &v) {
+    h8 h;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = to_half<TI>(v[e]);
+    return h;
+  }
+  __device__ __forceinline__ void load(const TI *base, long long sx, long long sk, int x0, int k0, int xn, int kn, bool vec) {
 #pragma unroll
     for (int q = 0; q < CHUNKS; ++q) {
       if (TOTAL % THREADS && (int)threadIdx.x + q * THREADS >= TOTAL) break;
       int x, k;
       where(threadIdx.x + q * THREADS, x, k);
-      const half_t *src = base + (long long)(x0 + x) * sx + (long long)(k0 + k) * sk;
+      const TI *src = base + (long long)(x0 + x) * sx + (long long)(k0 + k) * sk;
       if constexpr (!GUARD) {
-        r[q] = *reinterpret_cast<const h8 *>(src);
+        r[q] = widen(*reinterpret_cast<const raw8 *>(src));
       } else {
         const bool whole = KC ? (x0 + x < xn && k0 + k + 8 <= kn) : (x0 + x + 8 <= xn && k0 + k < kn);
         if (vec && whole) {
-          r[q] = *reinterpret_cast<const h8 *>(src);
+          r[q] = widen(*reinterpret_cast<const raw8 *>(src));
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int xe = x0 + x + (KC ? 0 : e), ke = k0 + k + (KC ? e : 0);
-            r[q][e] = (xe < xn && ke < kn) ? src[(KC ? sk : sx) * e] : half_t(0);
+            r[q][e] = (xe < xn && ke < kn) ? to_half<TI>(src[(KC ? sk : sx) * e]) : half_t(0);
           }
         }
       }
@@ -115,12 +134,15 @@ template <int X, bool KC, bool GUARD> struct Stager {
   }
 };
 
-template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD, int TR = 8, int NG = 2>
+template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD, int TR = 8, int NG = 2, typename TI = half_t>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void half_tile_kernel(Problem p) {
   constexpr int BM = 16 * TR, BN = 128 * NG;
+  constexpr bool BYTES = std::is_same<TI, int8_t>::value;
+  typedef typename out_of<TI>::type TO;
+  typedef typename vec8<TO>::type out8;
   typedef typename frag_of<TR>::type rows_t;
   __shared__ __attribute__((aligned(16))) Smem<TR, NG> sm;
-  select_batch<half_t>(p);
+  select_batch<TO, TI>(p);
   const int tiles_n = (p.n + BN - 1) / BN;
   const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
   const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
@@ -129,8 +151,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
     kb = blockIdx.y * p.k_per_slice;
     ke = min(p.k, kb + p.k_per_slice);
   }
-  const half_t *A = reinterpret_cast<const half_t *>(p.A), *B = reinterpret_cast<const half_t *>(p.B);
-  const half_t ident = scalar_as<half_t>(p.add_identity);
+  const TI *A = reinterpret_cast<const TI *>(p.A), *B = reinterpret_cast<const TI *>(p.B);
+  // int8 operands: the loop starts from the binary16 infinity of its add; the caller's identity joins at the end
+  const half_t ident = BYTES ? half_t(ADD == kMinimum ? __builtin_inff() : -__builtin_inff()) : scalar_as<half_t>(p.add_identity);
 
   h2 acc[TR][4 * NG];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
 #pragma unroll
@@ -138,11 +161,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int j = 0; j < 4 * NG; ++j) acc[i][j] = both(ident);
 
-  Stager<BM, A_KC, GUARD> sa;
-  Stager<BN, B_KC, GUARD> sb;
+  Stager<BM, A_KC, GUARD, TI> sa;
+  Stager<BN, B_KC, GUARD, TI> sb;
   // (tile origins are multiples of 8 in x; the k origin is one if the slice's is)
-  const bool vec_a = reinterpret_cast<uintptr_t>(A) % 16 == 0 && (A_KC ? p.sa_m : p.sa_k) % 8 == 0 && kb % 8 == 0;
-  const bool vec_b = reinterpret_cast<uintptr_t>(B) % 16 == 0 && (B_KC ? p.sb_n : p.sb_k) % 8 == 0 && kb % 8 == 0;
+  const bool vec_a = reinterpret_cast<uintptr_t>(A) % (8 * sizeof(TI)) == 0 && (A_KC ? p.sa_m : p.sa_k) % 8 == 0 && kb % 8 == 0;
+  const bool vec_b = reinterpret_cast<uintptr_t>(B) % (8 * sizeof(TI)) == 0 && (B_KC ? p.sb_n : p.sb_k) % 8 == 0 && kb % 8 == 0;
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   if (tiles_k > 0) {
     sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke, vec_a);
@@ -199,25 +222,26 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   }
 
   // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or the raw accumulators of a k-slice
-  const EpilogueScalars<half_t> e = resolve_scalars<half_t>(p, MUL);
-  half_t *ws = p.workspace ? reinterpret_cast<half_t *>(p.workspace) + (long long)blockIdx.y * p.m * p.n : nullptr;
-  const half_t *C = reinterpret_cast<const half_t *>(p.C);
-  half_t *D = reinterpret_cast<half_t *>(p.D);
+  const EpilogueScalars<TO> e = resolve_scalars<TO>(p, MUL);
+  TO *ws = p.workspace ? reinterpret_cast<TO *>(p.workspace) + (long long)blockIdx.y * p.m * p.n : nullptr;
+  const TO *C = reinterpret_cast<const TO *>(p.C);
+  TO *D = reinterpret_cast<TO *>(p.D);
 #pragma unroll
   for (int i = 0; i < TR; ++i) {
     const int row = m0 + ty * TR + i;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
       const int col = n0 + g * 128 + tx * 8;
-      h8 v;
+      out8 v;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        v[2 * j] = acc[i][g * 4 + j][0];
-        v[2 * j + 1] = acc[i][g * 4 + j][1];
+      for (int j = 0; j < 8; ++j) {
+        const half_t a = acc[i][g * 4 + j / 2][j % 2];
+        if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
+        else v[j] = a;
       }
       if (ws) {
         if constexpr (!GUARD) {
-          *reinterpret_cast<h8 *>(ws + (long long)row * p.n + col) = v;
+          *reinterpret_cast<out8 *>(ws + (long long)row * p.n + col) = v;
         } else {
 #pragma unroll
           for (int x = 0; x < 8; ++x)
@@ -225,26 +249,26 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         }
         continue;
       }
-      h8 c;
+      out8 c;
 #pragma unroll
       for (int x = 0; x < 8; ++x) c[x] = e.ident;
       if (e.source_needed) {
         if constexpr (!GUARD) {
-          c = *reinterpret_cast<const h8 *>(C + (long long)row * p.ldc + col);
+          c = *reinterpret_cast<const out8 *>(C + (long long)row * p.ldc + col);
         } else {
 #pragma unroll
           for (int x = 0; x < 8; ++x)
             if ((unsigned)row < (unsigned)p.m && (unsigned)(col + x) < (unsigned)p.n) c[x] = C[(long long)row * p.ldc + col + x];
         }
       }
-      h8 out;
+      out8 out;
 #pragma unroll
       for (int x = 0; x < 8; ++x) {
         out[x] = Op<MUL>::apply(e.alpha, v[x]);
         if (e.source_needed) out[x] = fold_epilogue<ADD, MUL>(out[x], Op<MUL>::apply(e.beta, c[x]));
       }
       if constexpr (!GUARD) {
-        *reinterpret_cast<h8 *>(D + (long long)row * p.ldd + col) = out;
+        *reinterpret_cast<out8 *>(D + (long long)row * p.ldd + col) = out;
       } else {
 #pragma unroll
         for (int x = 0; x < 8; ++x)
@@ -254,30 +278,34 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   }
 }
 
-// whole tiles, whole 16-byte vectors at 16-byte boundaries everywhere: the unguarded kernel
-static bool exact(const Problem &p, bool a_kc, bool b_kc) {
-  auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+// whole tiles, whole vectors at vector boundaries everywhere: the unguarded kernel
+template <typename TI> static bool exact(const Problem &p, bool a_kc, bool b_kc) {
+  typedef typename out_of<TI>::type TO;
+  constexpr uintptr_t in_bytes = 8 * sizeof(TI);            // a chunk of 8 operands
+  constexpr long long out_step = 16 / sizeof(TO);           // elements of C / D per 16 bytes
+  auto al = [](const void *q, uintptr_t to) { return reinterpret_cast<uintptr_t>(q) % to == 0; };
   if (p.m % 128 || p.n % 256 || p.k % BK || p.k == 0) return false;
-  if (p.workspace && (p.k_per_slice % BK || !al16(p.workspace))) return false;
+  if (p.workspace && (p.k_per_slice % BK || !al(p.workspace, 16))) return false;
   if ((a_kc ? p.sa_m : p.sa_k) % 8 || (b_kc ? p.sb_n : p.sb_k) % 8) return false;
-  if (!al16(p.A) || !al16(p.B) || !al16(p.D) || p.ldd % 8) return false;
-  if (p.C && (!al16(p.C) || p.ldc % 8)) return false;
-  if (p.batch > 1 && (p.batch_a % 8 || p.batch_b % 8 || p.batch_c % 8 || p.batch_d % 8)) return false;
+  if (!al(p.A, in_bytes) || !al(p.B, in_bytes) || !al(p.D, 16) || p.ldd % out_step) return false;
+  if (p.C && (!al(p.C, 16) || p.ldc % out_step)) return false;
+  if (p.batch > 1 && (p.batch_a % 8 || p.batch_b % 8 || p.batch_c % out_step || p.batch_d % out_step)) return false;
   return true;
 }
 
-template <int ADD, int MUL, bool GUARD, int TR, int NG> static hipError_t launch_tile(const Problem &p, bool a_kc, bool b_kc, hipStream_t s) {
+template <int ADD, int MUL, bool GUARD, int TR, int NG, typename TI>
+static hipError_t launch_tile(const Problem &p, bool a_kc, bool b_kc, hipStream_t s) {
   const long long tiles = (long long)((p.m + 16 * TR - 1) / (16 * TR)) * ((p.n + 128 * NG - 1) / (128 * NG));
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(THREADS);
-#define CUASR_HALF_LAUNCH(AK, BK_) launch_kernel((half_tile_kernel<ADD, MUL, AK, BK_, GUARD, TR, NG>), grid, block, 0, s, p)
+#define CUASR_HALF_LAUNCH(AK, BK_) launch_kernel((half_tile_kernel<ADD, MUL, AK, BK_, GUARD, TR, NG, TI>), grid, block, 0, s, p)
   if (a_kc) { if (b_kc) CUASR_HALF_LAUNCH(true, true); else CUASR_HALF_LAUNCH(true, false); }
   else { if (b_kc) CUASR_HALF_LAUNCH(false, true); else CUASR_HALF_LAUNCH(false, false); }
 #undef CUASR_HALF_LAUNCH
   return take_launch_status();
 }
 
-template <int ADD, int MUL> static hipError_t launch(const Problem &p, hipStream_t s) {
+template <int ADD, int MUL, typename TI = half_t> static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   // one direction of each operand is contiguous (the C ABI produces nothing else)
   if ((p.sa_m != 1 && p.sa_k != 1) || (p.sb_n != 1 && p.sb_k != 1)) return hipErrorNotSupported;
@@ -293,11 +321,11 @@ template <int ADD, int MUL> static hipError_t launch(const Problem &p, hipStream
   };
   const long long full = cost(128, 256, 100), mid = cost(64, 128, 70), small = cost(32, 128, 55);
   if (full <= mid && full <= small) {
-    if (exact(p, a_kc, b_kc)) return launch_tile<ADD, MUL, false, 8, 2>(p, a_kc, b_kc, s);
-    return launch_tile<ADD, MUL, true, 8, 2>(p, a_kc, b_kc, s);
+    if (exact<TI>(p, a_kc, b_kc)) return launch_tile<ADD, MUL, false, 8, 2, TI>(p, a_kc, b_kc, s);
+    return launch_tile<ADD, MUL, true, 8, 2, TI>(p, a_kc, b_kc, s);
   }
-  if (mid <= small) return launch_tile<ADD, MUL, true, 4, 1>(p, a_kc, b_kc, s);
-  return launch_tile<ADD, MUL, true, 2, 1>(p, a_kc, b_kc, s);
+  if (mid <= small) return launch_tile<ADD, MUL, true, 4, 1, TI>(p, a_kc, b_kc, s);
+  return launch_tile<ADD, MUL, true, 2, 1, TI>(p, a_kc, b_kc, s);
 }
 
 }  // namespace half_tile
@@ -313,6 +341,18 @@ launch_fn find_valu_f16(int add_op, int mult_op) {
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
   PAIR(kPlus, kMultiplies)
+#undef PAIR
+  return nullptr;
+}
+
+// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16)
+launch_fn find_valu_i8(int add_op, int mult_op) {
+#define PAIR(ADD, MUL) \
+  if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL, int8_t>;
+  PAIR(kMinimum, kPlus)
+  PAIR(kMaximum, kPlus)
+  PAIR(kMinimum, kMaximum)
+  PAIR(kMaximum, kMinimum)
 #undef PAIR
   return nullptr;
 }

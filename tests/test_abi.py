@@ -91,8 +91,9 @@ def test_half_and_int8_element_types(lib):
     assert ok(d) == 0
     d.D = 0x10002
     assert ok(d) == 1
-    assert sel(desc(dtype="i8")) == b"naive" and ok(desc(dtype="i8", add="bit_xor", mult="bit_and")) == 0
-    assert ok(desc(dtype="i8", kernel="valu")) == 5
+    assert sel(desc(dtype="i8")) == b"valu" and ok(desc(dtype="i8", kernel="valu")) == 0   # min-plus: exact in binary16
+    assert ok(desc(dtype="i8", add="bit_xor", mult="bit_and")) == 0 and sel(desc(dtype="i8", add="bit_xor", mult="bit_and")) == b"naive"
+    assert ok(desc(dtype="i8", add="plus", mult="multiplies", kernel="valu")) == 5
     assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "i8") == 4 * 100 * 7 * 3
     d = desc()
     d.dtype = 6

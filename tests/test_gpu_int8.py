@@ -55,7 +55,8 @@ def test_selected_family(lib):
     dA = to_device(np.zeros((128, 64), np.int8))
     dB = to_device(np.zeros((64, 256), np.int8))
     dD = to_device(np.zeros((128, 256), np.int32))
-    for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"naive"), (("bit_xor", "bit_and"), b"naive")]:
+    for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"valu"), (("maximum", "minimum"), b"valu"),
+                              (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"naive")]:
         desc = cuasr_amd.make_desc(add, mult, "i8", dA, dB, dD, dD, 1, 0, 0, 1)
         assert lib.cuasr_amd_selected_kernel(desc) == name
 
@@ -67,6 +68,36 @@ def test_every_pair_on_widened_operands(oracle, lib, sr):
     for layouts in ("ccc", "rcr"):
         check(oracle, *sr, 70, 90, 33, layouts, "auto")
         check(oracle, *sr, 70, 90, 33, layouts, "naive")
+
+
+@pytest.mark.parametrize("sr", [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum")])
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_tropical_pairs_on_the_packed_tile(oracle, lib, sr, layouts):
+    """Sums, minima and maxima of two int8 values are exact in binary16: these pairs run on the packed
+    half-precision tile (operands converted on their way to LDS, integer epilogue).  Every tile size, aligned and
+    ragged, identities and scalars that are not the semiring's own."""
+    check(oracle, *sr, 100, 300, 45, layouts, "valu")                        # 32 x 128 tiles, ragged
+    check(oracle, *sr, 1, 1, 1, layouts, "valu")
+    check(oracle, *sr, 2048, 2048, 96, layouts, "valu", alpha=7, beta=-3)    # 64 x 128 tiles
+    check(oracle, *sr, 4096, 4096, 64, layouts, "valu")                      # full tiles, unguarded
+    check(oracle, *sr, 4000, 4100, 70, layouts, "valu", alpha=-100, beta=100)  # full tiles, guarded
+
+
+def test_tropical_identity_that_is_not_infinite(oracle, lib):
+    """The caller's additive identity takes part in the result (here it beats some of the sums), also with no
+    terms at all."""
+    import torch
+    import cuasr_amd
+    for (m, n, k) in [(70, 90, 33), (70, 90, 0)]:
+        A, B, C = operands(m, n, k, "col", "row", "col", seed=5)
+        C[:] = 1000                                                   # (out of the way: D = min(acc, 0 + C))
+        want = oracle.srgemm("minimum", "plus", A, B, C, 0, 0, -225)
+        dA, dB, dC = to_device(A), to_device(B), to_device(C)
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm("minimum", "plus", dA, dB, dC, dD, 0, 0, -225, 0, dtype="i8", kernel="valu")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"identity -225, k = {k}")
+        assert k == 0 or (want == -225).any() and (want < -225).any()
 
 
 @pytest.mark.parametrize("slices", [1, 3, 8])
