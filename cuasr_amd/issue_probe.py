@@ -131,6 +131,8 @@ def kernels():
     k["add_u32_sdwa_bytes"] = (only("v_add_u32_sdwa v{t}, sext(v{b}), sext(v{a}) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:BYTE_2"), 192, 0, "f32")
     k["min3_i32"] = (only("v_min3_i32 v{acc}, v{acc}, v{b}, v{a}"), 192, 0, "f32")
     k["mix_i8_sdwa"] = (flat(mix_i8()), 192, 128, "f32")
+    # an operand fetched from another lane of the quad by the add itself (a fragment shared by four lanes)
+    k["add_f32_dpp_quad"] = (only("v_add_f32_dpp v{t}, v{b}, v{a} quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf"), 192, 0, "f32")
     k["mix"] = (flat(mix()), 192, 128, "f32")
     k["mix_sgpr_b"] = (flat(mix(True)), 192, 128, "f32")
     for n in (4, 8, 16):
