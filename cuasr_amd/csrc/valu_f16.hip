@@ -75,6 +75,8 @@ template <> __device__ __forceinline__ half_t to_half<half_t>(half_t v) { return
 // memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
 template <int X, bool KC, bool GUARD, typename TI> struct Stager {
   typedef typename vec8<TI>::type raw8;
+  // the same eight operands at any element boundary (the hardware takes a vector load at any address)
+  typedef TI loose8 __attribute__((ext_vector_type(8), aligned(sizeof(TI))));
   static constexpr int TOTAL = X * BK / 8, CHUNKS = (TOTAL + THREADS - 1) / THREADS;  // (a small panel leaves threads idle)
   h8 r[CHUNKS];
 
@@ -85,16 +87,16 @@ template <int X, bool KC, bool GUARD, typename TI> struct Stager {
   }
 
   // base: the operand's element (x = 0, k = 0); sx, sk: element strides; x0, k0: the tile's origin;
-  // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored);
-  // vec (guarded form): chunks of this operand lie at vector boundaries, so one that is wholly inside the
-  // extents is read as a vector all the same
+  // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored).
+  // In the guarded form a chunk that lies wholly inside the extents is read as a vector all the same, at whatever
+  // element boundary it starts; only chunks across an edge are read element by element
   static __device__ __forceinline__ h8 widen(const raw8 &v) {
     h8 h;
 #pragma unroll
     for (int e = 0; e < 8; ++e) h[e] = to_half<TI>(v[e]);
     return h;
   }
-  __device__ __forceinline__ void load(const TI *base, long long sx, long long sk, int x0, int k0, int xn, int kn, bool vec) {
+  __device__ __forceinline__ void load(const TI *base, long long sx, long long sk, int x0, int k0, int xn, int kn) {
 #pragma unroll
     for (int q = 0; q < CHUNKS; ++q) {
       if (TOTAL % THREADS && (int)threadIdx.x + q * THREADS >= TOTAL) break;
@@ -105,8 +107,8 @@ template <int X, bool KC, bool GUARD, typename TI> struct Stager {
         r[q] = widen(*reinterpret_cast<const raw8 *>(src));
       } else {
         const bool whole = KC ? (x0 + x < xn && k0 + k + 8 <= kn) : (x0 + x + 8 <= xn && k0 + k < kn);
-        if (vec && whole) {
-          r[q] = widen(*reinterpret_cast<const raw8 *>(src));
+        if (whole) {
+          r[q] = widen(*reinterpret_cast<const loose8 *>(src));
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
@@ -163,13 +165,10 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
   Stager<BM, A_KC, GUARD, TI> sa;
   Stager<BN, B_KC, GUARD, TI> sb;
-  // (tile origins are multiples of 8 in x; the k origin is one if the slice's is)
-  const bool vec_a = reinterpret_cast<uintptr_t>(A) % (8 * sizeof(TI)) == 0 && (A_KC ? p.sa_m : p.sa_k) % 8 == 0 && kb % 8 == 0;
-  const bool vec_b = reinterpret_cast<uintptr_t>(B) % (8 * sizeof(TI)) == 0 && (B_KC ? p.sb_n : p.sb_k) % 8 == 0 && kb % 8 == 0;
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   if (tiles_k > 0) {
-    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke, vec_a);
-    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke, vec_b);
+    sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke);
+    sb.load(B, p.sb_n, p.sb_k, n0, kb, p.n, ke);
     sa.store(sm.a[0]);
     sb.store(sm.b[0]);
   }
@@ -177,8 +176,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   for (int t = 0; t < tiles_k; ++t) {
     const int s = t & 1, k0 = kb + t * BK;
     if (t + 1 < tiles_k) {
-      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke, vec_a);
-      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke, vec_b);
+      sa.load(A, p.sa_m, p.sa_k, m0, k0 + BK, p.m, ke);
+      sb.load(B, p.sb_n, p.sb_k, n0, k0 + BK, p.n, ke);
     }
     const half_t(*pa)[BM] = sm.a[s];
     const half_t(*pb)[BN] = sm.b[s];
