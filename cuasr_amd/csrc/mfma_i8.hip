@@ -50,7 +50,10 @@ template <int X, bool KC, bool GUARD> struct Stager {
       return *reinterpret_cast<const v4i *>(src);
     } else {
       v4i v = {0, 0, 0, 0};
-      if (live) {
+      typedef int loose4 __attribute__((ext_vector_type(4), aligned(1)));  // (a vector load may start at any byte)
+      if (live && first + 16 <= limit) {
+        v = *reinterpret_cast<const loose4 *>(src);
+      } else if (live) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int byte = (first + e < limit) ? (int)(unsigned char)src[e] : 0;
