@@ -85,5 +85,10 @@ static inline bool can_run(const Problem &p) {
   return true;
 }
 
+// what the element-aligned form of the compiled plus-times kernel asks for: one contiguous direction per operand
+static inline bool loose_can_run(const Problem &p) {
+  return (p.sa_m == 1 || p.sa_k == 1) && (p.sb_n == 1 || p.sb_k == 1);
+}
+
 }  // namespace mfma_panel
 }  // namespace cuasr_amd

@@ -249,6 +249,11 @@ launch_fn find_mfma_f32(int add_op, int mult_op) {
   return nullptr;
 }
 
-bool mfma_f32_can_run(const Problem &p) { return mfma_panel::can_run(p); }
+bool mfma_gemm_f32_can_run(const Problem &);
+// (plus-times has an element-aligned form; the tropical tile needs 16-byte vectors)
+bool mfma_f32_can_run(const Problem &p) {
+  if (p.add_op == kPlus && p.mult_op == kMultiplies) return mfma_gemm_f32_can_run(p);
+  return mfma_panel::can_run(p);
+}
 
 }  // namespace cuasr_amd

@@ -50,11 +50,19 @@ template <int NB> struct Smem {
 // src[] points at the vectors of the FIRST k-tile (x clamped to the matrix) and
 // advances by `step` per tile; lds[] is the float index inside a stage where
 // element 0 of each vector goes (row stride LD per k for k-contiguous vectors).
-struct Mover {
+// LOOSE: operands of any extent, leading dimension and 4-byte alignment.  The vector loads are made at element
+// alignment (the hardware takes them at any 4-byte boundary), and a vector that would cross the end of its row
+// (x contiguous) or of the k range (k contiguous) is read element by element with clamped indices instead --
+// what lands in the places past the end is never used (rows / columns past the edge are not stored, k past the
+// end is zeroed in the ragged tile).
+typedef float v4f_loose __attribute__((ext_vector_type(4), aligned(4)));
+
+template <bool LOOSE> struct Mover {
   const float *src[2];
   long long step;
   int lds[2];
   bool x_contig;
+  int x_left;    // LOOSE, x contiguous: elements from this thread's vector start to the end of the row (<= 0: none)
 
   __device__ __forceinline__ void init(const float *base, long long s_x, long long s_k, int x0, int x_end, int k0,
                                        bool xc) {
@@ -63,7 +71,8 @@ struct Mover {
     step = (long long)BK * s_k;
     if (xc) {
       const int xg = tid & 31, kq = (tid >> 5) & 3, half = tid >> 7;
-      const int xx = min(x0 + xg * 4, x_end - 4);
+      const int xx = LOOSE ? min(x0 + xg * 4, x_end - 1) : min(x0 + xg * 4, x_end - 4);
+      x_left = x_end - (x0 + xg * 4);
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int kk = kq * 4 + half * 2 + j;
@@ -82,10 +91,22 @@ struct Mover {
       }
     }
   }
+  // 4 consecutive x from `at`, of which x_left lie inside the row (LOOSE; at itself is inside)
+  __device__ __forceinline__ v4f row_vector(const float *at) const {
+    if (x_left >= 4) return *reinterpret_cast<const v4f_loose *>(at);
+    v4f v;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = at[min(e, max(x_left - 1, 0))];
+    return v;
+  }
   // whole k-tile: nothing to clamp along k
   __device__ __forceinline__ void load(v4f (&r)[2]) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) r[j] = *reinterpret_cast<const v4f *>(src[j]);
+    for (int j = 0; j < 2; ++j) {
+      if constexpr (!LOOSE) r[j] = *reinterpret_cast<const v4f *>(src[j]);
+      else if (x_contig) r[j] = row_vector(src[j]);
+      else r[j] = *reinterpret_cast<const v4f_loose *>(src[j]);
+    }
   }
   // ragged last k-tile with `kcount` (< BK) valid k: vectors that start past the end re-read the
   // last valid one (never used); k-contiguous extents are multiples of 4, so no vector straddles the end
@@ -97,8 +118,22 @@ struct Mover {
       if (x_contig) {
         const int kk = ((tid >> 5) & 3) * 4 + (tid >> 7) * 2 + j;
         back = (long long)max(kk - (kcount - 1), 0) * s_k;
+        if constexpr (LOOSE) {
+          r[j] = row_vector(src[j] - back);
+          continue;
+        }
       } else {
         const int kg = ((tid + 256 * j) >> 4) & 3;
+        if constexpr (LOOSE) {
+          // element e is k = 4 kg + e of the tile; past the end, the last valid k instead
+          if (kg * 4 + 4 <= kcount) {
+            r[j] = *reinterpret_cast<const v4f_loose *>(src[j]);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[j][e] = src[j][min(kg * 4 + e, kcount - 1) - kg * 4];
+          }
+          continue;
+        }
         back = max(kg * 4 - (kcount - 4), 0);
       }
       r[j] = *reinterpret_cast<const v4f *>(src[j] - back);
@@ -121,7 +156,7 @@ struct Mover {
   }
 };
 
-template <int NB>
+template <int NB, bool LOOSE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_kernel(Problem p) {
   constexpr int BN = 128 * NB, WN = 64 * NB, QB = 2 * NB;  // tile columns, wave columns, 32-column blocks per wave
   __shared__ Smem<NB> sm;
@@ -163,7 +198,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int r = 0; r < 16; ++r) acc[bi][bj][r] = p.add_identity.f32;  // 0 for plus
 
   const int ntiles = (ke - kb + BK - 1) / BK;
-  Mover ma, mb[NB];
+  Mover<LOOSE> ma, mb[NB];
   ma.init(A, p.sa_m, p.sa_k, m0, p.m, kb, a_xc);
 #pragma unroll
   for (int h = 0; h < NB; ++h) mb[h].init(B, p.sb_n, p.sb_k, n0 + 128 * h, p.n, kb, b_xc);
@@ -318,7 +353,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
-  if (!can_run(p)) return hipErrorNotSupported;
+  if (!loose_can_run(p)) return hipErrorNotSupported;
+  const bool loose = !can_run(p);
   const long long tiles_m = (p.m + BM - 1) / BM, slices = p.workspace ? p.slices : 1;
   const long long tiles = tiles_m * ((p.n + 127) / 128), wide = tiles_m * ((p.n + 255) / 256);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
@@ -328,21 +364,29 @@ static hipError_t launch(const Problem &p, hipStream_t s) {
   // tile, 5120^3: 133 against 117, 6144^3: 150 against 136); where both fill theirs (4096^3: 149.1 and 149.8) the
   // wide one, which moves a quarter less data per flop.
   const long long batch = p.batch > 1 ? p.batch : 1;
-  if (mfma_direct_f32_can_run(p)) {
+  if (!loose && mfma_direct_f32_can_run(p)) {
     auto fill = [](long long groups) { return (double)groups / (256.0 * (double)((groups + 255) / 256)); };
     return mfma_direct_f32_launch(p, fill(wide * slices * batch) >= 0.995 * fill(tiles * slices * batch), s);
   }
   if (batch > 1) return hipErrorNotSupported;  // the compiled kernels take one product per launch
   // the 128 x 256 tile when its workgroups fill >= 7/8 of whole rounds of 512 (two per compute unit)
   const long long rounds = (wide * slices + 511) / 512;
-  if (wide * slices * 8 >= rounds * 512 * 7)
-    launch_kernel(gemm_mfma_kernel<2>, dim3((unsigned)wide, (unsigned)slices), dim3(256), 0, s, p);
-  else
-    launch_kernel(gemm_mfma_kernel<1>, dim3((unsigned)tiles, (unsigned)slices), dim3(256), 0, s, p);
+  const bool wide_tile = wide * slices * 8 >= rounds * 512 * 7;
+  const dim3 grid((unsigned)(wide_tile ? wide : tiles), (unsigned)slices);
+  if (loose) {
+    if (wide_tile) launch_kernel((gemm_mfma_kernel<2, true>), grid, dim3(256), 0, s, p);
+    else launch_kernel((gemm_mfma_kernel<1, true>), grid, dim3(256), 0, s, p);
+  } else {
+    if (wide_tile) launch_kernel((gemm_mfma_kernel<2, false>), grid, dim3(256), 0, s, p);
+    else launch_kernel((gemm_mfma_kernel<1, false>), grid, dim3(256), 0, s, p);
+  }
   return take_launch_status();
 }
 
 }  // namespace gemm_mfma
+
+// plus-times runs on the matrix cores whatever the operands' extents and alignment
+bool mfma_gemm_f32_can_run(const Problem &p) { return mfma_panel::loose_can_run(p); }
 
 launch_fn find_mfma_gemm_f32(int add_op, int mult_op) {
   if (add_op == kPlus && mult_op == kMultiplies) return gemm_mfma::launch;

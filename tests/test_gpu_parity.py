@@ -187,6 +187,19 @@ def test_plus_times_mfma_small_integers(oracle, lib, shape, layouts):
         run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", beta_one)
 
 
+@pytest.mark.parametrize("shape", [(1001, 997, 333), (130, 66, 6), (257, 129, 17), (1, 1, 1), (3, 5, 2), (2501, 2303, 70), (63, 1, 5)])
+@pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"])
+def test_plus_times_mfma_any_extent(oracle, lib, shape, layouts):
+    """Extents, leading dimensions and k that are not multiples of the 16-byte vector: the matrix-core kernel's
+    element-aligned form (vectors that would cross the end of a row or of the k range are read element by
+    element).  Small integers, so the host reference's bits are the answer."""
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for beta_one in (False, True):
+        run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", beta_one)
+    if shape[2] > 64:
+        run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", True, splitk=3)
+
+
 @pytest.mark.parametrize("shape", [(3584, 4096, 16), (3588, 4092, 48), (3588, 4092, 160), (3584, 4096, 32)])
 @pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr"])
 def test_plus_times_mfma_hand_scheduled(oracle, lib, shape, layouts):
@@ -309,7 +322,8 @@ def test_unaligned_views(oracle, lib, sr, layouts):
         order = "F" if lc == "col" else "C"
         want = oracle.srgemm(add, mult, np.asarray(A, order=("F" if la == "col" else "C")), np.asarray(B, order=("F" if lb == "col" else "C")),
                              np.asarray(C, order=order), one, one, ident)
-        for kernel in ("auto", "valu"):
+        # (plus-times on the matrix cores has an element-aligned form for such operands)
+        for kernel in ("auto", "valu") + (("mfma",) if (add, mult, dtype) == ("plus", "multiplies", "f32") else ()):
             dD = dD0.clone() if False else dD0  # the window of D is written in place
             cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dtype, kernel=kernel)
             torch.cuda.synchronize()
