@@ -53,11 +53,18 @@ __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, in
 // four 16-byte vectors (x contiguous: 2 consecutive x at one k; k contiguous: 2
 // consecutive k at one x).  src[] points at the vectors of the first k-tile, x
 // clamped to the matrix, and advances by one k-tile per load.
-struct Mover {
+// LOOSE: operands of any extent, leading dimension and 8-byte alignment.  The vector loads are made at element
+// alignment, and a vector that would cross the end of its row (x contiguous) or of the k range (k contiguous) is
+// read element by element with clamped indices -- what lands in the places past the end is never used (rows /
+// columns past the edge are not stored, k past the end is zeroed in the ragged tile).
+typedef double v2d_loose __attribute__((ext_vector_type(2), aligned(8)));
+
+template <bool LOOSE> struct Mover {
   const double *src[VECS];
   long long step;
   int lds[VECS];  // index of element 0 of each vector inside a stage
   bool x_contig;
+  bool lone[VECS];  // LOOSE, x contiguous: only the vector's first element (or none: src is clamped) lies inside the row
 
   // the vector's first k inside a k-tile
   static __device__ __forceinline__ int k_local(int v, bool xc) { return xc ? v >> 6 : ((v >> 4) & 7) * 2; }
@@ -72,12 +79,14 @@ struct Mover {
       const int v = tid + 256 * p, kl = k_local(v, xc);
       if (xc) {
         const int x = (v & 63) * 2;
-        src[p] = base + (long long)(k0 + kl) * s_k + min(x0 + x, x_end - 2);
+        src[p] = base + (long long)(k0 + kl) * s_k + (LOOSE ? min(x0 + x, x_end - 1) : min(x0 + x, x_end - 2));
+        lone[p] = x0 + x + 2 > x_end;
         lds[p] = kl * LD + x;
       } else {
         // lanes 0..15: 16 consecutive x of k-pair 0, lanes 16..31: the same x of k-pair 1, ...
         const int x = ((v >> 7) << 4) | (v & 15);
         src[p] = base + (long long)min(x0 + x, x_end - 1) * s_x + k0 + kl;
+        lone[p] = false;
         lds[p] = kl * LD + x;
       }
     }
@@ -85,9 +94,15 @@ struct Mover {
   __device__ __forceinline__ void load(v2d (&r)[VECS]) {
 #pragma unroll
     for (int p = 0; p < VECS; ++p) {
-      r[p] = *reinterpret_cast<const v2d *>(src[p]);
+      r[p] = fetch(src[p], p);
       src[p] += step;
     }
+  }
+  // two consecutive elements from `at` (x contiguous: of a row, where the second may lie past its end)
+  __device__ __forceinline__ v2d fetch(const double *at, int p) const {
+    if constexpr (!LOOSE) return *reinterpret_cast<const v2d *>(at);
+    else if (lone[p]) return v2d{at[0], at[0]};
+    else return *reinterpret_cast<const v2d_loose *>(at);
   }
   // ragged last k-tile with kcount (< BK) valid k: vectors past the end re-read the last valid one
   __device__ __forceinline__ void load_ragged(v2d (&r)[VECS], long long s_k, int kcount) {
@@ -95,8 +110,13 @@ struct Mover {
 #pragma unroll
     for (int p = 0; p < VECS; ++p) {
       const int kl = k_local(tid + 256 * p, x_contig);
-      const int back = max(kl - (kcount - (x_contig ? 1 : 2)), 0);
-      r[p] = *reinterpret_cast<const v2d *>(src[p] - (long long)back * s_k);
+      if (LOOSE && !x_contig) {
+        // elements are k = kl, kl + 1 of the tile; past the end, the last valid k instead
+        r[p] = v2d{src[p][min(kl, kcount - 1) - kl], src[p][min(kl + 1, kcount - 1) - kl]};
+      } else {
+        const int back = max(kl - (kcount - (x_contig ? 1 : 2)), 0);
+        r[p] = fetch(src[p] - (long long)back * s_k, p);
+      }
       src[p] += step;
     }
   }
@@ -113,6 +133,7 @@ struct Mover {
   }
 };
 
+template <bool LOOSE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_mfma_f64_kernel(Problem p) {
   __shared__ Smem sm;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -144,7 +165,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
       for (int r = 0; r < 4; ++r) acc[bi][bj][r] = p.add_identity.f64;  // 0 for plus
 
   const int ntiles = (ke - kb + BK - 1) / BK;
-  Mover ma, mb;
+  Mover<LOOSE> ma, mb;
   ma.init(A, p.sa_m, p.sa_k, m0, p.m, kb, a_xc);
   mb.init(B, p.sb_n, p.sb_k, n0, p.n, kb, b_xc);
   v2d ra[VECS], rb[VECS];
@@ -266,17 +287,22 @@ static bool can_run(const Problem &p) {
   return true;
 }
 
+// the element-aligned form asks for one contiguous direction per operand only
+static bool loose_can_run(const Problem &p) { return (p.sa_m == 1 || p.sa_k == 1) && (p.sb_n == 1 || p.sb_k == 1); }
+
 static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
-  if (!can_run(p)) return hipErrorNotSupported;
+  if (!loose_can_run(p)) return hipErrorNotSupported;
+  const bool loose = !can_run(p);
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   // whole k-tiles, loadable straight into LDS: the hand-scheduled form of the same tile (faster at every size
   // measured, also where a round of workgroups is mostly empty: 2048^3 71.9 against 54.8 TFLOP/s)
-  if (mfma_direct_f64_can_run(p)) return mfma_direct_f64_launch(p, s);
+  if (!loose && mfma_direct_f64_can_run(p)) return mfma_direct_f64_launch(p, s);
   if (p.batch > 1) return hipErrorNotSupported;  // the compiled kernel takes one product per launch
   dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1);
-  launch_kernel(gemm_mfma_f64_kernel, grid, dim3(256), 0, s, p);
+  if (loose) launch_kernel(gemm_mfma_f64_kernel<true>, grid, dim3(256), 0, s, p);
+  else launch_kernel(gemm_mfma_f64_kernel<false>, grid, dim3(256), 0, s, p);
   return take_launch_status();
 }
 
@@ -287,6 +313,6 @@ launch_fn find_mfma_f64(int add_op, int mult_op) {
   return nullptr;
 }
 
-bool mfma_f64_can_run(const Problem &p) { return gemm_mfma_f64::can_run(p); }
+bool mfma_f64_can_run(const Problem &p) { return gemm_mfma_f64::loose_can_run(p); }
 
 }  // namespace cuasr_amd

@@ -190,14 +190,15 @@ def test_plus_times_mfma_small_integers(oracle, lib, shape, layouts):
 @pytest.mark.parametrize("shape", [(1001, 997, 333), (130, 66, 6), (257, 129, 17), (1, 1, 1), (3, 5, 2), (2501, 2303, 70), (63, 1, 5)])
 @pytest.mark.parametrize("layouts", ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"])
 def test_plus_times_mfma_any_extent(oracle, lib, shape, layouts):
-    """Extents, leading dimensions and k that are not multiples of the 16-byte vector: the matrix-core kernel's
-    element-aligned form (vectors that would cross the end of a row or of the k range are read element by
-    element).  Small integers, so the host reference's bits are the answer."""
+    """Extents, leading dimensions and k that are not multiples of the 16-byte vector: the matrix-core kernels'
+    element-aligned forms (vectors that would cross the end of a row or of the k range are read element by
+    element), float and double.  Small integers, so the host reference's bits are the answer."""
     la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
-    for beta_one in (False, True):
-        run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", beta_one)
-    if shape[2] > 64:
-        run(oracle, "plus", "multiplies", "f32", *shape, la, lb, lc, "mfma", True, splitk=3)
+    for dtype in ("f32", "f64"):
+        for beta_one in (False, True):
+            run(oracle, "plus", "multiplies", dtype, *shape, la, lb, lc, "mfma", beta_one)
+        if shape[2] > 64:
+            run(oracle, "plus", "multiplies", dtype, *shape, la, lb, lc, "mfma", True, splitk=3)
 
 
 @pytest.mark.parametrize("shape", [(3584, 4096, 16), (3588, 4092, 48), (3588, 4092, 160), (3584, 4096, 32)])
