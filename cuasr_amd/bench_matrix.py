@@ -30,7 +30,7 @@ SEMIRINGS = [("plus", "multiplies"), ("minimum", "plus"), ("maximum", "plus"), (
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--sizes", default="256,512,1024,2048,4096")
-    ap.add_argument("--dtypes", default="f32,f64")
+    ap.add_argument("--dtypes", default="f32,f64", help="any of f32, f64, f16, i8")
     ap.add_argument("--layouts", default="nn,nt,tn,tt")
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--json", default=None)
@@ -62,14 +62,20 @@ def main():
         if t_start.elapsed_time(t_end) > 300.0:
             break
     for dt in args.dtypes.split(","):
-        npd, tdt = {"f32": (np.float32, torch.float32), "f64": (np.float64, torch.float64)}[dt]
+        # (f16: binary16 throughout; i8: int8 A and B, int32 C and D)
+        npd, tdt = {"f32": (np.float32, torch.float32), "f64": (np.float64, torch.float64), "f16": (np.float16, torch.float16),
+                    "i8": (np.int32, torch.int32)}[dt]
         print(f"\n{dt}: TOPS (2 ops per term), layouts of A and B = {' '.join(layouts)}; C, D column-major; kernel = {args.kernel}")
         print("| add-mult | " + " | ".join(f"N={n}" for n in sizes) + " |")
         print("|---|" + "---|" * len(sizes))
         data = {}
         for n in sizes:
             # one buffer per operand and size; a layout is only a way of reading it
-            data[n] = [torch.from_numpy(inputs.uniform(901 + i, n, n, -1.0, 1.0, npd, "C")).cuda() for i in range(3)]
+            if dt == "i8":
+                data[n] = [torch.from_numpy(inputs.integers(901 + i, n, n, -128, 127, np.int8, "C")).cuda() for i in range(2)]
+                data[n].append(torch.from_numpy(inputs.integers(903, n, n, -1000, 1000, np.int32, "C")).cuda())
+            else:
+                data[n] = [torch.from_numpy(inputs.uniform(901 + i, n, n, -1.0, 1.0, npd, "C")).cuda() for i in range(3)]
             data[n].append(torch.empty(n, n, dtype=tdt, device="cuda"))
         for add, mult in SEMIRINGS:
             ident = cuasr_amd.op_identity(add, dt, True)
