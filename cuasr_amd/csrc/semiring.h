@@ -44,7 +44,16 @@ template <> __device__ __forceinline__ double hw_max<double>(double l, double r)
 // so kernels use the strict form wherever `multiplies` feeds a min or max.
 template <int OP> struct Op {
   template <typename T> static __device__ __forceinline__ T strict(T l, T r) {
-    if constexpr (OP == kMinimum) return r < l ? r : l;
+    if constexpr (std::is_same<T, half_t>::value && (OP == kMinimum || OP == kMaximum)) {
+      // binary16: compared and chosen as integers (sign-magnitude to two's complement, so +0 and -0 tie), because
+      // the compiler turns the floating-point form of this comparison into the min / max instruction, which
+      // returns -0 for that tie whatever the operand order.  (NaN-free data, as everywhere on the fast paths.)
+      const unsigned short rb = __builtin_bit_cast(unsigned short, r), lb = __builtin_bit_cast(unsigned short, l);
+      const int rk = (rb & 0x8000) ? -(int)(rb & 0x7fff) : (int)(rb & 0x7fff);
+      const int lk = (lb & 0x8000) ? -(int)(lb & 0x7fff) : (int)(lb & 0x7fff);
+      const bool take_r = OP == kMinimum ? rk < lk : lk < rk;
+      return __builtin_bit_cast(half_t, (unsigned short)(take_r ? rb : lb));
+    } else if constexpr (OP == kMinimum) return r < l ? r : l;
     else if constexpr (OP == kMaximum) return l < r ? r : l;
     else return apply(l, r);
   }

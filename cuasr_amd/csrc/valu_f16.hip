@@ -136,10 +136,21 @@ template <int X, bool KC, bool GUARD, typename TI> struct Stager {
   }
 };
 
+// the last product of a k range that is zero (acc itself when there is none); not inlined: it runs after the main loop
+static __device__ __attribute__((noinline)) half_t last_zero_product(const half_t *a_row, long long sa_k, const half_t *b_col,
+                                                                     long long sb_k, int kcount, half_t acc) {
+  for (int kk = kcount - 1; kk >= 0; --kk) {
+    const half_t prod = a_row[(long long)kk * sa_k] * b_col[(long long)kk * sb_k];
+    if (prod == half_t(0)) return prod;
+  }
+  return acc;
+}
+
 template <int ADD, int MUL, bool A_KC, bool B_KC, bool GUARD, int TR = 8, int NG = 2, typename TI = half_t>
 __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void half_tile_kernel(Problem p) {
   constexpr int BM = 16 * TR, BN = 128 * NG;
   constexpr bool BYTES = std::is_same<TI, int8_t>::value;
+  constexpr bool ZERO_SIGN = !BYTES && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum);
   typedef typename out_of<TI>::type TO;
   typedef typename vec8<TO>::type out8;
   typedef typename frag_of<TR>::type rows_t;
@@ -237,6 +248,14 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         const half_t a = acc[i][g * 4 + j / 2][j % 2];
         if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
         else v[j] = a;
+        if constexpr (ZERO_SIGN) {
+          // a minimum / maximum that is zero: the reference's comparison keeps the newer of two equal operands
+          // (host_srgemm.h:87 with functional.h:132, :172), so its zero has the sign of the LAST zero product of
+          // the k range, where the packed instruction keeps -0.  Looked up for the few accumulators that end at zero.
+          if (a == half_t(0) && (unsigned)row < (unsigned)p.m && (unsigned)(col + j) < (unsigned)p.n)
+            v[j] = last_zero_product(A + (long long)row * p.sa_m + (long long)kb * p.sa_k, p.sa_k,
+                                     B + (long long)(col + j) * p.sb_n + (long long)kb * p.sb_k, p.sb_k, ke - kb, a);
+        }
       }
       if (ws) {
         if constexpr (!GUARD) {
@@ -329,9 +348,9 @@ template <int ADD, int MUL, typename TI = half_t> static hipError_t launch(const
 
 }  // namespace half_tile
 
-// The semirings whose operators are each one packed instruction with nothing to watch: sums, minima and
-// maxima of data free of -0 never produce -0 (products do: min-times and max-times stay on the naive kernel,
-// as do the logical pairs).
+// The semirings whose operators are each one packed instruction.  Sums, minima and maxima of data free of -0
+// never produce -0; products do, so min-times and max-times settle the sign of a zero result in the epilogue
+// (ZERO_SIGN in the kernel).  The logical pairs stay on the naive kernel.
 launch_fn find_valu_f16(int add_op, int mult_op) {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL>;
@@ -340,6 +359,8 @@ launch_fn find_valu_f16(int add_op, int mult_op) {
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
   PAIR(kPlus, kMultiplies)
+  PAIR(kMinimum, kMultiplies)
+  PAIR(kMaximum, kMultiplies)
 #undef PAIR
   return nullptr;
 }

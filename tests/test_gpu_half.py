@@ -8,8 +8,9 @@ from helpers import assert_same_bits, order_of, to_device
 
 pytestmark = pytest.mark.gpu
 
-TILE_PAIRS = [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"), ("plus", "multiplies")]
-OTHER_PAIRS = [("minimum", "multiplies"), ("maximum", "multiplies"), ("logical_or", "logical_and")]
+TILE_PAIRS = [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"), ("plus", "multiplies"),
+              ("minimum", "multiplies"), ("maximum", "multiplies")]
+OTHER_PAIRS = [("logical_or", "logical_and")]
 LAYOUTS = ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"]
 
 
@@ -82,7 +83,8 @@ def test_selected_family(lib):
     dA = to_device(np.zeros((128, 64), np.float16))
     dB = to_device(np.zeros((64, 256), np.float16))
     dD = to_device(np.zeros((128, 256), np.float16))
-    for (add, mult), name in [(("minimum", "plus"), b"valu"), (("plus", "multiplies"), b"valu"), (("minimum", "multiplies"), b"naive")]:
+    for (add, mult), name in [(("minimum", "plus"), b"valu"), (("plus", "multiplies"), b"valu"), (("minimum", "multiplies"), b"valu"),
+                              (("logical_or", "logical_and"), b"naive")]:
         ident, one, zero = scalars(add, mult, False)
         desc = cuasr_amd.make_desc(add, mult, "f16", dA, dB, dD, dD, one, zero, ident, one)
         assert lib.cuasr_amd_selected_kernel(desc) == name
@@ -97,6 +99,37 @@ def test_every_pair(oracle, lib, sr, kernel):
     for layouts in ("ccc", "rcr"):
         check(oracle, *sr, 70, 90, 33, layouts, kernel)
         check(oracle, *sr, 128, 256, 64, layouts, kernel, beta_one=False)
+
+
+@pytest.mark.parametrize("add", ["minimum", "maximum"])
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr"])
+def test_sign_of_a_zero_extremum(oracle, lib, add, layouts):
+    """min-times / max-times whose result is a zero: the reference's comparison keeps the newer of two equal
+    operands, so the zero carries the sign of the last zero product of the k range.  Operands drawn from
+    {+0, -0} and values of one sign make every result such a zero or a proper extremum."""
+    import torch
+    import cuasr_amd
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    rng = np.random.default_rng(17)
+    sign = 1.0 if add == "minimum" else -1.0          # products are >= 0 (min) or <= 0 (max), zeros of both signs
+    # (not through split-K: which zero a split product keeps depends on where the slices end)
+    for (m, n, k), slices in [((130, 258, 67), 0), ((64, 128, 40), 0), ((2048, 2048, 40), 0)]:
+        A = np.asarray(rng.choice(np.array([0.0, -0.0, 1.0, 2.5], np.float16), (m, k)), order=order_of(la))
+        B = np.asarray(rng.choice(np.array([0.0, -0.0, sign * 1.0, sign * 3.0], np.float16), (k, n)), order=order_of(lb))
+        C = np.asarray(rng.choice(np.array([0.0, -0.0, sign * 5.0], np.float16), (m, n)), order=order_of(lc))
+        ident, one, _ = scalars(add, "multiplies", True)
+        want = oracle.srgemm(add, "multiplies", A, B, C, one, one, ident)
+        assert (want.view(np.uint16) == 0x8000).any() and (want.view(np.uint16) == 0).any()   # zeros of both signs
+        for kernel in ("valu", "naive"):
+            dA, dB, dC = to_device(A), to_device(B), to_device(C)
+            dD = to_device(np.zeros_like(C))
+            if slices:
+                ws = torch.empty(m * n * slices + 8, dtype=torch.float16, device="cuda")
+                cuasr_amd.srgemm_splitk(add, "multiplies", dA, dB, dC, dD, slices, ws, one, one, ident, one, dtype="f16", kernel=kernel)
+            else:
+                cuasr_amd.srgemm(add, "multiplies", dA, dB, dC, dD, one, one, ident, one, dtype="f16", kernel=kernel)
+            torch.cuda.synchronize()
+            assert_same_bits(dD.cpu().numpy(), want, f"{add}-times zeros {m}x{n}x{k} {layouts} {kernel} slices={slices}")
 
 
 def test_scaled_epilogue(oracle, lib):
