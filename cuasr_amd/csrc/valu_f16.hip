@@ -49,7 +49,19 @@ template <int OP> __device__ __forceinline__ h2 pk(h2 l, h2 r) {
 }
 
 // acc <- add(acc, mult(a0, b0), mult(a1, b1)), the two terms in this order
+// or-and: `lhs && rhs`, `lhs || rhs` (functional.h:212, :252) only look at whether an operand is zero, so the
+// panels go to LDS as 16-bit masks (all ones / zero) and a term is one three-input bit operation acc | (a & b)
+// on a register of two masks
+template <int ADD, int MUL> struct masked : std::integral_constant<bool, ADD == kLogicalOr && MUL == kLogicalAnd> {};
+__device__ __forceinline__ h2 or_and_pair(h2 acc, h2 a, h2 b) {
+  return __builtin_bit_cast(h2, or_and_term(__builtin_bit_cast(uint32_t, acc), __builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b)));
+}
+
 template <int ADD, int MUL> __device__ __forceinline__ void two_terms(h2 &acc, h2 a0, h2 b0, h2 a1, h2 b1) {
+  if constexpr (masked<ADD, MUL>::value) {
+    acc = or_and_pair(or_and_pair(acc, a0, b0), a1, b1);
+    return;
+  }
   const h2 t0 = pk<MUL>(a0, b0), t1 = pk<MUL>(a1, b1);
   // the three-input forms (v_pk_minimum3_f16 / v_pk_maximum3_f16) differ from min / max only on NaN
   if constexpr (ADD == kMinimum) acc = __builtin_elementwise_minimum(__builtin_elementwise_minimum(acc, t0), t1);
@@ -57,7 +69,8 @@ template <int ADD, int MUL> __device__ __forceinline__ void two_terms(h2 &acc, h
   else acc = pk<ADD>(pk<ADD>(acc, t0), t1);
 }
 template <int ADD, int MUL> __device__ __forceinline__ void one_term(h2 &acc, h2 a, h2 b) {
-  acc = pk<ADD>(acc, pk<MUL>(a, b));
+  if constexpr (masked<ADD, MUL>::value) acc = or_and_pair(acc, a, b);
+  else acc = pk<ADD>(acc, pk<MUL>(a, b));
 }
 
 __device__ __forceinline__ h2 both(half_t v) { return h2{v, v}; }
@@ -73,7 +86,12 @@ template <> __device__ __forceinline__ half_t to_half<half_t>(half_t v) { return
 // One operand's share of a k-tile on its way from memory to LDS.  The panel is X wide (X = BM for A, BN
 // for B); a chunk is 8 elements: of one k and 8 consecutive x when x is the contiguous direction in
 // memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
-template <int X, bool KC, bool GUARD, typename TI> struct Stager {
+template <int X, bool KC, bool GUARD, typename TI, bool MASK = false> struct Stager {
+  // what goes to LDS for one operand: its binary16 value, or (MASK) all ones / zero for non-zero / zero
+  static __device__ __forceinline__ half_t staged(TI v) {
+    if constexpr (MASK) return __builtin_bit_cast(half_t, (unsigned short)(v != TI(0) ? 0xffff : 0));
+    else return to_half<TI>(v);
+  }
   typedef typename vec8<TI>::type raw8;
   // the same eight operands at any element boundary (the hardware takes a vector load at any address)
   typedef TI loose8 __attribute__((ext_vector_type(8), aligned(sizeof(TI))));
@@ -90,10 +108,10 @@ template <int X, bool KC, bool GUARD, typename TI> struct Stager {
   // xn, kn: the extents (elements beyond them read as zero and are never used in a result that is stored).
   // In the guarded form a chunk that lies wholly inside the extents is read as a vector all the same, at whatever
   // element boundary it starts; only chunks across an edge are read element by element
-  static __device__ __forceinline__ h8 widen(const raw8 &v) {
+  template <typename V> static __device__ __forceinline__ h8 widen(const V v) {
     h8 h;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) h[e] = to_half<TI>(v[e]);
+    for (int e = 0; e < 8; ++e) h[e] = staged(v[e]);
     return h;
   }
   __device__ __forceinline__ void load(const TI *base, long long sx, long long sk, int x0, int k0, int xn, int kn) {
@@ -113,7 +131,7 @@ template <int X, bool KC, bool GUARD, typename TI> struct Stager {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
             const int xe = x0 + x + (KC ? 0 : e), ke = k0 + k + (KC ? e : 0);
-            r[q][e] = (xe < xn && ke < kn) ? to_half<TI>(src[(KC ? sk : sx) * e]) : half_t(0);
+            r[q][e] = (xe < xn && ke < kn) ? staged(src[(KC ? sk : sx) * e]) : half_t(0);
           }
         }
       }
@@ -151,6 +169,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   constexpr int BM = 16 * TR, BN = 128 * NG;
   constexpr bool BYTES = std::is_same<TI, int8_t>::value;
   constexpr bool ZERO_SIGN = !BYTES && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum);
+  constexpr bool MASKED = masked<ADD, MUL>::value;
   typedef typename out_of<TI>::type TO;
   typedef typename vec8<TO>::type out8;
   typedef typename frag_of<TR>::type rows_t;
@@ -166,7 +185,9 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   }
   const TI *A = reinterpret_cast<const TI *>(p.A), *B = reinterpret_cast<const TI *>(p.B);
   // int8 operands: the loop starts from the binary16 infinity of its add; the caller's identity joins at the end
-  const half_t ident = BYTES ? half_t(ADD == kMinimum ? __builtin_inff() : -__builtin_inff()) : scalar_as<half_t>(p.add_identity);
+  // (or-and: the loop ors masks, starting from none; the caller's identity joins at the end as well)
+  const half_t ident = MASKED ? half_t(0)
+                       : BYTES ? half_t(ADD == kMinimum ? __builtin_inff() : -__builtin_inff()) : scalar_as<half_t>(p.add_identity);
 
   h2 acc[TR][4 * NG];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
 #pragma unroll
@@ -174,8 +195,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int j = 0; j < 4 * NG; ++j) acc[i][j] = both(ident);
 
-  Stager<BM, A_KC, GUARD, TI> sa;
-  Stager<BN, B_KC, GUARD, TI> sb;
+  Stager<BM, A_KC, GUARD, TI, MASKED> sa;
+  Stager<BN, B_KC, GUARD, TI, MASKED> sb;
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   if (tiles_k > 0) {
     sa.load(A, p.sa_m, p.sa_k, m0, kb, p.m, ke);
@@ -246,7 +267,11 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const half_t a = acc[i][g * 4 + j / 2][j % 2];
-        if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
+        if constexpr (MASKED) {
+          // the reference's accumulator after k > 0 terms: 1 if any term or the identity is non-zero, else 0
+          const bool any = __builtin_bit_cast(unsigned short, a) != 0 || e.ident != TO(0);
+          v[j] = tiles_k > 0 ? TO(any ? 1 : 0) : e.ident;
+        } else if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
         else v[j] = a;
         if constexpr (ZERO_SIGN) {
           // a minimum / maximum that is zero: the reference's comparison keeps the newer of two equal operands
@@ -350,7 +375,7 @@ template <int ADD, int MUL, typename TI = half_t> static hipError_t launch(const
 
 // The semirings whose operators are each one packed instruction.  Sums, minima and maxima of data free of -0
 // never produce -0; products do, so min-times and max-times settle the sign of a zero result in the epilogue
-// (ZERO_SIGN in the kernel).  The logical pairs stay on the naive kernel.
+// (ZERO_SIGN in the kernel).  or-and runs on masks.
 launch_fn find_valu_f16(int add_op, int mult_op) {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL>;
@@ -361,11 +386,12 @@ launch_fn find_valu_f16(int add_op, int mult_op) {
   PAIR(kPlus, kMultiplies)
   PAIR(kMinimum, kMultiplies)
   PAIR(kMaximum, kMultiplies)
+  PAIR(kLogicalOr, kLogicalAnd)
 #undef PAIR
   return nullptr;
 }
 
-// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16)
+// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16), and or-and
 launch_fn find_valu_i8(int add_op, int mult_op) {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL, int8_t>;
@@ -373,6 +399,7 @@ launch_fn find_valu_i8(int add_op, int mult_op) {
   PAIR(kMaximum, kPlus)
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
+  PAIR(kLogicalOr, kLogicalAnd)
 #undef PAIR
   return nullptr;
 }

@@ -83,7 +83,8 @@ def test_half_and_int8_element_types(lib):
     assert sel(desc(dtype="f16")) == b"valu" and sel(desc(dtype="f16", m=63, n=1, k=5)) == b"valu"
     assert sel(desc(dtype="f16", add="plus", mult="multiplies")) == b"valu"
     assert sel(desc(dtype="f16", add="minimum", mult="multiplies")) == b"valu"
-    assert sel(desc(dtype="f16", add="logical_or", mult="logical_and")) == b"naive"
+    assert sel(desc(dtype="f16", add="logical_or", mult="logical_and")) == b"valu"
+    assert sel(desc(dtype="f16", add="plus", mult="maximum")) == b"naive"
     assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "f16") == 2 * 100 * 7 * 3
     # int8 operands, int32 everything else: A and B at any byte, C and D at four; every integer pair is defined
     d = desc(dtype="i8", add="plus", mult="multiplies")

@@ -9,8 +9,8 @@ from helpers import assert_same_bits, order_of, to_device
 pytestmark = pytest.mark.gpu
 
 TILE_PAIRS = [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"), ("plus", "multiplies"),
-              ("minimum", "multiplies"), ("maximum", "multiplies")]
-OTHER_PAIRS = [("logical_or", "logical_and")]
+              ("minimum", "multiplies"), ("maximum", "multiplies"), ("logical_or", "logical_and")]
+OTHER_PAIRS = [("plus", "maximum"), ("logical_or", "plus")]     # (pairs no tile serves: the naive kernel)
 LAYOUTS = ["ccc", "rrr", "crc", "rcr", "rcc", "crr", "ccr", "rrc"]
 
 
@@ -22,8 +22,9 @@ def operands(add, mult, m, n, k, la, lb, lc, seed=1):
     B = inputs.uniform(seed + 1, k, n, lo, hi, np.float16, order_of(lb))
     C = inputs.uniform(seed + 2, m, n, lo, hi, np.float16, order_of(lc))
     if mult == "logical_and":
-        A[A < 30] = 0
-        B[B < 30] = 0
+        A[A < 97] = 0          # sparse, and zeros of both signs: -0 is false as well
+        B[B < 97] = 0
+        A[::3, ::5] = np.float16(-0.0)
     return A, B, C
 
 
@@ -84,7 +85,7 @@ def test_selected_family(lib):
     dB = to_device(np.zeros((64, 256), np.float16))
     dD = to_device(np.zeros((128, 256), np.float16))
     for (add, mult), name in [(("minimum", "plus"), b"valu"), (("plus", "multiplies"), b"valu"), (("minimum", "multiplies"), b"valu"),
-                              (("logical_or", "logical_and"), b"naive")]:
+                              (("logical_or", "logical_and"), b"valu"), (("plus", "maximum"), b"naive")]:
         ident, one, zero = scalars(add, mult, False)
         desc = cuasr_amd.make_desc(add, mult, "f16", dA, dB, dD, dD, one, zero, ident, one)
         assert lib.cuasr_amd_selected_kernel(desc) == name
@@ -99,6 +100,18 @@ def test_every_pair(oracle, lib, sr, kernel):
     for layouts in ("ccc", "rcr"):
         check(oracle, *sr, 70, 90, 33, layouts, kernel)
         check(oracle, *sr, 128, 256, 64, layouts, kernel, beta_one=False)
+
+
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc"])
+def test_boolean_closure_on_masks(oracle, lib, layouts):
+    """or-and (functional.h:212, :252): the tile works on 16-bit masks; sparse operands so that the answer is
+    not all ones, every tile size, an identity that is not zero, alpha / beta that are zero or not."""
+    check(oracle, "logical_or", "logical_and", 1024, 1024, 64, layouts, "valu")      # 32 x 128 tiles
+    check(oracle, "logical_or", "logical_and", 2048, 2048, 40, layouts, "valu")      # 64 x 128 tiles
+    check(oracle, "logical_or", "logical_and", 4096, 4096, 32, layouts, "valu")      # full tiles, unguarded
+    check(oracle, "logical_or", "logical_and", 4000, 4100, 37, layouts, "valu", beta_one=False)
+    check(oracle, "logical_or", "logical_and", 300, 200, 45, layouts, "valu", alpha=0.0, beta=2.5)
+    check(oracle, "logical_or", "logical_and", 300, 200, 45, layouts, "valu", alpha=-3.0, beta=0.0)
 
 
 @pytest.mark.parametrize("add", ["minimum", "maximum"])

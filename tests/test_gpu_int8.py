@@ -56,7 +56,7 @@ def test_selected_family(lib):
     dB = to_device(np.zeros((64, 256), np.int8))
     dD = to_device(np.zeros((128, 256), np.int32))
     for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"valu"), (("maximum", "minimum"), b"valu"),
-                              (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"naive")]:
+                              (("logical_or", "logical_and"), b"valu"), (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"naive")]:
         desc = cuasr_amd.make_desc(add, mult, "i8", dA, dB, dD, dD, 1, 0, 0, 1)
         assert lib.cuasr_amd_selected_kernel(desc) == name
 
@@ -81,6 +81,27 @@ def test_tropical_pairs_on_the_packed_tile(oracle, lib, sr, layouts):
     check(oracle, *sr, 2048, 2048, 96, layouts, "valu", alpha=7, beta=-3)    # 64 x 128 tiles
     check(oracle, *sr, 4096, 4096, 64, layouts, "valu")                      # full tiles, unguarded
     check(oracle, *sr, 4000, 4100, 70, layouts, "valu", alpha=-100, beta=100)  # full tiles, guarded
+
+
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc"])
+def test_boolean_closure_on_masks(oracle, lib, layouts):
+    """or-and on int8 operands: sparse (most entries zero), so that the answer is not all ones; every tile size;
+    an identity that is not zero."""
+    import torch
+    import cuasr_amd
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    rng = np.random.default_rng(23)
+    for (m, n, k), ident in [((1024, 1024, 64), 0), ((2048, 2048, 40), 0), ((4096, 4096, 32), 0), ((4000, 4100, 37), 0),
+                             ((300, 200, 45), 7), ((70, 90, 1), 0)]:
+        A = np.asarray(np.where(rng.random((m, k)) < 0.03, rng.integers(-128, 128, (m, k)), 0).astype(np.int8), order=order_of(la))
+        B = np.asarray(np.where(rng.random((k, n)) < 0.03, rng.integers(-128, 128, (k, n)), 0).astype(np.int8), order=order_of(lb))
+        C = np.asarray(np.where(rng.random((m, n)) < 0.1, rng.integers(-5, 6, (m, n)), 0).astype(np.int32), order=order_of(lc))
+        want = oracle.srgemm("logical_or", "logical_and", A, B, C, 1, 1, ident)
+        assert ident != 0 or 0.02 < (want != 0).mean() < 0.98
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm("logical_or", "logical_and", to_device(A), to_device(B), to_device(C), dD, 1, 1, ident, 1, dtype="i8", kernel="valu")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"or-and i8 {m}x{n}x{k} {layouts} identity {ident}")
 
 
 def test_tropical_identity_that_is_not_infinite(oracle, lib):
