@@ -157,7 +157,18 @@ template <int X, bool KC, bool GUARD, typename TI, bool MASK = false> struct Sta
 // the last product of a k range that is zero (acc itself when there is none); not inlined: it runs after the main loop
 static __device__ __attribute__((noinline)) half_t last_zero_product(const half_t *a_row, long long sa_k, const half_t *b_col,
                                                                      long long sb_k, int kcount, half_t acc) {
-  for (int kk = kcount - 1; kk >= 0; --kk) {
+  // sixteen k at a time, so that the loads of a step are in flight together (one lane scans alone: a step costs a
+  // memory latency whatever it fetches)
+  int kk = kcount - 1;
+  for (; kk >= 15; kk -= 16) {
+    half_t prod[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) prod[u] = a_row[(long long)(kk - u) * sa_k] * b_col[(long long)(kk - u) * sb_k];
+#pragma unroll
+    for (int u = 0; u < 16; ++u)
+      if (prod[u] == half_t(0)) return prod[u];
+  }
+  for (; kk >= 0; --kk) {
     const half_t prod = a_row[(long long)kk * sa_k] * b_col[(long long)kk * sb_k];
     if (prod == half_t(0)) return prod;
   }

@@ -12,7 +12,8 @@ _M2 = np.uint64(0x94D049BB133111EB)
 
 
 def splitmix64(seed, count, offset=0):
-    """``count`` 64-bit words: word i is mix(seed*G + (offset+i+1)*G)."""
+    """``count`` 64-bit words: word i is mix(seed*G + (offset+i+1)*G).  (So seed s + 1 gives the stream of
+    seed s moved on by one word: matrices that must be unrelated take seeds further apart than their size.)"""
     with np.errstate(over="ignore"):
         idx = np.arange(offset + 1, offset + count + 1, dtype=np.uint64)
         z = (np.uint64(seed) * _GOLDEN + np.uint64(0x632BE59BD9B4E019)) + idx * _GOLDEN
