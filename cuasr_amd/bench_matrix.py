@@ -71,7 +71,6 @@ def main():
         data = {}
         for n in sizes:
             # one buffer per operand and size; a layout is only a way of reading it
-            if dt == "i8":
             # (seeds far apart: the generator is counter-based, and neighbouring seeds give the same stream shifted
             # by one element -- B would be A moved down a row)
             if dt == "i8":
