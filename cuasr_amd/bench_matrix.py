@@ -71,13 +71,13 @@ def main():
         data = {}
         for n in sizes:
             # one buffer per operand and size; a layout is only a way of reading it
-            # (seeds far apart: the generator is counter-based, and neighbouring seeds give the same stream shifted
-            # by one element -- B would be A moved down a row)
+            # (seeds further apart than a matrix has elements: the generator is counter-based, and seed s + d gives the
+            # stream of seed s moved on by d words -- B would be A moved down by d rows)
             if dt == "i8":
-                data[n] = [torch.from_numpy(inputs.integers(901 + 1000 * i, n, n, -128, 127, np.int8, "C")).cuda() for i in range(2)]
-                data[n].append(torch.from_numpy(inputs.integers(2901, n, n, -1000, 1000, np.int32, "C")).cuda())
+                data[n] = [torch.from_numpy(inputs.integers(901 + (i << 40), n, n, -128, 127, np.int8, "C")).cuda() for i in range(2)]
+                data[n].append(torch.from_numpy(inputs.integers(901 + (2 << 40), n, n, -1000, 1000, np.int32, "C")).cuda())
             else:
-                data[n] = [torch.from_numpy(inputs.uniform(901 + 1000 * i, n, n, -1.0, 1.0, npd, "C")).cuda() for i in range(3)]
+                data[n] = [torch.from_numpy(inputs.uniform(901 + (i << 40), n, n, -1.0, 1.0, npd, "C")).cuda() for i in range(3)]
             data[n].append(torch.empty(n, n, dtype=tdt, device="cuda"))
         for add, mult in SEMIRINGS:
             ident = cuasr_amd.op_identity(add, dt, True)
