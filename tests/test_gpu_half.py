@@ -213,3 +213,29 @@ def test_no_terms(oracle, lib):
     # k = 0: the accumulator is the additive identity and only the epilogue runs
     check(oracle, "minimum", "plus", 40, 50, 0, "ccc", "auto")
     check(oracle, "plus", "multiplies", 128, 256, 0, "rcr", "valu")
+
+
+@pytest.mark.parametrize("slices", [1, 2, 5])
+def test_serial_splitk(oracle, lib, slices):
+    """The serial split-K chain of epilogues in binary16 (small integers: the sums inside a slice are exact in
+    any order; alpha multiplies every slice's partial product, as in the reference)."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    for (add, mult, alpha, beta, ident, one), layouts in [(("minimum", "plus", 3.0, 0.0, np.inf, 0.0), "ccc"),
+                                                           (("plus", "multiplies", 2.0, -3.0, 0.0, 1.0), "rcr"),
+                                                           (("maximum", "minimum", 5.0, np.inf, -np.inf, np.inf), "crc")]:
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        m, n, k = 130, 258, 200
+        A = inputs.integers(31, m, k, -4, 4, np.float16, order_of(la))
+        B = inputs.integers(1031, k, n, -4, 4, np.float16, order_of(lb))
+        C = inputs.integers(2031, m, n, -4, 4, np.float16, order_of(lc))
+        f = np.float16
+        want = oracle.srgemm_splitk_serial(add, mult, A, B, C, f(alpha), f(beta), f(ident), f(one), slices)
+        nbytes = cuasr_amd.splitk_serial_workspace_bytes(m, n, slices, "f16")
+        assert nbytes == (2 * m * n * slices if slices > 1 else 0)
+        ws = torch.full((nbytes // 2 + 8,), float("nan"), dtype=torch.float16, device="cuda") if nbytes else None
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm_splitk_serial(add, mult, to_device(A), to_device(B), to_device(C), dD, slices, ws, f(alpha), f(beta), f(ident), f(one), dtype="f16")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"serial split-K f16 {add}-{mult} {layouts} S={slices}")

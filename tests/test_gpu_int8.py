@@ -174,3 +174,23 @@ def test_batch_in_the_grid(oracle, lib):
         for i in range(batch):
             want = oracle.srgemm("plus", "multiplies", A[i], B[i], C[i], 1, 1, 0)
             assert_same_bits(got[i], want, f"batch product {i} of {m}x{n}x{k}")
+
+
+@pytest.mark.parametrize("slices", [1, 2, 5])
+def test_serial_splitk(oracle, lib, slices):
+    """The serial split-K chain of epilogues on int8 operands (integer arithmetic: exact in any order)."""
+    import torch
+    import cuasr_amd
+    for (add, mult, alpha, beta, ident, one), layouts in [(("plus", "multiplies", 2, -3, 0, 1), "rcr"),
+                                                           (("minimum", "plus", 3, 0, 2 ** 31 - 1, 0), "ccc")]:
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        m, n, k = 130, 258, 200
+        A, B, C = operands(m, n, k, la, lb, lc, seed=41)
+        want = oracle.srgemm_splitk_serial(add, mult, A, B, C, alpha, beta, ident, one, slices)
+        nbytes = cuasr_amd.splitk_serial_workspace_bytes(m, n, slices, "i8")
+        assert nbytes == (4 * m * n * slices if slices > 1 else 0)
+        ws = torch.full((nbytes // 4 + 4,), 0x7FC00000, dtype=torch.int32, device="cuda") if nbytes else None
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm_splitk_serial(add, mult, to_device(A), to_device(B), to_device(C), dD, slices, ws, alpha, beta, ident, one, dtype="i8")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"serial split-K i8 {add}-{mult} {layouts} S={slices}")
