@@ -31,7 +31,11 @@ bool mfma_f64_can_run(const Problem &);
 bool mfma_direct_f32_can_run(const Problem &);
 bool mfma_direct_f64_can_run(const Problem &);
 
+launch_fn find_or_and_on_masks(int dtype);
+
 launch_fn find_valu(int dtype, int add_op, int mult_op) {
+  if (add_op == kLogicalOr && mult_op == kLogicalAnd)
+    if (launch_fn f = find_or_and_on_masks(dtype)) return f;  // float, double: the packed mask tile for large outputs
   switch (dtype) {
     case CUASR_AMD_F32: return find_valu_f32(add_op, mult_op);
     case CUASR_AMD_F64: return find_valu_f64(add_op, mult_op);

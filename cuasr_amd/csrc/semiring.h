@@ -42,6 +42,22 @@ template <> __device__ __forceinline__ double hw_max<double>(double l, double r)
 // The two differ only when the operands are +0 and -0 (or NaN).  Sums, minima
 // and maxima of data free of -0 never produce -0; products do (0 * negative),
 // so kernels use the strict form wherever `multiplies` feeds a min or max.
+// What the logical operators ask of an operand: is it anything but zero?  +0 and -0 are false, NaN is true
+// (functional.h:212, :252 convert to bool).  Floating point is asked by its bit pattern, and the pattern passes
+// through an empty asm statement: the compiler recognises the integer test of a bit-cast float as a floating-point
+// comparison, and in a translation unit that lets it assume NaN-free data it then picks the ordered one (NaN false).
+template <typename T> __device__ __forceinline__ bool truth(T x) {
+  if constexpr (is_fp<T>::value) {
+    typedef typename std::conditional<sizeof(T) == 8, uint64_t, typename std::conditional<sizeof(T) == 4, uint32_t, uint16_t>::type>::type bits_t;
+    typedef typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type reg_t;
+    reg_t bits = __builtin_bit_cast(bits_t, x);
+    asm("" : "+v"(bits));
+    return reg_t(bits << (sizeof(T) == 2 ? 17 : 1)) != 0;
+  } else {
+    return x != T(0);
+  }
+}
+
 template <int OP> struct Op {
   template <typename T> static __device__ __forceinline__ T strict(T l, T r) {
     if constexpr (std::is_same<T, half_t>::value && (OP == kMinimum || OP == kMaximum)) {
@@ -62,8 +78,8 @@ template <int OP> struct Op {
     else if constexpr (OP == kMultiplies) return l * r;
     else if constexpr (OP == kMinimum) return hw_min<T>(l, r);
     else if constexpr (OP == kMaximum) return hw_max<T>(l, r);
-    else if constexpr (OP == kLogicalAnd) return T((l != T(0)) && (r != T(0)));
-    else if constexpr (OP == kLogicalOr) return T((l != T(0)) || (r != T(0)));
+    else if constexpr (OP == kLogicalAnd) return T(truth(l) && truth(r));
+    else if constexpr (OP == kLogicalOr) return T(truth(l) || truth(r));
     else if constexpr (!is_fp<T>::value) {
       if constexpr (OP == kBitAnd) return l & r;
       else if constexpr (OP == kBitOr) return l | r;

@@ -1,0 +1,38 @@
+// The packed half-precision tile (half_tile.h) for operands that are not binary16: int8 (exact in binary16 for the
+// tropical pairs), and float / double for or-and, whose operands reach LDS as masks.
+#include "half_tile.h"
+
+namespace cuasr_amd {
+
+// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16), and or-and
+launch_fn find_valu_i8(int add_op, int mult_op) {
+#define PAIR(ADD, MUL) \
+  if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL, int8_t>;
+  PAIR(kMinimum, kPlus)
+  PAIR(kMaximum, kPlus)
+  PAIR(kMinimum, kMaximum)
+  PAIR(kMaximum, kMinimum)
+  PAIR(kLogicalOr, kLogicalAnd)
+#undef PAIR
+  return nullptr;
+}
+
+// or-and on float / double operands.  The operators only ask whether an operand is zero, so nothing of the
+// element type survives the trip to LDS: large outputs take the 16-bit mask form of the packed tile (two terms per
+// three-input bit operation; 4096^3: 128 TOPS against 84 on the staged tile's 32-bit masks), smaller ones, which the
+// packed tile's large workgroups would leave most of the chip idle on, stay on the staged tile.
+launch_fn find_valu_f32(int add_op, int mult_op);
+launch_fn find_valu_f64(int add_op, int mult_op);
+template <typename T> static hipError_t or_and_on_masks(const Problem &p, hipStream_t s) {
+  const long long full = (long long)((p.m + 127) / 128) * ((p.n + 255) / 256) * (p.workspace ? p.slices : 1) * p.batch;
+  if (full >= 384) return half_tile::launch<kLogicalOr, kLogicalAnd, T>(p, s);
+  const launch_fn staged = sizeof(T) == 8 ? find_valu_f64(kLogicalOr, kLogicalAnd) : find_valu_f32(kLogicalOr, kLogicalAnd);
+  return staged ? staged(p, s) : hipErrorNotSupported;
+}
+launch_fn find_or_and_on_masks(int dtype) {
+  if (dtype == CUASR_AMD_F32) return or_and_on_masks<float>;
+  if (dtype == CUASR_AMD_F64) return or_and_on_masks<double>;
+  return nullptr;
+}
+
+}  // namespace cuasr_amd

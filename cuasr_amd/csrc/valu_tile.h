@@ -65,7 +65,7 @@ struct ValuTile {
   using S = typename std::conditional<MASKED, uint32_t, T>::type;  // what LDS, fragments and accumulators hold
   typedef S svec_t __attribute__((ext_vector_type(VW)));
   static __device__ __forceinline__ S staged(T x) {
-    if constexpr (MASKED) return x != T(0) ? 0xFFFFFFFFu : 0u;
+    if constexpr (MASKED) return truth(x) ? 0xFFFFFFFFu : 0u;
     else return x;
   }
   static constexpr bool FUSED = fused_bit_term<ADD, MUL, T>::value;

@@ -76,7 +76,22 @@ def test_every_tile_size(oracle, lib, layouts):
     check(oracle, "maximum", "minimum", 4000, 4100, 70, layouts, "valu", False)    # full tiles, ragged: guarded
     check(oracle, "minimum", "plus", 2048, 2048, 96, layouts, "valu")              # 64 x 128 tiles
     check(oracle, "plus", "multiplies", 1000, 2000, 50, layouts, "valu")           # 64 x 128 tiles, ragged
-    check(oracle, "maximum", "plus", 1024, 1024, 64, layouts, "valu")              # 32 x 128 tiles
+    check(oracle, "maximum", "plus", 1536, 1536, 64, layouts, "valu")              # 32 x 128 tiles, k shared out between the waves
+    check(oracle, "maximum", "plus", 1024, 1024, 64, layouts, "valu")              # 16 x 128 tiles, likewise
+    check(oracle, "plus", "multiplies", 1024, 1024, 64, layouts, "valu")           # 32 x 128 tiles, whole k-tiles per thread
+
+
+@pytest.mark.parametrize("sr", [x for x in TILE_PAIRS if x[0] != "plus"])
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc"])
+def test_k_shared_out_between_waves(oracle, lib, sr, layouts):
+    """The two small tiles of the order-free adds: each wave takes a quarter of every k-tile and the four partial
+    accumulators meet in LDS.  k that ends inside the first, second, third, fourth quarter of a tile; one tile; k
+    shorter than a quarter; extents that are no multiple of anything; and the split-K forms on top."""
+    for k in (3, 9, 17, 31, 32, 45, 64, 250):
+        check(oracle, *sr, 520, 390, k, layouts, "valu", beta_one=bool(k & 1))       # 16 x 128 tiles
+    check(oracle, *sr, 1530, 1300, 77, layouts, "valu")                             # 32 x 128 tiles
+    check(oracle, *sr, 1530, 1300, 32, layouts, "valu", beta_one=False)
+    check(oracle, *sr, 300, 260, 500, layouts, "valu", splitk=5)
 
 
 def test_selected_family(lib):

@@ -115,6 +115,9 @@ def test_or_and_on_truth_values_of_arbitrary_operands(oracle, lib, dtype, kernel
         la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
         A, B = sparse(11, m, k, npd, order_of(la)), sparse(12, k, n, npd, order_of(lb))
         C = sparse(13, m, n, npd, order_of(lc), 0.3)
+        if dtype in ("f32", "f64"):
+            A.flat[::17], B.flat[::19], C.flat[::23] = npd("nan"), npd("-inf"), npd("nan")   # true, all of them
+            A.flat[1::17] = npd(-0.0)                                                        # false
         for alpha, beta in ((1, 0), (1, 1), (0, 1), (7, 3)):   # any non-zero scalar is "true"
             want = oracle.srgemm("logical_or", "logical_and", A, B, C, alpha, beta, 0)
             try:
@@ -130,6 +133,50 @@ def test_or_and_on_truth_values_of_arbitrary_operands(oracle, lib, dtype, kernel
     if not ran:
         pytest.skip(f"{kernel} does not run or-and on {dtype}")
     assert ones > 1000 and zeros > 1000, "the inputs must produce both truth values"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc", "rrr", "ccr"])
+def test_or_and_large_outputs_on_packed_masks(oracle, lib, dtype, layouts):
+    """From 384 tiles of 128 x 256 on, float and double or-and runs on the 16-bit mask tile: whole tiles of aligned
+    operands, ragged extents, an identity that is not zero, scalars that are zero, and operands that hold -0 (false),
+    NaN and infinities (true, functional.h:212)."""
+    import cuasr_amd
+    npd = NPD[dtype]
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for (m, n, k), ident, alpha, beta in (((4096, 3072, 64), 0, 1, 1), ((4000, 4100, 37), 0, 1, 0), ((4000, 4100, 37), 0, 0, 1),
+                                          ((3968, 3328, 33), 2.5, 1, 1)):
+        A, B = sparse(31, m, k, npd, order_of(la), 0.06), sparse(32, k, n, npd, order_of(lb), 0.06)
+        C = sparse(33, m, n, npd, order_of(lc), 0.3)
+        A[::7, ::3] = npd(-0.0)
+        A[5::11, 1::4] = npd("nan")
+        B[2::13, ::5] = npd("inf")
+        want = oracle.srgemm("logical_or", "logical_and", A, B, C, alpha, beta, ident)
+        print(f"or-and {dtype} {m}x{n}x{k} {layouts} ident={ident} alpha={alpha} beta={beta}", flush=True)
+        for kernel in ("auto", "valu"):
+            got = launch("logical_or", "logical_and", dtype, A, B, C, alpha, beta, ident, 1, kernel)
+            assert_same_bits(got, want, f"or-and {dtype} {m}x{n}x{k} {layouts} {kernel} ident={ident} alpha={alpha} beta={beta}")
+        if ident == 0 and (alpha, beta) == (1, 0):
+            assert 0.1 < (want == 1).mean() < 0.9, "the inputs must produce both truth values"
+    dA = to_device(np.zeros((4096, 64), npd))
+    dB = to_device(np.zeros((64, 3072), npd))
+    dD = to_device(np.zeros((4096, 3072), npd))
+    assert lib.cuasr_amd_selected_kernel(cuasr_amd.make_desc("logical_or", "logical_and", dtype, dA, dB, dD, dD, 1, 1, 0, 1)) == b"valu"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f64"])
+def test_or_and_split_k_on_packed_masks(oracle, lib, dtype):
+    """Slices count towards the 384 workgroups: 8 x 8 tiles in 6 or 7 slices run the mask tile into the workspace."""
+    npd = NPD[dtype]
+    m, n, k = 1024, 2048, 700
+    A, B, C = sparse(41, m, k, npd, "C", 0.02), sparse(42, k, n, npd, "F", 0.02), sparse(43, m, n, npd, "C", 0.3)
+    for slices in (6, 7):
+        for beta in (0, 1):
+            want = oracle.srgemm("logical_or", "logical_and", A, B, C, 1, beta, 0)
+            got = launch("logical_or", "logical_and", dtype, A, B, C, 1, beta, 0, 1, "valu", splitk=slices)
+            assert_same_bits(got, want, f"split-K or-and {dtype} S={slices} beta={beta}")
+            got = launch("logical_or", "logical_and", dtype, A, B, C, 1, beta, 0, 1, "valu", splitk=slices, serial=True)
+            assert_same_bits(got, want, f"serial split-K or-and {dtype} S={slices} beta={beta}")
 
 
 @pytest.mark.parametrize("dtype", ["f32", "i32"])

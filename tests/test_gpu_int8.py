@@ -76,7 +76,9 @@ def test_tropical_pairs_on_the_packed_tile(oracle, lib, sr, layouts):
     """Sums, minima and maxima of two int8 values are exact in binary16: these pairs run on the packed
     half-precision tile (operands converted on their way to LDS, integer epilogue).  Every tile size, aligned and
     ragged, identities and scalars that are not the semiring's own."""
-    check(oracle, *sr, 100, 300, 45, layouts, "valu")                        # 32 x 128 tiles, ragged
+    check(oracle, *sr, 100, 300, 45, layouts, "valu")                        # 16 x 128 tiles, k shared out between the waves, ragged
+    check(oracle, *sr, 1530, 1300, 77, layouts, "valu", alpha=3, beta=-2)    # 32 x 128 tiles, likewise
+    check(oracle, *sr, 520, 390, 9, layouts, "valu")                         # k shorter than a tile
     check(oracle, *sr, 1, 1, 1, layouts, "valu")
     check(oracle, *sr, 2048, 2048, 96, layouts, "valu", alpha=7, beta=-3)    # 64 x 128 tiles
     check(oracle, *sr, 4096, 4096, 64, layouts, "valu")                      # full tiles, unguarded
@@ -92,7 +94,7 @@ def test_boolean_closure_on_masks(oracle, lib, layouts):
     la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
     rng = np.random.default_rng(23)
     for (m, n, k), ident in [((1024, 1024, 64), 0), ((2048, 2048, 40), 0), ((4096, 4096, 32), 0), ((4000, 4100, 37), 0),
-                             ((300, 200, 45), 7), ((70, 90, 1), 0)]:
+                             ((300, 200, 45), 7), ((70, 90, 1), 0), ((1530, 1300, 50), 0)]:
         A = np.asarray(np.where(rng.random((m, k)) < 0.03, rng.integers(-128, 128, (m, k)), 0).astype(np.int8), order=order_of(la))
         B = np.asarray(np.where(rng.random((k, n)) < 0.03, rng.integers(-128, 128, (k, n)), 0).astype(np.int8), order=order_of(lb))
         C = np.asarray(np.where(rng.random((m, n)) < 0.1, rng.integers(-5, 6, (m, n)), 0).astype(np.int32), order=order_of(lc))
