@@ -90,6 +90,8 @@ template <typename TI> struct out_of { typedef half_t type; };
 template <> struct out_of<int8_t> { typedef int32_t type; };
 template <> struct out_of<float> { typedef float type; };    // (or-and only: the operands go to LDS as masks)
 template <> struct out_of<double> { typedef double type; };
+template <> struct out_of<int32_t> { typedef int32_t type; };
+template <> struct out_of<uint32_t> { typedef uint32_t type; };
 template <typename T> struct vec8 { typedef T type __attribute__((ext_vector_type(8), aligned(sizeof(T) * 8 < 16 ? sizeof(T) * 8 : 16))); };
 template <typename TI> __device__ __forceinline__ half_t to_half(TI v) { return half_t(float(v)); }
 template <> __device__ __forceinline__ half_t to_half<half_t>(half_t v) { return v; }
