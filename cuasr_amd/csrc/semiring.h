@@ -69,6 +69,14 @@ template <int OP> struct Op {
       const int lk = (lb & 0x8000) ? -(int)(lb & 0x7fff) : (int)(lb & 0x7fff);
       const bool take_r = OP == kMinimum ? rk < lk : lk < rk;
       return __builtin_bit_cast(half_t, (unsigned short)(take_r ? rb : lb));
+    } else if constexpr (is_fp<T>::value && (OP == kMinimum || OP == kMaximum)) {
+      // float, double: the operand the comparison may pick passes through an empty asm statement.  Written plainly,
+      // in a translation unit that assumes NaN-free data the compiler turns compare-and-select into the min / max
+      // instruction, which returns -0 for a +0 / -0 tie whatever the operand order (min(+0, 0 * C) with C < 0 then
+      // comes out as -0 where the reference keeps the left operand).
+      T picked = r;
+      asm("" : "+v"(picked));
+      return (OP == kMinimum ? r < l : l < r) ? picked : l;
     } else if constexpr (OP == kMinimum) return r < l ? r : l;
     else if constexpr (OP == kMaximum) return l < r ? r : l;
     else return apply(l, r);
