@@ -34,7 +34,7 @@ inline cuasr_amd_srgemm_desc make_desc(Args const &a, int kernel) {
   cuasr_amd_srgemm_desc d{};
   d.add_op = op_tag<typename Op::AdditionOp>::value;
   d.mult_op = op_tag<typename Op::MultiplicationOp>::value;
-  d.dtype = dtype_tag<Element>::value;
+  d.dtype = element_types<typename Op::ElementA, typename Op::ElementB, Element, typename Op::ElementAccumulator>::value;
   d.layout_a = Op::LayoutA::kAbiTag;
   d.layout_b = Op::LayoutB::kAbiTag;
   d.layout_c = Op::LayoutC::kAbiTag;
@@ -115,10 +115,12 @@ class Srgemm {
   /// specialisation): the kernel is then built from the functors' operator() in this translation unit
   /// (cuasr/gemm/kernel/functor_srgemm.h), which needs hipcc; split-K is not offered for such functors
   static bool const kUserFunctors = op_tag<AdditionOp>::value < 0 || op_tag<MultiplicationOp>::value < 0;
+  static_assert(!kUserFunctors || (std::is_same<ElementA, ElementC>::value && sizeof(ElementC) >= 4),
+                "kernels built from user functors: float, double, int32_t or uint32_t throughout");
 
-  static_assert(std::is_same<ElementA, ElementC>::value && std::is_same<ElementB, ElementC>::value &&
-                    std::is_same<ElementAccumulator, ElementC>::value,
-                "A, B, C and the accumulator share one element type (as in every reference configuration)");
+  static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
+                "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
+                "are int8_t with int32_t C and accumulator");
 
   struct Arguments {
     GemmCoord problem_size;

@@ -77,9 +77,9 @@ class SrgemmSplitKParallel {
   using MultiplicationOp = MultiplicationOp_;
   static int const kStages = Stages;
 
-  static_assert(std::is_same<ElementA, ElementC>::value && std::is_same<ElementB, ElementC>::value &&
-                    std::is_same<ElementAccumulator, ElementC>::value,
-                "A, B, C and the accumulator share one element type");
+  static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
+                "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
+                "are int8_t with int32_t C and accumulator");
 
   struct Arguments {
     GemmCoord problem_size;

@@ -126,6 +126,131 @@ template <typename Add, typename Mul, typename T> static void testbed_sweep_seri
   report(ok, name);
 }
 
+// ---- the wider element types through the same operator templates: binary16 throughout (cuasr::half_t), and int8
+// operands with int32 results (the element types of the reference's dp4a cores, default_srmma_core_simt.h:747-757)
+template <typename Add, typename Mul, typename LA, typename LB, typename LC>
+static bool int8_case(int m, int n, int k, int32_t alpha, int32_t beta, int slices = 1) {
+  using Op = cuasr::gemm::device::Srgemm<Add, Mul, int8_t, LA, int8_t, LB, int32_t, LC, int32_t>;
+  const long long lda = ld_of<LA>(m, k), ldb = ld_of<LB>(k, n), ldc = ld_of<LC>(m, n);
+  std::vector<int8_t> A(size_t(m) * k), B(size_t(k) * n);
+  std::vector<int32_t> C(size_t(m) * n), D(size_t(m) * n, 0), R(size_t(m) * n, 0);
+  fill_int(A, 2019, -128, 127);
+  fill_int(B, 2018, -128, 127);
+  fill_int(C, 2017, -100000, 100000);
+  DeviceBuf<int8_t> dA(A), dB(B);
+  DeviceBuf<int32_t> dC(C), dD(D);
+  typename Op::Arguments args({m, n, k}, {dA.p, lda}, {dB.p, ldb}, {dC.p, ldc}, {dD.p, ldc}, {alpha, beta}, slices);
+  Op op;
+  if (Op::can_implement(args) != Status::kSuccess) return false;
+  if (op(args, nullptr) != Status::kSuccess) return false;
+  HIP_OK(hipDeviceSynchronize());
+  cuasr::reference::host::Srgemm<Add, Mul, int8_t, LA, int8_t, LB, int32_t, LC, int32_t, int32_t> ref;
+  ref({m, n, k}, alpha, {A.data(), lda}, {B.data(), ldb}, beta, {C.data(), ldc}, {R.data(), ldc}, Add::Identity);
+  D = dD.download();
+  return std::memcmp(D.data(), R.data(), D.size() * sizeof(int32_t)) == 0;
+}
+
+static void wider_element_types() {
+  using cuasr::half_t;
+  // the conversions of the host-side type, at the places where rounding decides
+  bool ok = half_t(1.0f).bits == 0x3c00 && half_t(-2.0f).bits == 0xc000 && half_t(65504.0f).bits == 0x7bff &&
+            half_t(65519.9f).bits == 0x7bff && half_t(65520.0f).bits == 0x7c00 && half_t(1.0f + 1.0f / 2048).bits == 0x3c00 &&
+            half_t(1.0f + 3.0f / 2048).bits == 0x3c02 && half_t(5.9604645e-8f).bits == 0x0001 && half_t(2.9802322e-8f).bits == 0x0000 &&
+            half_t(2.9802326e-8f).bits == 0x0001 && half_t(6.097555e-5f).bits == 0x03ff && half_t(6.1035156e-5f).bits == 0x0400 &&
+            half_t(-0.0f).bits == 0x8000 && float(half_t::from_bits(0x0001)) == 5.9604645e-8f && float(half_t::from_bits(0x7bff)) == 65504.0f &&
+            float(half_t::from_bits(0xfc00)) == -std::numeric_limits<float>::infinity();
+  for (uint32_t b = 0; b < 0x10000 && ok; ++b) {   // every pattern survives the round trip (NaN stays NaN)
+    const half_t h = half_t::from_bits(uint16_t(b));
+    const float f = float(h);
+    ok = (f != f) ? ((half_t(f).bits & 0x7c00) == 0x7c00 && (half_t(f).bits & 0x3ff) != 0) : half_t(f).bits == b;
+  }
+  report(ok, "cuasr::half_t: conversions round to nearest-even, every pattern survives the round trip");
+
+  ok = true;
+  const int ms[2] = {1, 509}, ns[2] = {1, 510}, ks[2] = {1, 23};
+  for (int m : ms)
+    for (int n : ns)
+      for (int k : ks) {
+        ok = ok && testbed_case<cuasr::minimum<half_t>, cuasr::plus<half_t>, half_t, ColumnMajor, ColumnMajor, ColumnMajor>(m, n, k, half_t(0), half_t(0));
+        ok = ok && testbed_case<cuasr::maximum<half_t>, cuasr::minimum<half_t>, half_t, RowMajor, ColumnMajor, RowMajor>(m, n, k, cuasr::minimum<half_t>::Identity, cuasr::minimum<half_t>::Identity);
+        ok = ok && testbed_case<cuasr::plus<half_t>, cuasr::multiplies<half_t>, half_t, ColumnMajor, RowMajor, RowMajor>(m, n, k, half_t(1), half_t(1));
+        ok = ok && testbed_case<cuasr::binary_or<half_t>, cuasr::binary_and<half_t>, half_t, RowMajor, RowMajor, ColumnMajor>(m, n, k, half_t(1), half_t(1));
+      }
+  ok = ok && testbed_case<cuasr::inf::minimum<half_t>, cuasr::plus<half_t>, half_t, RowMajor, ColumnMajor, RowMajor>(256, 512, 96, half_t(0), half_t(0));
+  report(ok, "binary16 throughout: min-plus, max-min, plus-times, or-and on the testbed sweep shapes");
+
+  ok = true;
+  for (int m : ms)
+    for (int n : ns)
+      for (int k : ks) {
+        ok = ok && int8_case<cuasr::plus<int32_t>, cuasr::multiplies<int32_t>, RowMajor, ColumnMajor, RowMajor>(m, n, k, 1, 0);
+        ok = ok && int8_case<cuasr::plus<int32_t>, cuasr::multiplies<int32_t>, ColumnMajor, ColumnMajor, ColumnMajor>(m, n, k, 3, -2);
+        ok = ok && int8_case<cuasr::minimum<int32_t>, cuasr::plus<int32_t>, ColumnMajor, RowMajor, RowMajor>(m, n, k, 0, 0);
+        ok = ok && int8_case<cuasr::maximum<int32_t>, cuasr::minimum<int32_t>, RowMajor, RowMajor, ColumnMajor>(m, n, k, cuasr::minimum<int32_t>::Identity, cuasr::minimum<int32_t>::Identity);
+      }
+  ok = ok && int8_case<cuasr::plus<int32_t>, cuasr::multiplies<int32_t>, RowMajor, ColumnMajor, RowMajor>(256, 384, 192, 1, 1);
+  report(ok, "int8 operands, int32 results: plus-times, min-plus, max-min on the testbed sweep shapes");
+
+  // parallel split-K on both: the workspace holds elements of C (2 or 4 bytes each)
+  {
+    using Add = cuasr::minimum<half_t>;
+    using Mul = cuasr::plus<half_t>;
+    using SplitK = cuasr::gemm::device::SrgemmSplitKParallel<Add, Mul, half_t, RowMajor, half_t, ColumnMajor, half_t, RowMajor, half_t>;
+    using Plain = cuasr::gemm::device::Srgemm<Add, Mul, half_t, RowMajor, half_t, ColumnMajor, half_t, RowMajor, half_t>;
+    const int M = 128, N = 96, K = 1000;
+    std::vector<half_t> a(size_t(M) * K), b(size_t(K) * N), c(size_t(M) * N);
+    fill_unit(a, 21, 0.5, 100.0);
+    fill_unit(b, 22, 0.5, 100.0);
+    fill_unit(c, 23, 0.5, 100.0);
+    DeviceBuf<half_t> da(a), db(b), dc(c), d1(std::vector<half_t>(size_t(M) * N)), d2(std::vector<half_t>(size_t(M) * N));
+    ok = true;
+    for (int slices : {3, 8}) {
+      SplitK::Arguments args({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d1.p, N}, {Mul::Identity, Mul::Identity}, slices);
+      const size_t bytes = SplitK::get_workspace_size(args);
+      DeviceBuf<uint8_t> ws(bytes);
+      SplitK op;
+      ok = ok && bytes == sizeof(half_t) * size_t(M) * N * slices;
+      ok = ok && op.initialize(args, ws.p) == Status::kSuccess && op() == Status::kSuccess;
+      Plain::Arguments pargs({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {Mul::Identity, Mul::Identity});
+      Plain plain;
+      ok = ok && plain(pargs) == Status::kSuccess;
+      HIP_OK(hipDeviceSynchronize());
+      const std::vector<half_t> x = d1.download(), y = d2.download();
+      ok = ok && std::memcmp(x.data(), y.data(), x.size() * sizeof(half_t)) == 0;
+    }
+    report(ok, "binary16 parallel split-K == non-split");
+  }
+  {
+    using Add = cuasr::plus<int32_t>;
+    using Mul = cuasr::multiplies<int32_t>;
+    using SplitK = cuasr::gemm::device::SrgemmSplitKParallel<Add, Mul, int8_t, RowMajor, int8_t, ColumnMajor, int32_t, RowMajor, int32_t>;
+    using Plain = cuasr::gemm::device::Srgemm<Add, Mul, int8_t, RowMajor, int8_t, ColumnMajor, int32_t, RowMajor, int32_t>;
+    const int M = 128, N = 96, K = 1000;
+    std::vector<int8_t> a(size_t(M) * K), b(size_t(K) * N);
+    std::vector<int32_t> c(size_t(M) * N);
+    fill_int(a, 31, -128, 127);
+    fill_int(b, 32, -128, 127);
+    fill_int(c, 33, -1000, 1000);
+    DeviceBuf<int8_t> da(a), db(b);
+    DeviceBuf<int32_t> dc(c), d1(std::vector<int32_t>(size_t(M) * N)), d2(std::vector<int32_t>(size_t(M) * N));
+    ok = true;
+    for (int slices : {3, 8}) {
+      SplitK::Arguments args({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d1.p, N}, {2, -3}, slices);
+      const size_t bytes = SplitK::get_workspace_size(args);
+      DeviceBuf<uint8_t> ws(bytes);
+      SplitK op;
+      ok = ok && bytes == sizeof(int32_t) * size_t(M) * N * slices;
+      ok = ok && op.initialize(args, ws.p) == Status::kSuccess && op() == Status::kSuccess;
+      Plain::Arguments pargs({M, N, K}, {da.p, K}, {db.p, K}, {dc.p, N}, {d2.p, N}, {2, -3});
+      Plain plain;
+      ok = ok && plain(pargs) == Status::kSuccess;
+      HIP_OK(hipDeviceSynchronize());
+      ok = ok && d1.download() == d2.download();   // (sums of int32 wrap in any order)
+    }
+    report(ok, "int8 parallel split-K == non-split");
+  }
+}
+
 // ---- a user-defined functor, as in examples/01_userdefined_semiring: defined
 // by the user, made known to the library by specialising cuasr::op_tag
 namespace {
@@ -343,6 +468,7 @@ int main() {
   testbed_sweep_serial<cuasr::binary_or<float>, cuasr::binary_and<float>, float>("testbed serial split-K or-and f32");
   testbed_sweep<cuasr::inf::minimum<float>, cuasr::inf::plus<float>, float>("testbed inf::minimum-plus f32");
   testbed_sweep<cuasr::inf::maximum<double>, cuasr::inf::plus_for_max<double>, double>("testbed inf::maximum-plus f64");
+  wider_element_types();
   std::printf("%d checks, %d failed\n", g_run, g_fail);
   return g_fail;
 }
