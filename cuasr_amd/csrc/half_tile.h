@@ -28,6 +28,7 @@
 // their minima are exact; the operands are converted on their way to LDS, the accumulators on their way out,
 // and the epilogue (the caller's additive identity included) is integer arithmetic.  On the vector ALU that is
 // twice the rate integers get (three-input integer minima and byte-selecting adds issue at half rate).
+// min-times and max-times on int8 operands use the kernel with int16 lanes (int16_lanes below).
 #pragma once
 #include "semiring.h"
 
@@ -60,7 +61,23 @@ __device__ __forceinline__ h2 or_and_pair(h2 acc, h2 a, h2 b) {
   return __builtin_bit_cast(h2, or_and_term(__builtin_bit_cast(uint32_t, acc), __builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b)));
 }
 
-template <int ADD, int MUL> __device__ __forceinline__ void two_terms(h2 &acc, h2 a0, h2 b0, h2 a1, h2 b1) {
+// int8 operands under min-times / max-times: a product of two int8 values is a 16-bit integer (|a b| <= 16384) but no
+// binary16 value, so the lanes hold int16 and the instructions are the packed 16-bit integer ones (v_pk_mul_lo_u16,
+// v_pk_min_i16 / v_pk_max_i16; there is no three-input packed integer minimum: four instructions per four terms)
+typedef short s2 __attribute__((ext_vector_type(2)));
+template <int ADD, int MUL, typename TI> struct int16_lanes
+    : std::integral_constant<bool, std::is_same<TI, int8_t>::value && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum)> {};
+template <int ADD> __device__ __forceinline__ h2 int16_fold(h2 l, h2 r) {
+  const s2 x = __builtin_bit_cast(s2, l), y = __builtin_bit_cast(s2, r);
+  return __builtin_bit_cast(h2, ADD == kMinimum ? __builtin_elementwise_min(x, y) : __builtin_elementwise_max(x, y));
+}
+__device__ __forceinline__ h2 int16_product(h2 a, h2 b) { return __builtin_bit_cast(h2, __builtin_bit_cast(s2, a) * __builtin_bit_cast(s2, b)); }
+
+template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ void two_terms(h2 &acc, h2 a0, h2 b0, h2 a1, h2 b1) {
+  if constexpr (I16) {
+    acc = int16_fold<ADD>(int16_fold<ADD>(acc, int16_product(a0, b0)), int16_product(a1, b1));
+    return;
+  }
   if constexpr (masked<ADD, MUL>::value) {
     acc = or_and_pair(or_and_pair(acc, a0, b0), a1, b1);
     return;
@@ -71,14 +88,16 @@ template <int ADD, int MUL> __device__ __forceinline__ void two_terms(h2 &acc, h
   else if constexpr (ADD == kMaximum) acc = __builtin_elementwise_maximum(__builtin_elementwise_maximum(acc, t0), t1);
   else acc = pk<ADD>(pk<ADD>(acc, t0), t1);
 }
-template <int ADD, int MUL> __device__ __forceinline__ void one_term(h2 &acc, h2 a, h2 b) {
-  if constexpr (masked<ADD, MUL>::value) acc = or_and_pair(acc, a, b);
+template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ void one_term(h2 &acc, h2 a, h2 b) {
+  if constexpr (I16) acc = int16_fold<ADD>(acc, int16_product(a, b));
+  else if constexpr (masked<ADD, MUL>::value) acc = or_and_pair(acc, a, b);
   else acc = pk<ADD>(acc, pk<MUL>(a, b));
 }
 
 // add(l, r) of two partial accumulators (or-and: of two masks)
-template <int ADD, int MUL> __device__ __forceinline__ h2 fold(h2 l, h2 r) {
-  if constexpr (masked<ADD, MUL>::value) return __builtin_bit_cast(h2, __builtin_bit_cast(uint32_t, l) | __builtin_bit_cast(uint32_t, r));
+template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ h2 fold(h2 l, h2 r) {
+  if constexpr (I16) return int16_fold<ADD>(l, r);
+  else if constexpr (masked<ADD, MUL>::value) return __builtin_bit_cast(h2, __builtin_bit_cast(uint32_t, l) | __builtin_bit_cast(uint32_t, r));
   else return pk<ADD>(l, r);
 }
 
@@ -99,10 +118,12 @@ template <> __device__ __forceinline__ half_t to_half<half_t>(half_t v) { return
 // One operand's share of a k-tile on its way from memory to LDS.  The panel is X wide (X = BM for A, BN
 // for B); a chunk is 8 elements: of one k and 8 consecutive x when x is the contiguous direction in
 // memory, of one x and 8 consecutive k otherwise (KC).  CHUNKS chunks per thread.
-template <int X, bool KC, bool GUARD, typename TI, bool MASK = false> struct Stager {
-  // what goes to LDS for one operand: its binary16 value, or (MASK) all ones / zero for non-zero / zero
+template <int X, bool KC, bool GUARD, typename TI, bool MASK = false, bool I16 = false> struct Stager {
+  // what goes to LDS for one operand: its binary16 value, or (MASK) all ones / zero for non-zero / zero, or (I16)
+  // the 16-bit integer
   static __device__ __forceinline__ half_t staged(TI v) {
-    if constexpr (MASK) return __builtin_bit_cast(half_t, (unsigned short)(truth(v) ? 0xffff : 0));
+    if constexpr (I16) return __builtin_bit_cast(half_t, (short)v);
+    else if constexpr (MASK) return __builtin_bit_cast(half_t, (unsigned short)(truth(v) ? 0xffff : 0));
     else return to_half<TI>(v);
   }
   typedef typename vec8<TI>::type raw8;
@@ -202,6 +223,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   constexpr bool BYTES = std::is_same<TI, int8_t>::value;
   constexpr bool ZERO_SIGN = !BYTES && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum);
   constexpr bool MASKED = masked<ADD, MUL>::value;
+  constexpr bool I16 = int16_lanes<ADD, MUL, TI>::value;
   typedef typename out_of<TI>::type TO;
   typedef typename vec8<TO>::type out8;
   typedef typename frag_of<TR>::type rows_t;
@@ -224,6 +246,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   // int8 operands: the loop starts from the binary16 infinity of its add; the caller's identity joins at the end
   // (or-and: the loop ors masks, starting from none; the caller's identity joins at the end as well)
   const half_t ident = MASKED ? half_t(0)
+                       : I16   ? __builtin_bit_cast(half_t, (short)(ADD == kMinimum ? 32767 : -32768))
                        : BYTES ? half_t(ADD == kMinimum ? __builtin_inff() : -__builtin_inff()) : scalar_as<half_t>(p.add_identity);
 
   h2 acc[TR][4 * NG];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
@@ -234,8 +257,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
   // AHEAD = 2: the loads of k-tile t + 2 are issued before the terms of tile t, into the registers that tile t
   // passed through (a workgroup alone on its compute unit has nobody to hide a memory latency behind)
-  Stager<BM, A_KC, GUARD, TI, MASKED> sa[AHEAD];
-  Stager<BN, B_KC, GUARD, TI, MASKED> sb[AHEAD];
+  Stager<BM, A_KC, GUARD, TI, MASKED, I16> sa[AHEAD];
+  Stager<BN, B_KC, GUARD, TI, MASKED, I16> sb[AHEAD];
   const int tiles_k = ke > kb ? (ke - kb + BK - 1) / BK : 0;
   auto fetch = [&](auto set, int t) {
     sa[set.value].load(A, p.sa_m, p.sa_k, m0, kb + t * BK, p.m, ke);
@@ -271,7 +294,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
           for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int g = 0; g < NG; ++g)
-              two_terms<ADD, MUL>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j), both(a1[i]), pair_of(b1[g], j));
+              two_terms<ADD, MUL, I16>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j), both(a1[i]), pair_of(b1[g], j));
       }
     } else {
       for (int kk = kf; kk < min(kf + KW, ke - k0); ++kk) {  // the ragged last k-tile
@@ -284,7 +307,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
           for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int g = 0; g < NG; ++g) one_term<ADD, MUL>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j));
+            for (int g = 0; g < NG; ++g) one_term<ADD, MUL, I16>(acc[i][4 * g + j], both(a0[i]), pair_of(b0[g], j));
       }
     }
     if (t + 1 < tiles_k) {
@@ -319,7 +342,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
       for (int j = 0; j < 4 * NG; ++j) {
         h2 v = red[0][(part * IR + i) * 4 * NG + j][lane];
 #pragma unroll
-        for (int w = 1; w < KS; ++w) v = fold<ADD, MUL>(v, red[w][(part * IR + i) * 4 * NG + j][lane]);
+        for (int w = 1; w < KS; ++w) v = fold<ADD, MUL, I16>(v, red[w][(part * IR + i) * 4 * NG + j][lane]);
         fin[i][j] = v;
       }
   }
@@ -343,7 +366,8 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
           // the reference's accumulator after k > 0 terms: 1 if any term or the identity is non-zero, else 0
           const bool any = __builtin_bit_cast(unsigned short, a) != 0 || truth(e.ident);
           v[j] = tiles_k > 0 ? TO(any ? 1 : 0) : e.ident;
-        } else if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
+        } else if constexpr (I16) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(__builtin_bit_cast(short, a))) : e.ident;
+        else if constexpr (BYTES) v[j] = tiles_k > 0 ? Op<ADD>::apply(e.ident, TO(float(a))) : e.ident;  // (an exact integer)
         else v[j] = a;
         if constexpr (ZERO_SIGN) {
           // a minimum / maximum that is zero: the reference's comparison keeps the newer of two equal operands

@@ -4,7 +4,8 @@
 
 namespace cuasr_amd {
 
-// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16), and or-and
+// int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16), the two
+// whose terms are products (exact as 16-bit integers), and or-and
 launch_fn find_valu_i8(int add_op, int mult_op) {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL, int8_t>;
@@ -12,6 +13,8 @@ launch_fn find_valu_i8(int add_op, int mult_op) {
   PAIR(kMaximum, kPlus)
   PAIR(kMinimum, kMaximum)
   PAIR(kMaximum, kMinimum)
+  PAIR(kMinimum, kMultiplies)   // (int16 lanes)
+  PAIR(kMaximum, kMultiplies)
   PAIR(kLogicalOr, kLogicalAnd)
 #undef PAIR
   return nullptr;

@@ -56,7 +56,8 @@ def test_selected_family(lib):
     dB = to_device(np.zeros((64, 256), np.int8))
     dD = to_device(np.zeros((128, 256), np.int32))
     for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"valu"), (("maximum", "minimum"), b"valu"),
-                              (("logical_or", "logical_and"), b"valu"), (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"naive")]:
+                              (("logical_or", "logical_and"), b"valu"), (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"valu"),
+                              (("maximum", "multiplies"), b"valu")]:
         desc = cuasr_amd.make_desc(add, mult, "i8", dA, dB, dD, dD, 1, 0, 0, 1)
         assert lib.cuasr_amd_selected_kernel(desc) == name
 
@@ -70,12 +71,14 @@ def test_every_pair_on_widened_operands(oracle, lib, sr):
         check(oracle, *sr, 70, 90, 33, layouts, "naive")
 
 
-@pytest.mark.parametrize("sr", [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum")])
+@pytest.mark.parametrize("sr", [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"),
+                                ("minimum", "multiplies"), ("maximum", "multiplies")])
 @pytest.mark.parametrize("layouts", LAYOUTS)
 def test_tropical_pairs_on_the_packed_tile(oracle, lib, sr, layouts):
     """Sums, minima and maxima of two int8 values are exact in binary16: these pairs run on the packed
-    half-precision tile (operands converted on their way to LDS, integer epilogue).  Every tile size, aligned and
-    ragged, identities and scalars that are not the semiring's own."""
+    half-precision tile (operands converted on their way to LDS, integer epilogue); products of two int8 values are
+    exact as 16-bit integers: min-times and max-times run on the same tile with int16 lanes.  Every tile size,
+    aligned and ragged, identities and scalars that are not the semiring's own."""
     check(oracle, *sr, 100, 300, 45, layouts, "valu")                        # 16 x 128 tiles, k shared out between the waves, ragged
     check(oracle, *sr, 1530, 1300, 77, layouts, "valu", alpha=3, beta=-2)    # 32 x 128 tiles, likewise
     check(oracle, *sr, 520, 390, 9, layouts, "valu")                         # k shorter than a tile
@@ -104,6 +107,29 @@ def test_boolean_closure_on_masks(oracle, lib, layouts):
         cuasr_amd.srgemm("logical_or", "logical_and", to_device(A), to_device(B), to_device(C), dD, 1, 1, ident, 1, dtype="i8", kernel="valu")
         torch.cuda.synchronize()
         assert_same_bits(dD.cpu().numpy(), want, f"or-and i8 {m}x{n}x{k} {layouts} identity {ident}")
+
+
+def test_products_at_the_ends_of_the_int16_range(oracle, lib):
+    """min-times / max-times: (-128) (-128) = 16384 is the largest product, (-128) 127 = -16256 the smallest; rows and
+    columns that hold nothing else, identities inside and outside the int16 range."""
+    import torch
+    import cuasr_amd
+    rng = np.random.default_rng(5)
+    for add in ("minimum", "maximum"):
+        for (m, n, k), ident in [((130, 260, 40), 2 ** 31 - 1), ((130, 260, 40), 100), ((64, 128, 3), -40000), ((520, 390, 77), -(2 ** 31)),
+                                 ((70, 90, 1), 12345)]:
+            A = np.asarray(rng.choice(np.array([-128, 127, -1, 1], np.int8), (m, k)), order="C")
+            B = np.asarray(rng.choice(np.array([-128, 127, -1, 1], np.int8), (k, n)), order="F")
+            if k:
+                A[::3, :] = -128
+                B[:, ::5] = -128       # (rows x columns of nothing but 16384)
+                B[:, 1::5] = 127
+            C = np.asarray(rng.integers(-50000, 50000, (m, n)).astype(np.int32), order="C")
+            want = oracle.srgemm(add, "multiplies", A, B, C, 1, 0, ident)
+            dD = to_device(np.zeros_like(C))
+            cuasr_amd.srgemm(add, "multiplies", to_device(A), to_device(B), to_device(C), dD, 1, 0, ident, 1, dtype="i8", kernel="valu")
+            torch.cuda.synchronize()
+            assert_same_bits(dD.cpu().numpy(), want, f"{add}-times i8 {m}x{n}x{k} identity {ident}")
 
 
 def test_tropical_identity_that_is_not_infinite(oracle, lib):
