@@ -9,6 +9,7 @@ only as handles to device memory.  There is no CPU fallback: if the library
 has not been built, loading raises.
 """
 import ctypes
+import struct
 import os
 
 import numpy as np
@@ -164,7 +165,10 @@ def _set_scalar(s, value, dtype):
     elif dtype in ("i32", "i8"):
         s.i32 = int(value)
     elif dtype == "f16":
-        s.f16 = int(np.array([value], dtype=np.float16).view(np.uint16)[0])   # the binary16 bit pattern
+        try:                                                   # the binary16 bit pattern, rounded to nearest-even
+            s.f16 = struct.unpack("<H", struct.pack("<e", float(value)))[0]
+        except OverflowError:                                  # beyond 65504: struct refuses, numpy rounds to infinity
+            s.f16 = int(np.array([value], dtype=np.float16).view(np.uint16)[0])
     else:
         s.u32 = int(value) & 0xFFFFFFFF
 

@@ -14,6 +14,7 @@ groups of add, add, min3 = 128 terms per lane) or a variation of it, run by 256-
     mix + N waits / nops / scalar adds    what an instruction that does no arithmetic costs
     packed fp16 add / min / minimum3 / mix the same for two fp16 terms per instruction
     SDWA byte add / min3_i32 / mix         int8 operands widened by the add's own byte selects
+    packed int16 multiply / min / mix      int8 operands as 16-bit integers (products fit): min-times, max-times
     fp64 add / max / mix (+ the same)     the same questions for 8-byte elements
 Times are HIP events around the second of two launches; the clock is read inside the kernel
 (shader cycle counter against the 100 MHz wall clock), so cycle figures are per measured clock.
@@ -58,6 +59,23 @@ def mix_f16():
             groups.append([f"v_pk_add_f16 v{t0}, v{A0[i]}, v{B0[j]} op_sel_hi:[0,1]",
                            f"v_pk_add_f16 v{t1}, v{A0[i]}, v{B1[j]} op_sel:[1,0] op_sel_hi:[1,1]",
                            f"v_pk_minimum3_f16 v{acc}, v{acc}, v{t0}, v{t1}"])
+    return groups
+
+
+def mix_i16():
+    """min-times on int8 operands widened to packed int16 (a product of two int8 values is a 16-bit integer): two
+    products and two minima per group of four terms -- there is no three-input packed integer minimum; 256 terms per
+    lane in 256 instructions"""
+    groups, t = [], 0
+    for i in range(8):
+        for j in range(8):
+            t0, t1 = T[t % 8], T[(t + 1) % 8]
+            t += 2
+            acc = ACC[i * 8 + j]
+            groups.append([f"v_pk_mul_lo_u16 v{t0}, v{A0[i]}, v{B0[j]} op_sel_hi:[0,1]",
+                           f"v_pk_mul_lo_u16 v{t1}, v{A0[i]}, v{B1[j]} op_sel:[1,0] op_sel_hi:[1,1]",
+                           f"v_pk_min_i16 v{acc}, v{acc}, v{t0}",
+                           f"v_pk_min_i16 v{acc}, v{acc}, v{t1}"])
     return groups
 
 
@@ -131,6 +149,10 @@ def kernels():
     k["add_u32_sdwa_bytes"] = (only("v_add_u32_sdwa v{t}, sext(v{b}), sext(v{a}) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 src1_sel:BYTE_2"), 192, 0, "f32")
     k["min3_i32"] = (only("v_min3_i32 v{acc}, v{acc}, v{b}, v{a}"), 192, 0, "f32")
     k["mix_i8_sdwa"] = (flat(mix_i8()), 192, 128, "f32")
+    # int8 operands as packed int16 (min-times / max-times)
+    k["pk_mul_lo_u16"] = (only("v_pk_mul_lo_u16 v{t}, v{b}, v{a}"), 192, 0, "f32")
+    k["pk_min_i16"] = (only("v_pk_min_i16 v{acc}, v{acc}, v{b}"), 192, 0, "f32")
+    k["mix_i16"] = (flat(mix_i16()), 256, 256, "f32")
     # an operand fetched from another lane of the quad by the add itself (a fragment shared by four lanes)
     k["add_f32_dpp_quad"] = (only("v_add_f32_dpp v{t}, v{b}, v{a} quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf"), 192, 0, "f32")
     k["mix"] = (flat(mix()), 192, 128, "f32")
