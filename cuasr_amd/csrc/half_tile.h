@@ -28,7 +28,7 @@
 // their minima are exact; the operands are converted on their way to LDS, the accumulators on their way out,
 // and the epilogue (the caller's additive identity included) is integer arithmetic.  On the vector ALU that is
 // twice the rate integers get (three-input integer minima and byte-selecting adds issue at half rate).
-// min-times and max-times on int8 operands use the kernel with int16 lanes (int16_lanes below).
+// min-times, max-times and the bitwise pairs on int8 operands use the kernel with int16 lanes (int16_lanes below).
 #pragma once
 #include "semiring.h"
 
@@ -63,19 +63,34 @@ __device__ __forceinline__ h2 or_and_pair(h2 acc, h2 a, h2 b) {
 
 // int8 operands under min-times / max-times: a product of two int8 values is a 16-bit integer (|a b| <= 16384) but no
 // binary16 value, so the lanes hold int16 and the instructions are the packed 16-bit integer ones (v_pk_mul_lo_u16,
-// v_pk_min_i16 / v_pk_max_i16; there is no three-input packed integer minimum: four instructions per four terms)
+// v_pk_min_i16 / v_pk_max_i16; there is no three-input packed integer minimum: four instructions per four terms).
+// The bitwise pairs on int8 operands (xor-and, or-and on bits) use the same lanes: the operators act on the widened
+// values, and the bitwise and / xor / or of sign-extended 8-bit values are the sign extensions of the 8-bit results,
+// at 16 bits as at 32; a term is one three-input bit operation on a register of two lanes.
 typedef short s2 __attribute__((ext_vector_type(2)));
 template <int ADD, int MUL, typename TI> struct int16_lanes
-    : std::integral_constant<bool, std::is_same<TI, int8_t>::value && MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum)> {};
+    : std::integral_constant<bool, std::is_same<TI, int8_t>::value &&
+                                       ((MUL == kMultiplies && (ADD == kMinimum || ADD == kMaximum)) ||
+                                        (MUL == kBitAnd && (ADD == kBitXor || ADD == kBitOr)))> {};
 template <int ADD> __device__ __forceinline__ h2 int16_fold(h2 l, h2 r) {
   const s2 x = __builtin_bit_cast(s2, l), y = __builtin_bit_cast(s2, r);
-  return __builtin_bit_cast(h2, ADD == kMinimum ? __builtin_elementwise_min(x, y) : __builtin_elementwise_max(x, y));
+  if constexpr (ADD == kBitXor) return __builtin_bit_cast(h2, x ^ y);
+  else if constexpr (ADD == kBitOr) return __builtin_bit_cast(h2, x | y);
+  else return __builtin_bit_cast(h2, ADD == kMinimum ? __builtin_elementwise_min(x, y) : __builtin_elementwise_max(x, y));
 }
 __device__ __forceinline__ h2 int16_product(h2 a, h2 b) { return __builtin_bit_cast(h2, __builtin_bit_cast(s2, a) * __builtin_bit_cast(s2, b)); }
+template <int ADD, int MUL> __device__ __forceinline__ h2 int16_term(h2 acc, h2 a, h2 b) {
+  if constexpr (MUL == kBitAnd) {
+    const uint32_t x = __builtin_bit_cast(uint32_t, acc), u = __builtin_bit_cast(uint32_t, a), v = __builtin_bit_cast(uint32_t, b);
+    return __builtin_bit_cast(h2, ADD == kBitXor ? xor_and_term(x, u, v) : or_and_term(x, u, v));
+  } else {
+    return int16_fold<ADD>(acc, int16_product(a, b));
+  }
+}
 
 template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ void two_terms(h2 &acc, h2 a0, h2 b0, h2 a1, h2 b1) {
   if constexpr (I16) {
-    acc = int16_fold<ADD>(int16_fold<ADD>(acc, int16_product(a0, b0)), int16_product(a1, b1));
+    acc = int16_term<ADD, MUL>(int16_term<ADD, MUL>(acc, a0, b0), a1, b1);
     return;
   }
   if constexpr (masked<ADD, MUL>::value) {
@@ -89,7 +104,7 @@ template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ void tw
   else acc = pk<ADD>(pk<ADD>(acc, t0), t1);
 }
 template <int ADD, int MUL, bool I16 = false> __device__ __forceinline__ void one_term(h2 &acc, h2 a, h2 b) {
-  if constexpr (I16) acc = int16_fold<ADD>(acc, int16_product(a, b));
+  if constexpr (I16) acc = int16_term<ADD, MUL>(acc, a, b);
   else if constexpr (masked<ADD, MUL>::value) acc = or_and_pair(acc, a, b);
   else acc = pk<ADD>(acc, pk<MUL>(a, b));
 }
@@ -210,7 +225,8 @@ static __device__ __attribute__((noinline)) half_t last_zero_product(const half_
 }
 
 // TR rows and NG groups of 8 columns per thread.  KS = 1: the 256 threads are 16 x 16, the tile 16 TR x 128 NG.
-// KS = 4 (adds that do not care about order or repetition: min, max, or): a wave is 16 x 4 threads and covers a
+// KS = 4 (adds that do not care about order, and about repetition of the value every part starts from -- min, max,
+// or, and xor, which starts from zero): a wave is 16 x 4 threads and covers a
 // tile of 4 TR x 128 NG by itself, each of the four waves takes a quarter of every k-tile, and the four partial
 // accumulators meet in LDS before the epilogue.  A small output then still gives every SIMD a wave, and the wave
 // the full tile's work per LDS read.
@@ -246,7 +262,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   // int8 operands: the loop starts from the binary16 infinity of its add; the caller's identity joins at the end
   // (or-and: the loop ors masks, starting from none; the caller's identity joins at the end as well)
   const half_t ident = MASKED ? half_t(0)
-                       : I16   ? __builtin_bit_cast(half_t, (short)(ADD == kMinimum ? 32767 : -32768))
+                       : I16   ? __builtin_bit_cast(half_t, (short)(ADD == kMinimum ? 32767 : ADD == kMaximum ? -32768 : 0))
                        : BYTES ? half_t(ADD == kMinimum ? __builtin_inff() : -__builtin_inff()) : scalar_as<half_t>(p.add_identity);
 
   h2 acc[TR][4 * NG];  // [row][column pair]: pairs 0..3 = columns tx*8 .. +7, pairs 4..7 = the same 128 further on
@@ -462,7 +478,7 @@ template <int ADD, int MUL, typename TI = half_t> static hipError_t launch(const
     return groups / 512 * (512 * area / paired) + (rest > 256 ? 512 * area / paired : rest > 0 ? 256 * area / alone : 0);
   };
   // (or-and: the full tile's term is half an instruction; the smaller tiles are bound by what surrounds the terms)
-  const bool bits = masked<ADD, MUL>::value;
+  const bool bits = masked<ADD, MUL>::value || MUL == kBitAnd;
   const long long full = bits ? cost(128, 256, 95, 128) : cost(128, 256, 63, 83), mid = bits ? cost(64, 128, 50, 76) : cost(64, 128, 50, 68);
   if constexpr (ADD == kPlus) {
     // the sum's order is the reference's: every k-tile whole in one thread

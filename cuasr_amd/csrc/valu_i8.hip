@@ -5,7 +5,7 @@
 namespace cuasr_amd {
 
 // int8 operands: the pairs whose terms are sums, minima or maxima of two int8 values (exact in binary16), the two
-// whose terms are products (exact as 16-bit integers), and or-and
+// whose terms are products (exact as 16-bit integers), the bitwise pairs (the same lanes), and or-and
 launch_fn find_valu_i8(int add_op, int mult_op) {
 #define PAIR(ADD, MUL) \
   if (add_op == ADD && mult_op == MUL) return half_tile::launch<ADD, MUL, int8_t>;
@@ -15,6 +15,8 @@ launch_fn find_valu_i8(int add_op, int mult_op) {
   PAIR(kMaximum, kMinimum)
   PAIR(kMinimum, kMultiplies)   // (int16 lanes)
   PAIR(kMaximum, kMultiplies)
+  PAIR(kBitXor, kBitAnd)
+  PAIR(kBitOr, kBitAnd)
   PAIR(kLogicalOr, kLogicalAnd)
 #undef PAIR
   return nullptr;

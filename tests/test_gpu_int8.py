@@ -56,7 +56,8 @@ def test_selected_family(lib):
     dB = to_device(np.zeros((64, 256), np.int8))
     dD = to_device(np.zeros((128, 256), np.int32))
     for (add, mult), name in [(("plus", "multiplies"), b"mfma"), (("minimum", "plus"), b"valu"), (("maximum", "minimum"), b"valu"),
-                              (("logical_or", "logical_and"), b"valu"), (("bit_xor", "bit_and"), b"naive"), (("minimum", "multiplies"), b"valu"),
+                              (("logical_or", "logical_and"), b"valu"), (("bit_xor", "bit_and"), b"valu"), (("bit_or", "bit_and"), b"valu"),
+                              (("bit_xor", "logical_and"), b"naive"), (("minimum", "multiplies"), b"valu"),
                               (("maximum", "multiplies"), b"valu")]:
         desc = cuasr_amd.make_desc(add, mult, "i8", dA, dB, dD, dD, 1, 0, 0, 1)
         assert lib.cuasr_amd_selected_kernel(desc) == name
@@ -72,12 +73,13 @@ def test_every_pair_on_widened_operands(oracle, lib, sr):
 
 
 @pytest.mark.parametrize("sr", [("minimum", "plus"), ("maximum", "plus"), ("minimum", "maximum"), ("maximum", "minimum"),
-                                ("minimum", "multiplies"), ("maximum", "multiplies")])
+                                ("minimum", "multiplies"), ("maximum", "multiplies"), ("bit_xor", "bit_and"), ("bit_or", "bit_and")])
 @pytest.mark.parametrize("layouts", LAYOUTS)
 def test_tropical_pairs_on_the_packed_tile(oracle, lib, sr, layouts):
     """Sums, minima and maxima of two int8 values are exact in binary16: these pairs run on the packed
     half-precision tile (operands converted on their way to LDS, integer epilogue); products of two int8 values are
-    exact as 16-bit integers: min-times and max-times run on the same tile with int16 lanes.  Every tile size,
+    exact as 16-bit integers: min-times and max-times run on the same tile with int16 lanes, and so do the bitwise
+    pairs (and / xor / or of sign-extended bytes are the sign extensions of the byte results).  Every tile size,
     aligned and ragged, identities and scalars that are not the semiring's own."""
     check(oracle, *sr, 100, 300, 45, layouts, "valu")                        # 16 x 128 tiles, k shared out between the waves, ragged
     check(oracle, *sr, 1530, 1300, 77, layouts, "valu", alpha=3, beta=-2)    # 32 x 128 tiles, likewise
