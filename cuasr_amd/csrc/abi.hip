@@ -17,6 +17,7 @@ launch_fn find_valu_i8(int, int);
 launch_fn find_mfma_f32(int, int);
 launch_fn find_mfma_f64(int, int);
 launch_fn find_mfma_i8(int, int);
+launch_fn find_mfma_f16(int, int);
 launch_fn find_direct_f32(int, int);
 launch_fn find_direct_i32(int, int);
 launch_fn find_direct_u32(int, int);
@@ -70,6 +71,7 @@ launch_fn find_mfma(int dtype, int add_op, int mult_op) {
   if (dtype == CUASR_AMD_F32) return find_mfma_f32(add_op, mult_op);
   if (dtype == CUASR_AMD_F64) return find_mfma_f64(add_op, mult_op);
   if (dtype == CUASR_AMD_I8) return find_mfma_i8(add_op, mult_op);
+  if (dtype == CUASR_AMD_F16) return find_mfma_f16(add_op, mult_op);  // (float accumulation: by request only)
   return nullptr;
 }
 
@@ -93,6 +95,7 @@ static Problem canonical(const cuasr_amd_srgemm_desc *d);
 static bool mfma_usable(const cuasr_amd_srgemm_desc *d) {
   if (!find_mfma(d->dtype, d->add_op, d->mult_op)) return false;
   if (d->dtype == CUASR_AMD_I8) return true;  // its kernel has a guarded form for every extent and alignment
+  if (d->dtype == CUASR_AMD_F16) return d->split_k_slices == 1;  // likewise; its float sums have no binary16 split-K form
   return d->dtype == CUASR_AMD_F64 ? mfma_f64_can_run(canonical(d)) : mfma_f32_can_run(canonical(d));
 }
 
@@ -197,7 +200,9 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   // plus-times is the one semiring a matrix instruction computes as is
   // (its tile is 128 x 128: below 128 tiles half the compute units and more stand idle, and the
   // vector-ALU tiles, which are smaller, are faster -- 1024^3: 31 against 22 TFLOP/s)
-  if (d->add_op == kPlus && d->mult_op == kMultiplies && mfma_usable(d)) {
+  // (binary16: the matrix-core kernel accumulates in float and is not bit-identical to the binary16 sums of the
+  // vector-ALU tile and the oracle, so it runs only when the descriptor asks for it)
+  if (d->add_op == kPlus && d->mult_op == kMultiplies && d->dtype != CUASR_AMD_F16 && mfma_usable(d)) {
     const long long mfma_tiles = (long long)((d->m + 127) / 128) * ((d->n + 127) / 128) * d->split_k_slices * batch;
     if (mfma_tiles >= 128 || !find_valu(d->dtype, d->add_op, d->mult_op)) return kMfma;
   }
@@ -406,7 +411,7 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
     probe.batch = batch < 65535 ? batch : 65535;
     probe.batch_a = col ? stride_b : stride_a;
     probe.batch_b = col ? stride_a : stride_b;
-    in_grid = desc->dtype == CUASR_AMD_I8 ? true : desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
+    in_grid = (desc->dtype == CUASR_AMD_I8 || desc->dtype == CUASR_AMD_F16) ? true : desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
   }
   if (in_grid) {
     const launch_fn fn = family_fn(family, desc);

@@ -43,6 +43,19 @@ template <int X, bool KC, bool GUARD> struct Stager {
   static constexpr int NUNITS = (X / 16) * (BK / 4);                // otherwise: units in the tile ...
   static constexpr int UNITS = (NUNITS + THREADS - 1) / THREADS;    // ... and per thread
   v4i r[KC ? CHUNKS : 4 * UNITS];
+  // unit u -> (x, k) of its first element.  XB neighbouring lanes take neighbouring blocks of 16 x at one group of 4 k,
+  // the next lanes the next groups of k: the lanes of one LDS store then write XB rows (16 apart: the same bank) at
+  // 64 / XB consecutive words each -- a two-way bank conflict where x-fastest lanes had an eight-way one.
+#ifndef CUASR_I8_XB
+#define CUASR_I8_XB 2
+#endif
+  static constexpr int XB = CUASR_I8_XB;
+  static_assert((X / 16) % XB == 0, "blocks of x split evenly");
+  static __device__ __forceinline__ void where(int u, int &x, int &k) {
+    const int lo = u % XB, kg = (u / XB) % (BK / 4), hi = u / (XB * (BK / 4));
+    x = (hi * XB + lo) * 16;
+    k = kg * 4;
+  }
 
   static __device__ __forceinline__ v4i fetch(const int8_t *src, int first, int limit, bool live) {
     // 16 consecutive bytes; byte e is element first + e of a run that ends at `limit`
@@ -76,7 +89,8 @@ template <int X, bool KC, bool GUARD> struct Stager {
       for (int q = 0; q < UNITS; ++q) {
         const int u = threadIdx.x + q * THREADS;
         if (u < NUNITS) {
-          const int x = (u % (X / 16)) * 16, k = (u / (X / 16)) * 4;
+          int x, k;
+          where(u, x, k);
 #pragma unroll
           for (int kk = 0; kk < 4; ++kk)
             r[4 * q + kk] = fetch(base + (x0 + x) + (long long)(k0 + k + kk) * sk, x0 + x, xn, k0 + k + kk < kn);
@@ -97,7 +111,8 @@ template <int X, bool KC, bool GUARD> struct Stager {
       for (int q = 0; q < UNITS; ++q) {
         const int u = threadIdx.x + q * THREADS;
         if (u < NUNITS) {
-          const int x = (u % (X / 16)) * 16, k = (u / (X / 16)) * 4;
+          int x, k;
+          where(u, x, k);
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             // words d of the four loads hold x = 4d .. 4d+3 at k, k+1, k+2, k+3: a 4 x 4 byte transpose

@@ -96,7 +96,10 @@ typedef enum cuasr_amd_kernel {
   CUASR_AMD_KERNEL_AUTO = 0,
   CUASR_AMD_KERNEL_NAIVE = 1, /* one thread per output element               */
   CUASR_AMD_KERNEL_VALU = 2,  /* LDS-staged, register-blocked vector-ALU tile */
-  CUASR_AMD_KERNEL_MFMA = 3,  /* matrix-core assisted tile                    */
+  CUASR_AMD_KERNEL_MFMA = 3,  /* matrix-core assisted tile.  For CUASR_AMD_F16 plus-times this family accumulates
+                                 in float and rounds D to binary16 once (the reference's ElementAccumulator =
+                                 float); AUTO never picks it there, because AUTO's binary16 sums are rounded
+                                 term by term like the reference's all-half instantiation */
   CUASR_AMD_KERNEL_VALU_DIRECT = 4, /* vector-ALU tile fed by direct-to-LDS loads;
                                        needs 16-byte aligned, vector-sized operands */
   CUASR_AMD_KERNEL_VALU_STREAMK = 5 /* the same tile with the k-tiles of all output tiles shared out evenly over

@@ -82,6 +82,10 @@ def test_half_and_int8_element_types(lib):
     assert ok(desc(dtype="f16", kernel="mfma")) == 5 and ok(desc(dtype="f16", kernel="direct")) == 5
     assert sel(desc(dtype="f16")) == b"valu" and sel(desc(dtype="f16", m=63, n=1, k=5)) == b"valu"
     assert sel(desc(dtype="f16", add="plus", mult="multiplies")) == b"valu"
+    # the matrix cores accumulate binary16 plus-times in float: by request only, at any size, and with no split-K form
+    assert sel(desc(dtype="f16", add="plus", mult="multiplies", m=4096, n=4096)) == b"valu"
+    assert ok(desc(dtype="f16", add="plus", mult="multiplies", kernel="mfma")) == 0
+    assert sel(desc(dtype="f16", add="plus", mult="multiplies", kernel="mfma")) == b"mfma"
     assert sel(desc(dtype="f16", add="minimum", mult="multiplies")) == b"valu"
     assert sel(desc(dtype="f16", add="logical_or", mult="logical_and")) == b"valu"
     assert sel(desc(dtype="f16", add="plus", mult="maximum")) == b"naive"
@@ -94,7 +98,9 @@ def test_half_and_int8_element_types(lib):
     d.D = 0x10002
     assert ok(d) == 1
     assert sel(desc(dtype="i8")) == b"valu" and ok(desc(dtype="i8", kernel="valu")) == 0   # min-plus: exact in binary16
-    assert ok(desc(dtype="i8", add="bit_xor", mult="bit_and")) == 0 and sel(desc(dtype="i8", add="bit_xor", mult="bit_and")) == b"naive"
+    assert ok(desc(dtype="i8", add="bit_xor", mult="bit_and")) == 0 and sel(desc(dtype="i8", add="bit_xor", mult="bit_and")) == b"valu"
+    assert sel(desc(dtype="i8", add="minimum", mult="multiplies")) == b"valu"      # (int16 lanes)
+    assert ok(desc(dtype="i8", add="bit_xor", mult="logical_and")) == 0 and sel(desc(dtype="i8", add="bit_xor", mult="logical_and")) == b"naive"
     assert ok(desc(dtype="i8", add="plus", mult="multiplies", kernel="valu")) == 5
     assert cuasr_amd.splitk_workspace_bytes(100, 7, 3, "i8") == 4 * 100 * 7 * 3
     d = desc()

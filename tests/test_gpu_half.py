@@ -224,6 +224,111 @@ def test_batch_in_the_grid(oracle, lib):
             assert_same_bits(got[i], want, f"batch product {i} of {m}x{n}x{k}")
 
 
+@pytest.mark.parametrize("layouts", LAYOUTS)
+def test_plus_times_matrix_cores_exact_on_small_integers(oracle, lib, layouts):
+    """kernel = mfma on binary16 operands accumulates in float (the reference's ElementAccumulator = float).  On
+    small integers every product, every partial sum in either precision and the result are exact, so the output
+    must equal the oracle's binary16 sums bit for bit: this checks the fragment layouts, the transposing stager,
+    the guards and the epilogue.  Whole tiles (the unguarded kernel), ragged everything, single element, thin."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for (m, n, k), (alpha, beta) in [((128, 128, 64), (1, 0)), ((256, 384, 192), (1, 1)), ((100, 70, 45), (2, -1)), ((1, 1, 1), (1, 1)),
+                                     ((130, 258, 67), (-1, 2)), ((64, 8, 200), (1, 1)), ((16, 16, 16), (1, 0)), ((512, 256, 128), (1, 1))]:
+        A = inputs.integers(21, m, k, -2, 2, np.float16, order_of(la))
+        B = inputs.integers(22, k, n, -2, 2, np.float16, order_of(lb))
+        C = inputs.integers(23, m, n, -8, 8, np.float16, order_of(lc))
+        want = oracle.srgemm("plus", "multiplies", A, B, C, np.float16(alpha), np.float16(beta), np.float16(0))
+        assert np.abs(want.astype(np.float64)).max() <= 2048
+        dD = to_device(np.full_like(C, 7))
+        print(f"half plus-times mfma {m}x{n}x{k} {layouts} alpha={alpha} beta={beta}", flush=True)
+        cuasr_amd.srgemm("plus", "multiplies", to_device(A), to_device(B), to_device(C), dD, np.float16(alpha), np.float16(beta),
+                         np.float16(0), np.float16(1), dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"plus-times f16 mfma {m}x{n}x{k} {layouts}")
+
+
+@pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc"])
+def test_plus_times_matrix_cores_float_accumulation(lib, layouts):
+    """On data whose sums do not fit binary16, the matrix-core kernel must be within one binary16 rounding of
+    alpha * (A B) + beta * C computed in double, plus the error of a float sum: |d - r| <= 2^-11 |r| + 1e-5 sum |a||b|
+    (the vector-ALU tile, which rounds every partial sum to binary16, is far outside that bound at k = 1024)."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+    for (m, n, k) in [(256, 256, 1024), (1000, 900, 333)]:
+        A = inputs.uniform(31, m, k, -1.0, 1.0, np.float16, order_of(la))
+        B = inputs.uniform(32, k, n, -1.0, 1.0, np.float16, order_of(lb))
+        C = inputs.uniform(33, m, n, -4.0, 4.0, np.float16, order_of(lc))
+        alpha, beta = np.float16(0.75), np.float16(-1.5)
+        r = float(alpha) * (A.astype(np.float64) @ B.astype(np.float64)) + float(beta) * C.astype(np.float64)
+        bound = 2.0 ** -11 * np.abs(r) + 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + 1e-7
+        dD = to_device(np.zeros_like(C))
+        cuasr_amd.srgemm("plus", "multiplies", to_device(A), to_device(B), to_device(C), dD, alpha, beta, np.float16(0), np.float16(1),
+                         dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        err = np.abs(dD.cpu().numpy().astype(np.float64) - r)
+        assert (err <= bound).all(), f"{m}x{n}x{k} {layouts}: worst excess {(err - bound).max():.3e}"
+
+
+def test_matrix_cores_only_on_request(lib):
+    """The library's own choice for binary16 plus-times stays the tile that is bit-identical to the oracle; the
+    float-accumulating kernel has no split-K form (its partial sums would have to leave as binary16)."""
+    import torch
+    import cuasr_amd
+    dA = to_device(np.zeros((4096, 64), np.float16))
+    dB = to_device(np.zeros((64, 4096), np.float16))
+    dD = to_device(np.zeros((4096, 4096), np.float16))
+    desc = cuasr_amd.make_desc("plus", "multiplies", "f16", dA, dB, dD, dD, 1, 0, 0, 1)
+    assert lib.cuasr_amd_selected_kernel(desc) == b"valu"
+    desc = cuasr_amd.make_desc("plus", "multiplies", "f16", dA, dB, dD, dD, 1, 0, 0, 1, kernel="mfma")
+    assert lib.cuasr_amd_srgemm_can_implement(desc) == 0 and lib.cuasr_amd_selected_kernel(desc) == b"mfma"
+    desc = cuasr_amd.make_desc("minimum", "plus", "f16", dA, dB, dD, dD, 0, 0, float("inf"), 0, kernel="mfma")
+    assert lib.cuasr_amd_srgemm_can_implement(desc) == 5
+    ws = torch.empty(4096 * 4096 * 2, dtype=torch.float16, device="cuda")
+    with pytest.raises(cuasr_amd.CuasrError) as e:
+        cuasr_amd.srgemm_splitk("plus", "multiplies", dA, dB, dD, dD, 2, ws, 1, 0, 0, 1, dtype="f16", kernel="mfma")
+    assert e.value.status == 5
+
+
+def test_plus_times_matrix_cores_batch_and_views(oracle, lib):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    for (m, n, k, batch) in [(128, 128, 64, 5), (50, 30, 70, 4)]:
+        A = inputs.integers(3, batch * m, k, -2, 2, np.float16, "C").reshape(batch, m, k)
+        B = inputs.integers(4, batch * k, n, -2, 2, np.float16, "C").reshape(batch, k, n)
+        C = inputs.integers(5, batch * m, n, -8, 8, np.float16, "C").reshape(batch, m, n)
+        dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), torch.from_numpy(C).cuda()
+        dD = torch.zeros_like(dC)
+        cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, np.float16(1), np.float16(1), np.float16(0), np.float16(1), dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        for i in range(batch):
+            want = oracle.srgemm("plus", "multiplies", A[i], B[i], C[i], np.float16(1), np.float16(1), np.float16(0))
+            assert_same_bits(got[i], want, f"batch product {i} of {m}x{n}x{k}")
+    # operands inside larger allocations, two bytes off every vector boundary
+    m, n, k = 131, 257, 67
+    for layouts in ("ccc", "rcr"):
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        A = inputs.integers(6, m + 3, k + 3, -2, 2, np.float16, order_of(la))
+        B = inputs.integers(7, k + 3, n + 3, -2, 2, np.float16, order_of(lb))
+        C = inputs.integers(8, m + 3, n + 3, -8, 8, np.float16, order_of(lc))
+        want = oracle.srgemm("plus", "multiplies", A[1:1 + m, 1:1 + k], B[1:1 + k, 1:1 + n], C[1:1 + m, 1:1 + n], np.float16(1), np.float16(1), np.float16(0))
+        dA, dB, dC = to_device(A), to_device(B), to_device(C)
+        dD = to_device(np.full_like(C, 7))
+        cuasr_amd.srgemm("plus", "multiplies", dA[1:1 + m, 1:1 + k], dB[1:1 + k, 1:1 + n], dC[1:1 + m, 1:1 + n], dD[1:1 + m, 1:1 + n],
+                         np.float16(1), np.float16(1), np.float16(0), np.float16(1), dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        assert_same_bits(got[1:1 + m, 1:1 + n], want, f"view {layouts}")
+        frame = got.copy()
+        frame[1:1 + m, 1:1 + n] = 7
+        assert (frame == 7).all(), "wrote outside the view"
+
+
 def test_no_terms(oracle, lib):
     # k = 0: the accumulator is the additive identity and only the epilogue runs
     check(oracle, "minimum", "plus", 40, 50, 0, "ccc", "auto")
