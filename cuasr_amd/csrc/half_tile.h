@@ -149,8 +149,20 @@ template <int X, bool KC, bool GUARD, typename TI, bool MASK = false, bool I16 =
 
   // chunk c -> (x, k) of its first element, tile-relative
   static __device__ __forceinline__ void where(int c, int &x, int &k) {
-    if constexpr (KC) { k = (c % (BK / 8)) * 8; x = c / (BK / 8); }
-    else { x = (c % (X / 8)) * 8; k = c / (X / 8); }
+    if constexpr (KC) {
+      // KL neighbouring lanes take neighbouring chunks of k of one x, the next lanes the next x: the 2-byte stores of
+      // one instruction then go to KL rows of the panel (8 apart: the same banks) at 64 / KL consecutive x each
+#ifndef CUASR_HALF_KL
+#define CUASR_HALF_KL 2
+#endif
+      constexpr int KL = CUASR_HALF_KL;
+      static_assert((BK / 8) % KL == 0, "chunks of k split evenly");
+      k = ((c / (KL * X)) * KL + c % KL) * 8;
+      x = (c / KL) % X;
+    } else {
+      x = (c % (X / 8)) * 8;
+      k = c / (X / 8);
+    }
   }
 
   // base: the operand's element (x = 0, k = 0); sx, sk: element strides; x0, k0: the tile's origin;
