@@ -53,6 +53,9 @@ inline cuasr_amd_srgemm_desc make_desc(Args const &a, int kernel) {
   d.alpha_ptr = a.epilogue.alpha_ptr;
   d.beta_ptr = a.epilogue.beta_ptr;
   d.kernel = kernel;
+  // half operands with a float accumulator: the matrix-core kernel is the one that accumulates in float
+  if (std::is_same<typename Op::ElementC, half_t>::value && std::is_same<typename Op::ElementAccumulator, float>::value)
+    d.kernel = CUASR_AMD_KERNEL_MFMA;
   d.reserved = 0;
   return d;
 }
@@ -120,7 +123,7 @@ class Srgemm {
 
   static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
                 "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
-                "are int8_t with int32_t C and accumulator");
+                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator");
 
   struct Arguments {
     GemmCoord problem_size;

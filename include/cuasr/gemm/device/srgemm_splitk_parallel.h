@@ -79,7 +79,7 @@ class SrgemmSplitKParallel {
 
   static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
                 "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
-                "are int8_t with int32_t C and accumulator");
+                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator");
 
   struct Arguments {
     GemmCoord problem_size;

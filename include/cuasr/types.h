@@ -190,6 +190,12 @@ template <> struct element_types<int8_t, int8_t, int32_t, int32_t> {
   static bool const valid = true;
   static int const value = CUASR_AMD_I8;
 };
+/// binary16 operands and results with a float accumulator: plus-times on the matrix cores, sums in float, D rounded
+/// to binary16 once (the library runs this only when asked to: device::Srgemm asks by this accumulator type)
+template <> struct element_types<half_t, half_t, half_t, float> {
+  static bool const valid = true;
+  static int const value = CUASR_AMD_F16;
+};
 
 template <typename T> inline cuasr_amd_scalar make_scalar(T v);
 template <> inline cuasr_amd_scalar make_scalar<half_t>(half_t v) { cuasr_amd_scalar s; s.bits = 0; s.f16 = v.bits; return s; }

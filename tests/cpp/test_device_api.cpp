@@ -191,6 +191,39 @@ static void wider_element_types() {
   ok = ok && int8_case<cuasr::plus<int32_t>, cuasr::multiplies<int32_t>, RowMajor, ColumnMajor, RowMajor>(256, 384, 192, 1, 1);
   report(ok, "int8 operands, int32 results: plus-times, min-plus, max-min on the testbed sweep shapes");
 
+  // half operands with a float accumulator (the reference's spelling of mixed precision): plus-times on the matrix
+  // cores, sums in float, D rounded once.  On small integers everything is exact, so the host reference with the same
+  // accumulator type must agree bit for bit; a min-plus with that accumulator has no kernel and is refused
+  {
+    using Add = cuasr::plus<float>;
+    using Mul = cuasr::multiplies<float>;
+    using Op = cuasr::gemm::device::Srgemm<Add, Mul, half_t, RowMajor, half_t, ColumnMajor, half_t, RowMajor, float>;
+    ok = true;
+    for (int m : {1, 509, 256})
+      for (int k : {1, 23, 192}) {
+        const int n = m == 256 ? 384 : 510;
+        std::vector<half_t> A(size_t(m) * k), B(size_t(k) * n), C(size_t(m) * n), D(size_t(m) * n), R(size_t(m) * n);
+        fill_int(A, 41, -2, 2);
+        fill_int(B, 42, -2, 2);
+        fill_int(C, 43, -8, 8);
+        DeviceBuf<half_t> dA(A), dB(B), dC(C), dD(D);
+        Op::Arguments args({m, n, k}, {dA.p, k}, {dB.p, k}, {dC.p, n}, {dD.p, n}, {2.0f, -1.0f});
+        Op op;
+        ok = ok && Op::can_implement(args) == Status::kSuccess && op(args) == Status::kSuccess;
+        HIP_OK(hipDeviceSynchronize());
+        cuasr::reference::host::Srgemm<Add, Mul, half_t, RowMajor, half_t, ColumnMajor, half_t, RowMajor, float, float> ref;
+        ref({m, n, k}, 2.0f, {A.data(), k}, {B.data(), k}, -1.0f, {C.data(), n}, {R.data(), n}, Add::Identity);
+        D = dD.download();
+        ok = ok && std::memcmp(D.data(), R.data(), D.size() * sizeof(half_t)) == 0;
+      }
+    using MinPlus = cuasr::gemm::device::Srgemm<cuasr::minimum<float>, cuasr::plus<float>, half_t, RowMajor, half_t, ColumnMajor, half_t, RowMajor, float>;
+    std::vector<half_t> z(64 * 64);
+    DeviceBuf<half_t> dz(z);
+    MinPlus::Arguments margs({64, 64, 64}, {dz.p, 64}, {dz.p, 64}, {dz.p, 64}, {dz.p, 64}, {0.0f, 0.0f});
+    ok = ok && MinPlus::can_implement(margs) == Status::kErrorNotSupported;
+    report(ok, "binary16 operands, float accumulator: plus-times on the matrix cores == host reference on small integers");
+  }
+
   // parallel split-K on both: the workspace holds elements of C (2 or 4 bytes each)
   {
     using Add = cuasr::minimum<half_t>;
