@@ -32,6 +32,7 @@ sys.path.insert(0, ROOT)
 FP32_VECTOR_PEAK = 157.3   # TFLOP/s, FMA counted as 2 flops (also the fp32 matrix-core peak)
 FP64_VECTOR_PEAK = 78.6    # also the fp64 matrix-core peak
 INT8_MATRIX_PEAK = 5000.0  # TOP/s, dense int8 on the matrix cores
+F16_MATRIX_PEAK = 2500.0   # TFLOP/s, dense binary16 on the matrix cores
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant kernel come from profiles/traffic.json, which the profiling
@@ -308,15 +309,17 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         def step(i):
             cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dt, kernel=args.kernel)
 
-        desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one)
-        matrix = add == "plus" and mult == "multiplies" and dt in ("f32", "f64", "i8")
+        desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one, kernel=args.kernel)
+        # (binary16 plus-times runs on the matrix cores, with float accumulation, only when asked to)
+        matrix = add == "plus" and mult == "multiplies" and (dt in ("f32", "f64", "i8") or (dt == "f16" and args.kernel == "mfma"))
         return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=desc, host=(add, mult, A, B, C, one, one, ident),
                     result=lambda: dD.cpu().numpy(),
                     metric=f"{dt} {add}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"{add}-{mult} SRGEMM {dt}, M=N=K={n}, layouts (A, B, C) = {args.layouts} "
                              "(c = column-major, r = row-major), beta = one with a seeded C",
                     bound="mfma" if matrix else "valu",
-                    peak=FP64_VECTOR_PEAK if dt == "f64" else INT8_MATRIX_PEAK if (dt == "i8" and matrix) else FP32_VECTOR_PEAK,
+                    peak=FP64_VECTOR_PEAK if dt == "f64" else INT8_MATRIX_PEAK if (dt == "i8" and matrix)
+                    else F16_MATRIX_PEAK if (dt == "f16" and matrix) else FP32_VECTOR_PEAK,
                     instr_per_term=None)
 
     raise SystemExit(f"bench.py: unknown workload {w!r}")
@@ -430,6 +433,23 @@ def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
     out.append(entry(wl, ms, steps, family_of(wl, "?"), bit_exact=bool(np.asfortranarray(got).tobytes() == np.asfortranarray(want).tobytes()),
                      checked="first 64 rows of the output",
                      note="packed binary16 instructions issue at half the rate of 4-byte ones: two terms per instruction, the same vector peak"))
+    del wl
+    torch.cuda.empty_cache()
+
+    # binary16 plus-times with float accumulation on the matrix cores (the reference's ElementAccumulator = float for
+    # half operands; by request only: kernel = mfma), 4096^3, A row-major and B column-major; the first 256 rows
+    # against a double-precision product: one binary16 rounding of the result plus the error of a float sum
+    wl = build_workload(ns(workload="srgemm", add="plus", mult="multiplies", dtype="f16", layouts="rcr", size=4096, kernel="mfma"),
+                        np, torch, cuasr_amd, inputs)
+    ms, steps = measure(wl)
+    add, mult, A, B, C, alpha, beta, ident = wl["host"]
+    a64, b64 = A[:256].astype(np.float64), B.astype(np.float64)
+    want = float(alpha) * (a64 @ b64) + float(beta) * C[:256].astype(np.float64)
+    bound = 2.0 ** -11 * np.abs(want) + 1e-5 * (np.abs(a64) @ np.abs(b64)) + 1e-7
+    got = wl["result"]()[:256].astype(np.float64)
+    out.append(entry(wl, ms, steps, "mfma", within_tolerance=bool((np.abs(got - want) <= bound).all()),
+                     tolerance="|d - r| <= 2^-11 |r| + 1e-5 * sum_k |a||b| against a double-precision product, first 256 rows",
+                     note="float accumulation: not bit-identical to the all-binary16 sums the library computes by default (65 TFLOP/s on the vector ALU)"))
     del wl
     torch.cuda.empty_cache()
 
