@@ -38,7 +38,8 @@ template <typename T> static launch_fn staged_or_and() {
 }
 template <typename T> static hipError_t or_and_on_masks(const Problem &p, hipStream_t s) {
   const long long full = (long long)((p.m + 127) / 128) * ((p.n + 255) / 256) * (p.workspace ? p.slices : 1) * p.batch;
-  if (full >= 384) return half_tile::launch<kLogicalOr, kLogicalAnd, T>(p, s);
+  // (8-byte operands from 128 such tiles on: their staged tile is slower, 2048^3 58 against 65 - 68 TOPS)
+  if (full >= (sizeof(T) == 8 ? 128 : 384)) return half_tile::launch<kLogicalOr, kLogicalAnd, T>(p, s);
   const launch_fn staged = staged_or_and<T>();
   return staged ? staged(p, s) : hipErrorNotSupported;
 }

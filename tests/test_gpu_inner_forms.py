@@ -138,14 +138,14 @@ def test_or_and_on_truth_values_of_arbitrary_operands(oracle, lib, dtype, kernel
 @pytest.mark.parametrize("dtype", ["f32", "f64", "i32", "u32"])
 @pytest.mark.parametrize("layouts", ["ccc", "rcr", "crr", "rrc", "rrr", "ccr"])
 def test_or_and_large_outputs_on_packed_masks(oracle, lib, dtype, layouts):
-    """From 384 tiles of 128 x 256 on, or-and on 4- and 8-byte operands runs on the 16-bit mask tile: whole tiles of
+    """From 384 tiles of 128 x 256 on (double: 128), or-and on 4- and 8-byte operands runs on the 16-bit mask tile: whole tiles of
     aligned operands, ragged extents, an identity that is not zero, scalars that are zero, and floating-point operands
     that hold -0 (false), NaN and infinities (true, functional.h:212)."""
     import cuasr_amd
     npd = NPD[dtype]
     la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
     for (m, n, k), ident, alpha, beta in (((4096, 3072, 64), 0, 1, 1), ((4000, 4100, 37), 0, 1, 0), ((4000, 4100, 37), 0, 0, 1),
-                                          ((3968, 3328, 33), 2.5, 1, 1)):
+                                          ((3968, 3328, 33), 2.5, 1, 1), ((2048, 2048, 40), 0, 1, 0)):   # (the last: on masks for f64 only)
         A, B = sparse(31, m, k, npd, order_of(la), 0.06), sparse(32, k, n, npd, order_of(lb), 0.06)
         C = sparse(33, m, n, npd, order_of(lc), 0.3)
         if dtype in ("f32", "f64"):
