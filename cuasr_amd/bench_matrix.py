@@ -6,7 +6,7 @@ in powers of two with alpha = beta = the multiplicative identity and reports 2 *
 shapes are the library's business here, so the matrix is semiring x type x layout x size.
 
     python -m cuasr_amd.bench_matrix [--sizes 256,512,1024,2048,4096] [--dtypes f32,f64]
-                                     [--layouts nn,nt,tn,tt] [--kernel auto] [--json out.jsonl]
+                                     [--layouts nn,nt,tn,tt] [--kernel auto] [--json out.jsonl] [--bitwise]
 
 Layouts name A and B as the reference does (n = column-major, t = row-major); C and D are
 column-major.  Prints a table of TOPS (2 ops per term) and, with --json, one JSON object per case.
@@ -25,6 +25,8 @@ import sys
 
 SEMIRINGS = [("plus", "multiplies"), ("minimum", "plus"), ("maximum", "plus"), ("minimum", "multiplies"),
              ("maximum", "multiplies"), ("minimum", "maximum"), ("maximum", "minimum"), ("logical_or", "logical_and")]
+# the pairs on bits (the reference's user-defined example is xor-and, examples/01_userdefined_semiring): integer types only
+BITWISE = [("bit_xor", "bit_and"), ("bit_or", "bit_and")]
 
 
 def main():
@@ -35,6 +37,7 @@ def main():
     ap.add_argument("--kernel", default="auto")
     ap.add_argument("--json", default=None)
     ap.add_argument("--tune", action="store_true", help="also time every forced kernel family; list where auto loses")
+    ap.add_argument("--bitwise", action="store_true", help="add xor-and and or-and on bits (dtypes i32, u32, i8)")
     args = ap.parse_args()
 
     import numpy as np
@@ -64,7 +67,10 @@ def main():
     for dt in args.dtypes.split(","):
         # (f16: binary16 throughout; i8: int8 A and B, int32 C and D)
         npd, tdt = {"f32": (np.float32, torch.float32), "f64": (np.float64, torch.float64), "f16": (np.float16, torch.float16),
-                    "i8": (np.int32, torch.int32)}[dt]
+                    "i8": (np.int32, torch.int32), "i32": (np.int32, torch.int32), "u32": (np.uint32, torch.int32)}[dt]
+        integer = dt in ("i8", "i32", "u32")
+        if args.bitwise and not integer:
+            sys.exit("bench_matrix: --bitwise needs integer dtypes (i32, u32, i8)")
         print(f"\n{dt}: TOPS (2 ops per term), layouts of A and B = {' '.join(layouts)}; C, D column-major; kernel = {args.kernel}")
         print("| add-mult | " + " | ".join(f"N={n}" for n in sizes) + " |")
         print("|---|" + "---|" * len(sizes))
@@ -76,10 +82,14 @@ def main():
             if dt == "i8":
                 data[n] = [torch.from_numpy(inputs.integers(901 + (i << 40), n, n, -128, 127, np.int8, "C")).cuda() for i in range(2)]
                 data[n].append(torch.from_numpy(inputs.integers(901 + (2 << 40), n, n, -1000, 1000, np.int32, "C")).cuda())
+            elif integer:
+                # random words for the pairs on bits; (small values would suit the arithmetic pairs, which this table
+                # times on the floating-point types)
+                data[n] = [torch.from_numpy(inputs.words32(901 + (i << 40), n, n, "C").view(np.int32)).cuda() for i in range(3)]
             else:
                 data[n] = [torch.from_numpy(inputs.uniform(901 + (i << 40), n, n, -1.0, 1.0, npd, "C")).cuda() for i in range(3)]
             data[n].append(torch.empty(n, n, dtype=tdt, device="cuda"))
-        for add, mult in SEMIRINGS:
+        for add, mult in (BITWISE if args.bitwise else SEMIRINGS):
             ident = cuasr_amd.op_identity(add, dt, True)
             one = cuasr_amd.op_identity(mult, dt, True)
             cells = []
