@@ -234,7 +234,10 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   // both operands k-contiguous, 4-byte types: the direct tile has no hand-scheduled loop for that pair of
   // panel forms (two k-quad operands do not fit 128 registers) and its 2-wave variant is slower than the
   // staged tile (4096^3 min-plus: 70.4 against 72.9 TOPS)
-  const bool both_kc = !f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
+  // (not so for xor-and / or-and on words, one instruction per term: there the 2-wave direct tile wins, 4096^3 87 - 88
+  // against 77 TOPS)
+  const bool one_instruction = d->mult_op == kBitAnd && (d->add_op == kBitXor || d->add_op == kBitOr);
+  const bool both_kc = !f64 && !one_instruction && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
   if (streamk_preferred(d, batch)) return kStreamK;
   if (direct_usable(d) && ((fills && !((both_kc || masked) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
