@@ -234,12 +234,16 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   // both operands k-contiguous, 4-byte types: the direct tile has no hand-scheduled loop for that pair of
   // panel forms (two k-quad operands do not fit 128 registers) and its 2-wave variant is slower than the
   // staged tile (4096^3 min-plus: 70.4 against 72.9 TOPS)
-  // (not so for xor-and / or-and on words, one instruction per term: there the 2-wave direct tile wins, 4096^3 87 - 88
-  // against 77 TOPS)
-  const bool one_instruction = d->mult_op == kBitAnd && (d->add_op == kBitXor || d->add_op == kBitOr);
-  const bool both_kc = !f64 && !one_instruction && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
+  // (float only: on the integer types the 2-wave direct tile wins that case -- xor-and / or-and on words 87 - 88
+  // against 77 TOPS at 4096^3, min-plus 47.7 against 45.1, plus-times 45.9 against 41.8)
+  const bool kc2 = c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1;
+  const bool both_kc = d->dtype == CUASR_AMD_F32 && kc2;
+  // integer plus-times on the 4-wave direct tile is a compiled multiply-add loop that spills: 22.6 against 41.9 TOPS
+  // on the staged tile (4096^3); its 2-wave form for two k-contiguous operands does not
+  const bool slow_direct = (d->dtype == CUASR_AMD_I32 || d->dtype == CUASR_AMD_U32) && d->add_op == kPlus &&
+                           d->mult_op == kMultiplies && !kc2;
   if (streamk_preferred(d, batch)) return kStreamK;
-  if (direct_usable(d) && ((fills && !((both_kc || masked) && have_valu)) || !have_valu)) return kDirect;
+  if (direct_usable(d) && ((fills && !((both_kc || masked || slow_direct) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
   return kNaive;
@@ -258,6 +262,8 @@ static Block direct_block(const cuasr_amd_srgemm_desc *d, const Problem &c) {
   // or-and and 4-byte operands that are both k-contiguous prefer the staged tile at any size (pick_family)
   if (d->add_op == kLogicalOr && d->mult_op == kLogicalAnd) return none;
   if (!f64 && c.sa_k == 1 && c.sa_m != 1 && c.sb_k == 1 && c.sb_n != 1) return none;
+  // ... and so does integer plus-times (the direct tile's compiled multiply-add loop is the slower one)
+  if ((d->dtype == CUASR_AMD_I32 || d->dtype == CUASR_AMD_U32) && d->add_op == kPlus && d->mult_op == kMultiplies) return none;
   const int tile_m = f64 ? 128 : 256;
   const int tile_n = 128;
   const long long slots = 512;
