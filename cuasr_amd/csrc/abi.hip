@@ -118,6 +118,11 @@ static bool streamk_usable(const cuasr_amd_srgemm_desc *d) {
 
 // ... and worth it: the plain tiles would leave a good part of their last round of 512 places empty, and every
 // workgroup's share of the k-tiles is long enough to carry a tile's prologue and fold
+// 70 % or more of the compute units get one tile each and none gets two: the plain direct tile then beats both the
+// shared tiles, whose folds cost more than the idle units (2560^3 min-plus: 60 - 66 against 54 - 57 TOPS), and the
+// staged tile (2816^3: 71 against 60)
+static bool one_tile_each(long long tiles) { return tiles <= 256 && tiles * 10 >= 256 * 7; }
+
 static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
   if (batch != 1 || d->split_k_slices != 1 || !streamk_usable(d)) return false;
   // min-max and max-min spend two instructions per term and their staged tile is within 5 % of the direct one:
@@ -127,6 +132,7 @@ static bool streamk_preferred(const cuasr_amd_srgemm_desc *d, long long batch) {
   const long long tiles = (long long)((c.m + 255) / 256) * ((c.n + 127) / 128), ktiles = (c.k + 15) / 16;
   const long long rounds = (tiles + 511) / 512;
   if (tiles * 10 >= rounds * 512 * 9) return false;   // >= 90 % of the places filled: nothing to gain
+  if (d->mult_op == kPlus && one_tile_each(tiles)) return false;   // (the plain tile, one per compute unit: pick_family)
   return tiles >= 64 && tiles * ktiles >= 512 * 48;
 }
 
@@ -243,6 +249,11 @@ static int pick_family(const cuasr_amd_srgemm_desc *d, long long batch = 1) {
   const bool slow_direct = (d->dtype == CUASR_AMD_I32 || d->dtype == CUASR_AMD_U32) && d->add_op == kPlus &&
                            d->mult_op == kMultiplies && !kc2;
   if (streamk_preferred(d, batch)) return kStreamK;
+  // min-plus / max-plus, which would otherwise share their tiles out (measured for those only: generalised to every
+  // pair and type, the rule lost as often as it won; xor-and on words at 2560^3: 63 against 66 TOPS on the staged tile)
+  if (batch == 1 && d->split_k_slices == 1 && streamk_usable(d) && d->mult_op == kPlus &&
+      one_tile_each((long long)((c.m + 255) / 256) * ((c.n + 127) / 128)))
+    return kDirect;
   if (direct_usable(d) && ((fills && !((both_kc || masked || slow_direct) && have_valu)) || !have_valu)) return kDirect;
   if (have_valu) return kValu;
   if (mfma_usable(d)) return kMfma;
