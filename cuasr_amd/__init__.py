@@ -113,6 +113,8 @@ def load():
                                                 ctypes.c_int64, ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p]
         lib.cuasr_amd_selected_kernel.restype = ctypes.c_char_p
         lib.cuasr_amd_selected_kernel.argtypes = [ctypes.POINTER(SrgemmDesc)]
+        lib.cuasr_amd_selected_kernel_batched.restype = ctypes.c_char_p
+        lib.cuasr_amd_selected_kernel_batched.argtypes = [ctypes.POINTER(SrgemmDesc), ctypes.c_int] + [ctypes.c_int64] * 4
         _lib = lib
     return _lib
 

@@ -64,30 +64,20 @@ def build(jobs=None, verbose=True):
     return LIB
 
 
-def build_cpp_tests():
-    """The C++ operator-API test program (tests/cpp), linked against the library."""
+def build_functor_bench():
+    """cuasr_amd/functor_bench.hip -> cuasr_amd/lib/functor_bench: the throughput of kernels built from user functors
+    (what `bench.py --workload functor` runs), compiled the way a user's translation unit is."""
     root = os.path.dirname(HERE)
-    src = os.path.join(root, "tests", "cpp", "test_device_api.cpp")
-    out = os.path.join(root, "tests", "cpp", "test_device_api")
-    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
-    # plain host C++: the operator templates need only the HIP runtime API header
-    subprocess.check_call([os.environ.get("CXX", "g++"), "-std=c++17", "-O1", "-D__HIP_PLATFORM_AMD__",
-                           "-I", os.path.join(rocm, "include"),
-                           "-I", os.path.join(root, "include"), "-I", os.path.join(root, "oracle", "include"),
-                           src, "-L", LIB_DIR, "-lcuasr_amd", "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
-                           "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,$ORIGIN/../../cuasr_amd/lib", "-o", out])
-    # the functor path of the operator templates needs hipcc: its kernel is built in the user's translation unit
-    src2 = os.path.join(root, "tests", "cpp", "test_user_functor.hip")
-    out2 = os.path.join(root, "tests", "cpp", "test_user_functor")
-    subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-O2", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-                           "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
-                           "-I", os.path.join(root, "include"), "-I", os.path.join(root, "oracle", "include"),
-                           src2, "-L", LIB_DIR, "-lcuasr_amd", "-Wl,-rpath," + LIB_DIR,
-                           "-Wl,-rpath,$ORIGIN/../../cuasr_amd/lib", "-o", out2], stderr=subprocess.DEVNULL)
+    out = os.path.join(LIB_DIR, "functor_bench")
+    cmd = [HIPCC] + [f for f in FLAGS if f != "-fPIC"] + ["-I", os.path.join(root, "include"), os.path.join(HERE, "functor_bench.hip"),
+                                                          "-L", LIB_DIR, "-lcuasr_amd", "-Wl,-rpath," + LIB_DIR, "-Wl,-rpath,$ORIGIN", "-o", out]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on functor_bench.hip:\n" + r.stderr[-4000:])
     return out
 
 
 if __name__ == "__main__":
     j = int(sys.argv[sys.argv.index("-j") + 1]) if "-j" in sys.argv else None
     print(build(j))
-    print(build_cpp_tests())
+    print(build_functor_bench())

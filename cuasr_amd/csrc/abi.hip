@@ -336,6 +336,41 @@ static launch_fn family_fn(int family, const cuasr_amd_srgemm_desc *d) {
   }
 }
 
+// Which family a strided batch runs on, and whether the product index goes into the grid (one launch for
+// the whole batch) or the batch becomes a sequence of launches.  -1: the descriptor names the direct-to-LDS
+// tile and the batch strides do not keep its 16-byte alignment.
+static int batched_family(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a, int64_t stride_b, int64_t stride_c,
+                          int64_t stride_d, bool *in_grid_out) {
+  const bool col = desc->layout_c == CUASR_AMD_COLUMN_MAJOR;
+  int family = pick_family(desc, batch);
+  if (family == kDirect && batch > 1) {
+    // the direct-to-LDS tiles fetch 16-byte vectors: a batch stride that is no multiple of 16 bytes leaves the
+    // later products misaligned; the staged tile takes any element alignment, with the batch still in the grid
+    Problem probe = canonical(desc);
+    probe.batch = batch < 65535 ? batch : 65535;
+    probe.batch_a = col ? stride_b : stride_a;
+    probe.batch_b = col ? stride_a : stride_b;
+    probe.batch_c = stride_c;
+    probe.batch_d = stride_d;
+    if (!(desc->dtype == CUASR_AMD_F64 ? direct64_can_run(probe) : direct_can_run(probe))) {
+      if (desc->kernel == CUASR_AMD_KERNEL_VALU_DIRECT) return -1;  // asked for by name
+      family = find_valu(desc->dtype, desc->add_op, desc->mult_op) ? kValu : kNaive;
+    }
+  }
+  bool in_grid = (family == kValu || family == kDirect) && batch > 1;
+  if (family == kMfma && batch > 1 && desc->add_op == kPlus && desc->mult_op == kMultiplies) {
+    // the hand-scheduled matrix-core tiles take a batch in the grid too; the compiled ones (ragged k, unaligned
+    // products) do not: ask with the first launch's problem
+    Problem probe = canonical(desc);
+    probe.batch = batch < 65535 ? batch : 65535;
+    probe.batch_a = col ? stride_b : stride_a;
+    probe.batch_b = col ? stride_a : stride_b;
+    in_grid = (desc->dtype == CUASR_AMD_I8 || desc->dtype == CUASR_AMD_F16) ? true : desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
+  }
+  *in_grid_out = in_grid;
+  return family;
+}
+
 }  // namespace cuasr_amd
 
 using namespace cuasr_amd;
@@ -371,6 +406,20 @@ const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc) {
     case kStreamK: return "valu_streamk";
     case kValu: return direct_block(desc, canonical(desc)).rows ? "valu_direct+valu" : "valu";  // a block + two strips
     default: return "naive";
+  }
+}
+
+const char *cuasr_amd_selected_kernel_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a, int64_t stride_b,
+                                              int64_t stride_c, int64_t stride_d) {
+  if (!desc || batch < 1 || stride_a < 0 || stride_b < 0 || stride_c < 0 || stride_d < 0) return nullptr;
+  if (validate(desc, false) != CUASR_AMD_SUCCESS) return nullptr;
+  bool in_grid = false;
+  switch (batched_family(desc, batch, stride_a, stride_b, stride_c, stride_d, &in_grid)) {
+    case kMfma: return in_grid ? "mfma" : "mfma, a launch per product";
+    case kDirect: return in_grid ? "valu_direct" : "valu_direct, a launch per product";
+    case kValu: return in_grid ? "valu" : "valu, a launch per product";
+    case -1: return nullptr;
+    default: return "a launch per product";   // each product picks for itself (cuasr_amd_selected_kernel)
   }
 }
 
@@ -422,17 +471,9 @@ int cuasr_amd_srgemm_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64
   if (batch > 1 && outer > 0 && inner > 0 && stride_d < (outer - 1) * desc->ldd + inner) return CUASR_AMD_ERROR_INVALID_PROBLEM;
   if (batch == 0) return CUASR_AMD_SUCCESS;
   const int64_t es = int64_t(elem_size(desc->dtype)), os = int64_t(operand_size(desc->dtype));
-  const int family = pick_family(desc, batch);
-  bool in_grid = (family == kValu || family == kDirect) && batch > 1;
-  if (family == kMfma && batch > 1 && desc->add_op == kPlus && desc->mult_op == kMultiplies) {
-    // the hand-scheduled matrix-core tiles take a batch in the grid too; the compiled ones (ragged k, unaligned
-    // products) do not: ask with the first launch's problem
-    Problem probe = canonical(desc);
-    probe.batch = batch < 65535 ? batch : 65535;
-    probe.batch_a = col ? stride_b : stride_a;
-    probe.batch_b = col ? stride_a : stride_b;
-    in_grid = (desc->dtype == CUASR_AMD_I8 || desc->dtype == CUASR_AMD_F16) ? true : desc->dtype == CUASR_AMD_F64 ? mfma_direct_f64_can_run(probe) : mfma_direct_f32_can_run(probe);
-  }
+  bool in_grid = false;
+  const int family = batched_family(desc, batch, stride_a, stride_b, stride_c, stride_d, &in_grid);
+  if (family < 0) return CUASR_AMD_ERROR_MISALIGNED_OPERAND;  // the direct-to-LDS tile asked for by name, strides off 16 bytes
   if (in_grid) {
     const launch_fn fn = family_fn(family, desc);
     if (!fn) return CUASR_AMD_ERROR_NOT_SUPPORTED;

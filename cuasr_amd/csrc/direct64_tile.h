@@ -261,6 +261,8 @@ static inline bool direct64_ok(const Problem &p) {
   auto al = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
   const bool a_kc = p.sa_k == 1 && p.sa_m != 1, b_kc = p.sb_k == 1 && p.sb_n != 1;
   if (p.k <= 0 || !al(p.A) || !al(p.B)) return false;
+  // every product of a batch in the grid starts at base + index * stride: the strides keep the 16-byte alignment
+  if (p.batch > 1 && ((p.batch_a | p.batch_b | p.batch_c | p.batch_d) % 2)) return false;
   // 32-bit byte offsets inside one tile
   const long long span = 8LL * 128 * (p.sa_m > p.sa_k ? p.sa_m : p.sa_k), span_b = 8LL * 128 * (p.sb_n > p.sb_k ? p.sb_n : p.sb_k);
   if (span >= (1LL << 31) || span_b >= (1LL << 31)) return false;

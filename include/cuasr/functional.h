@@ -24,6 +24,7 @@
 #pragma once
 #include <limits>
 
+#include "array.h"
 #include "types.h"
 
 namespace cuasr {
@@ -45,17 +46,28 @@ template <typename T> constexpr T neg_inf() {
 }
 }  // namespace detail
 
-#if defined(__HIPCC__)
-#define CUASR_HOST_DEVICE __host__ __device__
-#else
-#define CUASR_HOST_DEVICE
-#endif
-
+// Besides the scalar form every functor has the reference's three element-wise forms on Array<T, N>
+// (functional.h:52-79 and the same three per functor): array with array, array with scalar, scalar with array.
 #define CUASR_AMD_FUNCTOR(NAME, IDENT, ANNIH, EXPR)                               \
   template <typename T, int N = 1> struct NAME {                                  \
     static constexpr T Identity = IDENT;                                          \
     static constexpr T Annihilator = ANNIH;                                       \
     CUASR_HOST_DEVICE constexpr T operator()(T lhs, T const &rhs) const { return EXPR; } \
+    CUASR_HOST_DEVICE constexpr Array<T, N> operator()(Array<T, N> const &lhs, Array<T, N> const &rhs) const { \
+      Array<T, N> result{};                                                       \
+      for (int i = 0; i < N; ++i) result[i] = (*this)(lhs[i], rhs[i]);            \
+      return result;                                                              \
+    }                                                                             \
+    CUASR_HOST_DEVICE constexpr Array<T, N> operator()(Array<T, N> const &lhs, T const &scalar) const { \
+      Array<T, N> result{};                                                       \
+      for (int i = 0; i < N; ++i) result[i] = (*this)(lhs[i], scalar);            \
+      return result;                                                              \
+    }                                                                             \
+    CUASR_HOST_DEVICE constexpr Array<T, N> operator()(T const &scalar, Array<T, N> const &rhs) const { \
+      Array<T, N> result{};                                                       \
+      for (int i = 0; i < N; ++i) result[i] = (*this)(scalar, rhs[i]);            \
+      return result;                                                              \
+    }                                                                             \
   };                                                                              \
   template <typename T, int N> constexpr T NAME<T, N>::Identity;                  \
   template <typename T, int N> constexpr T NAME<T, N>::Annihilator;

@@ -19,6 +19,7 @@
 
 #include "default_srgemm_configuration.h"
 #if defined(__HIPCC__)
+#include "../../reduction/kernel/reduce_split_k.h"
 #include "../kernel/functor_srgemm.h"
 #endif
 
@@ -53,12 +54,97 @@ inline cuasr_amd_srgemm_desc make_desc(Args const &a, int kernel) {
   d.alpha_ptr = a.epilogue.alpha_ptr;
   d.beta_ptr = a.epilogue.beta_ptr;
   d.kernel = kernel;
-  // half operands with a float accumulator: the matrix-core kernel is the one that accumulates in float
+  // half operands with a float accumulator (plus-times only, see the operator's static_assert): the matrix-core
+  // kernel is the one that accumulates in float
   if (std::is_same<typename Op::ElementC, half_t>::value && std::is_same<typename Op::ElementAccumulator, float>::value)
     d.kernel = CUASR_AMD_KERNEL_MFMA;
   d.reserved = 0;
   return d;
 }
+/// k-tile depth the reference's default configurations slice K by (ThreadblockShape::kK = 8 in every one of
+/// them, device/default_srgemm_configuration.h:44-275); kernels built from user functors follow its slice
+/// rules with this depth, because their results may depend on where a slice ends.
+static int const kReferenceTileK = 8;
+
+/// The host-side checks of a problem that runs on kernels built from user functors (no C-ABI descriptor to validate).
+template <typename Op, typename Args> inline Status functor_check(Args const &args) {
+  const long long m = args.problem_size.m(), n = args.problem_size.n(), k = args.problem_size.k();
+  if (m < 0 || n < 0 || k < 0 || args.split_k_slices < 1 || args.split_k_slices > 65535) return Status::kErrorInvalidProblem;
+  auto ld_ok = [](long long ld, bool column_major, long long rows, long long cols) { return ld >= (column_major ? rows : cols); };
+  if (m > 0 && k > 0 && !ld_ok(args.ref_A.stride(0), Op::LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, k)) return Status::kErrorInvalidProblem;
+  if (n > 0 && k > 0 && !ld_ok(args.ref_B.stride(0), Op::LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, k, n)) return Status::kErrorInvalidProblem;
+  if (m > 0 && n > 0) {
+    if (!args.ref_D.data() || !ld_ok(args.ref_D.stride(0), Op::LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
+    if (args.ref_C.data() && !ld_ok(args.ref_C.stride(0), Op::LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
+    if (k > 0 && (!args.ref_A.data() || !args.ref_B.data())) return Status::kErrorInvalidProblem;
+  }
+  return Status::kSuccess;
+}
+
+#if defined(__HIPCC__)
+/// Typed arguments -> the parameters of the functor kernel (one slice, epilogue in the kernel).
+template <typename Op, typename Args> inline kernel::FunctorSrgemmParams<typename Op::ElementC> functor_params(Args const &a) {
+  using Element = typename Op::ElementC;
+  kernel::FunctorSrgemmParams<Element> p{};
+  p.m = a.problem_size.m();
+  p.n = a.problem_size.n();
+  p.k = a.problem_size.k();
+  auto strides = [](long long ld, bool column_major, long long &s_row, long long &s_col) {
+    s_row = column_major ? 1 : ld;
+    s_col = column_major ? ld : 1;
+  };
+  p.A = a.ref_A.data();
+  strides(a.ref_A.stride(0), Op::LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sa_m, p.sa_k);
+  p.B = a.ref_B.data();
+  strides(a.ref_B.stride(0), Op::LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sb_k, p.sb_n);
+  p.C = a.ref_C.data();
+  strides(a.ref_C.stride(0), Op::LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sc_m, p.sc_n);
+  p.D = a.ref_D.data();
+  strides(a.ref_D.stride(0), Op::LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sd_m, p.sd_n);
+  p.alpha = a.epilogue.alpha;
+  p.beta = a.epilogue.beta;
+  p.alpha_ptr = static_cast<Element const *>(a.epilogue.alpha_ptr);
+  p.beta_ptr = static_cast<Element const *>(a.epilogue.beta_ptr);
+  p.workspace = nullptr;
+  p.slices = 1;
+  p.k_per_slice = p.k;
+  p.last_takes_rest = 0;
+  return p;
+}
+
+/// Both split-K forms on kernels built from the functors: the slices' raw accumulators into the workspace
+/// (one launch, the slice index in the grid), then the fold + epilogue.  k_per_slice follows the reference:
+/// parallel ((K / 8) / S) * 8 with the last slice running on to K (kernel/srgemm_splitk_parallel.h:86-89,
+/// :136-142), serial ceil(ceil(K / 8) / S) * 8 with every slice cut off at K (kernel/srgemm.h:97-100, :184-189).
+template <typename Op, typename Args> inline Status functor_splitk(Args const &a, void *workspace, bool serial, hipStream_t stream) {
+  using Element = typename Op::ElementC;
+  using Add = typename Op::AdditionOp;
+  using Mult = typename Op::MultiplicationOp;
+  kernel::FunctorSrgemmParams<Element> p = functor_params<Op>(a);
+  const int slices = a.split_k_slices;
+  p.workspace = static_cast<Element *>(workspace);
+  p.slices = slices;
+  const long long tk = kReferenceTileK;
+  if (serial) {
+    const long long iterations = (p.k + tk - 1) / tk;
+    p.k_per_slice = (int)(((iterations + slices - 1) / slices) * tk);
+    p.last_takes_rest = 0;
+  } else {
+    p.k_per_slice = (int)(((p.k / tk) / slices) * tk);
+    p.last_takes_rest = 1;
+  }
+  if (kernel::launch_functor_srgemm<Add, Mult, Element>(p, stream) != hipSuccess) return Status::kErrorInternal;
+  reduction::kernel::FunctorReduceParams<Element> r{};
+  r.m = p.m; r.n = p.n; r.slices = slices;
+  r.workspace = p.workspace;
+  r.C = p.C; r.sc_m = p.sc_m; r.sc_n = p.sc_n;
+  r.D = p.D; r.sd_m = p.sd_m; r.sd_n = p.sd_n;
+  r.alpha = p.alpha; r.beta = p.beta; r.alpha_ptr = p.alpha_ptr; r.beta_ptr = p.beta_ptr;
+  return reduction::kernel::launch_functor_reduce<Add, Mult, Element>(r, serial, stream) == hipSuccess ? Status::kSuccess
+                                                                                                      : Status::kErrorInternal;
+}
+#endif
+
 template <typename OperatorClass> struct kernel_of { static int const value = CUASR_AMD_KERNEL_AUTO; };
 template <> struct kernel_of<arch::OpClassMatrixCore> { static int const value = CUASR_AMD_KERNEL_MFMA; };
 template <> struct kernel_of<arch::OpClassVectorAlu> { static int const value = CUASR_AMD_KERNEL_VALU; };
@@ -116,14 +202,17 @@ class Srgemm {
   static bool const kSplitKSerial = SplitKSerial;
   /// true when AdditionOp or MultiplicationOp is none of the library's operators (no cuasr::op_tag
   /// specialisation): the kernel is then built from the functors' operator() in this translation unit
-  /// (cuasr/gemm/kernel/functor_srgemm.h), which needs hipcc; split-K is not offered for such functors
+  /// (cuasr/gemm/kernel/functor_srgemm.h), which needs hipcc; the serial split-K runs on the same kernel plus the
+  /// replay of the slices' epilogues in cuasr/reduction/kernel/reduce_split_k.h
   static bool const kUserFunctors = op_tag<AdditionOp>::value < 0 || op_tag<MultiplicationOp>::value < 0;
   static_assert(!kUserFunctors || (std::is_same<ElementA, ElementC>::value && sizeof(ElementC) >= 4),
                 "kernels built from user functors: float, double, int32_t or uint32_t throughout");
 
   static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
                 "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
-                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator");
+                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator (plus-times "
+                "only: every other pair computes in binary16 throughout and is refused by can_implement with that "
+                "accumulator -- name half_t as the accumulator type instead)");
 
   struct Arguments {
     GemmCoord problem_size;
@@ -149,20 +238,7 @@ class Srgemm {
   static Status can_implement(Arguments const &args) {
     if (!kSplitKSerial && args.split_k_slices > 1) return Status::kErrorInvalidProblem;
     if (args.split_k_slices < 1) return Status::kErrorInvalidProblem;
-    if constexpr (kUserFunctors) {
-      if (args.split_k_slices > 1) return Status::kErrorNotSupported;
-      const long long m = args.problem_size.m(), n = args.problem_size.n(), k = args.problem_size.k();
-      if (m < 0 || n < 0 || k < 0) return Status::kErrorInvalidProblem;
-      auto ld_ok = [](long long ld, bool column_major, long long rows, long long cols) { return ld >= (column_major ? rows : cols); };
-      if (m > 0 && k > 0 && !ld_ok(args.ref_A.stride(0), LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, k)) return Status::kErrorInvalidProblem;
-      if (n > 0 && k > 0 && !ld_ok(args.ref_B.stride(0), LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, k, n)) return Status::kErrorInvalidProblem;
-      if (m > 0 && n > 0) {
-        if (!args.ref_D.data() || !ld_ok(args.ref_D.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
-        if (args.ref_C.data() && !ld_ok(args.ref_C.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, m, n)) return Status::kErrorInvalidProblem;
-        if (k > 0 && (!args.ref_A.data() || !args.ref_B.data())) return Status::kErrorInvalidProblem;
-      }
-      return Status::kSuccess;
-    }
+    if constexpr (kUserFunctors) return detail::functor_check<Srgemm>(args);
     cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
     d.split_k_slices = 1;  // the slice count is checked above; the rest is the plain problem's check
     return static_cast<Status>(cuasr_amd_srgemm_can_implement(&d));
@@ -175,6 +251,8 @@ class Srgemm {
   /// function, as the reference's callers do.
   static size_t get_workspace_size(Arguments const &args) {
     if (!kSplitKSerial || args.split_k_slices <= 1) return 0;
+    if constexpr (kUserFunctors)
+      return sizeof(ElementC) * size_t(args.problem_size.m()) * size_t(args.problem_size.n()) * size_t(args.split_k_slices);
     cuasr_amd_srgemm_desc d = detail::make_desc<Srgemm>(args, detail::kernel_of<OperatorClass>::value);
     return cuasr_amd_splitk_serial_workspace_bytes(&d);
   }
@@ -218,26 +296,8 @@ class Srgemm {
     if (!ready_) return Status::kErrorInternal;
     if constexpr (kUserFunctors) {
 #if defined(__HIPCC__)
-      kernel::FunctorSrgemmParams<ElementC> p;
-      p.m = args_.problem_size.m();
-      p.n = args_.problem_size.n();
-      p.k = args_.problem_size.k();
-      auto strides = [](long long ld, bool column_major, long long &s_row, long long &s_col) {
-        s_row = column_major ? 1 : ld;
-        s_col = column_major ? ld : 1;
-      };
-      p.A = args_.ref_A.data();
-      strides(args_.ref_A.stride(0), LayoutA::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sa_m, p.sa_k);
-      p.B = args_.ref_B.data();
-      strides(args_.ref_B.stride(0), LayoutB::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sb_k, p.sb_n);
-      p.C = args_.ref_C.data();
-      strides(args_.ref_C.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sc_m, p.sc_n);
-      p.D = args_.ref_D.data();
-      strides(args_.ref_D.stride(0), LayoutC::kAbiTag == CUASR_AMD_COLUMN_MAJOR, p.sd_m, p.sd_n);
-      p.alpha = args_.epilogue.alpha;
-      p.beta = args_.epilogue.beta;
-      p.alpha_ptr = static_cast<ElementC const *>(args_.epilogue.alpha_ptr);
-      p.beta_ptr = static_cast<ElementC const *>(args_.epilogue.beta_ptr);
+      if (kSplitKSerial && args_.split_k_slices > 1) return detail::functor_splitk<Srgemm>(args_, workspace_, true, stream);
+      const kernel::FunctorSrgemmParams<ElementC> p = detail::functor_params<Srgemm>(args_);
       return kernel::launch_functor_srgemm<AdditionOp, MultiplicationOp, ElementC>(p, stream) == hipSuccess ? Status::kSuccess
                                                                                                            : Status::kErrorInternal;
 #else

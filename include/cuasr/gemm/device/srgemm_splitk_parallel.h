@@ -50,12 +50,6 @@ template <typename AdditionOp_, typename MultiplicationOp_, typename ElementA_, 
                                                     AdditionOp_, MultiplicationOp_, ArchTag_>::kStages,
           int kAlignmentA = 1, int kAlignmentB = 1>
 class SrgemmSplitKParallel {
-  static_assert(op_tag<AdditionOp_>::value >= 0 && op_tag<MultiplicationOp_>::value >= 0,
-                "cuasr::gemm::device::SrgemmSplitKParallel: split-K is offered for the library's operators only (plus, "
-                "multiplies, minimum, maximum, binary_and, binary_or, binary_xor, bitwise_and, bitwise_or); a functor that "
-                "computes one of them can say so by specialising cuasr::op_tag; any other functor runs through "
-                "cuasr::gemm::device::Srgemm, which builds its kernel from the functor");
-
  public:
   using ElementA = ElementA_;
   using LayoutA = LayoutA_;
@@ -76,10 +70,18 @@ class SrgemmSplitKParallel {
   using AdditionOp = AdditionOp_;
   using MultiplicationOp = MultiplicationOp_;
   static int const kStages = Stages;
+  /// true when AdditionOp or MultiplicationOp is none of the library's operators: the slice kernel and the
+  /// reduction are then built from the functors' operator() in this translation unit
+  /// (cuasr/gemm/kernel/functor_srgemm.h, cuasr/reduction/kernel/reduce_split_k.h), which needs hipcc
+  static bool const kUserFunctors = op_tag<AdditionOp>::value < 0 || op_tag<MultiplicationOp>::value < 0;
+  static_assert(!kUserFunctors || (std::is_same<ElementA, ElementC>::value && sizeof(ElementC) >= 4),
+                "kernels built from user functors: float, double, int32_t or uint32_t throughout");
 
   static_assert(element_types<ElementA, ElementB, ElementC, ElementAccumulator>::valid,
                 "A, B, C and the accumulator share one element type (as in every reference configuration), or A and B "
-                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator");
+                "are int8_t with int32_t C and accumulator, or all three are half_t with a float accumulator (plus-times "
+                "only: every other pair computes in binary16 throughout and is refused by can_implement with that "
+                "accumulator -- name half_t as the accumulator type instead)");
 
   struct Arguments {
     GemmCoord problem_size;
@@ -108,6 +110,7 @@ class SrgemmSplitKParallel {
   /// descriptor is validated, slices must be >= 1.
   static Status can_implement(Arguments const &args) {
     if (args.split_k_slices < 1) return Status::kErrorInvalidProblem;
+    if constexpr (kUserFunctors) return detail::functor_check<SrgemmSplitKParallel>(args);
     Arguments one = args;
     one.split_k_slices = 1;
     cuasr_amd_srgemm_desc d = detail::make_desc<SrgemmSplitKParallel>(one, detail::kernel_of<OperatorClass>::value);
@@ -115,6 +118,10 @@ class SrgemmSplitKParallel {
   }
 
   static size_t get_workspace_size(Arguments const &args) {
+    if constexpr (kUserFunctors) {
+      if (args.problem_size.m() < 0 || args.problem_size.n() < 0 || args.split_k_slices < 1) return 0;
+      return sizeof(ElementAccumulator) * size_t(args.problem_size.m()) * size_t(args.problem_size.n()) * size_t(args.split_k_slices);
+    }
     cuasr_amd_srgemm_desc d = detail::make_desc<SrgemmSplitKParallel>(args, CUASR_AMD_KERNEL_AUTO);
     return cuasr_amd_splitk_workspace_bytes(&d);
   }
@@ -123,7 +130,8 @@ class SrgemmSplitKParallel {
     if (!workspace) return Status::kErrorWorkspaceNull;
     Status s = can_implement(args);
     if (s != Status::kSuccess) return s;
-    desc_ = detail::make_desc<SrgemmSplitKParallel>(args, detail::kernel_of<OperatorClass>::value);
+    args_ = args;
+    if constexpr (!kUserFunctors) desc_ = detail::make_desc<SrgemmSplitKParallel>(args, detail::kernel_of<OperatorClass>::value);
     workspace_ = workspace;
     ready_ = true;
     return Status::kSuccess;
@@ -132,6 +140,10 @@ class SrgemmSplitKParallel {
   Status update(Arguments const &args, void *workspace = nullptr) {
     if (!workspace) return Status::kErrorWorkspaceNull;
     if (!ready_) return Status::kErrorInternal;
+    args_.ref_A = args.ref_A;
+    args_.ref_B = args.ref_B;
+    args_.ref_C = args.ref_C;
+    args_.ref_D = args.ref_D;
     desc_.A = args.ref_A.data();
     desc_.B = args.ref_B.data();
     desc_.C = args.ref_C.data();
@@ -142,6 +154,17 @@ class SrgemmSplitKParallel {
 
   Status run(hipStream_t stream = nullptr) {
     if (!ready_) return Status::kErrorInternal;
+    if constexpr (kUserFunctors) {
+#if defined(__HIPCC__)
+      return detail::functor_splitk<SrgemmSplitKParallel>(args_, workspace_, false, stream);
+#else
+      static_assert(!kUserFunctors,
+                    "cuasr::gemm::device::SrgemmSplitKParallel: AdditionOp / MultiplicationOp is not one of the library's "
+                    "operators (no cuasr::op_tag specialisation), so its kernels have to be built from the functors: "
+                    "compile this translation unit with hipcc, or specialise cuasr::op_tag if the functor is one of them");
+      return Status::kErrorNotSupported;
+#endif
+    }
     return static_cast<Status>(cuasr_amd_srgemm_splitk(&desc_, workspace_, stream));
   }
 
@@ -153,6 +176,7 @@ class SrgemmSplitKParallel {
   }
 
  private:
+  Arguments args_;
   cuasr_amd_srgemm_desc desc_;
   void *workspace_;
   bool ready_;

@@ -205,3 +205,7 @@ template <> inline cuasr_amd_scalar make_scalar<int32_t>(int32_t v) { cuasr_amd_
 template <> inline cuasr_amd_scalar make_scalar<uint32_t>(uint32_t v) { cuasr_amd_scalar s; s.bits = 0; s.u32 = v; return s; }
 
 }  // namespace cuasr
+
+#if !defined(CUASR_AMD_NO_CUTLASS_NAMES) && !defined(CUTLASS_HOST_DEVICE)
+#include "cutlass_names.h"
+#endif

@@ -321,6 +321,14 @@ int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64_t ld, int3
  * is invalid. */
 const char *cuasr_amd_selected_kernel(const cuasr_amd_srgemm_desc *desc);
 
+/* The same for cuasr_amd_srgemm_batched with these strides: the family, followed by ", a launch per product"
+ * when the product index does not go into the grid ("a launch per product" alone: every product chooses as
+ * cuasr_amd_selected_kernel says).  A batch whose strides are not multiples of 16 bytes stays off the
+ * direct-to-LDS tiles, whose vector loads need that alignment for every product, and runs on the staged tile.
+ * NULL for an invalid call. */
+const char *cuasr_amd_selected_kernel_batched(const cuasr_amd_srgemm_desc *desc, int batch, int64_t stride_a,
+                                              int64_t stride_b, int64_t stride_c, int64_t stride_d);
+
 #ifdef __cplusplus
 }
 #endif

@@ -131,6 +131,30 @@ def test_kernel_selection(lib):
     assert sel(desc(m=3072, n=3072, k=64)) == b"valu"               # 288 direct tiles fill no round
 
 
+def test_batched_kernel_selection_looks_at_the_strides(lib):
+    """The direct-to-LDS tiles fetch 16-byte vectors, so every product of a batch in the grid has to start at a
+    multiple of 16 bytes: strides that do not keep that alignment route the batch to the staged tile."""
+    sel = lambda d, batch, *strides: lib.cuasr_amd_selected_kernel_batched(ctypes.byref(d), batch, *strides)
+    d = desc(m=512, n=512, k=512)                                   # min-plus f32: 8 direct tiles per product
+    whole = 512 * 512
+    assert sel(d, 256, whole, whole, whole, whole) == b"valu_direct"
+    for odd in range(4):                                            # one stride off by an element is enough
+        strides = [whole] * 4
+        strides[odd] += 1
+        assert sel(d, 256, *strides) == b"valu", odd
+        strides[odd] += 3                                           # four floats further: aligned again
+        assert sel(d, 256, *strides) == b"valu_direct", odd
+    assert sel(d, 256, whole, 0, whole, whole) == b"valu_direct"   # a shared operand (stride 0)
+    d = desc(m=512, n=512, k=512, kernel="direct")
+    assert sel(d, 256, whole + 1, whole, whole, whole) is None      # asked for by name: refused, not rerouted
+    assert lib.cuasr_amd_srgemm_batched(ctypes.byref(d), 256, whole + 1, whole, whole, whole, None) == 1
+    d = desc(m=512, n=512, k=512, dtype="f64", add="maximum")
+    assert sel(d, 64, whole, whole, whole, whole) == b"valu_direct"
+    assert sel(d, 64, whole + 1, whole, whole, whole) == b"valu"    # 8-byte elements: multiples of two
+    assert sel(d, 64, whole + 2, whole, whole, whole) == b"valu_direct"
+    assert sel(d, 0, whole, whole, whole, whole) is None and sel(d, 4, -1, whole, whole, whole) is None
+
+
 def test_splitk_host_errors(lib):
     d = desc(m=256, n=256, k=4096, slices=8)
     assert cuasr_amd.splitk_workspace_bytes(256, 256, 8, "f32") == 4 * 256 * 256 * 8

@@ -112,8 +112,13 @@ def test_no_instruction_touches_a_register_an_asm_lds_read_is_filling(tmp_path):
         texts = list(ex.map(lambda s: _listing(s, str(tmp_path)), FILES))
     kernels = 0
     for src, text in zip(FILES, texts):
-        res = asm_inflight.check_listing(text, "gemm_mfma_direct" if src.startswith("mfma") else "fwgemm_direct_kernel" if src.startswith("fwgemm") else "srgemm_kernel")
+        # every kernel of the direct_*.hip files: the plain tiles and the stream-K form, which inlines the tile's
+        # segment twice inside run-time loops and so gets a register allocation of its own
+        res = asm_inflight.check_listing(text, "gemm_mfma_direct" if src.startswith("mfma") else "fwgemm_direct_kernel" if src.startswith("fwgemm") else "_kernel")
         assert res, f"{src}: no kernels found in the listing"
+        if src in ("direct_f32.hip", "direct_i32.hip", "direct_u32.hip"):
+            assert any("streamk_kernel" in k for k in res), f"{src}: no stream-K kernel was checked"
+            assert any("srgemm_kernel" in k for k in res), f"{src}: no plain tile was checked"
         kernels += len(res)
         bad = {k: v[:3] for k, v in res.items() if v}
         assert not bad, f"{src}: {len(bad)} kernels touch in-flight registers, e.g. {next(iter(bad.items()))}"

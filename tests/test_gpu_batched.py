@@ -139,3 +139,38 @@ def test_plus_times_batch_on_the_matrix_cores(oracle, dtype, kernel):
         want = oracle.srgemm("plus", "multiplies", np.asfortranarray(At[i].T), np.asfortranarray(Bt[i].T),
                              np.zeros((m, n), dtype, order="F"), 1.0, 0.0, 0.0)
         assert_same_bits(np.ascontiguousarray(got[i]), np.ascontiguousarray(want), f"{kernel} column-major product {i}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_batch_strides_off_the_vector_alignment(oracle, dtype):
+    """Products whose operands start at odd element offsets (strides of one matrix + 1, + 3 ...): the batch
+    stays in the grid but leaves the direct-to-LDS tiles, whose 16-byte loads need every product aligned."""
+    import torch
+    batch, m, n, k = 64, 512, 512, 96      # 512 direct tiles: with aligned strides this batch takes the direct-to-LDS tile
+    rng = np.random.default_rng(23)
+    tdt = torch.float32 if dtype == np.float32 else torch.float64
+
+    def strided(rows, cols, extra, lo, hi):
+        flat = rng.uniform(lo, hi, batch * (rows * cols + extra)).astype(dtype)
+        dev = torch.from_numpy(flat).cuda()
+        view = torch.as_strided(dev, (batch, rows, cols), (rows * cols + extra, cols, 1))
+        host = np.lib.stride_tricks.as_strided(flat, (batch, rows, cols), ((rows * cols + extra) * flat.itemsize, cols * flat.itemsize, flat.itemsize))
+        return dev, view, host
+
+    _, dA, A = strided(m, k, 1, 0, 10)
+    _, dB, B = strided(k, n, 3, 0, 10)
+    _, dC, C = strided(m, n, 5, 0, 30)
+    flatD = torch.full((batch * (m * n + 7),), -5, dtype=tdt, device="cuda")
+    dD = torch.as_strided(flatD, (batch, m, n), (m * n + 7, n, 1))
+    d = cuasr_amd.make_desc("minimum", "plus", "f32" if dtype == np.float32 else "f64", dA[0], dB[0], dC[0], dD[0], 0.0, 0.0, np.inf, 0.0, 1, "auto")
+    import ctypes
+    name = cuasr_amd.load().cuasr_amd_selected_kernel_batched(ctypes.byref(d), batch, dA.stride(0), dB.stride(0), dC.stride(0), dD.stride(0))
+    assert name == b"valu"
+    whole = cuasr_amd.load().cuasr_amd_selected_kernel_batched(ctypes.byref(d), batch, m * k, k * n, m * n, m * n)
+    assert whole == b"valu_direct"
+    cuasr_amd.srgemm_batched("minimum", "plus", dA, dB, dC, dD, 0.0, 0.0, float("inf"), 0.0)
+    got = torch.as_strided(flatD, (batch, m, n), (m * n + 7, n, 1)).cpu().numpy()
+    for i in list(range(0, batch, 7)) + [1, batch - 1]:
+        want = oracle.srgemm("minimum", "plus", np.ascontiguousarray(A[i]), np.ascontiguousarray(B[i]), np.ascontiguousarray(C[i]), 0.0, 0.0, np.inf)
+        assert_same_bits(np.ascontiguousarray(got[i]), want, f"product {i}")
+    assert (flatD.cpu().numpy().reshape(batch, m * n + 7)[:, m * n:] == -5).all()      # the gaps between the outputs are untouched

@@ -6,17 +6,15 @@ import subprocess
 
 import pytest
 
+import build_cpp
+
 pytestmark = pytest.mark.gpu
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-BIN = os.path.join(HERE, "cpp", "test_device_api")
 
 
 def test_cpp_operator_api(lib):
-    if not os.path.exists(BIN):
-        from cuasr_amd import build
-        build.build_cpp_tests()
-    r = subprocess.run([BIN], capture_output=True, text=True, timeout=600)
+    r = subprocess.run([build_cpp.ensure("test_device_api")], capture_output=True, text=True, timeout=600)
     print(r.stdout[-4000:])
     print(r.stderr[-2000:])
     assert r.returncode == 0, r.stdout[-4000:]
@@ -26,11 +24,7 @@ def test_cpp_operator_api(lib):
 def test_cpp_user_defined_functors(lib):
     """tests/cpp/test_user_functor.hip: device::Srgemm with functors the library has no operator for (the
     kernel is built from the functors, in a translation unit compiled by hipcc) against the host reference."""
-    binary = os.path.join(HERE, "cpp", "test_user_functor")
-    if not os.path.exists(binary):
-        from cuasr_amd import build
-        build.build_cpp_tests()
-    r = subprocess.run([binary], capture_output=True, text=True, timeout=600)
+    r = subprocess.run([build_cpp.ensure("test_user_functor")], capture_output=True, text=True, timeout=600)
     print(r.stdout[-4000:])
     print(r.stderr[-2000:])
     assert r.returncode == 0, r.stdout[-4000:]
