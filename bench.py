@@ -18,6 +18,9 @@ Other workloads (same JSON shape; one step = one SRGEMM on fixed inputs):
     plustimes_f32             fp32 plus-times on the matrix cores, 4096^3, N(0,1)
     plustimes_f64             fp64 plus-times on the matrix cores, 4096^3, N(0,1)
     srgemm                    any --add / --mult / --dtype / --layouts at --size (the reference's benchmark matrix)
+    functor                   kernels built from user functors (cuasr/gemm/kernel/functor_srgemm.h), fp32 at --size^3:
+                              runs cuasr_amd/lib/functor_bench, a program of its own because such kernels are compiled
+                              in the user's translation unit; `value` is the pair that computes min-plus through fminf
 """
 import argparse
 import json
@@ -325,6 +328,22 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
     raise SystemExit(f"bench.py: unknown workload {w!r}")
 
 
+FUNCTOR_BENCH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cuasr_amd", "lib", "functor_bench")
+
+
+def functor_lines(size, steps, warmup):
+    """Kernels built from user functors (cuasr/gemm/kernel/functor_srgemm.h) are compiled in the user's translation
+    unit, so they are measured by a program of their own, cuasr_amd/lib/functor_bench (built from
+    cuasr_amd/functor_bench.hip by `python -m cuasr_amd.build`): its JSON lines, parsed."""
+    import subprocess
+    if not os.path.exists(FUNCTOR_BENCH):
+        raise SystemExit("bench.py: cuasr_amd/lib/functor_bench is not built (python -m cuasr_amd.build)")
+    r = subprocess.run([FUNCTOR_BENCH, str(size), str(steps), str(warmup)], capture_output=True, text=True, timeout=600)
+    if r.returncode != 0:
+        raise SystemExit(f"bench.py: functor_bench failed ({r.returncode}): {r.stderr[-500:]}")
+    return [json.loads(line) for line in r.stdout.splitlines() if line.startswith("{")]
+
+
 def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
     """The other BASELINE configs, timed in the same process (a few launches each) and checked against the
     oracle on a sample: [{workload, ms, tops, frac, kernel_family, bit_exact | within_tolerance}]."""
@@ -386,7 +405,7 @@ def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
 
     # C4: split-K 256 x 256 x 65536, 8 and 64 slices; the reduction kernel on its own as well
     want = None
-    for slices in (8, 64):
+    for slices in (8, 16, 32, 64):
         wl = build_workload(ns(workload="splitk", slices=slices), np, torch, cuasr_amd, inputs)
         ms, steps = measure(wl)
         add, mult, A, B, C, alpha, beta, ident = wl["host"]
@@ -466,6 +485,18 @@ def extra_configs(np, torch, cuasr_amd, inputs, oracle, base_args):
     del wl
     torch.cuda.empty_cache()
 
+    # Kernels built from user functors (none of the library's operators): fp32 at 4096^3 for a functor pair that
+    # computes min-plus (compared bit for bit, by the program itself, with the tuned min-plus kernel, which the
+    # headline's check pins against the oracle), one spelled as the reference spells its minimum, one no library
+    # operator computes; the quarter-size tile at 1024^3; split-K 256 x 256 x 65536
+    for line in functor_lines(4096, 10, 5):
+        e = {"workload": line["workload"], "ms": line["ms"], "tops": line["tops"], "frac": round(line["tops"] / 157.3, 4),
+             "peak": 157.3, "bound": "valu", "kernel_family": "functor_srgemm_kernel (built from the user's functors by hipcc)"}
+        if line.get("bit_identical_to_tuned_min_plus") is not None:
+            e["bit_exact"] = bool(line["bit_identical_to_tuned_min_plus"])
+            e["checked"] = "whole matrix against the library's tuned min-plus kernel on the same operands"
+        out.append(e)
+
     # All-pairs shortest paths with predecessors on top of SRGEMM (README.md:338-342 of the reference,
     # cpu_fwgemm_naive): a whole job at n = 4096 by blocked Floyd-Warshall, counted as 2 n^3 operations, and the
     # same kind of graph at n = 1024 against the oracle's blocked iteration, dist and parent bit for bit
@@ -493,7 +524,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="apsp",
                     choices=["apsp", "maxplus_f64", "maxmin_f64", "splitk", "xorand_u32", "plustimes_f32", "plustimes_f64",
-                             "srgemm", "fwgemm", "apsp_blocked"])
+                             "srgemm", "fwgemm", "apsp_blocked", "functor"])
     ap.add_argument("--add", default="minimum", help="workload srgemm: the semiring's add operator")
     ap.add_argument("--mult", default="plus", help="workload srgemm: the semiring's multiply operator")
     ap.add_argument("--dtype", default="f32", choices=["f32", "f64", "i32", "u32", "f16", "i8"], help="workload srgemm")
@@ -512,6 +543,24 @@ def main():
         print("bench.py: this library runs on ONE GPU; --gpus N with N > 1 is not supported "
               "(no collectives, no sharding in this build).", file=sys.stderr)
         sys.exit(2)
+
+    if args.workload == "functor":
+        # measured by a program of its own (the kernels are built in the user's translation unit); --steps / --warmup
+        # are launches per functor pair
+        n = args.size or 4096
+        lines = functor_lines(n, args.steps, args.warmup)
+        head = lines[0]
+        print(json.dumps({
+            "metric": f"fp32 min-plus SRGEMM GOPS at {n}^3 (2 ops/term) on a kernel built from user functors, 1 GPU",
+            "value": round(head["tops"] * 1e3, 1), "unit": "GOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": head["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+            "data": "synthetic", "config": {"workload": head["workload"], "m": n, "n": n, "k": n,
+                                            "kernel_family": "functor_srgemm_kernel (built from the user's functors by hipcc)"},
+            "roofline": {"bound": "valu", "achieved": head["tops"], "peak": 157.3, "unit": "TOPS", "frac": round(head["tops"] / 157.3, 4),
+                         "traffic": None},
+            "bit_identical_to_tuned_min_plus": head.get("bit_identical_to_tuned_min_plus"),
+            "extra": {"functor_pairs": lines}}), flush=True)
+        return
 
     import numpy as np
     import torch

@@ -152,6 +152,8 @@ int main(int argc, char **argv) {
   run_pair<fmin_op<float>, user_plus<float>>("fmin / user plus (min-plus through the math library's fminf)", n, steps, warmup, b, true);
   run_pair<ternary_min<float>, user_plus<float>>("ternary min / user plus (min-plus as a comparison and a select)", n, steps, warmup, b, true);
   run_pair<fmin_op<float>, saturating_plus<float>>("fmin / saturating plus (no library operator)", n, steps, warmup, b, false);
+  // a size whose full-size tiles would leave three quarters of the chip idle: the quarter-size tile
+  run_pair<fmin_op<float>, user_plus<float>>("fmin / user plus (min-plus through the math library's fminf)", 1024, 4 * steps, 4 * warmup, b, true);
   run_splitk<fmin_op<float>, user_plus<float>>("fmin / user plus", 256, 65536, 8, steps, warmup, b);
   run_splitk<fmin_op<float>, user_plus<float>>("fmin / user plus", 256, 65536, 64, steps, warmup, b);
   return 0;

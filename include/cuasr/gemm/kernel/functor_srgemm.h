@@ -82,12 +82,18 @@ template <typename T> __device__ __forceinline__ T opaque(T v) {
   return v;
 }
 
-template <typename T> struct Tile {
+// SMALL: a quarter of the tile (4 x 4 accumulators per thread for 4-byte elements, 4 x 2 for 8-byte ones) for
+// outputs whose full-size tiles would leave most of the chip without work
+template <typename T, bool SMALL = false> struct Tile {
   static constexpr int VW = 16 / sizeof(T);
-  static constexpr int TM = 8, TN = sizeof(T) == 8 ? 4 : 8;
-  static constexpr int BM = 16 * TM, BN = 16 * TN, BK = 16;
+  static constexpr int TM = SMALL ? 4 : 8, TN = (SMALL ? 4 : 8) / (sizeof(T) == 8 ? 2 : 1);
+#ifndef CUASR_AMD_FUNCTOR_BK
+#define CUASR_AMD_FUNCTOR_BK 16
+#endif
+  static constexpr int BM = 16 * TM, BN = 16 * TN, BK = CUASR_AMD_FUNCTOR_BK;
   static constexpr int HM = TM / VW, GN = TN / VW;
   static constexpr int LDA = BM + VW, LDB = BN + VW;
+  static_assert(BM * BK / VW >= 256 && BN * BK / VW >= 256, "a panel gives every thread a vector");
   static constexpr int A_VECS = BM * BK / VW / 256, B_VECS = BN * BK / VW / 256;
   static_assert(sizeof(T) == 4 || sizeof(T) == 8, "4- and 8-byte element types");
   typedef T vec_t __attribute__((ext_vector_type(VW)));
@@ -98,12 +104,13 @@ template <typename T> struct Tile {
 // how an operand's panel is fetched: along which direction its 16-byte vectors run
 enum PanelMode { kElements = 0, kVectorsAlongX = 1, kVectorsAlongK = 2 };
 
-// Global -> registers: VECS vectors per thread of a ROWS x BK panel whose first row / column is x0 and first k
-// is k0.  Indices outside [0, x_end) x [0, k_end) are clamped to the last valid one: what is fetched there is
-// never used (rows and columns past the edge are not stored, k past the end is not iterated).
+// Global -> registers, the guarded form: VECS vectors per thread of a ROWS x BK panel whose first row / column
+// is x0 and first k is k0, for any strides and any position.  Indices outside [0, x_end) x [0, k_end) are
+// clamped to the last valid one: what is fetched there is never used (rows and columns past the edge are not
+// stored, k past the end is not iterated).  A vector that lies wholly inside is one 16-byte load.
 template <typename T, int ROWS, int VECS>
-__device__ __forceinline__ void load_panel(typename Tile<T>::vec_t (&r)[VECS], const T *base, long long s_x, long long s_k,
-                                           int x0, int x_end, int k0, int k_end, int mode) {
+__device__ __forceinline__ void load_panel_guarded(typename Tile<T>::vec_t (&r)[VECS], const T *base, long long s_x,
+                                                   long long s_k, int x0, int x_end, int k0, int k_end, int mode) {
   using Ti = Tile<T>;
   constexpr int VW = Ti::VW;
   const int tid = threadIdx.x;
@@ -137,6 +144,34 @@ __device__ __forceinline__ void load_panel(typename Tile<T>::vec_t (&r)[VECS], c
     }
   }
 }
+
+// Global -> registers, the fast form, for a panel that lies wholly inside the matrix and the k range: a thread's
+// vectors sit at fixed 32-bit byte offsets from the panel's first element, whose address is the same for the
+// whole workgroup (a scalar register pair that moves on by one k-tile per iteration) -- one register per vector
+// instead of an address pair and its guards.
+template <typename T, int ROWS, int VECS, int MODE> struct FastPanel {
+  using Ti = Tile<T>;
+  unsigned offset[VECS];
+  __device__ __forceinline__ void init(long long s_x, long long s_k) {
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int p = 0; p < VECS; ++p) {
+      const int v = tid + 256 * p;
+      if (MODE == kVectorsAlongK) offset[p] = (unsigned)(((long long)(v % ROWS) * s_x + (v / ROWS) * Ti::VW) * (long long)sizeof(T));
+      else offset[p] = (unsigned)(((long long)(v / (ROWS / Ti::VW)) * s_k + (v % (ROWS / Ti::VW)) * Ti::VW) * (long long)sizeof(T));
+    }
+  }
+  __device__ __forceinline__ void load(typename Ti::vec_t (&r)[VECS], const T *panel) const {
+#pragma unroll
+    for (int p = 0; p < VECS; ++p)
+      r[p] = *reinterpret_cast<const typename Ti::gvec_t *>(reinterpret_cast<const char *>(panel) + offset[p]);
+  }
+  // do all of a panel's offsets fit 32 bits?
+  static __device__ __forceinline__ bool fits(long long s_x, long long s_k) {
+    const long long last = MODE == kVectorsAlongK ? (long long)(ROWS - 1) * s_x + Ti::BK : (long long)(Ti::BK - 1) * s_k + ROWS;
+    return last * (long long)sizeof(T) < (1LL << 32);
+  }
+};
 
 // registers -> LDS, k-major.  A vector along x is stored as it is; a vector along k is transposed, the lanes of
 // a store instruction going to consecutive x, i.e. consecutive banks.
@@ -179,11 +214,128 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
 
 }  // namespace functor_detail
 
-// (two waves per SIMD at least: without the attribute the compiler may take all 512 registers of a lane)
-template <typename AddOp, typename MultOp, typename T>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void functor_srgemm_kernel(FunctorSrgemmParams<T> p) {
+// (CUASR_AMD_FUNCTOR_WAVES waves per SIMD at least: without the attribute the compiler may take all 512 registers of a lane)
+#ifndef CUASR_AMD_FUNCTOR_WAVES
+#define CUASR_AMD_FUNCTOR_WAVES 2
+#endif
+
+/// The kernel's pieces, as static members so that the main loop can be instantiated per pair of panel forms.
+template <typename AddOp, typename MultOp, typename T, bool SMALL> struct FunctorSrgemmBody {
+  using Ti = functor_detail::Tile<T, SMALL>;
+  using vec_t = typename Ti::vec_t;
+  static constexpr int VW = Ti::VW, TM = Ti::TM, TN = Ti::TN, BM = Ti::BM, BN = Ti::BN, BK = Ti::BK, HM = Ti::HM, GN = Ti::GN;
+  typedef T APanel[BK][Ti::LDA];
+  typedef T BPanel[BK][Ti::LDB];
+
+  // one k of the panels in LDS: the thread's 8 rows of A and 8 (4) columns of B
+  struct Fragment {
+    vec_t a[HM], b[GN];
+  };
+  static __device__ __forceinline__ void fetch(Fragment &f, const APanel &as, const BPanel &bs, int kk, int ty, int tx) {
+#pragma unroll
+    for (int g = 0; g < HM; ++g) f.a[g] = *reinterpret_cast<const vec_t *>(&as[kk][g * 16 * VW + ty * VW]);
+#pragma unroll
+    for (int g = 0; g < GN; ++g) f.b[g] = *reinterpret_cast<const vec_t *>(&bs[kk][g * 16 * VW + tx * VW]);
+  }
+  static __device__ __forceinline__ void terms(T (&acc)[TM][TN], const Fragment &f) {
+    AddOp add_op;
+    MultOp mult_op;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = add_op(functor_detail::opaque(mult_op(f.a[i / VW][i % VW], f.b[j / VW][j % VW])), acc[i][j]);
+  }
+  // a whole k-tile, two k at a time: the reads of the next pair are issued before the current pair is computed
+  // (two fragment sets), and nothing moves across a pair's boundary -- left alone, the scheduler hoists the
+  // whole tile's reads and the kernel ends up with one wave per SIMD
+  static __device__ __forceinline__ void whole_tile(T (&acc)[TM][TN], const APanel &as, const BPanel &bs, int ty, int tx) {
+    Fragment f[2][2];
+    fetch(f[0][0], as, bs, 0, ty, tx);
+    fetch(f[0][1], as, bs, 1, ty, tx);
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      const int s = (kk >> 1) & 1;
+      if (kk + 2 < BK) {
+        fetch(f[s ^ 1][0], as, bs, kk + 2, ty, tx);
+        fetch(f[s ^ 1][1], as, bs, kk + 3, ty, tx);
+      }
+      terms(acc, f[s][0]);
+      terms(acc, f[s][1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  static __device__ __forceinline__ void part_tile(T (&acc)[TM][TN], const APanel &as, const BPanel &bs, int kcount, int ty, int tx) {
+    for (int kk = 0; kk < kcount; ++kk) {
+      Fragment f;
+      fetch(f, as, bs, kk, ty, tx);
+      terms(acc, f);
+    }
+  }
+
+  // `tiles` whole k-tiles of panels that lie wholly inside the matrix, fetched in their fast form.  Branch-free
+  // inside: every iteration fetches the next tile (the last one fetches itself again), computes, stores, and
+  // passes one barrier; the loads of tile t + 1 are in flight while tile t is computed.
+  template <int A_MODE, int B_MODE>
+  static __device__ __forceinline__ void fast_tiles(T (&acc)[TM][TN], APanel *As, BPanel *Bs, const T *a_panel, long long sa_x, long long sa_k,
+                                                    const T *b_panel, long long sb_x, long long sb_k, int tiles, int ty, int tx) {
+    using namespace functor_detail;
+    FastPanel<T, BM, Ti::A_VECS, A_MODE> fa;
+    FastPanel<T, BN, Ti::B_VECS, B_MODE> fb;
+    fa.init(sa_x, sa_k);
+    fb.init(sb_x, sb_k);
+    const long long a_step = (long long)BK * sa_k, b_step = (long long)BK * sb_k;
+    vec_t ra[Ti::A_VECS], rb[Ti::B_VECS];
+    fa.load(ra, a_panel);
+    fb.load(rb, b_panel);
+    store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[0], ra, A_MODE);
+    store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[0], rb, B_MODE);
+    __syncthreads();
+    for (int t = 0; t < tiles; ++t) {
+      const int next = min(t + 1, tiles - 1), cur = t & 1;
+      fa.load(ra, a_panel + next * a_step);
+      fb.load(rb, b_panel + next * b_step);
+      whole_tile(acc, As[cur], Bs[cur], ty, tx);
+      store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[cur ^ 1], ra, A_MODE);
+      store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[cur ^ 1], rb, B_MODE);
+      __syncthreads();
+    }
+  }
+
+  // k in [kb, ke) with every guard: any strides, panels that reach past the matrix edge, a ragged last k-tile
+  static __device__ __forceinline__ void guarded_tiles(T (&acc)[TM][TN], APanel *As, BPanel *Bs, FunctorSrgemmParams<T> const &p, int m0, int n0,
+                                                       int kb, int ke, int a_mode, int b_mode, int ty, int tx) {
+    using namespace functor_detail;
+    vec_t ra[Ti::A_VECS], rb[Ti::B_VECS];
+    load_panel_guarded<T, BM, Ti::A_VECS>(ra, p.A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_mode);
+    load_panel_guarded<T, BN, Ti::B_VECS>(rb, p.B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_mode);
+    store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[0], ra, a_mode);
+    store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[0], rb, b_mode);
+    __syncthreads();
+    int cur = 0;
+    for (int k0 = kb; k0 < ke; k0 += BK) {
+      const bool more = k0 + BK < ke;
+      if (more) {
+        load_panel_guarded<T, BM, Ti::A_VECS>(ra, p.A, p.sa_m, p.sa_k, m0, p.m, k0 + BK, ke, a_mode);
+        load_panel_guarded<T, BN, Ti::B_VECS>(rb, p.B, p.sb_n, p.sb_k, n0, p.n, k0 + BK, ke, b_mode);
+      }
+      if (k0 + BK <= ke) whole_tile(acc, As[cur], Bs[cur], ty, tx);
+      else part_tile(acc, As[cur], Bs[cur], ke - k0, ty, tx);
+      if (more) {
+        store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[cur ^ 1], ra, a_mode);
+        store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[cur ^ 1], rb, b_mode);
+      }
+      __syncthreads();
+      cur ^= 1;
+    }
+  }
+};
+
+template <typename AddOp, typename MultOp, typename T, bool SMALL = false>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(CUASR_AMD_FUNCTOR_WAVES))) void functor_srgemm_kernel(FunctorSrgemmParams<T> p) {
   using namespace functor_detail;
-  using Ti = Tile<T>;
+  using Body = FunctorSrgemmBody<AddOp, MultOp, T, SMALL>;
+  using Ti = Tile<T, SMALL>;
   using vec_t = typename Ti::vec_t;
   using gvec_t = typename Ti::gvec_t;
   constexpr int VW = Ti::VW, TM = Ti::TM, TN = Ti::TN, BM = Ti::BM, BN = Ti::BN, BK = Ti::BK, HM = Ti::HM, GN = Ti::GN;
@@ -216,71 +368,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
   const int a_mode = p.sa_m == 1 ? kVectorsAlongX : p.sa_k == 1 ? kVectorsAlongK : kElements;
   const int b_mode = p.sb_n == 1 ? kVectorsAlongX : p.sb_k == 1 ? kVectorsAlongK : kElements;
 
-  // one k of the panels in LDS: the thread's 8 rows of A and 8 (4) columns of B
-  struct Fragment {
-    vec_t a[HM], b[GN];
-  };
-  auto fetch = [&](Fragment &f, int cur, int kk) {
-#pragma unroll
-    for (int g = 0; g < HM; ++g) f.a[g] = *reinterpret_cast<const vec_t *>(&As[cur][kk][g * 16 * VW + ty * VW]);
-#pragma unroll
-    for (int g = 0; g < GN; ++g) f.b[g] = *reinterpret_cast<const vec_t *>(&Bs[cur][kk][g * 16 * VW + tx * VW]);
-  };
-  auto compute = [&](const Fragment &f) {
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = add_op(opaque(mult_op(f.a[i / VW][i % VW], f.b[j / VW][j % VW])), acc[i][j]);
-  };
-
-  if (ke > kb) {
-    vec_t ra[Ti::A_VECS], rb[Ti::B_VECS];
-    load_panel<T, BM, Ti::A_VECS>(ra, p.A, p.sa_m, p.sa_k, m0, p.m, kb, ke, a_mode);
-    load_panel<T, BN, Ti::B_VECS>(rb, p.B, p.sb_n, p.sb_k, n0, p.n, kb, ke, b_mode);
-    store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[0], ra, a_mode);
-    store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[0], rb, b_mode);
-    __syncthreads();
-    int cur = 0;
-    for (int k0 = kb; k0 < ke; k0 += BK) {
-      const bool more = k0 + BK < ke;
-      if (more) {
-        load_panel<T, BM, Ti::A_VECS>(ra, p.A, p.sa_m, p.sa_k, m0, p.m, k0 + BK, ke, a_mode);
-        load_panel<T, BN, Ti::B_VECS>(rb, p.B, p.sb_n, p.sb_k, n0, p.n, k0 + BK, ke, b_mode);
-      }
-      if (k0 + BK <= ke) {
-        // whole k-tile, two k at a time: the reads of the next pair are issued before the current pair is
-        // computed (two fragment sets), and nothing moves across a pair's boundary -- left alone, the
-        // scheduler hoists the whole tile's reads and the kernel ends up with one wave per SIMD
-        Fragment f[2][2];
-        fetch(f[0][0], cur, 0);
-        fetch(f[0][1], cur, 1);
-#pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-          const int s = (kk >> 1) & 1;
-          if (kk + 2 < BK) {
-            fetch(f[s ^ 1][0], cur, kk + 2);
-            fetch(f[s ^ 1][1], cur, kk + 3);
-          }
-          compute(f[s][0]);
-          compute(f[s][1]);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      } else {
-        for (int kk = 0; kk < ke - k0; ++kk) {
-          Fragment f;
-          fetch(f, cur, kk);
-          compute(f);
-        }
-      }
-      if (more) {
-        store_panel<T, BM, Ti::LDA, Ti::A_VECS>(As[cur ^ 1], ra, a_mode);
-        store_panel<T, BN, Ti::LDB, Ti::B_VECS>(Bs[cur ^ 1], rb, b_mode);
-      }
-      __syncthreads();
-      cur ^= 1;
-    }
+  // the whole k-tiles of a tile that lies wholly inside the output run in the branch-free loop of their pair of
+  // panel forms; everything else -- tiles on the edge, strides that are not 1 in either direction, operands so
+  // large that a panel's byte offsets outgrow 32 bits, and the ragged last k-tile -- in the guarded loop
+  int k_done = kb;
+  const int whole = (ke - kb) / BK;
+  if (whole > 0 && m0 + BM <= p.m && n0 + BN <= p.n && a_mode != kElements && b_mode != kElements) {
+    const T *a_panel = p.A + (long long)m0 * p.sa_m + (long long)kb * p.sa_k;
+    const T *b_panel = p.B + (long long)n0 * p.sb_n + (long long)kb * p.sb_k;
+    bool done = true;
+    if (a_mode == kVectorsAlongX && b_mode == kVectorsAlongX && FastPanel<T, BM, Ti::A_VECS, kVectorsAlongX>::fits(p.sa_m, p.sa_k) &&
+        FastPanel<T, BN, Ti::B_VECS, kVectorsAlongX>::fits(p.sb_n, p.sb_k))
+      Body::template fast_tiles<kVectorsAlongX, kVectorsAlongX>(acc, As, Bs, a_panel, p.sa_m, p.sa_k, b_panel, p.sb_n, p.sb_k, whole, ty, tx);
+    else if (a_mode == kVectorsAlongX && b_mode == kVectorsAlongK && FastPanel<T, BM, Ti::A_VECS, kVectorsAlongX>::fits(p.sa_m, p.sa_k) &&
+             FastPanel<T, BN, Ti::B_VECS, kVectorsAlongK>::fits(p.sb_n, p.sb_k))
+      Body::template fast_tiles<kVectorsAlongX, kVectorsAlongK>(acc, As, Bs, a_panel, p.sa_m, p.sa_k, b_panel, p.sb_n, p.sb_k, whole, ty, tx);
+    else if (a_mode == kVectorsAlongK && b_mode == kVectorsAlongX && FastPanel<T, BM, Ti::A_VECS, kVectorsAlongK>::fits(p.sa_m, p.sa_k) &&
+             FastPanel<T, BN, Ti::B_VECS, kVectorsAlongX>::fits(p.sb_n, p.sb_k))
+      Body::template fast_tiles<kVectorsAlongK, kVectorsAlongX>(acc, As, Bs, a_panel, p.sa_m, p.sa_k, b_panel, p.sb_n, p.sb_k, whole, ty, tx);
+    else if (a_mode == kVectorsAlongK && b_mode == kVectorsAlongK && FastPanel<T, BM, Ti::A_VECS, kVectorsAlongK>::fits(p.sa_m, p.sa_k) &&
+             FastPanel<T, BN, Ti::B_VECS, kVectorsAlongK>::fits(p.sb_n, p.sb_k))
+      Body::template fast_tiles<kVectorsAlongK, kVectorsAlongK>(acc, As, Bs, a_panel, p.sa_m, p.sa_k, b_panel, p.sb_n, p.sb_k, whole, ty, tx);
+    else
+      done = false;
+    if (done) k_done = kb + whole * BK;
   }
+  if (k_done < ke) Body::guarded_tiles(acc, As, Bs, p, m0, n0, k_done, ke, a_mode, b_mode, ty, tx);
 
   auto row_of = [&](int i) { return m0 + (i / VW) * 16 * VW + ty * VW + i % VW; };
   auto col_of = [&](int j) { return n0 + (j / VW) * 16 * VW + tx * VW + j % VW; };
@@ -380,17 +493,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void f
 }
 
 /// Launch on `stream`; hipSuccess or the launch's error.  With p.workspace set, p.slices slices run side by
-/// side (grid dimension y) and no epilogue is applied.
+/// side (grid dimension y) and no epilogue is applied.  The quarter-size tile is launched when the full-size
+/// one would give the chip's 256 compute units fewer than two workgroups each.
 template <typename AddOp, typename MultOp, typename T>
 inline hipError_t launch_functor_srgemm(FunctorSrgemmParams<T> const &p, hipStream_t stream) {
-  using Ti = functor_detail::Tile<T>;
+  using Full = functor_detail::Tile<T, false>;
+  using Quarter = functor_detail::Tile<T, true>;
   if (p.m <= 0 || p.n <= 0) return hipSuccess;
-  const long long tiles = (long long)((p.m + Ti::BM - 1) / Ti::BM) * ((p.n + Ti::BN - 1) / Ti::BN);
   const int slices = p.workspace ? p.slices : 1;
-  if (tiles > 0x7fffffffLL || slices < 1 || slices > 65535) return hipErrorInvalidValue;
+  if (slices < 1 || slices > 65535) return hipErrorInvalidValue;
+  long long tiles = (long long)((p.m + Full::BM - 1) / Full::BM) * ((p.n + Full::BN - 1) / Full::BN);
+  const bool quarter = tiles * slices < 512;
+  if (quarter) tiles = (long long)((p.m + Quarter::BM - 1) / Quarter::BM) * ((p.n + Quarter::BN - 1) / Quarter::BN);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   void *args[] = {const_cast<void *>(static_cast<const void *>(&p))};
-  return hipLaunchKernel(reinterpret_cast<const void *>(&functor_srgemm_kernel<AddOp, MultOp, T>),
-                         dim3((unsigned)tiles, (unsigned)slices), dim3(256), args, 0, stream);
+  const void *fn = quarter ? reinterpret_cast<const void *>(&functor_srgemm_kernel<AddOp, MultOp, T, true>)
+                           : reinterpret_cast<const void *>(&functor_srgemm_kernel<AddOp, MultOp, T, false>);
+  return hipLaunchKernel(fn, dim3((unsigned)tiles, (unsigned)slices), dim3(256), args, 0, stream);
 }
 
 }  // namespace kernel

@@ -12,8 +12,8 @@
 #include "cuasr/functional.h"
 #include "cuasr/reference/srgemm/host_srgemm_splitk.h"
 
-// value i of stream `seed`: multiples of 1/16 in [-3, 3.25], not integers, so that float sums round
-static float value(unsigned seed, unsigned i) { return float((i * 37u + seed * 11u + (i >> 3) * 5u) % 101u) / 16.0f - 3.0f; }
+// value i of stream `seed`: sevenths in [-3, 11.3): products and sums round
+static float value(unsigned seed, unsigned i) { return float((i * 37u + seed * 11u + (i >> 3) * 5u) % 101u) / 7.0f - 3.0f; }
 
 template <typename Add, typename Mul> static void run(bool serial, int m, int n, int k, int slices, float alpha, float beta) {
   using Col = cuasr::layout::ColumnMajor;

@@ -193,6 +193,16 @@ int main() {
     // both user-defined, a non-associative add in double: only the host's own order gives these bits
     run_case<leaky_plus<double>, saturating_plus<double>, double, Col, Col, Row>(s[0], s[1], s[2], 1.5, 0.5, 15, "leaky-plus / saturating-plus f64 ccr");
   }
+  // outputs of 512 full-size tiles and more (below that the launcher takes the quarter-size tile): whole, and with ragged edges
+  run_case<abs_max<float>, cuasr::multiplies<float>, float, Col, Row, Col>(2048, 4096, 24, 1.0f, 1.0f, 31, "abs-max / times f32 crc, full-size tiles");
+  run_case<abs_max<float>, cuasr::multiplies<float>, float, Row, Col, Row>(2100, 4000, 35, -2.0f, 0.5f, 32, "abs-max / times f32 rcr, full-size tiles, ragged");
+  run_case<abs_max<float>, cuasr::multiplies<float>, float, Row, Row, Row>(2048, 4096, 17, 1.0f, 1.0f, 33, "abs-max / times f32 rrr, full-size tiles");
+  run_case<abs_max<float>, cuasr::multiplies<float>, float, Col, Col, Col>(2101, 4001, 18, 1.0f, 1.0f, 34, "abs-max / times f32 ccc, full-size tiles, odd extents");
+  run_case<leaky_plus<double>, saturating_plus<double>, double, Col, Col, Row>(2048, 2048, 33, 1.5, 0.5, 35, "leaky-plus / saturating-plus f64 ccr, full-size tiles");
+  run_case<leaky_plus<double>, saturating_plus<double>, double, Row, Col, Col>(2050, 2100, 20, 1.5, 0.5, 36, "leaky-plus / saturating-plus f64 rcc, full-size tiles, ragged");
+  run_splitk_case<abs_max<float>, cuasr::multiplies<float>, float, Row, Col, Col, false>(2048, 2048, 70, -2.0f, 0.5f, 2, 37, "abs-max / times f32 rcc, full-size tiles");
+  run_splitk_case<leaky_plus<double>, saturating_plus<double>, double, Col, Col, Row, true>(1024, 2048, 50, 1.5, 0.5, 3, 38, "leaky-plus / saturating-plus f64 ccr, full-size tiles");
+
   // xor-and on 0 / 1 integers with the example's own addition functor (the multiplication is the library's)
   run_case<example_xor<int>, cuasr::binary_and<int>, int, Row, Row, Row>(512, 512, 512, 1, 1, 16, "example xor / binary_and i32 rrr");
   run_case<example_xor<int>, cuasr::binary_and<int>, int, Row, Row, Row>(130, 70, 33, 1, 0, 17, "example xor / binary_and i32 rrr, beta = 0");

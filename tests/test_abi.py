@@ -2,6 +2,7 @@
 every function include/cuasr_amd.h declares, and validates descriptors like the
 reference's can_implement / initialize do."""
 import ctypes
+import os
 import re
 
 import numpy as np
@@ -315,3 +316,11 @@ int main() {
     src.write_text(src.read_text().replace("my_op<float>", "cuasr::minimum<float>"))
     r = subprocess.run(cmd, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_reference_call_sites_compile():
+    """A program that spells its operators the way the reference's examples do (cutlass:: names, a user functor
+    with Array overloads, split-K with an owning workspace buffer) compiles against this library's headers --
+    hipcc cross-compiles it here; tests/test_gpu_cpp_api.py runs it on the GPU."""
+    import build_cpp
+    assert os.path.exists(build_cpp.build("test_reference_call_sites"))

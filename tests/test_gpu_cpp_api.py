@@ -29,3 +29,13 @@ def test_cpp_user_defined_functors(lib):
     print(r.stderr[-2000:])
     assert r.returncode == 0, r.stdout[-4000:]
     assert "0 failed" in r.stdout
+
+
+def test_cpp_reference_call_sites(lib):
+    """tests/cpp/test_reference_call_sites.hip: the three call shapes of the reference's examples, spelled with
+    cutlass:: names, a user functor with Array overloads and a cutlass::device_memory workspace."""
+    r = subprocess.run([build_cpp.ensure("test_reference_call_sites")], capture_output=True, text=True, timeout=600)
+    print(r.stdout[-4000:])
+    print(r.stderr[-2000:])
+    assert r.returncode == 0, r.stdout[-4000:]
+    assert "0 failed" in r.stdout

@@ -538,3 +538,35 @@ def test_blocked_fw_leading_dimensions(oracle):
     oracle.apsp_blocked(dist, parent, 16)
     assert np.array_equal(big[:n], dist) and np.array_equal(pbig[:n], parent)
     assert (big[n:] == -3.0).all() and (pbig[n:] == -9).all()
+
+
+# ---- the C++ split-K models that check the kernels built from user functors ----------------------------------
+
+@pytest.mark.parametrize("form", ["parallel", "serial"])
+@pytest.mark.parametrize("pair", ["plustimes", "mintimes"])
+def test_cpp_splitk_models_agree_with_the_c_oracle(oracle, form, pair):
+    """oracle/include/cuasr/reference/srgemm/host_srgemm_splitk.h restates, for any functor pair, the two split-K
+    models that oracle/host_srgemm.c holds for the library's operators (pinned above against literal Python
+    chains).  On floating-point plus-times with non-integer data, and on min-times under a negative alpha, the
+    bits depend on where a slice ends and on the order of the fold, so agreement pins both."""
+    import subprocess
+    import build_cpp
+    binary = build_cpp.build("host_splitk_models")
+    add, mult, alpha, beta, ident = ("plus", "multiplies", 1.25, 0.5, 0.0) if pair == "plustimes" else ("minimum", "multiplies", -1.5, 1.0, np.finfo(np.float32).max)
+    value = lambda seed, count: (((np.arange(count, dtype=np.uint32) * 37 + seed * 11 + (np.arange(count, dtype=np.uint32) >> 3) * 5) % 101).astype(np.float32) / np.float32(7) - np.float32(3))
+    differs = 0
+    for m, n, k, slices in [(3, 2, 20, 2), (5, 7, 100, 3), (4, 6, 77, 8), (9, 3, 301, 5), (2, 2, 7, 4), (6, 5, 64, 1)]:
+        out = subprocess.run([binary, form, pair, str(m), str(n), str(k), str(slices)], capture_output=True, text=True, check=True).stdout.split()
+        got = np.array([int(x, 16) for x in out], dtype=np.uint32).view(np.float32).reshape(n, m).T    # column-major m x n
+        A = value(1, m * k).reshape(k, m).T            # column-major m x k
+        B = value(2, k * n).reshape(k, n)              # row-major k x n
+        C = np.asfortranarray(value(3, m * n).reshape(n, m).T)
+        model = oracle.srgemm_splitk if form == "parallel" else oracle.srgemm_splitk_serial
+        want = model(add, mult, np.asfortranarray(A), np.ascontiguousarray(B), C, alpha, beta, ident, 1.0, slices, tbk=8)
+        assert_same_bits(np.ascontiguousarray(got), np.ascontiguousarray(want), f"{form} {pair} {m}x{n}x{k} S={slices}")
+        plain = oracle.srgemm(add, mult, np.asfortranarray(A), np.ascontiguousarray(B), C, alpha, beta, ident)
+        differs += int(np.ascontiguousarray(plain).tobytes() != np.ascontiguousarray(want).tobytes())
+    # (the parallel form folds raw minima and scales once: with an order-free add it cannot differ from the unsplit
+    # result, whatever the slices -- which the assertion above has just shown for the C++ model)
+    if not (pair == "mintimes" and form == "parallel"):
+        assert differs >= 2, "cases whose split-K result equals the unsplit one pin nothing about the slices"
