@@ -512,6 +512,37 @@ size_t cuasr_amd_splitk_workspace_bytes(const cuasr_amd_srgemm_desc *desc) {
   return elem_size(desc->dtype) * size_t(desc->m) * size_t(desc->n) * size_t(desc->split_k_slices);
 }
 
+// fills `count` 4-byte words with `bits` (a plain kernel rather than a memset node: this may run under stream capture)
+static __global__ __launch_bounds__(256) void fill_words_kernel(uint32_t *dst, long long count, uint32_t bits) {
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i + 4 <= count) {
+    *reinterpret_cast<uint4 *>(dst + i) = make_uint4(bits, bits, bits, bits);
+  } else {
+    for (long long j = i; j < count; ++j) dst[j] = bits;
+  }
+}
+
+// Split-K of a small output on the staged tiles: how many workgroups share one slice's k range (Problem::k_sub).
+// The quarter-size tile runs with four groups of waves per workgroup, one workgroup per compute unit; fewer than
+// half as many (tile, slice) pairs as compute units leave the rest of the chip idle (256 x 256 x 65536 in 8
+// slices: 128 workgroups, 31.9 TOPS against 51.5 in 16 slices).  Only where the parts can meet through native
+// atomics (4-byte minimum / maximum, or / xor on words) and every part keeps a long run of k-tiles.
+static int sub_slices(const cuasr_amd_srgemm_desc *d, const Problem &p, int units) {
+  if (units <= 0 || p.batch != 1 || p.slices < 1) return 1;
+  const bool fp = d->dtype == CUASR_AMD_F32;
+  if (!fp && d->dtype != CUASR_AMD_I32 && d->dtype != CUASR_AMD_U32) return 1;
+  const bool minmax = d->add_op == kMinimum || d->add_op == kMaximum;
+  if (!(minmax || (!fp && (d->add_op == kBitOr || d->add_op == kBitXor)))) return 1;
+  if (fp && d->mult_op == kMultiplies) return 1;   // a zero result's sign depends on the whole k range
+  if (reinterpret_cast<uintptr_t>(p.workspace) % 16) return 1;
+  const long long groups = (long long)((p.m + 63) / 64) * ((p.n + 63) / 64) * p.slices;
+  if (groups * 2 > units) return 1;
+  long long sub = units / groups;
+  const long long max_sub = p.k_per_slice / 1024;   // at least 32 k-tiles of 32 per part
+  if (sub > max_sub) sub = max_sub;
+  return sub >= 2 ? (int)sub : 1;
+}
+
 // Both split-K forms: partial products of the K-slices into the workspace, then one
 // reduction kernel (`serial` picks the ordered replay of the serial form's epilogues).
 // `stages`: 1 = the slice kernel, 2 = the reduction kernel, 3 = both.
@@ -545,6 +576,15 @@ static int run_splitk(const cuasr_amd_srgemm_desc *desc, void *workspace, void *
   const launch_fn red = serial ? find_reduce_serial(desc->dtype) : find_reduce(desc->dtype);
   if (!fn || !red) return CUASR_AMD_ERROR_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if ((stages & 1) && family == kValu && desc->kernel != CUASR_AMD_KERNEL_NAIVE) {
+    p.k_sub = sub_slices(desc, p, compute_units());
+    if (p.k_sub > 1) {
+      // the parts of a slice fold into its partial tile: start every partial tile at the additive identity
+      const long long words = (long long)p.m * p.n * p.slices;
+      fill_words_kernel<<<dim3((unsigned)((words + 1023) / 1024)), dim3(256), 0, s>>>(static_cast<uint32_t *>(workspace), words, p.add_identity.u32);
+      if (hipGetLastError() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+    }
+  }
   if ((stages & 1) && fn(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
   if ((stages & 2) && red(p, s) != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
   return CUASR_AMD_SUCCESS;

@@ -158,6 +158,41 @@ template <> __host__ __device__ __forceinline__ half_t scalar_as<half_t>(const c
   return __builtin_bit_cast(half_t, s.f16);
 }
 
+// add(v, *addr) into *addr, atomically at device scope and without waiting for an answer, for the adds that have a
+// native atomic on 4-byte elements: minimum and maximum (integers directly; floats through the integer atomics --
+// a float without sign bit orders like its bits as a signed integer, one with sign bit the other way round like its
+// bits as an unsigned integer, and every float of the second kind is below every float of the first both as a number
+// and as a signed integer / above as an unsigned one), or and xor on words.  NaN-free data, as everywhere the
+// hardware minimum is used; the results do not depend on the order in which the folds arrive.
+template <typename T, int ADD> struct has_native_fold
+    : std::integral_constant<bool, sizeof(T) == 4 && (ADD == kMinimum || ADD == kMaximum || (!is_fp<T>::value && (ADD == kBitOr || ADD == kBitXor)))> {};
+
+template <int ADD, typename T> __device__ __forceinline__ void native_fold(T *addr, T v) {
+  static_assert(has_native_fold<T, ADD>::value, "no native atomic for this add on this element type");
+  const int bits = __builtin_bit_cast(int, v);
+  int *si = reinterpret_cast<int *>(addr);
+  unsigned *ui = reinterpret_cast<unsigned *>(addr);
+  if constexpr (ADD == kBitXor) {
+    __hip_atomic_fetch_xor(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if constexpr (ADD == kBitOr) {
+    __hip_atomic_fetch_or(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else if constexpr (is_fp<T>::value) {
+    if constexpr (ADD == kMinimum) {
+      if (bits >= 0) __hip_atomic_fetch_min(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_fetch_max(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+      if (bits >= 0) __hip_atomic_fetch_max(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      else __hip_atomic_fetch_min(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  } else if constexpr (std::is_signed<T>::value) {
+    if constexpr (ADD == kMinimum) __hip_atomic_fetch_min(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else __hip_atomic_fetch_max(si, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    if constexpr (ADD == kMinimum) __hip_atomic_fetch_min(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else __hip_atomic_fetch_max(ui, (unsigned)bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 // The problem in kernel form.  The host has already turned a column-major C
 // into the transposed problem (C^T = B^T (x) A^T, as the reference does in
 // include/cuasr/gemm/device/srgemm.h:432-453, :513-523), so C and D are always
@@ -175,6 +210,11 @@ struct Problem {
   // partial accumulators go to workspace[z][m][n] (row-major, ld = n)
   int slices, k_per_slice;
   void *workspace;
+  // split-K of a small output on the staged tiles: every slice's k range is shared out over k_sub workgroups
+  // (blockIdx.y = slice * k_sub + part), which fold their accumulators into the slice's partial tile with one
+  // atomic per element; the host fills the workspace with the additive identity first.  0 or 1: one workgroup
+  // per tile and slice, plain stores.
+  int k_sub;
   // strided batch (tile kernels only): product blockIdx.z works on A, B, C, D moved on by z times
   // these element strides; batch = 1 for a single product
   int batch;

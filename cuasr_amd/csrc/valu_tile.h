@@ -356,10 +356,23 @@ struct ValuTile {
     kb = 0;
     ke = p.k;
     if (p.workspace) {
-      kb = blockIdx.y * p.k_per_slice;
-      ke = min(p.k, kb + p.k_per_slice);
+      if (p.k_sub > 1) {
+        // this workgroup's part of its slice: whole k-tiles, spread evenly over the slice's k_sub workgroups
+        const int slice = blockIdx.y / p.k_sub, part = blockIdx.y % p.k_sub;
+        const int sb = min(p.k, slice * p.k_per_slice), se = min(p.k, sb + p.k_per_slice);
+        const int per = ((se - sb + BK - 1) / BK + p.k_sub - 1) / p.k_sub * BK;
+        kb = min(se, sb + part * per);
+        ke = min(se, kb + per);
+      } else {
+        kb = blockIdx.y * p.k_per_slice;
+        ke = min(p.k, kb + p.k_per_slice);
+      }
     }
   }
+  // can the k range of a slice be shared out over several workgroups (Problem::k_sub)?  The parts meet in the
+  // workspace through one native atomic per element, so: an add that has one, and accumulators that are final
+  // as they stand (no mask to turn back, no zero whose sign depends on the rest of the range).
+  static constexpr bool SUB_SLICES = has_native_fold<T, ADD>::value && !MASKED && !ZERO_SIGN;
 
   static __device__ __forceinline__ void run(const Problem &p, Smem &sm) {
     int m0, n0, kb, ke;
@@ -467,7 +480,7 @@ struct ValuTile {
     const bool partial = p.workspace != nullptr;
     EpilogueScalars<T> e;
     if (partial) {
-      out = reinterpret_cast<T *>(p.workspace) + (long long)blockIdx.y * p.m * p.n;
+      out = reinterpret_cast<T *>(p.workspace) + (long long)(p.k_sub > 1 ? blockIdx.y / p.k_sub : blockIdx.y) * p.m * p.n;
       ld_out = p.n;
       e.alpha = e.beta = e.ident = ident;
       e.source_needed = false;
@@ -475,6 +488,23 @@ struct ValuTile {
       out = reinterpret_cast<T *>(p.D);
       ld_out = p.ldd;
       e = resolve_scalars<T>(p, MUL);
+    }
+    if constexpr (SUB_SLICES) {
+      if (partial && p.k_sub > 1) {
+        // one of several workgroups on this slice's tile: fold into the partial tile, which the host has filled
+        // with the additive identity
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int row = m0 + ty * VW + (i / VW) * 16 * VW + (i % VW);
+          if (row >= p.m) continue;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const int col = n0 + tx * VW + (j / VW) * 16 * VW + (j % VW);
+            if (col < p.n) native_fold<ADD>(out + (long long)row * ld_out + col, acc[i][j]);
+          }
+        }
+        return;
+      }
     }
     const T *C = reinterpret_cast<const T *>(p.C);
 #pragma unroll
@@ -614,6 +644,9 @@ template <typename T> static bool vector_possible(const Problem &p) {
   return p.k >= 1;
 }
 
+// grid dimension y: one workgroup per slice, or k_sub per slice
+static inline unsigned slice_groups(const Problem &p) { return p.workspace ? (unsigned)(p.slices * (p.k_sub > 1 ? p.k_sub : 1)) : 1u; }
+
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, int G>
 static void launch_ksplit(const Problem &p, dim3 grid, hipStream_t s) {
   if (vector_exact<T>(p))
@@ -629,12 +662,12 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
   const long long tiles = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
-  dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch);
+  dim3 grid((unsigned)tiles, slice_groups(p), p.batch);
   if constexpr (KSPLIT && order_free<T, ADD>::value) {
     // 256 compute units: up to 256 workgroups get four groups (1024 threads, four waves per SIMD),
     // up to 512 two; each group wants a few k-tiles of its own to be worth the fold at the end
     const long long groups = tiles * grid.y * grid.z;
-    const long long k_range = p.workspace ? p.k_per_slice : p.k;
+    const long long k_range = p.workspace ? p.k_per_slice / (p.k_sub > 1 ? p.k_sub : 1) : p.k;
     if (vector_possible<T>(p) && k_range >= 8LL * BK) {
       if (groups <= 256) {
         launch_ksplit<T, ADD, MUL, TM, TN, BK, 4>(p, grid, s);
@@ -670,15 +703,15 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, int TM_SMALL, int TN_SMALL, int BK_SMALL = BK>
 static hipError_t launch_valu_sized(const Problem &p, hipStream_t s) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
-  const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * (p.workspace ? p.slices : 1) * p.batch;
+  const long long groups = (long long)((p.m + BM - 1) / BM) * ((p.n + BN - 1) / BN) * slice_groups(p) * p.batch;
   const long long rounds = (groups + 1023) / 1024;
   if constexpr (order_free<T, ADD>::value) {
     // 192 .. 256 full-size workgroups (2048^2: exactly 256) are one per compute unit for most of the
     // chip: two groups per workgroup give every SIMD its two waves, and the full-size tile then runs
     // at the rate it has on large problems, which the quarter-size tile does not reach
-    const long long k_range = p.workspace ? p.k_per_slice : p.k;
+    const long long k_range = p.workspace ? p.k_per_slice / (p.k_sub > 1 ? p.k_sub : 1) : p.k;
     if (groups >= 192 && groups <= 256 && k_range >= 8LL * BK && vector_possible<T>(p) && p.m > 0 && p.n > 0) {
-      launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / (p.workspace ? p.slices : 1) / p.batch), p.workspace ? p.slices : 1, p.batch), s);
+      launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, dim3((unsigned)(groups / slice_groups(p) / p.batch), slice_groups(p), p.batch), s);
       return take_launch_status();
     }
   }

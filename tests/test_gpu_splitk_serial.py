@@ -162,3 +162,48 @@ def test_serial_splitk_plus_times_tolerance(oracle, lib):
     got = to_host(dD, "f32").astype(np.float64)
     bound = 1e-5 * (1.5 * np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64) + 0.5 * np.abs(C))
     assert (np.abs(got - want) <= bound).all()
+
+
+# ---- small outputs: several workgroups per slice --------------------------------------------------------------
+
+SHARED = {
+    "minplus_f32": ("minimum", "plus", "f32", 2.0, 0.0, INF, 0.0),
+    "maxplus_f32_beta_zero": ("maximum", "plus", "f32", 0.0, -INF, -INF, 0.0),
+    "maxmin_f32": ("maximum", "minimum", "f32", INF, INF, -INF, INF),
+    "minplus_i32": ("minimum", "plus", "i32", 1, 0, 2**31 - 1, 0),
+    "maxplus_u32": ("maximum", "plus", "u32", 0, 0, 0, 0),
+    "xorand_u32": ("bit_xor", "bit_and", "u32", FULL, FULL, 0, FULL),
+}
+
+
+@pytest.mark.parametrize("form", ["parallel", "serial"])
+@pytest.mark.parametrize("case", sorted(SHARED))
+def test_splitk_of_a_small_output_shares_each_slice_between_workgroups(oracle, lib, case, form):
+    """An output of few tiles in few slices (the shape of the 256 x 256 x 65536 split-K in 8 slices): the staged
+    tiles give every slice's k range to several workgroups, which fold their parts into the slice's partial
+    tile with native atomics after the workspace has been set to the additive identity.  Stale workspace
+    contents, ragged extents, k that does not divide, and the serial form's chain (alpha multiplies every
+    slice's partial) must all come out as the oracle's models say."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    add, mult, dtype, alpha, beta, ident, one = SHARED[case]
+    for (m, n, k, slices, layouts) in [(256, 256, 16384, 8, "rcr"), (250, 130, 9001, 3, "ccc"), (64, 64, 40000, 2, "crc"), (100, 300, 6144, 4, "rrc")]:
+        la, lb, lc = [{"c": "col", "r": "row"}[x] for x in layouts]
+        npd = NPD[dtype]
+        if dtype == "u32" and add == "bit_xor":
+            A, B, C = inputs.words32(31, m, k, order_of(la)), inputs.words32(32, k, n, order_of(lb)), inputs.words32(33, m, n, order_of(lc))
+        else:
+            lo, hi = (0, 1000) if dtype == "u32" else (-1000, 1000)
+            A = inputs.integers(31, m, k, lo, hi, npd, order_of(la))
+            B = inputs.integers(32, k, n, lo, hi, npd, order_of(lb))
+            C = inputs.integers(33, m, n, 2 * lo, 2 * hi, npd, order_of(lc))
+        model = oracle.srgemm_splitk if form == "parallel" else oracle.srgemm_splitk_serial
+        want = model(add, mult, A, B, C, alpha, beta, ident, one, slices, tbk=16 if form == "parallel" else 8)
+        dA, dB, dC = to_device(A), to_device(B), to_device(C)
+        dD = to_device(np.zeros_like(C))
+        ws = torch.full((m * n * slices,), 0x7FC00000, dtype=torch.int32, device="cuda")   # stale contents must not survive
+        run_it = cuasr_amd.srgemm_splitk if form == "parallel" else cuasr_amd.srgemm_splitk_serial
+        run_it(add, mult, dA, dB, dC, dD, slices, ws, alpha, beta, ident, one, dtype=dtype)
+        torch.cuda.synchronize()
+        assert_same_bits(to_host(dD, dtype), want, f"{form} split-K {case} {m}x{n}x{k} {layouts} S={slices}")
