@@ -46,7 +46,7 @@ def generate():
     spec = importlib.util.spec_from_file_location("gen_direct_asm", os.path.join(CSRC, "gen_direct_asm.py"))
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    return mod.generate(os.path.join(CSRC, "gen")) + mod.generate_mfma(os.path.join(CSRC, "gen")) + mod.generate_mfma64(os.path.join(CSRC, "gen")) + mod.generate_fwgemm_merge(os.path.join(CSRC, "gen"))
+    return mod.generate(os.path.join(CSRC, "gen")) + mod.generate_mfma(os.path.join(CSRC, "gen")) + mod.generate_mfma64(os.path.join(CSRC, "gen")) + mod.generate_narrow(os.path.join(CSRC, "gen")) + mod.generate_fwgemm_merge(os.path.join(CSRC, "gen"))
 
 
 def build(jobs=None, verbose=True):

@@ -596,6 +596,148 @@ def generate_mfma64(out_dir):
 
 
 # ---------------------------------------------------------------------------------------------
+# plus-times on the matrix cores for the narrow element types (mfma_direct_narrow.hip): int8 operands with
+# v_mfma_i32_32x32x32_i8, binary16 operands with v_mfma_f32_32x32x16_f16, both operands k-contiguous.
+#
+# Either instruction multiplies 32 rows by 32 columns over 32 BYTES of k per row, every lane supplying 16
+# consecutive bytes of one row (column): lanes 0..31 the first 16 bytes of the step, lanes 32..63 the second.  So
+# in bytes the two types are the same kernel:
+#   workgroup 256 threads = 4 waves (2 x 2), one wave per SIMD; output tile 256 x 256, wave tile 128 x 128 =
+#   4 x 4 blocks of 32 x 32
+#   a0 .. a255   accumulators, block (bm, bn) in a[16 (4 bm + bn) : +15]
+#   v0 .. v31    fragments, buffer 0: A blocks 0..3 (four registers = 16 bytes of k each), then B blocks 0..3
+#   v32 .. v63   fragments, buffer 1
+# A stage of the LDS ring holds 64 bytes of k of both panels = two steps of the instruction, in the image the
+# direct-to-LDS loads produce -- lane i of a load writes 16-byte slot i of its KiB -- with the lanes dealt to memory
+# so that four neighbouring lanes fetch the four 16-byte chunks of ONE row's 64 bytes (16 cache lines per load
+# instruction; with one row per lane it was 64, and the tag lookups, not the bytes, bounded the kernel), and so
+# that fragment reads stay free of bank conflicts: row r's chunk c sits in slot 4 r + (c ^ ((r >> 2) & 3)), which
+# spreads the 16 rows a quarter-wave reads at one chunk over all 16 slot positions of the banks.  A lane reads
+# chunk (2 step + half) of its row, so its address for step 1 is that for step 0 with the chunk's bit 1
+# flipped: two address registers per panel.  Four stages: a body works on stage t, fetches stage t + 3 behind the
+# matrix instructions of its second step (into the ring slot that stage t - 1 has left) and passes ONE barrier,
+# in its middle: before it every read of this stage has been issued and has returned, and this wave's loads of
+# stage t + 1 have landed; after it the reads of stage t + 1's first step are issued, under the second step's
+# matrix instructions.
+class NarrowMfmaBody(MfmaBody):
+    def __init__(self, instruction):
+        self.instruction = instruction
+        self.lines, self.inflight, self.groups = [], [], 0
+        self.stats = {"groups": 0, "lds": 0, "waits": 0, "other": 0}
+        self.content = {}
+
+    @staticmethod
+    def frag(operand, u, blk):
+        return u * 32 + (0 if operand == "A" else 16) + blk * 4
+
+    def reads(self, step):
+        """LDS reads of the fragments of absolute step `step` (0, 1 of this stage; 2 = the next stage's first,
+        through the already advanced addresses) into buffer step % 2."""
+        u, out = step % 2, []
+        for operand, addr in (("A", "a_addr"), ("B", "b_addr")):
+            for blk in range(4):
+                r = self.frag(operand, u, blk)
+                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}{step % 2}] offset:{blk * 32 * 64}",
+                            {r + i: (operand, blk, step) for i in range(4)}))
+        return out
+
+    def mfma(self, step, bm, bn):
+        u = step % 2
+        ra, rb = self.frag("A", u, bm), self.frag("B", u, bn)
+        for i in range(4):
+            assert self.content.get(ra + i) == ("A", bm, step) and self.content.get(rb + i) == ("B", bn, step)
+        self.require_exact({ra + i for i in range(4)} | {rb + i for i in range(4)})
+        acc = 16 * (4 * bm + bn)
+        self.lines.append(f'"{self.instruction} a[{acc}:{acc + 15}], v[{ra}:{ra + 3}], v[{rb}:{rb + 3}], a[{acc}:{acc + 15}]\\n"')
+        self.groups += 1
+        self.stats["groups"] += 1
+
+    def step(self, step, aux, first, last):
+        """The 16 matrix instructions of one step, the callables of `aux` spread behind instructions first .. last."""
+        order = [(bm, bn) for bn in range(4) for bm in range(4)]
+        behind = {}
+        for i, item in enumerate(aux):
+            slot = first + (i * (last - first + 1)) // len(aux)
+            behind.setdefault(slot, []).append(item)
+        for i, (bm, bn) in enumerate(order):
+            self.mfma(step, bm, bn)
+            for item in behind.get(i, []):
+                item()
+
+    def prime(self):
+        for item in self.reads(0):
+            self.read(item)
+        self.drain()
+        return self.lines
+
+    def dma_chunk(self, index):
+        """One 1 KiB piece of the stage three ahead (skipped when there is no such stage): 16 rows x 64 bytes of
+        this wave's 64 rows of the A panel (pieces 0..3) or of the B panel (4..7); consecutive pieces are
+        consecutive KiB of the ring slot (M0) and 16 rows apart in memory (a lane offset of their own each)."""
+        e = self.emit
+        name, h = ("a", index) if index < 4 else ("b", index - 4)
+        e("s_cmp_lt_i32 %[fetch], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_%=")
+        e(f"s_add_u32 m0, %[m0_{name}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[base_{name}]")
+        e(f".Lcuasr_nofetch{index}_%=:")
+
+    def tile(self):
+        e = self.emit
+        for operand in ("A", "B"):
+            for blk in range(4):
+                for i in range(4):
+                    self.content[self.frag(operand, 0, blk) + i] = (operand, blk, 0)
+        entry = dict(self.content)
+        # step 0 (buffer 0); the reads of step 1 (same stage) behind its first matrix instructions, so that the
+        # last eight (256 cycles) cover the latency of the last read
+        self.step(0, [(lambda it=it: self.read(it)) for it in self.reads(1)], 0, 7)
+        # every read of this stage has returned; this wave's part of stage t + 1 has landed (the eight loads of
+        # stage t + 2 are younger and stay in flight, if there is such a stage); after the barrier both hold for
+        # the workgroup: stage t + 1 may be read, and the slot of stage t - 1 refilled
+        e("s_cmp_lt_i32 %[fetch], 0")
+        e("s_cbranch_scc1 .Lcuasr_all_%=")
+        e("s_waitcnt vmcnt(8) lgkmcnt(0)")
+        e("s_branch .Lcuasr_join_%=")
+        e(".Lcuasr_all_%=:")
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        e(".Lcuasr_join_%=:")
+        self.inflight = []
+        e("s_barrier")
+        for name in ("a_addr0", "a_addr1", "b_addr0", "b_addr1"):
+            e(f"v_add_u32 %[{name}], %[step], %[{name}]")
+        e("s_mov_b32 %[m0_save], m0")
+        # step 1 (buffer 1): the next stage's first fragments behind the first eight matrix instructions, the
+        # eight loads of the stage three ahead behind the last eight
+        rd = [(lambda it=it: self.read(it)) for it in self.reads(2)]
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(8)]
+        self.step(1, rd + aux, 0, 15)
+        e("s_mov_b32 m0, %[m0_save]")
+        self.drain()
+        shifted = {r: (o, b, t - 2) for r, (o, b, t) in self.content.items() if t >= 2}
+        assert shifted == entry, "tile body does not reproduce its entry state"
+        return self.lines
+
+
+NARROW_VARIANTS = {"n_i8": "v_mfma_i32_32x32x32_i8", "n_f16": "v_mfma_f32_32x32x16_f16"}
+
+
+def generate_narrow(out_dir):
+    os.makedirs(out_dir, exist_ok=True)
+    report = []
+    for name, instruction in NARROW_VARIANTS.items():
+        b = NarrowMfmaBody(instruction)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_prime.inc"), "w") as f:
+            f.write(b.text(b.prime()))
+        b = NarrowMfmaBody(instruction)
+        with open(os.path.join(out_dir, f"mfma_asm_{name}_tile.inc"), "w") as f:
+            f.write(b.text(b.tile()))
+        report.append((name, dict(b.stats)))
+    return report
+
+
+# ---------------------------------------------------------------------------------------------
 # The bookkeeping of the predecessor-tracking product on the direct tile (fwgemm.hip, fwgemm_direct_kernel):
 # after a chunk of k the loop's 64 accumulators (v0 .. v63) are compared with their values before it
 # (v128 .. v191); where one is lower, the chunk's index goes into that element's 16 bits of v192 .. v223 and

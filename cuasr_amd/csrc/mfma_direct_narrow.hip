@@ -1,0 +1,264 @@
+// plus-times on the matrix cores for the narrow element types, hand-scheduled:
+//     int8 operands, int32 accumulation and results          v_mfma_i32_32x32x32_i8
+//     binary16 operands and results, float accumulation      v_mfma_f32_32x32x16_f16
+// for products whose operands are both k-contiguous (A row-major, B column-major in the canonical orientation),
+// whose extents are whole tiles of 256 x 256 and whose k range is a multiple of 64 bytes; everything else stays on
+// the compiled kernels (mfma_i8.hip, mfma_f16.hip), which take every extent, layout and alignment.  The element
+// types are those of the reference's dp4a threadblock cores (include/cuasr/gemm/threadblock/
+// default_srmma_core_simt.h:733-1381: int8 operands, never instantiated there) and of its ElementAccumulator =
+// float for half operands; the kernel's place is the reference's include/cuasr/gemm/kernel/srgemm.h:156-321.
+//
+// Either instruction multiplies 32 rows by 32 columns over 32 bytes of k per row, every lane supplying 16
+// consecutive bytes of one row (column), so in bytes the two element types are one kernel.  The compiled kernels
+// run the matrix cores 24 - 30 % busy: a 64 x 64 wave tile reads 4 KiB of fragments per 128 cycles of matrix work,
+// which is all a compute unit's LDS delivers, panels pass through registers, and every k-tile ends in a barrier
+// that nothing hides.  Here:
+//   - workgroup 256 threads = 2 x 2 waves, ONE wave per SIMD; output tile 256 x 256, wave tile 128 x 128 = 4 x 4
+//     blocks of 32 x 32: 8 fragment reads per 16 matrix instructions (half the LDS traffic per instruction), and
+//     64 KiB of panels per 2^24 operations (half the traffic from L2).  The 256 accumulator registers are the
+//     wave's AGPRs; fragments, addresses and the rest live in VGPRs;
+//   - panels go global -> LDS without passing registers (global_load_lds_dwordx4).  A stage of the LDS ring is 64
+//     bytes of k of both panels; four neighbouring lanes of a load fetch the four 16-byte chunks of one row's 64
+//     bytes, so an instruction touches 16 cache lines (one row per lane, 64 lines per instruction, ran into the
+//     rate at which a compute unit's L1 looks lines up: 1.2 POP/s, no better than the compiled kernel), and the
+//     chunks of a row are stored in an order that depends on the row -- slot 4 r + (c ^ ((r >> 2) & 3)) -- so
+//     that a fragment read (32 consecutive rows, one chunk) is free of bank conflicts.  Four stages of 32 KiB;
+//   - the main loop is one generated asm statement per stage (gen_direct_asm.py, NarrowMfmaBody): 32 matrix
+//     instructions, the 16 fragment reads of the next two steps and the 8 loads of the stage three ahead spread
+//     between them, one counted wait and one barrier in the middle of the stage.
+// Integer sums wrap modulo 2^32 in any order, so the int8 result is bit-identical to the k-ascending reference
+// loop; the binary16 result is the float sum of exact products, rounded to binary16 once (see mfma_f16.hip).
+#include "mfma_common.h"
+
+namespace cuasr_amd {
+namespace mfma_narrow {
+
+using mfma_panel::tile_coords;
+
+constexpr int BM = 256, BN = 256, STAGE_K_BYTES = 64, STAGES = 4;
+constexpr unsigned PANEL = STAGE_K_BYTES * 256;   // bytes of one panel in one stage: 16 KiB
+
+struct Smem {
+  unsigned char a[STAGES][PANEL];
+  unsigned char b[STAGES][PANEL];
+};
+
+typedef int asm_v32 __attribute__((ext_vector_type(32)));
+struct Regs {
+  asm_v32 acc[8];    // a0 .. a255: block (bm, bn) in a[16 (4 bm + bn) : +15]
+  asm_v32 frag[2];   // v0 .. v63: the two fragment buffers
+};
+
+__device__ __forceinline__ void dma16(const char *src, unsigned char *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                   (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
+
+#define CUASR_NARROW_ACC                                                                                                  \
+  "+{a[0:31]}"(r.acc[0]), "+{a[32:63]}"(r.acc[1]), "+{a[64:95]}"(r.acc[2]), "+{a[96:127]}"(r.acc[3]),                      \
+      "+{a[128:159]}"(r.acc[4]), "+{a[160:191]}"(r.acc[5]), "+{a[192:223]}"(r.acc[6]), "+{a[224:255]}"(r.acc[7])
+#define CUASR_NARROW_PRIME                                                                                                \
+  : "+{v[0:31]}"(r.frag[0]), "+{v[32:63]}"(r.frag[1]) : [a_addr0] "v"(a_addr[0]), [b_addr0] "v"(b_addr[0]) : "memory"
+#define CUASR_NARROW_TILE                                                                                                 \
+  : CUASR_NARROW_ACC, "+{v[0:31]}"(r.frag[0]), "+{v[32:63]}"(r.frag[1]), [a_addr0] "+v"(a_addr[0]),                       \
+    [a_addr1] "+v"(a_addr[1]), [b_addr0] "+v"(b_addr[0]), [b_addr1] "+v"(b_addr[1]), [m0_save] "=&s"(m0_save)             \
+  : [step] "s"(step), [fetch] "s"(fetch), [m0_a] "s"(m0_a), [m0_b] "s"(m0_b),                                             \
+    [off_a0] "v"(off_a[0]), [off_a1] "v"(off_a[1]), [off_a2] "v"(off_a[2]), [off_a3] "v"(off_a[3]),                       \
+    [off_b0] "v"(off_b[0]), [off_b1] "v"(off_b[1]), [off_b2] "v"(off_b[2]), [off_b3] "v"(off_b[3]),                       \
+    [base_a] "s"(base_a), [base_b] "s"(base_b)                                                                            \
+  : "scc", "memory"
+#define CUASR_NARROW_TILE_ARGS                                                                                            \
+  Regs &r, unsigned (&a_addr)[2], unsigned (&b_addr)[2], unsigned step, int fetch, unsigned m0_a, unsigned m0_b,          \
+      const unsigned (&off_a)[4], const unsigned (&off_b)[4], const char *base_a, const char *base_b
+
+// prime: the fragments of the first step into buffer 0; the stage must have landed in ring slot 0.
+// tile: one stage -- 32 matrix instructions per wave, the loads of the stage three ahead (if fetch > 0), the
+// workgroup barrier that hands a ring slot back, and the fragments of the next stage's first step.
+template <bool I8> struct Loop;
+template <> struct Loop<true> {
+  static __device__ __forceinline__ void prime(Regs &r, const unsigned (&a_addr)[2], const unsigned (&b_addr)[2]) {
+    asm volatile(
+#include "gen/mfma_asm_n_i8_prime.inc"
+        CUASR_NARROW_PRIME);
+  }
+  static __device__ __forceinline__ void tile(CUASR_NARROW_TILE_ARGS) {
+    unsigned m0_save;
+    asm volatile(
+#include "gen/mfma_asm_n_i8_tile.inc"
+        CUASR_NARROW_TILE);
+  }
+};
+template <> struct Loop<false> {
+  static __device__ __forceinline__ void prime(Regs &r, const unsigned (&a_addr)[2], const unsigned (&b_addr)[2]) {
+    asm volatile(
+#include "gen/mfma_asm_n_f16_prime.inc"
+        CUASR_NARROW_PRIME);
+  }
+  static __device__ __forceinline__ void tile(CUASR_NARROW_TILE_ARGS) {
+    unsigned m0_save;
+    asm volatile(
+#include "gen/mfma_asm_n_f16_tile.inc"
+        CUASR_NARROW_TILE);
+  }
+};
+
+template <bool I8>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mfma_narrow_kernel(Problem p) {
+  using Operand = typename std::conditional<I8, int8_t, half_t>::type;
+  using Result = typename std::conditional<I8, int32_t, half_t>::type;
+  constexpr long long E = sizeof(Operand);
+  __shared__ __attribute__((aligned(1024))) Smem sm;
+  select_batch<Result, Operand>(p);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;   // the host sends whole tiles only
+  int bm, bn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
+  const int m0 = bm * BM, n0 = bn * BN;
+
+  int kb = 0, ke = p.k;
+  if (p.workspace) {
+    kb = blockIdx.y * p.k_per_slice;
+    ke = min(p.k, kb + p.k_per_slice);
+  }
+  const int nstages = (int)((long long)max(ke - kb, 0) * E / STAGE_K_BYTES);   // (the host sends whole stages only)
+
+  Regs r;
+#pragma unroll
+  for (int v = 0; v < 8; ++v) r.acc[v] = asm_v32(0);
+#pragma unroll
+  for (int v = 0; v < 2; ++v) r.frag[v] = asm_v32(0);
+
+  if (nstages > 0) {
+    const char *base_a = reinterpret_cast<const char *>(p.A) + ((long long)m0 * p.sa_m + kb) * E;
+    const char *base_b = reinterpret_cast<const char *>(p.B) + ((long long)n0 * p.sb_n + kb) * E;
+    // this wave's 64 rows of each panel in four loads of 16 rows x 64 bytes: lane l of load h fetches row
+    // 64 wave + 16 h + l / 4, chunk (l % 4) ^ ((l / 16) % 4) -- the chunk that belongs in the LDS slot the lane writes
+    unsigned off_a[4], off_b[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const long long row = wave * 64 + 16 * h + lane / 4;
+      const unsigned chunk = (unsigned)((lane & 3) ^ ((lane >> 4) & 3));
+      off_a[h] = (unsigned)(row * p.sa_m * E) + 16u * chunk;
+      off_b[h] = (unsigned)(row * p.sb_n * E) + 16u * chunk;
+    }
+    auto fetch = [&](int stage) {
+#pragma unroll
+      for (int h = 0; h < 4; ++h) dma16(base_a + off_a[h], &sm.a[stage][(wave * 4 + h) * 1024]);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) dma16(base_b + off_b[h], &sm.b[stage][(wave * 4 + h) * 1024]);
+    };
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      if (s < nstages) fetch(s);
+      base_a += STAGE_K_BYTES;
+      base_b += STAGE_K_BYTES;
+    }
+    __syncthreads();  // waits for the loads first
+    // from here base_a / base_b point at stage 3
+
+    // lane's LDS byte addresses of its fragments for (ring slot 0, block 0), step 0 and step 1: row r's chunk c is
+    // in 16-byte slot 4 r + (c ^ ((r >> 2) & 3)); lanes 0..31 take a step's first chunk, lanes 32..63 the second
+    const unsigned a_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)&sm.a[0][0];
+    const unsigned b_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)&sm.b[0][0];
+    const unsigned turn = (unsigned)((l32 >> 2) & 3);
+    unsigned a_addr[2], b_addr[2];
+#pragma unroll
+    for (int st = 0; st < 2; ++st) {
+      const unsigned chunk = (unsigned)(2 * st + half) ^ turn;
+      a_addr[st] = a_lds + ((wm * 128 + l32) * 4 + chunk) * 16;
+      b_addr[st] = b_lds + ((wn * 128 + l32) * 4 + chunk) * 16;
+    }
+    const unsigned m0_a0 = __builtin_amdgcn_readfirstlane(a_lds + wave * 4096);
+    const unsigned m0_b0 = __builtin_amdgcn_readfirstlane(b_lds + wave * 4096);
+    typedef Loop<I8> L;
+    L::prime(r, a_addr, b_addr);
+    int stage = 0;
+    for (int t = 0; t < nstages; ++t) {
+      const int next = (stage + 1) & 3, slot3 = (stage + 3) & 3;
+      L::tile(r, a_addr, b_addr, (unsigned)((next - stage) * (int)PANEL), nstages - (t + 3),
+              m0_a0 + slot3 * PANEL, m0_b0 + slot3 * PANEL, off_a, off_b, base_a, base_b);
+      base_a += STAGE_K_BYTES;
+      base_b += STAGE_K_BYTES;
+      stage = next;
+    }
+    // the compiler does not see the matrix instructions inside the statements, so it cannot know that the
+    // accumulators it reads next may still be on their way: the last one written needs 18 wait states
+    asm volatile("s_nop 15\ns_nop 7" : CUASR_NARROW_ACC);
+  }
+
+  // ---- epilogue.  Block (bi, bj), register e of lane l: row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32: a
+  // store instruction writes 128 consecutive bytes of two rows.  (With the operands of the matrix instruction
+  // swapped a lane holds four consecutive columns per group of registers and stores vectors -- a quarter of the
+  // store instructions, but each touching 32 rows, a leading dimension apart: measured 25 % slower at 8192^3.)
+  const EpilogueScalars<Result> sc = resolve_scalars<Result>(p, kMultiplies);
+  const Result *C = reinterpret_cast<const Result *>(p.C);
+  Result *D = reinterpret_cast<Result *>(p.D);
+#pragma unroll
+  for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj) {
+      const int col = n0 + wn * 128 + bj * 32 + l32;
+      const int blk = 4 * bi + bj;
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int row = m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+        const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
+        if constexpr (I8) {
+          if (p.workspace) {
+            reinterpret_cast<int32_t *>(p.workspace)[((long long)blockIdx.y * p.m + row) * p.n + col] = bits;
+          } else {
+            // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
+            uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
+            if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)C[(long long)row * p.ldc + col];
+            D[(long long)row * p.ldd + col] = (int32_t)out;
+          }
+        } else {
+          // D = alpha * acc + beta * C in float, rounded to binary16 once
+          float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
+          if (sc.source_needed) out += float(sc.beta) * float(C[(long long)row * p.ldc + col]);
+          D[(long long)row * p.ldd + col] = half_t(out);
+        }
+      }
+    }
+}
+
+// whole tiles, whole stages, both operands k-contiguous with 16-byte aligned rows, a panel's 256 rows within 32
+// bits of byte offset
+static bool can_run(const Problem &p, long long esize) {
+  auto al16 = [](const void *q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
+  if (p.sa_k != 1 || p.sb_k != 1 || p.m <= 0 || p.n <= 0 || p.k <= 0) return false;
+  if (p.m % BM || p.n % BN || (p.k * esize) % STAGE_K_BYTES) return false;
+  if (p.workspace && (p.k_per_slice * esize) % STAGE_K_BYTES) return false;
+  if ((p.sa_m * esize) % 16 || (p.sb_n * esize) % 16 || !al16(p.A) || !al16(p.B)) return false;
+  if (256 * p.sa_m * esize >= (1LL << 32) || 256 * p.sb_n * esize >= (1LL << 32)) return false;
+  if (p.batch > 1 && ((p.batch_a * esize) % 16 || (p.batch_b * esize) % 16)) return false;
+  return true;
+}
+
+template <bool I8> static hipError_t launch(const Problem &p, hipStream_t s) {
+  const long long tiles = (long long)(p.m / BM) * (p.n / BN);
+  if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+  const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(256);
+  launch_kernel((mfma_narrow_kernel<I8>), grid, block, 0, s, p);
+  return take_launch_status();
+}
+
+}  // namespace mfma_narrow
+
+// One wave per SIMD and one workgroup per compute unit: a launch takes ceil(workgroups / compute units) tile
+// times, so the hand-scheduled tile is for launches that fill most of their last such round; smaller or oddly
+// sized ones are better served by the compiled kernels' 128 x 128 tiles, two per compute unit.
+static bool narrow_fills(const Problem &p, int units) {
+  if (units <= 0) units = 256;
+  const long long groups = (long long)(p.m / mfma_narrow::BM) * (p.n / mfma_narrow::BN) * (p.workspace ? p.slices : 1) * p.batch;
+  const long long rounds = (groups + units - 1) / units;
+  return groups * 4 >= rounds * units * 3;
+}
+
+bool mfma_narrow_i8_can_run(const Problem &p, int units) { return mfma_narrow::can_run(p, 1) && narrow_fills(p, units); }
+bool mfma_narrow_f16_can_run(const Problem &p, int units) { return !p.workspace && mfma_narrow::can_run(p, 2) && narrow_fills(p, units); }
+hipError_t launch_mfma_narrow_i8(const Problem &p, hipStream_t s) { return mfma_narrow::launch<true>(p, s); }
+hipError_t launch_mfma_narrow_f16(const Problem &p, hipStream_t s) { return mfma_narrow::launch<false>(p, s); }
+
+}  // namespace cuasr_amd

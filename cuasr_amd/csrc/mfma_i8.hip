@@ -21,6 +21,11 @@
 #include "semiring.h"
 
 namespace cuasr_amd {
+
+// the hand-scheduled form for whole 256 x 256 tiles of k-contiguous operands (mfma_direct_narrow.hip)
+bool mfma_narrow_i8_can_run(const Problem &p, int units);
+hipError_t launch_mfma_narrow_i8(const Problem &p, hipStream_t s);
+
 namespace mfma_i8 {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -237,6 +242,7 @@ static bool exact(const Problem &p, bool a_kc, bool b_kc) {
 
 static hipError_t launch(const Problem &p, hipStream_t s) {
   if (p.m == 0 || p.n == 0) return hipSuccess;
+  if (mfma_narrow_i8_can_run(p, 0)) return launch_mfma_narrow_i8(p, s);
   if ((p.sa_m != 1 && p.sa_k != 1) || (p.sb_n != 1 && p.sb_k != 1)) return hipErrorNotSupported;
   // (an operand with both strides 1 is a single row or column: either form reads it correctly)
   const bool a_kc = p.sa_k == 1, b_kc = p.sb_k == 1;

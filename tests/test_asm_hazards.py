@@ -13,7 +13,8 @@ import pytest
 import asm_inflight
 from cuasr_amd import build as B
 
-FILES = ["direct_f32.hip", "direct_i32.hip", "direct_u32.hip", "direct_f64.hip", "mfma_direct_f32.hip", "mfma_direct_f64.hip", "fwgemm.hip"]
+FILES = ["direct_f32.hip", "direct_i32.hip", "direct_u32.hip", "direct_f64.hip", "mfma_direct_f32.hip", "mfma_direct_f64.hip",
+         "mfma_direct_narrow.hip", "fwgemm.hip"]
 
 
 def _listing(src, out_dir):
@@ -114,7 +115,7 @@ def test_no_instruction_touches_a_register_an_asm_lds_read_is_filling(tmp_path):
     for src, text in zip(FILES, texts):
         # every kernel of the direct_*.hip files: the plain tiles and the stream-K form, which inlines the tile's
         # segment twice inside run-time loops and so gets a register allocation of its own
-        res = asm_inflight.check_listing(text, "gemm_mfma_direct" if src.startswith("mfma") else "fwgemm_direct_kernel" if src.startswith("fwgemm") else "_kernel")
+        res = asm_inflight.check_listing(text, "mfma_narrow_kernel" if src.startswith("mfma_direct_narrow") else "gemm_mfma_direct" if src.startswith("mfma") else "fwgemm_direct_kernel" if src.startswith("fwgemm") else "_kernel")
         assert res, f"{src}: no kernels found in the listing"
         if src in ("direct_f32.hip", "direct_i32.hip", "direct_u32.hip"):
             assert any("streamk_kernel" in k for k in res), f"{src}: no stream-K kernel was checked"

@@ -359,3 +359,39 @@ def test_serial_splitk(oracle, lib, slices):
         cuasr_amd.srgemm_splitk_serial(add, mult, to_device(A), to_device(B), to_device(C), dD, slices, ws, f(alpha), f(beta), f(ident), f(one), dtype="f16")
         torch.cuda.synchronize()
         assert_same_bits(dD.cpu().numpy(), want, f"serial split-K f16 {add}-{mult} {layouts} S={slices}")
+
+
+# ---- the hand-scheduled 256 x 256 matrix-core tile (whole tiles of k-contiguous operands that fill the chip) ----
+
+def test_hand_scheduled_matrix_core_tile(oracle, lib):
+    """192 tiles and more of 256 x 256, A row-major and B column-major, kernel = mfma: exact on small integers
+    (fragment layout, ring of stages, epilogue), one to nine stages of 32 k; then uniform data against a
+    double-precision product within one binary16 rounding plus the error of a float sum."""
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    m, n = 4096, 3072
+    for k, (alpha, beta) in [(32, (1, 0)), (64, (1, 1)), (96, (2, -1)), (288, (-1, 2))]:
+        A = inputs.integers(21 + k, m, k, -2, 2, np.float16, "C")
+        B = inputs.integers(22 + k, k, n, -2, 2, np.float16, "F")
+        C = inputs.integers(23 + k, m, n, -8, 8, np.float16, "C")
+        want = oracle.srgemm("plus", "multiplies", A, B, C, np.float16(alpha), np.float16(beta), np.float16(0))
+        assert np.abs(want.astype(np.float64)).max() <= 2048
+        dD = to_device(np.full_like(C, 7))
+        cuasr_amd.srgemm("plus", "multiplies", to_device(A), to_device(B), to_device(C), dD, np.float16(alpha), np.float16(beta),
+                         np.float16(0), np.float16(1), dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        assert_same_bits(dD.cpu().numpy(), want, f"plus-times f16 mfma {m}x{n}x{k}")
+    k = 1024
+    A = inputs.uniform(31, m, k, -1.0, 1.0, np.float16, "C")
+    B = inputs.uniform(32, k, n, -1.0, 1.0, np.float16, "F")
+    C = inputs.uniform(33, m, n, -4.0, 4.0, np.float16, "C")
+    alpha, beta = np.float16(0.75), np.float16(-1.5)
+    r = float(alpha) * (A.astype(np.float64) @ B.astype(np.float64)) + float(beta) * C.astype(np.float64)
+    bound = 2.0 ** -11 * np.abs(r) + 1e-5 * (np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)) + 1e-7
+    dD = to_device(np.zeros_like(C))
+    cuasr_amd.srgemm("plus", "multiplies", to_device(A), to_device(B), to_device(C), dD, alpha, beta, np.float16(0), np.float16(1),
+                     dtype="f16", kernel="mfma")
+    torch.cuda.synchronize()
+    err = np.abs(dD.cpu().numpy().astype(np.float64) - r)
+    assert (err <= bound).all(), f"worst excess {(err - bound).max():.3e}"

@@ -224,3 +224,38 @@ def test_serial_splitk(oracle, lib, slices):
         cuasr_amd.srgemm_splitk_serial(add, mult, to_device(A), to_device(B), to_device(C), dD, slices, ws, alpha, beta, ident, one, dtype="i8")
         torch.cuda.synchronize()
         assert_same_bits(dD.cpu().numpy(), want, f"serial split-K i8 {add}-{mult} {layouts} S={slices}")
+
+
+# ---- the hand-scheduled 256 x 256 tile (whole tiles of k-contiguous operands that fill the chip) ----------------
+
+def test_hand_scheduled_tile_plain(oracle, lib):
+    """192 tiles and more of 256 x 256 with A row-major and B column-major (both k-contiguous) take the
+    hand-scheduled tile: one, two, three (the ring's prologue) and nine stages of 64 k, scalars that are not the
+    semiring's own, and the same shape with one operand the other way round (the compiled kernel) for contrast."""
+    for k in (64, 128, 192, 576):
+        check(oracle, "plus", "multiplies", 4096, 3072, k, "rcr", "auto", alpha=3, beta=-2, seed=k)
+    check(oracle, "plus", "multiplies", 3072, 4096, 320, "rcc", "mfma", alpha=1, beta=0)   # column-major C: the transposed problem
+    check(oracle, "plus", "multiplies", 4096, 3072, 128, "ccr", "auto", alpha=1, beta=1)
+
+
+def test_hand_scheduled_tile_splitk_and_batch(oracle, lib):
+    import torch
+    import cuasr_amd
+    from cuasr_amd import inputs
+    # 16 tiles x 13 slices of 64 k: every slice one stage; then slices of five stages with a ragged last slice
+    check(oracle, "plus", "multiplies", 1024, 1024, 64 * 13, "rcr", "auto", alpha=2, beta=5, splitk=13)
+    check(oracle, "plus", "multiplies", 1024, 1024, 64 * 61, "rcr", "auto", alpha=1, beta=1, splitk=13)
+    # 13 products of 16 tiles each in one launch
+    m = n = 1024
+    k, batch = 192, 13
+    A = inputs.integers(3, batch * m, k, -128, 127, np.int8, "C").reshape(batch, m, k)
+    B = inputs.integers(4, batch * n, k, -128, 127, np.int8, "C").reshape(batch, n, k)        # column-major k x n slices
+    C = inputs.integers(5, batch * m, n, -1000, 1000, np.int32, "C").reshape(batch, m, n)
+    dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda().transpose(1, 2), torch.from_numpy(C).cuda()
+    dD = torch.zeros_like(dC)
+    cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, 1, 1, 0, 1, dtype="i8")
+    torch.cuda.synchronize()
+    got = dD.cpu().numpy()
+    for i in (0, 5, 12):
+        want = oracle.srgemm("plus", "multiplies", A[i], np.asfortranarray(B[i].T), C[i], 1, 1, 0)
+        assert_same_bits(got[i], want, f"batch product {i}")
