@@ -162,12 +162,22 @@ struct DirectTile {
     return KC ? i * XT + t : (i >> 2) * 4 * XT + t * 4 + (i & 3);
   }
 
+  // CUASR_AMD_TILE_ORDER (measurement only; see profiles/direct_srgemm_minplus_f32_apsp4096.md): 0 = the order
+  // described here, 1 = plain row-major tiles with no regard for the XCDs, 2 = blocks of 4 tile rows instead of 8
+#ifndef CUASR_AMD_TILE_ORDER
+#define CUASR_AMD_TILE_ORDER 0
+#endif
   static __device__ __forceinline__ void tile_coords(int id, int tiles_m, int tiles_n, int &bm, int &bn) {
     const int total = tiles_m * tiles_n;
+    if (CUASR_AMD_TILE_ORDER == 1) {
+      bm = id / tiles_n;
+      bn = id % tiles_n;
+      return;
+    }
     // consecutive workgroup ids land on consecutive XCDs (8, one L2 each):
     // give every XCD one contiguous run of the tile order
     if ((total & 7) == 0) id = (id & 7) * (total >> 3) + (id >> 3);
-    constexpr int GROUP = 8;
+    constexpr int GROUP = CUASR_AMD_TILE_ORDER == 2 ? 4 : 8;
     const int width = GROUP * tiles_n;
     const int group = id / width, first = group * GROUP;
     const int gsz = min(tiles_m - first, GROUP);
