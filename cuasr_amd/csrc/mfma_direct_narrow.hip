@@ -200,9 +200,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int bj = 0; bj < 4; ++bj) {
       const int col = n0 + wn * 128 + bj * 32 + l32;
       const int blk = 4 * bi + bj;
+      auto row_of = [&](int e) { return (long long)(m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4)); };
+      // a block's sixteen source elements are requested together, before any of its results is stored (D may be
+      // C, so the compiler cannot move a load of C above a store to D by itself: one load at a time, each waited
+      // for, made this epilogue as long as the product)
+      Result src[16];
+      if (!p.workspace && sc.source_needed) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) src[e] = C[row_of(e) * p.ldc + col];
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+        const long long row = row_of(e);
         const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
         if constexpr (I8) {
           if (p.workspace) {
@@ -210,14 +219,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           } else {
             // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
             uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
-            if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)C[(long long)row * p.ldc + col];
-            D[(long long)row * p.ldd + col] = (int32_t)out;
+            if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)src[e];
+            D[row * p.ldd + col] = (int32_t)out;
           }
         } else {
           // D = alpha * acc + beta * C in float, rounded to binary16 once
           float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
-          if (sc.source_needed) out += float(sc.beta) * float(C[(long long)row * p.ldc + col]);
-          D[(long long)row * p.ldd + col] = half_t(out);
+          if (sc.source_needed) out += float(sc.beta) * float(src[e]);
+          D[row * p.ldd + col] = half_t(out);
         }
       }
     }

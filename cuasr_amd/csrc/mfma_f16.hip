@@ -198,12 +198,22 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
       const int col = n0 + wn * 64 + bj * 32 + l32;
+      // a block's sixteen source elements are requested together, before any of its results is stored (D may be C,
+      // so the compiler cannot move a load of C above a store to D by itself)
+      half_t src[16];
+      if (sc.source_needed) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+          src[e] = (!GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) ? C[(long long)row * p.ldc + col] : half_t(0);
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
         if (GUARD && !((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) continue;
         float out = alpha * acc[bi][bj][e];
-        if (sc.source_needed) out += beta * float(C[(long long)row * p.ldc + col]);
+        if (sc.source_needed) out += beta * float(src[e]);
         D[(long long)row * p.ldd + col] = half_t(out);
       }
     }

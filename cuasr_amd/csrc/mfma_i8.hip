@@ -212,6 +212,16 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
       const int col = n0 + wn * 64 + bj * 32 + l32;
+      // a block's sixteen source elements are requested together, before any of its results is stored (D may be C,
+      // so the compiler cannot move a load of C above a store to D by itself)
+      int32_t src[16];
+      if (!ws && sc.source_needed) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
+          src[e] = (!GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) ? C[(long long)row * p.ldc + col] : 0;
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
         const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
@@ -222,7 +232,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
         } else {
           // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
           uint32_t out = (uint32_t)sc.alpha * (uint32_t)v;
-          if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)C[(long long)row * p.ldc + col];
+          if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)src[e];
           D[(long long)row * p.ldd + col] = (int32_t)out;
         }
       }
