@@ -261,25 +261,30 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         # a whole all-pairs shortest-path job with predecessor tracking by blocked Floyd-Warshall:
         # one step = reset dist and parent, then the n / 128 block steps (2 * n^3 operations in all)
         n = args.size or 4096
+        dt = args.dtype if args.dtype == "f64" else "f32"
         D0 = inputs.graph_distances(2024, n, density=0.10, lo=1.0, hi=100.0)
+        if dt == "f64":
+            D0 = D0.astype(np.float64)
         d0 = col_major(D0)
-        dist = torch.empty(n, n, device=dev).t()
+        dist = torch.empty(n, n, dtype=d0.dtype, device=dev).t()
         parent = torch.empty(n, n, dtype=torch.int32, device=dev).t()
-        ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, "f32"), dtype=torch.uint8, device=dev)
+        ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, dt), dtype=torch.uint8, device=dev)
 
         def step(i):
             dist.copy_(d0)
             parent.fill_(-1)
             cuasr_amd.apsp_blocked(dist, parent, ws)
 
-        return dict(step=step, m=n, n=n, k=n, dtype="f32", desc=None, host=(D0,), family="fwgemm_tile + fw_diagonal",
+        bits = "fp64" if dt == "f64" else "fp32"
+        return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=None, host=(D0,), family="fwgemm_tile + fw_close_dist",
                     fw=dict(dist=dist, parent=parent),
-                    metric=f"fp32 all-pairs shortest paths with predecessors, blocked Floyd-Warshall, GOPS at n={n} "
+                    metric=f"{bits} all-pairs shortest paths with predecessors, blocked Floyd-Warshall, GOPS at n={n} "
                            "(2 ops/term, 2*n^3 per job)",
-                    workload=f"whole APSP job with predecessor tracking by blocked Floyd-Warshall (128-vertex blocks), fp32, "
+                    workload=f"whole APSP job with predecessor tracking by blocked Floyd-Warshall (128-vertex blocks), {bits}, "
                              f"n={n}, column-major, 10% edges U[1,100), rest +inf; a step = reset of dist and parent + "
                              f"{(n + 127) // 128} block steps",
-                    bound="valu", peak=FP32_VECTOR_PEAK, instr_per_term=1.5)
+                    bound="valu", peak=FP64_VECTOR_PEAK if dt == "f64" else FP32_VECTOR_PEAK,
+                    instr_per_term=2.0 if dt == "f64" else 1.5)
 
     if w == "srgemm":
         # any operator pair / element type / layout combination at one size: the reference's
@@ -658,13 +663,15 @@ def main():
             # minutes at full size); the GPU runs that graph too and must match it bit for bit
             nc = min(n, 2048)
             Dc = inputs.graph_distances(2024, nc, density=0.10, lo=1.0, hi=100.0)
+            if wl["dtype"] == "f64":
+                Dc = Dc.astype(np.float64)
             hd, hp = Dc.copy(order="F"), np.full((nc, nc), -1, dtype=np.int32, order="F")   # (a copy: the oracle works in place)
             t1 = time.perf_counter()
             oracle.apsp_blocked(hd, hp, 128)
             cpu_s = time.perf_counter() - t1
             gd = torch.from_numpy(np.ascontiguousarray(Dc.T)).to("cuda:0").t()
             gp = torch.full((nc, nc), -1, dtype=torch.int32, device="cuda:0").t()
-            gws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(nc, "f32"), dtype=torch.uint8, device="cuda:0")
+            gws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(nc, wl["dtype"]), dtype=torch.uint8, device="cuda:0")
             cuasr_amd.apsp_blocked(gd, gp, gws)
             torch.cuda.synchronize()
             exact = bool(np.ascontiguousarray(gd.cpu().numpy()).tobytes() == np.ascontiguousarray(hd).tobytes()

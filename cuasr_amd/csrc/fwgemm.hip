@@ -44,8 +44,10 @@ struct FwArgs {
   void *out_t; int64_t ld_out_t;
   // tile kernel, blocked Floyd-Warshall only: the diagonal block that starts at (ahead0, ahead0) and has
   // ahead_bb (> 0) rows is the next block step's and has had this step's update already: the launch's
-  // first workgroup closes it (fw_close_256) while the others do the product, which leaves that tile alone
+  // first workgroup closes its distances (fw_close_dist) while the others do the product, which leaves that
+  // block alone.  hist: 3 x FW_BLOCK x FW_BLOCK elements that take what fw_parents_block needs afterwards.
   int ahead0, ahead_bb;
+  void *hist;
 };
 
 // cond ? a : b with a hidden from the optimiser: `x < y ? x : y` on floating point is
@@ -54,6 +56,14 @@ struct FwArgs {
 template <typename T> __device__ __forceinline__ T pick(bool cond, T a, T b) {
   asm("" : "+v"(a));
   return cond ? a : b;
+}
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a compile-time constant
+template <int N, int I = 0, typename F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<N, I + 1>(f);
+  }
 }
 
 // one thread per element, the literal scan; any extent, any leading dimension
@@ -221,21 +231,73 @@ template <typename T> __device__ __forceinline__ void fwgemm_rowcols_block(const
   }
 }
 
-// two independent products in one launch (the block row and the block column of a blocked
-// Floyd-Warshall step, each too small to fill the chip): the first blocks0 workgroups work on
-// g0, the others on g1
-template <typename T>
-__global__ void __launch_bounds__(256) fwgemm_pair_kernel(FwArgs g0, FwArgs g1, int blocks0) {
-  const int b = blockIdx.x;
-  if (b < blocks0) {
-    const int gx = (g0.m + 63) / 64;
-    fwgemm_rowcols_block<T>(g0, b % gx, b / gx);
-  } else {
-    const int gx = (g1.m + 63) / 64;
-    fwgemm_rowcols_block<T>(g1, (b - blocks0) % gx, (b - blocks0) / gx);
+// The improved elements of a tile, queued in LDS as (code = row in the tile | column << ROW_BITS | chunk <<
+// (ROW_BITS + COL_BITS), minimum), are looked up by groups of CHUNK / 4 lanes: each lane adds four of the chunk's
+// products (one 16- or 32-byte load from B's column and one from the k-contiguous image of A), the group agrees on
+// the first k whose product equals the minimum, and the lane that holds it stores that product -- the same single
+// addition of the same operands as in the main loop, so the comparison is exact and the stored distance has the sign
+// that the sequential scan would leave -- and the predecessor.  A wave's load then touches one cache line per
+// element where one lane per element would touch 64.  A group takes UN elements per turn and requests all their
+// operands before it looks at any: a turn costs one round trip to memory, and a tile has few turns.
+template <int G> __device__ __forceinline__ int group_min(int v) {
+  // minimum over the G (4 or 8) adjacent lanes of a group, by data-parallel moves inside the row of 16 lanes
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0xB1, 0xf, 0xf, true));   // lanes 1 0 3 2 of each four
+  v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x4E, 0xf, 0xf, true));   // lanes 2 3 0 1 of each four
+  if constexpr (G == 8) v = min(v, __builtin_amdgcn_update_dpp(v, v, 0x141, 0xf, 0xf, true));  // each eight mirrored
+  return v;
+}
+template <typename T, int THREADS, int CHUNK, bool HAS_AT, int ROW_BITS, int COL_BITS>
+__device__ __forceinline__ void lookup_queue(const FwArgs &g, const uint32_t *q_code, const T *q_want, int count, int tid,
+                                             int m0, int n0) {
+  typedef typename vec4_of<T>::type V4;
+  constexpr int G = CHUNK / 4, GROUPS = THREADS / G;
+  constexpr int UN = sizeof(T) == 4 ? 8 : 4;
+  static_assert(G == 4 || G == 8, "lanes per element");
+  const T *A = static_cast<const T *>(g.A), *B = static_cast<const T *>(g.B), *At = static_cast<const T *>(g.At);
+  T *dist = static_cast<T *>(g.dist);
+  const int sub = tid % G;
+  for (int e0 = tid / G; e0 < count; e0 += UN * GROUPS) {
+    int r[UN], c[UN], k0[UN];
+    T want[UN];
+    V4 pa[UN], pb[UN];
+    bool live[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      const int e = e0 + u * GROUPS;
+      live[u] = e < count;
+      const uint32_t code = q_code[live[u] ? e : e0];  // (a turn's last elements may not exist: their lanes look at the first again)
+      want[u] = q_want[live[u] ? e : e0];
+      r[u] = m0 + int(code & ((1u << ROW_BITS) - 1));
+      c[u] = n0 + int((code >> ROW_BITS) & ((1u << COL_BITS) - 1));
+      k0[u] = int(code >> (ROW_BITS + COL_BITS)) * CHUNK + 4 * sub;
+      pb[u] = *reinterpret_cast<const V4 *>(B + k0[u] + int64_t(c[u]) * g.ldb);
+      if constexpr (HAS_AT) {
+        pa[u] = *reinterpret_cast<const V4 *>(At + k0[u] + int64_t(r[u]) * g.ldat);
+      } else {
+#pragma unroll
+        for (int x = 0; x < 4; ++x) pa[u][x] = A[r[u] + int64_t(k0[u] + x) * g.lda];
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+      T value = want[u];
+      int first = 4;
+#pragma unroll
+      for (int x = 3; x >= 0; --x) {
+        const T prod = pa[u][x] + pb[u][x];
+        const bool hit = prod == want[u];
+        first = hit ? x : first;
+        value = pick(hit, prod, value);
+      }
+      const int key = first < 4 ? 4 * sub + first : CHUNK;  // where in the chunk my first hit is
+      const int best = group_min<G>(key);
+      if (live[u] && first < 4 && key == best) {
+        dist[r[u] + int64_t(c[u]) * g.ldc] = value;
+        g.parent[r[u] + int64_t(c[u]) * g.ldp] = g.k_base + k0[u] + first;
+      }
+    }
   }
 }
-
 
 // 256 threads as 16 x 16; each owns TM x TN outputs in groups of four rows /
 // columns that lie 64 apart, so a workgroup covers (16 TM) x (16 TN).
@@ -405,78 +467,73 @@ __device__ __forceinline__ void fwgemm_tile_body(const FwArgs &g, const int bloc
   asm volatile("" : "+v"(tx2), "+v"(ty2));
   if constexpr (!GUARD) {
     // Whole, aligned tiles.  Improved elements are few in most launches and scattered over the
-    // lanes, so they are first collected in a queue in LDS (the panels are no longer needed),
-    // one column j of the lanes' outputs at a time (at most 256 x TM entries), and the queue is
-    // then worked off by all 256 threads, one element per thread and turn: no lane waits for an
-    // element that did not improve.  Every lane looks at a chunk of its own, so each load of a
-    // column-major A touches 64 cache lines per wave; with the k-contiguous image of A an
-    // element's operands are two runs of BK values.
-    constexpr int CAP = 256 * TM;
-    static_assert(sizeof(as) >= 2 * CAP * sizeof(int) && sizeof(bs) >= CAP * sizeof(T), "the queue must fit in the panels");
-    __shared__ int q_count;
-    int *q_pos = reinterpret_cast<int *>(&as[0][0][0]);  // row | column << 8, inside the tile
-    int *q_ch = q_pos + CAP;                             // chunk
-    T *q_want = reinterpret_cast<T *>(&bs[0][0][0]);     // the minimum found
-    const T *At = static_cast<const T *>(g.At);
-#pragma unroll 1
+    // lanes, so they are first collected in a queue in LDS (the panels are no longer needed) and the
+    // queue is then worked off by all 256 threads (lookup_queue): no lane waits for an element that did
+    // not improve.  The queue takes as many whole columns j of the lanes' outputs as fit (one column
+    // always does: at most 256 x TM elements), so a tile with few improved elements -- the usual case --
+    // is done in one round of queueing, barrier and lookups, not one per column.
+    constexpr int CAP = (sizeof(as) / sizeof(int) < sizeof(bs) / sizeof(T) ? sizeof(as) / sizeof(int) : sizeof(bs) / sizeof(T)) / 256 * 256;
+    static_assert(CAP >= 256 * TM && BM <= 128 && BN <= 128, "a column of the lanes' outputs must fit in the panels");
+    // Where an element goes in the queue follows from counts alone, without a shared counter (whose every use is a
+    // round trip to LDS that the next one waits for): column by column, inside a column wave by wave, inside a wave
+    // row i by row i, inside a row lane by lane.  Each wave counts its improved elements per column first.
+    __shared__ int wave_count[4][TN];
+    uint32_t *q_code = reinterpret_cast<uint32_t *>(&as[0][0][0]);  // row | column << 7 | chunk << 14 (the host sees to k < 2^22)
+    T *q_want = reinterpret_cast<T *>(&bs[0][0][0]);                // the minimum found
+    const int wave = tid >> 6;
+    __syncthreads();  // everybody is done with the panels
+#pragma unroll
     for (int j = 0; j < TN; ++j) {
-      __syncthreads();  // everybody is done with the panels / with the queue of the column before
-      if (tid == 0) q_count = 0;
-      __syncthreads();
+      int n_improved = 0;  // in this column, over the wave
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        // (j is a run-time value here: the accumulators are read through a select chain over
-        // the TN columns, which is cheap next to the loop it replaces)
-        int ch = -1;
-        T want = T(0);
+      for (int i = 0; i < TM; ++i) n_improved += __builtin_popcountll(__builtin_amdgcn_ballot_w64(chunk[i][j] >= 0));
+      if ((tid & 63) == 0) wave_count[wave][j] = n_improved;
+    }
+    __syncthreads();
+    int before_me[TN], col_count[TN];  // improved elements of the column in the waves before mine / in all waves
 #pragma unroll
-        for (int jj = 0; jj < TN; ++jj)
-          if (jj == j) {
-            ch = chunk[i][jj];
-            want = acc[i][jj];
-          }
-        if (ch >= 0) {
-          const int slot = atomicAdd(&q_count, 1);
-          q_pos[slot] = ((i >> 2) * 64 + tx2 * 4 + (i & 3)) | (((j >> 2) * 64 + ty2 * 4 + (j & 3)) << 8);
-          q_ch[slot] = ch;
-          q_want[slot] = want;
-        }
+    for (int j = 0; j < TN; ++j) {
+      before_me[j] = col_count[j] = 0;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int n = __builtin_amdgcn_readfirstlane(wave_count[w][j]);
+        before_me[j] += w < wave ? n : 0;
+        col_count[j] += n;
       }
-      __syncthreads();
-      const int count = q_count;
-      for (int e = tid; e < count; e += 256) {
-        const int pos = q_pos[e], r = m0 + (pos & 255), c = n0 + (pos >> 8), k0 = q_ch[e] * BK;
-        const T want = q_want[e];
-        T pa[BK];
-        V4 pb[BK / 4];
-        const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(c) * g.ldb);
-        if constexpr (HAS_AT) {
-          const V4 *atp = reinterpret_cast<const V4 *>(At + k0 + int64_t(r) * g.ldat);
+    }
+    for (int j0 = 0; j0 < TN;) {  // (the same for every thread)
+      int total = 0, j1 = j0;
 #pragma unroll
-          for (int q = 0; q < BK / 4; ++q) {
-            const V4 v = atp[q];
-#pragma unroll
-            for (int x = 0; x < 4; ++x) pa[q * 4 + x] = v[x];
-          }
-        } else {
-          const T *ap = A + r + int64_t(k0) * g.lda;
-#pragma unroll
-          for (int kk = 0; kk < BK; ++kk) pa[kk] = ap[int64_t(kk) * g.lda];
-        }
-#pragma unroll
-        for (int q = 0; q < BK / 4; ++q) pb[q] = bp[q];
-        T value = want;
-        int first = 0;
-#pragma unroll
-        for (int kk = BK - 1; kk >= 0; --kk) {
-          const T prod = pa[kk] + pb[kk >> 2][kk & 3];
-          const bool hit = prod == want;
-          first = hit ? kk : first;
-          value = pick(hit, prod, value);
-        }
-        dist[r + int64_t(c) * g.ldc] = value;
-        g.parent[r + int64_t(c) * g.ldp] = g.k_base + k0 + first;
+      for (int j = 0; j < TN; ++j) {  // as many whole columns from j0 on as fit
+        if (j < j0 || j != j1) continue;
+        if (j > j0 && total + col_count[j] > CAP) continue;
+        total += col_count[j];
+        j1 = j + 1;
       }
+      if (total > 0) {
+        int base = 0;  // of the column in the queue
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if (j < j0 || j >= j1) continue;
+          int slot0 = base + before_me[j];  // of my wave's next row of this column
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+            const unsigned long long improved = __builtin_amdgcn_ballot_w64(chunk[i][j] >= 0);
+            if (chunk[i][j] >= 0) {
+              const int slot = slot0 + __builtin_amdgcn_mbcnt_hi(uint32_t(improved >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(improved), 0u));
+              q_code[slot] = uint32_t((i >> 2) * 64 + tx2 * 4 + (i & 3)) | uint32_t((j >> 2) * 64 + ty2 * 4 + (j & 3)) << 7 |
+                             uint32_t(chunk[i][j]) << 14;
+              q_want[slot] = acc[i][j];
+            }
+            slot0 += __builtin_popcountll(improved);
+          }
+          base += col_count[j];
+        }
+        __syncthreads();
+        lookup_queue<T, 256, BK, HAS_AT, 7, 7>(g, q_code, q_want, total, tid, m0, n0);
+        __syncthreads();  // the queue is free again
+      }
+      j0 = j1;
     }
     return;
   }
@@ -682,6 +739,293 @@ __device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *pare
     }
 }
 
+// ---- closing a diagonal block in two parts: distances first, predecessors afterwards
+//
+// Step k of the closure lowers d[i][j] to cand_k = d[i][k] + d[k][j] (row k and column k as they are before the
+// step) wherever that is strictly smaller, and the predecessor of (i, j) is the last k that did so.  A step that
+// lowers an element is a strict record of the sequence d0[i][j], cand_0, cand_1, ...; the last record of a
+// sequence is the first place its minimum is at.  So, given the rows and columns that the steps read, the
+// predecessors are those of one min-plus product with predecessor tracking (fwgemm's own semantics, strict
+// comparison, k ascending) of a matrix whose column k is "column k before step k" with one whose row k is
+// "row k before step k", started from the block as it was before the closure.  Nothing of that product is on the
+// critical path: nothing that follows reads a diagonal block's predecessors, and the product is spread over 64
+// workgroups of a later launch.
+//
+// What stays on the critical path is fw_close_dist: the 128 dependent steps for the distances alone, an addition
+// and a minimum per element and step (half the instructions of a step that also selects predecessors, and none
+// that reads a comparison mask), by one workgroup of 256 threads with an 8 x 8 patch per thread.  Every row and
+// column that a step publishes to LDS for the next one also goes to hist (row k and column k as step k reads them),
+// and the block as it was found goes there too.
+//
+// The hardware minimum prefers -0 to +0 where the strict comparison keeps whichever came first.  Sums and minima
+// of data free of -0 never produce one, so the block is searched for a -0 when it is loaded, and a block with
+// one takes the same steps with a comparison and a select (EXACT).
+//
+// hist: FW_BLOCK x FW_BLOCK elements each of  col[k * FW_BLOCK + i] = d[i][k] before step k,
+// row[k * FW_BLOCK + j] = d[k][j] before step k,  init[i + j * FW_BLOCK] = d[i][j] before the closure.
+// (returns false, with nothing done, when the block holds a -0 and EXACT is not set)
+template <typename T, bool EXACT>
+__device__ __forceinline__ bool fw_close_dist_as(T *d, int64_t ld, int bb, T *hist, T (*colbuf)[FW_BLOCK], T (*rowbuf)[FW_BLOCK]) {
+  typedef typename vec4_of<T>::type V4;
+  const int tid = threadIdx.x & 255, ti = tid & 15, tj = tid >> 4;  // rows 8 ti .. 8 ti + 7, columns 8 tj .. 8 tj + 7
+  const T inf = std::numeric_limits<T>::infinity();
+  T *hist_col = hist, *hist_row = hist + FW_BLOCK * FW_BLOCK, *init = hist + 2 * FW_BLOCK * FW_BLOCK;
+  T cur[8][8];  // [row in patch][column in patch]
+  // loads from clamped addresses, then a select (a branch per element would keep 64 lane masks alive); a column's
+  // addresses differ by the clamped row, so that the 64 loads in flight do not need 64 addresses in registers
+  int ic[8];
+#pragma unroll
+  for (int a = 0; a < 8; ++a) ic[a] = min(8 * ti + a, bb - 1);
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    const int j = 8 * tj + b;
+    const T *column = d + int64_t(min(j, bb - 1)) * ld;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const T v = column[ic[a]];
+      cur[a][b] = (8 * ti + a < bb && j < bb) ? v : inf;
+    }
+  }
+  if constexpr (!EXACT) {
+    // a block with a -0 is left to the other form, which loads the block for itself (with one copy of the
+    // block in registers across the branch, the registers that the other form needs would be taken from this one)
+    bool negative_zero = false;
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+#pragma unroll
+      for (int a = 0; a < 8; ++a) negative_zero |= cur[a][b] == T(0) && __builtin_signbit(cur[a][b]);
+    if (__syncthreads_or(negative_zero)) return false;
+  }
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      V4 v;
+#pragma unroll
+      for (int a = 0; a < 4; ++a) v[a] = cur[4 * h + a][b];
+      *reinterpret_cast<V4 *>(&init[8 * ti + 4 * h + (8 * tj + b) * FW_BLOCK]) = v;
+    }
+  }
+  // (the minimum as an instruction: from the builtin the compiler first "quiets" an operand whose origin it
+  // does not know, such as anything that comes round the loop, an instruction more per element)
+  auto relax = [](T &x, const T cand) {
+    if constexpr (EXACT) x = pick(cand < x, cand, x);
+    else if constexpr (sizeof(T) == 4) asm("v_min_f32 %0, %0, %1" : "+v"(x) : "v"(cand));
+    else asm("v_min_f64 %0, %0, %1" : "+v"(x) : "v"(cand));
+  };
+  // S = kn & 7, the row / column of the patch that is published, is a compile-time constant (the step
+  // loop is unrolled by eight): indexed by a run-time value the patch would live in scratch memory.
+  // Two elements per instruction, each from a register of its own: as 16-byte stores the compiler wants every
+  // row of the patch AND every column of it in four adjacent registers, cannot have both, and moves parts of the
+  // patch to scratch memory in the attempt.
+  const unsigned row_lds = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&rowbuf[0][8 * tj];
+  const unsigned col_lds = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&colbuf[0][8 * ti];
+  auto write2 = [](unsigned addr, const T x, const T y, auto at) {
+    constexpr int AT = decltype(at)::value;  // in elements
+    if constexpr (sizeof(T) == 4) asm volatile("ds_write2_b32 %0, %1, %2 offset0:%3 offset1:%4" ::"v"(addr), "v"(x), "v"(y), "n"(AT), "n"(AT + 1) : "memory");
+    else asm volatile("ds_write2_b64 %0, %1, %2 offset0:%3 offset1:%4" ::"v"(addr), "v"(x), "v"(y), "n"(AT), "n"(AT + 1) : "memory");
+  };
+  auto publish = [&](int kn, auto bufc, auto sc) {
+    constexpr int S = decltype(sc)::value, BUF = decltype(bufc)::value * FW_BLOCK;
+    if ((kn >> 3) == ti) {  // my patch holds row kn
+      write2(row_lds, cur[S][0], cur[S][1], std::integral_constant<int, BUF + 0>{});
+      write2(row_lds, cur[S][2], cur[S][3], std::integral_constant<int, BUF + 2>{});
+      write2(row_lds, cur[S][4], cur[S][5], std::integral_constant<int, BUF + 4>{});
+      write2(row_lds, cur[S][6], cur[S][7], std::integral_constant<int, BUF + 6>{});
+    }
+    if ((kn >> 3) == tj) {  // my patch holds column kn
+      write2(col_lds, cur[0][S], cur[1][S], std::integral_constant<int, BUF + 0>{});
+      write2(col_lds, cur[2][S], cur[3][S], std::integral_constant<int, BUF + 2>{});
+      write2(col_lds, cur[4][S], cur[5][S], std::integral_constant<int, BUF + 4>{});
+      write2(col_lds, cur[6][S], cur[7][S], std::integral_constant<int, BUF + 6>{});
+    }
+    // (the barrier that follows is the compiler's, which does not know of the instructions above)
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+  // what step kn reads goes to hist from the registers of the threads of the first patch row / column, which
+  // together have read all of it
+  auto record = [&](const T (&c)[8], const T (&r)[8], int kn) {
+    if (kn >= FW_BLOCK) return;
+    if (tj == 0) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        V4 v;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = c[4 * h + x];
+        *reinterpret_cast<V4 *>(&hist_col[kn * FW_BLOCK + 8 * ti + 4 * h]) = v;
+      }
+    }
+    if (ti == 0) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        V4 v;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) v[x] = r[4 * h + x];
+        *reinterpret_cast<V4 *>(&hist_row[kn * FW_BLOCK + 8 * tj + 4 * h]) = v;
+      }
+    }
+  };
+  T ci[8], rj[8];  // column k at my rows, row k at my columns, for the step in hand
+  auto fetch = [&](T (&c)[8], T (&r)[8], int buf) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const V4 cv = *reinterpret_cast<const V4 *>(&colbuf[buf][8 * ti + 4 * h]);
+      const V4 rv = *reinterpret_cast<const V4 *>(&rowbuf[buf][8 * tj + 4 * h]);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        c[4 * h + x] = cv[x];
+        r[4 * h + x] = rv[x];
+      }
+    }
+  };
+  // A step in two parts, because the steps depend on each other and everything between them (publishing row
+  // and column k + 1, the barrier, reading them back) would otherwise add its full latency to every step:
+  //   A. the patch's row and column (k + 1) & 7 -- every thread's, since which thread owns row / column
+  //      k + 1 is only known at run time -- then the owners publish them, then the barrier;
+  //   B. the reads of row / column k + 1 are issued, and the other 49 elements of step k are done while
+  //      they are on their way.
+  auto step = [&](int k, auto uc) {
+    constexpr int U = decltype(uc)::value;  // k & 7
+    constexpr int N = (U + 1) & 7;          // the row and the column of the patch that step k + 1 may need
+    constexpr int O[7] = {N > 0 ? 0 : 1, N > 1 ? 1 : 2, N > 2 ? 2 : 3, N > 3 ? 3 : 4, N > 4 ? 4 : 5, N > 5 ? 5 : 6, N > 6 ? 6 : 7};
+    const int buf = U & 1;
+    if constexpr (sizeof(T) == 8) {
+      // 8-byte elements: the patch takes half the register file, and a second set of rows and columns on its
+      // way beside the one in use pushes parts of the patch into scratch memory.  One part, then: the whole
+      // step, publish, barrier, read.  (The product beside this closure takes three times as long anyway.)
+#pragma unroll
+      for (int a = 0; a < 8; ++a)
+#pragma unroll
+        for (int b = 0; b < 8; ++b) relax(cur[a][b], ci[a] + rj[b]);
+      __builtin_amdgcn_sched_barrier(0);
+      publish(k + 1, std::integral_constant<int, (U & 1) ^ 1>{}, std::integral_constant<int, N>{});
+      __syncthreads();
+      fetch(ci, rj, buf ^ 1);
+      record(ci, rj, k + 1);
+      __builtin_amdgcn_sched_barrier(0);
+      return;
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) relax(cur[N][b], ci[N] + rj[b]);
+#pragma unroll
+    for (int i = 0; i < 7; ++i) relax(cur[O[i]][N], ci[O[i]] + rj[N]);
+    __builtin_amdgcn_sched_barrier(0);
+    // into the other pair of buffers: nobody reads it before the barrier, and nobody is still reading it
+    // from the step before (everybody has passed that step's barrier, and waited for its reads in part A)
+    publish(k + 1, std::integral_constant<int, (U & 1) ^ 1>{}, std::integral_constant<int, N>{});
+    __syncthreads();
+    T cn[8], rn[8];
+    fetch(cn, rn, buf ^ 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < 7; ++i)
+#pragma unroll
+      for (int j = 0; j < 7; ++j) relax(cur[O[i]][O[j]], ci[O[i]] + rj[O[j]]);
+    record(cn, rn, k + 1);
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      ci[x] = cn[x];
+      rj[x] = rn[x];
+    }
+  };
+  publish(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+  __syncthreads();
+  fetch(ci, rj, 0);
+  record(ci, rj, 0);
+  // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
+  // +infinity and improve nothing
+#pragma unroll 1
+  for (int k8 = 0; k8 < bb; k8 += 8) {
+    step(k8 + 0, std::integral_constant<int, 0>{});
+    step(k8 + 1, std::integral_constant<int, 1>{});
+    step(k8 + 2, std::integral_constant<int, 2>{});
+    step(k8 + 3, std::integral_constant<int, 3>{});
+    step(k8 + 4, std::integral_constant<int, 4>{});
+    step(k8 + 5, std::integral_constant<int, 5>{});
+    step(k8 + 6, std::integral_constant<int, 6>{});
+    step(k8 + 7, std::integral_constant<int, 7>{});
+  }
+#pragma unroll
+  for (int b = 0; b < 8; ++b)
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const int i = 8 * ti + a, j = 8 * tj + b;
+      if (i < bb && j < bb) d[i + int64_t(j) * ld] = cur[a][b];
+    }
+  return true;
+}
+
+template <typename T>
+__device__ __forceinline__ void fw_close_dist(T *d, int64_t ld, int bb, T *hist) {
+  __shared__ __attribute__((aligned(32))) T colbuf[2][FW_BLOCK];  // d[i][k] for the step that reads this buffer
+  __shared__ __attribute__((aligned(32))) T rowbuf[2][FW_BLOCK];  // d[k][j]
+  if (!fw_close_dist_as<T, false>(d, ld, bb, hist, colbuf, rowbuf)) fw_close_dist_as<T, true>(d, ld, bb, hist, colbuf, rowbuf);
+}
+
+// The predecessors of a diagonal block whose distances fw_close_dist has closed: workgroup b of 64 (256 threads)
+// takes rows 64 (b & 1) .. + 63 and columns 4 (b >> 1) .. + 3, one element per thread, and runs the literal scan
+// over the recorded columns and rows.  Only predecessors are written: the distances are those already there.
+template <typename T>
+__device__ __forceinline__ void fw_parents_block(const T *hist, int32_t *parent, int64_t ldp, int bb, int k_base, int b) {
+  const int row = (b & 1) * 64 + (threadIdx.x & 63);
+  const int col = __builtin_amdgcn_readfirstlane((b >> 1) * 4 + (threadIdx.x >> 6));
+  if (row >= bb || col >= bb) return;
+  const T *hc = hist + row, *hr = hist + FW_BLOCK * FW_BLOCK + col;
+  T curr = hist[2 * FW_BLOCK * FW_BLOCK + row + col * FW_BLOCK];
+  int32_t p = -1;
+  int k = 0;
+  for (; k + 16 <= bb; k += 16) {  // sixteen k at a time, their operands requested together
+    T cv[16], rv[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      cv[u] = hc[(k + u) * FW_BLOCK];
+      rv[u] = hr[(k + u) * FW_BLOCK];
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const T prod = cv[u] + rv[u];
+      const bool lower = prod < curr;
+      curr = pick(lower, prod, curr);
+      p = lower ? k + u : p;
+    }
+  }
+  for (; k < bb; ++k) {
+    const T prod = hc[k * FW_BLOCK] + hr[k * FW_BLOCK];
+    const bool lower = prod < curr;
+    curr = pick(lower, prod, curr);
+    p = lower ? k : p;
+  }
+  if (p >= 0) parent[row + int64_t(col) * ldp] = k_base + p;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fw_parents_kernel(const T *hist, int32_t *parent, int64_t ldp, int bb, int k_base) {
+  fw_parents_block<T>(hist, parent, ldp, bb, k_base, blockIdx.x);
+}
+constexpr int FW_PARENT_BLOCKS = (FW_BLOCK / 64) * (FW_BLOCK / 4);
+
+// two independent products in one launch (the block row and the block column of a blocked
+// Floyd-Warshall step, each too small to fill the chip): after the first FW_PARENT_BLOCKS workgroups, which
+// with hist set find the predecessors of the diagonal block at k_base (closed by fw_close_dist in the launch
+// before) and otherwise have nothing to do, the next blocks0 workgroups work on g0, the others on g1
+template <typename T>
+__global__ void __launch_bounds__(256) fwgemm_pair_kernel(FwArgs g0, FwArgs g1, int blocks0, const T *hist, int32_t *hist_parent,
+                                                          int64_t ldp, int hist_bb, int k_base) {
+  int b = blockIdx.x;
+  if (b < FW_PARENT_BLOCKS) {
+    if (hist) fw_parents_block<T>(hist, hist_parent, ldp, hist_bb, k_base, b);
+    return;
+  }
+  b -= FW_PARENT_BLOCKS;
+  if (b < blocks0) {
+    const int gx = (g0.m + 63) / 64;
+    fwgemm_rowcols_block<T>(g0, b % gx, b / gx);
+  } else {
+    const int gx = (g1.m + 63) / 64;
+    fwgemm_rowcols_block<T>(g1, (b - blocks0) % gx, (b - blocks0) / gx);
+  }
+}
+
 // The tile kernel.  Grid (tiles along m, tiles along n); with g.ahead_bb > 0 the grid has one more row,
 // whose first workgroup -- the first one the launch starts -- closes the next block step's diagonal
 // block while the workgroups of the other rows do the product's tiles, all but that block.  The block's
@@ -691,18 +1035,26 @@ __device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *pare
 template <typename T, int TM, int TN, int SN, int BK, bool GUARD, bool HAS_AT>
 __global__ void __launch_bounds__(256, 2) fwgemm_tile_kernel(FwArgs g) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
-  constexpr bool CAN_CLOSE = BM == FW_BLOCK && BN == FW_BLOCK && std::is_same<T, float>::value;
+  constexpr bool CAN_CLOSE = FW_BLOCK % BM == 0 && FW_BLOCK % BN == 0;
   int bx = blockIdx.x, by = blockIdx.y;
   if constexpr (CAN_CLOSE) {
     if (g.ahead_bb > 0) {
       if (by == 0) {
-        if (bx == 0)
-          fw_close_256(static_cast<float *>(g.dist) + g.ahead0 + int64_t(g.ahead0) * g.ldc, g.ldc,
-                       g.parent + g.ahead0 + int64_t(g.ahead0) * g.ldp, g.ldp, g.ahead_bb, g.ahead0);
+        // Which workgroup of the extra row closes the block: workgroups go to the chip's eight dies in turn, by
+        // their number in the launch, and a die starts them in order as places come free.  The closure holds
+        // its place for most of the launch, so it goes to the die that has the least to do: with a number of
+        // tile columns that is a multiple of eight, the tiles of the skipped rows -- which return at once --
+        // all have numbers that are bx modulo eight.  (On any other die the last tile waits for the
+        // closure's place and the launch ends 15 us later.)
+        const int closer = (gridDim.x % 8 == 0 && g.skip_r1 > g.skip_r0) ? (g.skip_r0 / BM) % 8 : 0;
+        if (bx == closer)
+          fw_close_dist<T>(static_cast<T *>(g.dist) + g.ahead0 + int64_t(g.ahead0) * g.ldc, g.ldc, g.ahead_bb,
+                           static_cast<T *>(g.hist));
         return;
       }
       by -= 1;
-      if (by * BN == g.ahead0 && bx * BM == g.ahead0) return;
+      const int r0 = bx * BM - g.ahead0, c0 = by * BN - g.ahead0;
+      if (r0 >= 0 && r0 < FW_BLOCK && c0 >= 0 && c0 < FW_BLOCK) return;
     }
   }
   fwgemm_tile_body<T, TM, TN, SN, BK, GUARD, HAS_AT>(g, bx, by);
@@ -810,67 +1162,75 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))
         : "v224", "vcc");
   }
 
-  // ---- improved elements: the first k of the recorded chunk whose sum equals the minimum.  One canonical row i
-  // (one dist column per thread) of the lanes' outputs at a time into a queue in LDS (the panels are done with),
-  // which all 512 threads then work off, one element per thread and turn.
-  constexpr int CAP = 512 * 8;
-  static_assert(sizeof(Tile::Smem) >= 3 * CAP * sizeof(int), "the queue must fit in the panels");
-  __shared__ int q_count;
-  int *q_pos = reinterpret_cast<int *>(&sm.a[0][0]);   // row | column << 8, inside the tile
-  int *q_ch = q_pos + CAP;
-  float *q_want = reinterpret_cast<float *>(q_ch + CAP);
-  const float *At = static_cast<const float *>(g.At);
+  // ---- improved elements: the first k of the recorded chunk whose sum equals the minimum.  As many whole canonical
+  // rows i (one dist column per thread each) of the lanes' outputs as fit go into a queue in LDS (the panels are done
+  // with; one row, at most 512 x 8 elements, always fits), which all 512 threads then work off (lookup_queue).
+  constexpr int CAP = sizeof(Tile::Smem) / 8 / 512 * 512;
+  static_assert(CAP >= 512 * 8, "a row of the lanes' outputs must fit in the panels");
+  // Where an element goes in the queue follows from counts alone, without a shared counter: row by row, inside a
+  // row wave by wave, inside a wave output j by output j, inside an output lane by lane.
+  __shared__ int wave_count[8][8];
+  uint32_t *q_code = reinterpret_cast<uint32_t *>(&sm.a[0][0]);   // row | column << 7 | chunk << 15, inside the tile
+  float *q_want = reinterpret_cast<float *>(q_code + CAP);
   int tx2 = tx, ty2 = ty;
   asm volatile("" : "+v"(tx2), "+v"(ty2));
-#pragma unroll 1
+  auto chunk_of = [&](auto ic, auto jc) -> uint32_t {
+    constexpr int I = decltype(ic)::value, J = decltype(jc)::value;
+    const uint32_t w = __builtin_bit_cast(uint32_t, (float)chunk[I >> 2][(I & 3) * 4 + (J >> 1)]);
+    return (J & 1) ? w >> 16 : w & 0xffffu;
+  };
+  __syncthreads();  // everybody is done with the panels
+  static_for<8>([&](auto ic) {
+    constexpr int I = decltype(ic)::value;
+    int n_improved = 0;  // in this row, over the wave
+    static_for<8>([&](auto jc) { n_improved += __builtin_popcountll(__builtin_amdgcn_ballot_w64(chunk_of(ic, jc) != 0xffffu)); });
+    if (lane == 0) wave_count[wave][I] = n_improved;
+  });
+  __syncthreads();
+  int before_me[8], row_count[8];  // improved elements of the row in the waves before mine / in all waves
+#pragma unroll
   for (int i = 0; i < 8; ++i) {
-    __syncthreads();  // everybody is done with the panels / with the queue of the row before
-    if (tid == 0) q_count = 0;
-    __syncthreads();
+    before_me[i] = row_count[i] = 0;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      // (i is a run-time value here: the registers are read through a select chain over the 8 rows)
-      uint32_t w = 0;
-      float want = 0.f;
-#pragma unroll
-      for (int ii = 0; ii < 8; ++ii)
-        if (ii == i) {
-          w = __builtin_bit_cast(uint32_t, (float)chunk[ii >> 2][(ii & 3) * 4 + (j >> 1)]);
-          want = run[ii >> 1][(ii & 1) * 8 + j];
-        }
-      const uint32_t ch = (j & 1) ? w >> 16 : w & 0xffffu;
-      if (ch != 0xffffu) {
-        const int slot = atomicAdd(&q_count, 1);
-        q_pos[slot] = (64 * (j >> 2) + 4 * tx2 + (j & 3)) | ((32 * i + ty2) << 8);
-        q_ch[slot] = (int)ch;
-        q_want[slot] = want;
-      }
+    for (int w = 0; w < 8; ++w) {
+      const int n = __builtin_amdgcn_readfirstlane(wave_count[w][i]);
+      before_me[i] += w < wave ? n : 0;
+      row_count[i] += n;
     }
-    __syncthreads();
-    const int count = q_count;
-    for (int e = tid; e < count; e += 512) {
-      const int pos = q_pos[e], row = m0 + (pos & 255), col = n0 + (pos >> 8), k0 = q_ch[e] * FWD_CHUNK;
-      const float want = q_want[e];
-      const V4 *ap = reinterpret_cast<const V4 *>(At + k0 + int64_t(row) * g.ldat);
-      const V4 *bp = reinterpret_cast<const V4 *>(B + k0 + int64_t(col) * g.ldb);
-      V4 pa[FWD_CHUNK / 4], pb[FWD_CHUNK / 4];
+  }
+  for (int i0 = 0; i0 < 8;) {  // (the same for every thread)
+    int total = 0, i1 = i0;
 #pragma unroll
-      for (int q = 0; q < FWD_CHUNK / 4; ++q) {
-        pa[q] = ap[q];
-        pb[q] = bp[q];
-      }
-      float value = want;
-      int first = 0;
-#pragma unroll
-      for (int kk = FWD_CHUNK - 1; kk >= 0; --kk) {
-        const float prod = pa[kk >> 2][kk & 3] + pb[kk >> 2][kk & 3];
-        const bool hit = prod == want;
-        first = hit ? kk : first;
-        value = pick(hit, prod, value);
-      }
-      dist[row + int64_t(col) * g.ldc] = value;
-      g.parent[row + int64_t(col) * g.ldp] = g.k_base + k0 + first;
+    for (int i = 0; i < 8; ++i) {  // as many whole rows from i0 on as fit
+      if (i < i0 || i != i1) continue;
+      if (i > i0 && total + row_count[i] > CAP) continue;
+      total += row_count[i];
+      i1 = i + 1;
     }
+    if (total > 0) {
+      int base = 0;  // of the row in the queue
+      static_for<8>([&](auto ic) {
+        constexpr int I = decltype(ic)::value;
+        if (I < i0 || I >= i1) return;
+        int slot0 = base + before_me[I];  // of my wave's next output of this row
+        static_for<8>([&](auto jc) {
+          constexpr int J = decltype(jc)::value;
+          const uint32_t ch = chunk_of(ic, jc);
+          const unsigned long long improved = __builtin_amdgcn_ballot_w64(ch != 0xffffu);
+          if (ch != 0xffffu) {
+            const int slot = slot0 + __builtin_amdgcn_mbcnt_hi(uint32_t(improved >> 32), __builtin_amdgcn_mbcnt_lo(uint32_t(improved), 0u));
+            q_code[slot] = uint32_t(64 * (J >> 2) + 4 * tx2 + (J & 3)) | uint32_t(32 * I + ty2) << 7 | ch << 15;
+            q_want[slot] = run[I >> 1][(I & 1) * 8 + J];
+          }
+          slot0 += __builtin_popcountll(improved);
+        });
+        base += row_count[I];
+      });
+      __syncthreads();
+      lookup_queue<float, 512, FWD_CHUNK, true, 7, 8>(g, q_code, q_want, total, tid, m0, n0);
+      __syncthreads();  // the queue is free again
+    }
+    i0 = i1;
   }
 }
 
@@ -890,11 +1250,12 @@ bool fwgemm_direct_ok(const FwArgs &g) {
 template <typename T, int TM, int TN, int SN, int BK>
 hipError_t launch_tile(const FwArgs &g, hipStream_t stream) {
   constexpr int BM = 16 * TM, BN = 16 * TN;
-  const bool whole = g.m % BM == 0 && g.n % BN == 0 && g.k % BK == 0;
+  // (the unguarded form queues improved elements with their chunk of BK k-values in 18 bits)
+  const bool whole = g.m % BM == 0 && g.n % BN == 0 && g.k % BK == 0 && g.k < (1 << 22);
   const size_t vec = 4 * sizeof(T);
   const bool aligned = reinterpret_cast<uintptr_t>(g.A) % vec == 0 && reinterpret_cast<uintptr_t>(g.B) % vec == 0 &&
                        g.lda % 4 == 0 && g.ldb % 4 == 0;
-  if (g.ahead_bb > 0 && (BM != FW_BLOCK || BN != FW_BLOCK)) return hipErrorInvalidValue;
+  if (g.ahead_bb > 0 && (FW_BLOCK % BM || FW_BLOCK % BN)) return hipErrorInvalidValue;
   dim3 grid((g.m + BM - 1) / BM, (g.n + BN - 1) / BN + (g.ahead_bb > 0 ? 1 : 0));
   if (g.At) {
     const bool at_aligned = reinterpret_cast<uintptr_t>(g.At) % vec == 0 && g.ldat % 4 == 0;
@@ -1079,6 +1440,7 @@ struct FwExtra {
   // blocked Floyd-Warshall: let the launch also close the diagonal block that starts at ahead0 (ahead_bb rows),
   // which the product then leaves alone.  Only the tile kernel can; *closed_ahead says whether this launch did.
   int ahead0 = 0, ahead_bb = 0;
+  void *hist = nullptr;
   bool *closed_ahead = nullptr;
 };
 // one-thread-per-element kernel or tiles: a launch of a few workgroups is better spread over one thread per
@@ -1095,12 +1457,13 @@ int fwgemm_run(int dtype, int m, int n, int k, const void *A, int64_t lda, const
   const int st = check(dtype, m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, kernel);
   if (st != CUASR_AMD_SUCCESS || m == 0 || n == 0 || k == 0) return st;
   FwArgs g{m, n, k, A, lda, B, ldb, dist, ldc, parent, ldp, x.At, x.ldat, x.k_base,
-           x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1, nullptr, 0, 0, 0};
+           x.skip_r0, x.skip_r1, x.skip_c0, x.skip_c1, nullptr, 0, 0, 0, nullptr};
   hipStream_t s = static_cast<hipStream_t>(stream);
   const bool naive = takes_naive_kernel(m, n, kernel);
-  if (!naive && x.ahead_bb > 0 && dtype == CUASR_AMD_F32) {  // (the 8-byte tile is half a diagonal block)
+  if (!naive && x.ahead_bb > 0 && x.hist) {
     g.ahead0 = x.ahead0;
     g.ahead_bb = x.ahead_bb;
+    g.hist = x.hist;
   }
   if (x.closed_ahead) *x.closed_ahead = g.ahead_bb > 0;
   hipError_t e;
@@ -1158,7 +1521,9 @@ extern "C" int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld,
 extern "C" size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n) {
   if (n <= 0 || (dtype != CUASR_AMD_F32 && dtype != CUASR_AMD_F64)) return 0;
   const size_t nn = (size_t(n) + 3) & ~size_t(3);
-  return 3 * size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * FW_BLOCK * nn;  // block row, block column, transposed block column
+  // block row, block column, transposed block column; then what closing a diagonal block records for its
+  // predecessors (fw_close_dist)
+  return 3 * size_t(dtype == CUASR_AMD_F64 ? 8 : 4) * FW_BLOCK * (nn + FW_BLOCK);
 }
 
 extern "C" int cuasr_amd_apsp_blocked(int dtype, int n, void *dist, int64_t ld, int32_t *parent, int64_t ldp,
@@ -1184,12 +1549,16 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
   char *R = static_cast<char *>(workspace);             // block row,    FW_BLOCK x n,  leading dimension FW_BLOCK
   char *C = R + es * FW_BLOCK * size_t(nn);             // block column, n x FW_BLOCK,  leading dimension nn
   char *Ct = C + es * FW_BLOCK * size_t(nn);            // updated block column with k contiguous, leading dimension FW_BLOCK
-  bool closed = false;  // this step's diagonal block was closed during the step before, beside its big product
+  char *H = Ct + es * FW_BLOCK * size_t(nn);            // columns, rows and first state of the diagonal block being closed
+  // this step's diagonal block had its distances closed during the step before, beside that step's big product;
+  // its predecessors are still to be found from what that closure recorded in H
+  bool closed = false;
   for (int k0 = 0; k0 < n; k0 += FW_BLOCK) {
     const int bb = n - k0 < FW_BLOCK ? n - k0 : FW_BLOCK;
     char *Dkk = D + es * (size_t(k0) + size_t(k0) * size_t(ld));
     int32_t *Pkk = parent + size_t(k0) + size_t(k0) * size_t(ldp);
     // 1. the diagonal block, closed by one workgroup
+    const bool parents_due = closed;
     if (!closed) {
       if (f64)
         launch_kernel(fw_diagonal_kernel<double>, dim3(1), dim3(1024), 0, s, reinterpret_cast<double *>(Dkk), ld, Pkk, ldp, bb, k0);
@@ -1230,10 +1599,20 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
       const FwArgs g1{n, bb, bb, C, nn, C + es * size_t(k0), nn, Dcol, ld, parent + size_t(k0) * size_t(ldp), ldp,
                       nullptr, 0, k0, k0, k0 + bb, 0, 0, Ct, FW_BLOCK, 0, 0};
       const int blocks0 = ((bb + 63) / 64) * ((n + 15) / 16), blocks1 = ((n + 63) / 64) * ((bb + 15) / 16);
-      if (f64) launch_kernel(fwgemm_pair_kernel<double>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
-      else launch_kernel(fwgemm_pair_kernel<float>, dim3(blocks0 + blocks1), dim3(256), 0, s, g0, g1, blocks0);
+      const dim3 grid(FW_PARENT_BLOCKS + blocks0 + blocks1);
+      if (f64)
+        launch_kernel(fwgemm_pair_kernel<double>, grid, dim3(256), 0, s, g0, g1, blocks0,
+                      reinterpret_cast<const double *>(parents_due ? H : nullptr), Pkk, ldp, bb, k0);
+      else
+        launch_kernel(fwgemm_pair_kernel<float>, grid, dim3(256), 0, s, g0, g1, blocks0,
+                      reinterpret_cast<const float *>(parents_due ? H : nullptr), Pkk, ldp, bb, k0);
       if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
     } else {
+      if (parents_due) {
+        if (f64) launch_kernel(fw_parents_kernel<double>, dim3(FW_PARENT_BLOCKS), dim3(256), 0, s, reinterpret_cast<const double *>(H), Pkk, ldp, bb, k0);
+        else launch_kernel(fw_parents_kernel<float>, dim3(FW_PARENT_BLOCKS), dim3(256), 0, s, reinterpret_cast<const float *>(H), Pkk, ldp, bb, k0);
+        if (take_launch_status() != hipSuccess) return CUASR_AMD_ERROR_INTERNAL;
+      }
       FwExtra xr = x, xc = x;
       xr.skip_c0 = xc.skip_r0 = k0;
       xr.skip_c1 = xc.skip_r1 = k0 + bb;
@@ -1254,13 +1633,14 @@ extern "C" int cuasr_amd_apsp_blocked_panels(int dtype, int n, void *dist, int64
     if (k0 + bb < n) {
       x.ahead0 = k0 + bb;
       x.ahead_bb = n - x.ahead0 < FW_BLOCK ? n - x.ahead0 : FW_BLOCK;
+      x.hist = H;
       x.closed_ahead = &closed;
     }
     x.At = Ct;
     x.ldat = FW_BLOCK;
     x.skip_r0 = x.skip_c0 = k0;
     x.skip_r1 = x.skip_c1 = k0 + bb;
-    if (x.ahead_bb > 0 && !f64 && !takes_naive_kernel(n, n, CUASR_AMD_KERNEL_AUTO)) {
+    if (x.ahead_bb > 0 && !takes_naive_kernel(n, n, CUASR_AMD_KERNEL_AUTO)) {
       // this step's update of that block, by a launch of its own (64 workgroups, a few microseconds): the
       // closure can then start with the big product instead of after one of its tiles
       const int a0 = x.ahead0, abb = x.ahead_bb;

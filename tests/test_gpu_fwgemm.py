@@ -211,6 +211,34 @@ def test_apsp_blocked_floyd_warshall(oracle, n, pad, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_apsp_blocked_keeps_the_sign_of_a_zero(oracle, dtype):
+    """Edges of weight +0 and -0: a sum of two -0 is -0, and the strict comparison keeps whichever zero was
+    there first, where a hardware minimum would prefer -0.  The diagonal blocks that hold a -0 are closed by
+    comparison and select; dist (bit for bit, so with its signs) and parent equal the oracle's."""
+    import torch
+    n = 1475
+    rng = np.random.default_rng(4242)
+    W = np.where(rng.random((n, n)) < 0.004, rng.integers(1, 9, (n, n)), np.inf).astype(dtype)
+    zeros = rng.random((n, n)) < 0.004
+    W[zeros] = rng.choice(np.array([0.0, -0.0], dtype), int(zeros.sum()))
+    # every diagonal block but the fourth has a -0 of its own
+    W[128 * 3:128 * 4, 128 * 3:128 * 4][W[128 * 3:128 * 4, 128 * 3:128 * 4] == 0] = 0.0
+    np.fill_diagonal(W, 0)
+    assert np.signbit(W[W == 0]).any()
+    dD = to_device(np.asfortranarray(W))
+    dP = torch.full((n, n), -1, dtype=torch.int32, device="cuda").t()
+    name = "f32" if dtype == np.float32 else "f64"
+    ws = torch.empty(cuasr_amd.apsp_blocked_workspace_bytes(n, name), dtype=torch.uint8, device="cuda")
+    cuasr_amd.apsp_blocked(dD, dP, ws)
+    want_d, want_p = np.asfortranarray(W), np.full((n, n), -1, np.int32, order="F")
+    oracle.apsp_blocked(want_d, want_p, 128)
+    dist = dD.cpu().numpy()
+    assert np.signbit(want_d[want_d == 0]).any() and not np.signbit(want_d[want_d == 0]).all()
+    assert_same_bits(np.ascontiguousarray(dist), np.ascontiguousarray(want_d), "dist")
+    assert np.array_equal(dP.cpu().numpy(), want_p)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("n,pad", [(100, 0), (384, 0), (513, 1), (700, 4), (1475, 1)])
 def test_apsp_blocked_with_tiled_panels(oracle, n, pad, dtype):
     """The way a block step updates its block row and column from n = 16257 on (two launches of the tiled
