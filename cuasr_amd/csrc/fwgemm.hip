@@ -572,173 +572,6 @@ __device__ __forceinline__ void fwgemm_tile_body(const FwArgs &g, const int bloc
 
 constexpr int FW_BLOCK = 128;  // vertices per block step of the blocked Floyd-Warshall
 
-// Floyd-Warshall inside one diagonal block of bb <= FW_BLOCK rows, by one workgroup of 256 threads that
-// holds the block in registers, an 8 x 8 patch per thread: the same element-by-element sequence as
-// fw_diagonal_kernel below (k ascending, d[i][j] > d[i][k] + d[k][j] => d[i][j] = the sum, parent =
-// k_base + k), for a caller that has only 256 threads: the tile kernel's first workgroup.
-//
-// Four instructions per element and step (add, compare, two selects), 64 elements per thread: a step is
-// 256 vector instructions per wave, which one wave per SIMD issues in about 1100 cycles -- and everything
-// else a step needs (publishing row and column k + 1 to LDS, the barrier, reading them back) would add
-// its full latency to that, because the steps depend on each other.  So a step is done in two parts:
-//   A. the patch's row and column (k + 1) & 7 -- every thread's, since which thread owns row / column
-//      k + 1 is only known at run time -- then the owners publish them, then the barrier;
-//   B. the reads of row / column k + 1 are issued, and the other 49 elements of step k are done while
-//      they are on their way.
-// relax4 / relax3: compare (strictly: -0 must not replace +0), select distance and parent, for four
-// (three) elements at a time.  Written out as instructions for two reasons.  Nothing reads the parents
-// before the end, and left alone the optimiser postpones their selects over a whole unrolled round of
-// steps and keeps 512 comparison results instead, which do not fit the scalar registers.  And a select
-// that directly follows its comparison waits for the mask: with three other instructions in between a
-// block took 100 us instead of 131.
-__device__ __forceinline__ void relax4(float &x0, float &x1, float &x2, float &x3, int32_t &p0, int32_t &p1, int32_t &p2,
-                                       int32_t &p3, float c0, float c1, float c2, float c3, int32_t kv) {
-  unsigned long long m0, m1, m2, m3;
-  asm volatile(
-      "v_cmp_lt_f32 %[m0], %[c0], %[x0]\n\tv_cmp_lt_f32 %[m1], %[c1], %[x1]\n\t"
-      "v_cmp_lt_f32 %[m2], %[c2], %[x2]\n\tv_cmp_lt_f32 %[m3], %[c3], %[x3]\n\t"
-      "v_cndmask_b32 %[x0], %[x0], %[c0], %[m0]\n\tv_cndmask_b32 %[x1], %[x1], %[c1], %[m1]\n\t"
-      "v_cndmask_b32 %[x2], %[x2], %[c2], %[m2]\n\tv_cndmask_b32 %[x3], %[x3], %[c3], %[m3]\n\t"
-      "v_cndmask_b32 %[p0], %[p0], %[kv], %[m0]\n\tv_cndmask_b32 %[p1], %[p1], %[kv], %[m1]\n\t"
-      "v_cndmask_b32 %[p2], %[p2], %[kv], %[m2]\n\tv_cndmask_b32 %[p3], %[p3], %[kv], %[m3]"
-      : [x0] "+v"(x0), [x1] "+v"(x1), [x2] "+v"(x2), [x3] "+v"(x3), [p0] "+v"(p0), [p1] "+v"(p1), [p2] "+v"(p2),
-        [p3] "+v"(p3), [m0] "=&s"(m0), [m1] "=&s"(m1), [m2] "=&s"(m2), [m3] "=&s"(m3)
-      : [c0] "v"(c0), [c1] "v"(c1), [c2] "v"(c2), [c3] "v"(c3), [kv] "v"(kv));
-}
-__device__ __forceinline__ void relax3(float &x0, float &x1, float &x2, int32_t &p0, int32_t &p1, int32_t &p2, float c0,
-                                       float c1, float c2, int32_t kv) {
-  unsigned long long m0, m1, m2;
-  asm volatile(
-      "v_cmp_lt_f32 %[m0], %[c0], %[x0]\n\tv_cmp_lt_f32 %[m1], %[c1], %[x1]\n\tv_cmp_lt_f32 %[m2], %[c2], %[x2]\n\t"
-      "v_cndmask_b32 %[x0], %[x0], %[c0], %[m0]\n\tv_cndmask_b32 %[x1], %[x1], %[c1], %[m1]\n\t"
-      "v_cndmask_b32 %[x2], %[x2], %[c2], %[m2]\n\t"
-      "v_cndmask_b32 %[p0], %[p0], %[kv], %[m0]\n\tv_cndmask_b32 %[p1], %[p1], %[kv], %[m1]\n\t"
-      "v_cndmask_b32 %[p2], %[p2], %[kv], %[m2]"
-      : [x0] "+v"(x0), [x1] "+v"(x1), [x2] "+v"(x2), [p0] "+v"(p0), [p1] "+v"(p1), [p2] "+v"(p2), [m0] "=&s"(m0),
-        [m1] "=&s"(m1), [m2] "=&s"(m2)
-      : [c0] "v"(c0), [c1] "v"(c1), [c2] "v"(c2), [kv] "v"(kv));
-}
-
-__device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *parent, int64_t ldp, int bb, int k_base) {
-  typedef vec4_of<float>::type V4;
-  __shared__ __attribute__((aligned(32))) float colbuf[2][FW_BLOCK];  // d[i][k] for the step that reads this buffer
-  __shared__ __attribute__((aligned(32))) float rowbuf[2][FW_BLOCK];  // d[k][j]
-  const int tid = threadIdx.x & 255, ti = tid & 15, tj = tid >> 4;  // rows 8 ti .. 8 ti + 7, columns 8 tj .. 8 tj + 7
-  const float inf = std::numeric_limits<float>::infinity();
-  float cur[8][8];  // [row in patch][column in patch]
-  int32_t par[8][8];
-  // (loads from clamped addresses, then a select: a branch per element would keep 64 lane masks alive)
-#pragma unroll
-  for (int b = 0; b < 8; ++b)
-#pragma unroll
-    for (int a = 0; a < 8; ++a) {
-      const int i = 8 * ti + a, j = 8 * tj + b;
-      const float v = d[min(i, bb - 1) + int64_t(min(j, bb - 1)) * ld];
-      cur[a][b] = (i < bb && j < bb) ? v : inf;
-      par[a][b] = -1;
-    }
-  // S = kn & 7, the row / column of the patch that is published, is a compile-time constant (the step
-  // loop is unrolled by eight): indexed by a run-time value the patch would live in scratch memory
-  auto publish = [&](int kn, int buf, auto sc) {
-    constexpr int S = decltype(sc)::value;
-    if ((kn >> 3) == ti) {  // my patch holds row kn
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        V4 v;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) v[b] = cur[S][4 * h + b];
-        *reinterpret_cast<V4 *>(&rowbuf[buf][8 * tj + 4 * h]) = v;
-      }
-    }
-    if ((kn >> 3) == tj) {  // my patch holds column kn
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        V4 v;
-#pragma unroll
-        for (int a = 0; a < 4; ++a) v[a] = cur[4 * h + a][S];
-        *reinterpret_cast<V4 *>(&colbuf[buf][8 * ti + 4 * h]) = v;
-      }
-    }
-  };
-  float ci[8], rj[8];  // column k at my rows, row k at my columns, for the step in hand
-  auto fetch = [&](float (&c)[8], float (&r)[8], int buf) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const V4 cv = *reinterpret_cast<const V4 *>(&colbuf[buf][8 * ti + 4 * h]);
-      const V4 rv = *reinterpret_cast<const V4 *>(&rowbuf[buf][8 * tj + 4 * h]);
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        c[4 * h + x] = cv[x];
-        r[4 * h + x] = rv[x];
-      }
-    }
-  };
-  auto step = [&](int k, auto uc) {
-    constexpr int U = decltype(uc)::value;  // k & 7
-    constexpr int N = (U + 1) & 7;          // the row and the column of the patch that step k + 1 may need
-    constexpr int O[7] = {N > 0 ? 0 : 1, N > 1 ? 1 : 2, N > 2 ? 2 : 3, N > 3 ? 3 : 4, N > 4 ? 4 : 5, N > 5 ? 5 : 6, N > 6 ? 6 : 7};
-    const int buf = U & 1;
-    int32_t kv = k_base + k;
-    asm volatile("" : "+v"(kv));  // one register for the step, not a constant folded into every select
-    // A. row N, then column N of the other rows
-    relax4(cur[N][0], cur[N][1], cur[N][2], cur[N][3], par[N][0], par[N][1], par[N][2], par[N][3], ci[N] + rj[0],
-           ci[N] + rj[1], ci[N] + rj[2], ci[N] + rj[3], kv);
-    relax4(cur[N][4], cur[N][5], cur[N][6], cur[N][7], par[N][4], par[N][5], par[N][6], par[N][7], ci[N] + rj[4],
-           ci[N] + rj[5], ci[N] + rj[6], ci[N] + rj[7], kv);
-    relax4(cur[O[0]][N], cur[O[1]][N], cur[O[2]][N], cur[O[3]][N], par[O[0]][N], par[O[1]][N], par[O[2]][N], par[O[3]][N],
-           ci[O[0]] + rj[N], ci[O[1]] + rj[N], ci[O[2]] + rj[N], ci[O[3]] + rj[N], kv);
-    relax3(cur[O[4]][N], cur[O[5]][N], cur[O[6]][N], par[O[4]][N], par[O[5]][N], par[O[6]][N], ci[O[4]] + rj[N],
-           ci[O[5]] + rj[N], ci[O[6]] + rj[N], kv);
-    // into the other pair of buffers: nobody reads it before the barrier, and nobody is still reading it
-    // from the step before (everybody has passed that step's barrier, and waited for its reads in part A)
-    publish(k + 1, buf ^ 1, std::integral_constant<int, N>{});
-    __syncthreads();
-    float cn[8], rn[8];
-    fetch(cn, rn, buf ^ 1);
-    // B. the rest of step k, under the latency of those reads
-#pragma unroll
-    for (int i = 0; i < 7; ++i) {
-      const int a = O[i];
-      relax4(cur[a][O[0]], cur[a][O[1]], cur[a][O[2]], cur[a][O[3]], par[a][O[0]], par[a][O[1]], par[a][O[2]], par[a][O[3]],
-             ci[a] + rj[O[0]], ci[a] + rj[O[1]], ci[a] + rj[O[2]], ci[a] + rj[O[3]], kv);
-      relax3(cur[a][O[4]], cur[a][O[5]], cur[a][O[6]], par[a][O[4]], par[a][O[5]], par[a][O[6]], ci[a] + rj[O[4]],
-             ci[a] + rj[O[5]], ci[a] + rj[O[6]], kv);
-    }
-#pragma unroll
-    for (int x = 0; x < 8; ++x) {
-      ci[x] = cn[x];
-      rj[x] = rn[x];
-    }
-  };
-  publish(0, 0, std::integral_constant<int, 0>{});
-  __syncthreads();
-  fetch(ci, rj, 0);
-  // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
-  // +infinity and improve nothing
-#pragma unroll 1
-  for (int k8 = 0; k8 < bb; k8 += 8) {
-    step(k8 + 0, std::integral_constant<int, 0>{});
-    step(k8 + 1, std::integral_constant<int, 1>{});
-    step(k8 + 2, std::integral_constant<int, 2>{});
-    step(k8 + 3, std::integral_constant<int, 3>{});
-    step(k8 + 4, std::integral_constant<int, 4>{});
-    step(k8 + 5, std::integral_constant<int, 5>{});
-    step(k8 + 6, std::integral_constant<int, 6>{});
-    step(k8 + 7, std::integral_constant<int, 7>{});
-  }
-  // (elements of the padding never improve: their parent is still -1)
-#pragma unroll
-  for (int b = 0; b < 8; ++b)
-#pragma unroll
-    for (int a = 0; a < 8; ++a) {
-      const int i = 8 * ti + a, j = 8 * tj + b;
-      if (par[a][b] >= 0) {
-        d[i + int64_t(j) * ld] = cur[a][b];
-        parent[i + int64_t(j) * ldp] = par[a][b];
-      }
-    }
-}
-
 // ---- closing a diagonal block in two parts: distances first, predecessors afterwards
 //
 // Step k of the closure lowers d[i][j] to cand_k = d[i][k] + d[k][j] (row k and column k as they are before the
@@ -762,14 +595,29 @@ __device__ __forceinline__ void fw_close_256(float *d, int64_t ld, int32_t *pare
 // one takes the same steps with a comparison and a select (EXACT).
 //
 // hist: FW_BLOCK x FW_BLOCK elements each of  col[k * FW_BLOCK + i] = d[i][k] before step k,
-// row[k * FW_BLOCK + j] = d[k][j] before step k,  init[i + j * FW_BLOCK] = d[i][j] before the closure.
+// row[k * FW_BLOCK + j] = d[k][j] before step k,  init[(8 * (i % 8) + j % 8) * 256 + i / 8 + 16 * (j / 8)] = d[i][j] before
+// the closure.
 // (returns false, with nothing done, when the block holds a -0 and EXACT is not set)
+// (A function of its own, not inlined: as part of a kernel that also holds the other form and a product's tile, the
+// compiler's register allocation moves parts of the patch to scratch memory inside the step loop, where any wait for
+// memory also waits for the stores to hist.  Alone, either form fits the registers.)
 template <typename T, bool EXACT>
-__device__ __forceinline__ bool fw_close_dist_as(T *d, int64_t ld, int bb, T *hist, T (*colbuf)[FW_BLOCK], T (*rowbuf)[FW_BLOCK]) {
+__device__ __attribute__((noinline)) bool fw_close_dist_as(T *d_anywhere, int64_t ld, int bb, T *hist_anywhere,
+                                                           __attribute__((address_space(3))) T *colbuf,
+                                                           __attribute__((address_space(3))) T *rowbuf) {
   typedef typename vec4_of<T>::type V4;
+  typedef __attribute__((address_space(3))) T LT;
+  typedef __attribute__((address_space(3))) V4 LV4;
+  // (both are device memory, which a function that is not a kernel has to be told: a store to "memory of some
+  // kind" counts as an LDS access as well, and the waits for LDS before each barrier would wait for it)
+  typedef __attribute__((address_space(1))) T GT;
+  typedef __attribute__((address_space(1))) V4 GV4;
+  GT *const d = (GT *)d_anywhere, *const hist = (GT *)hist_anywhere;
+  // colbuf, rowbuf: lines of FW_BLOCK elements in LDS for columns k (and k + 1) as the steps read them, and for
+  // the rows: two sets of one line for 8-byte elements (lines 0 and 2), four sets of two lines for 4-byte elements
   const int tid = threadIdx.x & 255, ti = tid & 15, tj = tid >> 4;  // rows 8 ti .. 8 ti + 7, columns 8 tj .. 8 tj + 7
   const T inf = std::numeric_limits<T>::infinity();
-  T *hist_col = hist, *hist_row = hist + FW_BLOCK * FW_BLOCK, *init = hist + 2 * FW_BLOCK * FW_BLOCK;
+  GT *hist_col = hist, *hist_row = hist + FW_BLOCK * FW_BLOCK, *init = hist + 2 * FW_BLOCK * FW_BLOCK;
   T cur[8][8];  // [row in patch][column in patch]
   // loads from clamped addresses, then a select (a branch per element would keep 64 lane masks alive); a column's
   // addresses differ by the clamped row, so that the 64 loads in flight do not need 64 addresses in registers
@@ -779,7 +627,7 @@ __device__ __forceinline__ bool fw_close_dist_as(T *d, int64_t ld, int bb, T *hi
 #pragma unroll
   for (int b = 0; b < 8; ++b) {
     const int j = 8 * tj + b;
-    const T *column = d + int64_t(min(j, bb - 1)) * ld;
+    const GT *column = d + int64_t(min(j, bb - 1)) * ld;
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
       const T v = column[ic[a]];
@@ -796,16 +644,12 @@ __device__ __forceinline__ bool fw_close_dist_as(T *d, int64_t ld, int bb, T *hi
       for (int a = 0; a < 8; ++a) negative_zero |= cur[a][b] == T(0) && __builtin_signbit(cur[a][b]);
     if (__syncthreads_or(negative_zero)) return false;
   }
+  // (element by element, a thread's elements 256 apart: written four at a time, the patch's registers would have
+  // to be adjacent in fours, and the compiler moves parts of the patch to scratch memory over that in the loop below)
 #pragma unroll
-  for (int b = 0; b < 8; ++b) {
+  for (int b = 0; b < 8; ++b)
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      V4 v;
-#pragma unroll
-      for (int a = 0; a < 4; ++a) v[a] = cur[4 * h + a][b];
-      *reinterpret_cast<V4 *>(&init[8 * ti + 4 * h + (8 * tj + b) * FW_BLOCK]) = v;
-    }
-  }
+    for (int a = 0; a < 8; ++a) init[(8 * a + b) * 256 + tid] = cur[a][b];
   // (the minimum as an instruction: from the builtin the compiler first "quiets" an operand whose origin it
   // does not know, such as anything that comes round the loop, an instruction more per element)
   auto relax = [](T &x, const T cand) {
@@ -813,187 +657,310 @@ __device__ __forceinline__ bool fw_close_dist_as(T *d, int64_t ld, int bb, T *hi
     else if constexpr (sizeof(T) == 4) asm("v_min_f32 %0, %0, %1" : "+v"(x) : "v"(cand));
     else asm("v_min_f64 %0, %0, %1" : "+v"(x) : "v"(cand));
   };
-  // S = kn & 7, the row / column of the patch that is published, is a compile-time constant (the step
-  // loop is unrolled by eight): indexed by a run-time value the patch would live in scratch memory.
-  // Two elements per instruction, each from a register of its own: as 16-byte stores the compiler wants every
-  // row of the patch AND every column of it in four adjacent registers, cannot have both, and moves parts of the
-  // patch to scratch memory in the attempt.
-  const unsigned row_lds = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&rowbuf[0][8 * tj];
-  const unsigned col_lds = (unsigned)(size_t)(__attribute__((address_space(3))) T *)&colbuf[0][8 * ti];
+  // two steps' candidates at once, in the steps' order
+  auto relax2 = [&](T &x, const T first, const T second) {
+    if constexpr (!EXACT && sizeof(T) == 4) {
+      asm("v_min3_f32 %0, %0, %1, %2" : "+v"(x) : "v"(first), "v"(second));
+    } else {
+      relax(x, first);
+      relax(x, second);
+    }
+  };
+  // Rows and columns go to LDS two elements per instruction, each from a register of its own: as 16-byte stores the
+  // compiler wants every row of the patch AND every column of it in four adjacent registers, cannot have both, and
+  // moves parts of the patch to scratch memory in the attempt.  colbuf / rowbuf: [2 * buffer + which of the pair]
+  auto lds = [](const LT *q) { return (unsigned)(size_t)q; };
   auto write2 = [](unsigned addr, const T x, const T y, auto at) {
     constexpr int AT = decltype(at)::value;  // in elements
     if constexpr (sizeof(T) == 4) asm volatile("ds_write2_b32 %0, %1, %2 offset0:%3 offset1:%4" ::"v"(addr), "v"(x), "v"(y), "n"(AT), "n"(AT + 1) : "memory");
     else asm volatile("ds_write2_b64 %0, %1, %2 offset0:%3 offset1:%4" ::"v"(addr), "v"(x), "v"(y), "n"(AT), "n"(AT + 1) : "memory");
   };
-  auto publish = [&](int kn, auto bufc, auto sc) {
-    constexpr int S = decltype(sc)::value, BUF = decltype(bufc)::value * FW_BLOCK;
-    if ((kn >> 3) == ti) {  // my patch holds row kn
-      write2(row_lds, cur[S][0], cur[S][1], std::integral_constant<int, BUF + 0>{});
-      write2(row_lds, cur[S][2], cur[S][3], std::integral_constant<int, BUF + 2>{});
-      write2(row_lds, cur[S][4], cur[S][5], std::integral_constant<int, BUF + 4>{});
-      write2(row_lds, cur[S][6], cur[S][7], std::integral_constant<int, BUF + 6>{});
-    }
-    if ((kn >> 3) == tj) {  // my patch holds column kn
-      write2(col_lds, cur[0][S], cur[1][S], std::integral_constant<int, BUF + 0>{});
-      write2(col_lds, cur[2][S], cur[3][S], std::integral_constant<int, BUF + 2>{});
-      write2(col_lds, cur[4][S], cur[5][S], std::integral_constant<int, BUF + 4>{});
-      write2(col_lds, cur[6][S], cur[7][S], std::integral_constant<int, BUF + 6>{});
-    }
-    // (the barrier that follows is the compiler's, which does not know of the instructions above)
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // row S of the patch to row_at, column S to col_at (S is a compile-time constant, the step loop being unrolled
+  // by eight: indexed by a run-time value the patch would live in scratch memory)
+  auto put_row = [&](unsigned row_at, auto sc, auto at) {
+    constexpr int S = decltype(sc)::value, AT = decltype(at)::value;
+    write2(row_at, cur[S][0], cur[S][1], std::integral_constant<int, AT + 0>{});
+    write2(row_at, cur[S][2], cur[S][3], std::integral_constant<int, AT + 2>{});
+    write2(row_at, cur[S][4], cur[S][5], std::integral_constant<int, AT + 4>{});
+    write2(row_at, cur[S][6], cur[S][7], std::integral_constant<int, AT + 6>{});
   };
-  // what step kn reads goes to hist from the registers of the threads of the first patch row / column, which
-  // together have read all of it
-  auto record = [&](const T (&c)[8], const T (&r)[8], int kn) {
-    if (kn >= FW_BLOCK) return;
-    if (tj == 0) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        V4 v;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] = c[4 * h + x];
-        *reinterpret_cast<V4 *>(&hist_col[kn * FW_BLOCK + 8 * ti + 4 * h]) = v;
-      }
-    }
-    if (ti == 0) {
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        V4 v;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) v[x] = r[4 * h + x];
-        *reinterpret_cast<V4 *>(&hist_row[kn * FW_BLOCK + 8 * tj + 4 * h]) = v;
-      }
-    }
+  auto put_col = [&](unsigned col_at, auto sc, auto at) {
+    constexpr int S = decltype(sc)::value, AT = decltype(at)::value;
+    write2(col_at, cur[0][S], cur[1][S], std::integral_constant<int, AT + 0>{});
+    write2(col_at, cur[2][S], cur[3][S], std::integral_constant<int, AT + 2>{});
+    write2(col_at, cur[4][S], cur[5][S], std::integral_constant<int, AT + 4>{});
+    write2(col_at, cur[6][S], cur[7][S], std::integral_constant<int, AT + 6>{});
   };
-  T ci[8], rj[8];  // column k at my rows, row k at my columns, for the step in hand
-  auto fetch = [&](T (&c)[8], T (&r)[8], int buf) {
+  auto get8 = [&](T (&x)[8], const LT *from) {
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const V4 cv = *reinterpret_cast<const V4 *>(&colbuf[buf][8 * ti + 4 * h]);
-      const V4 rv = *reinterpret_cast<const V4 *>(&rowbuf[buf][8 * tj + 4 * h]);
+      const V4 v = *reinterpret_cast<const LV4 *>(from + 4 * h);
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        c[4 * h + x] = cv[x];
-        r[4 * h + x] = rv[x];
-      }
+      for (int e = 0; e < 4; ++e) x[4 * h + e] = v[e];
     }
   };
-  // A step in two parts, because the steps depend on each other and everything between them (publishing row
-  // and column k + 1, the barrier, reading them back) would otherwise add its full latency to every step:
-  //   A. the patch's row and column (k + 1) & 7 -- every thread's, since which thread owns row / column
-  //      k + 1 is only known at run time -- then the owners publish them, then the barrier;
-  //   B. the reads of row / column k + 1 are issued, and the other 49 elements of step k are done while
-  //      they are on their way.
-  auto step = [&](int k, auto uc) {
-    constexpr int U = decltype(uc)::value;  // k & 7
-    constexpr int N = (U + 1) & 7;          // the row and the column of the patch that step k + 1 may need
-    constexpr int O[7] = {N > 0 ? 0 : 1, N > 1 ? 1 : 2, N > 2 ? 2 : 3, N > 3 ? 3 : 4, N > 4 ? 4 : 5, N > 5 ? 5 : 6, N > 6 ? 6 : 7};
-    const int buf = U & 1;
-    if constexpr (sizeof(T) == 8) {
-      // 8-byte elements: the patch takes half the register file, and a second set of rows and columns on its
-      // way beside the one in use pushes parts of the patch into scratch memory.  One part, then: the whole
-      // step, publish, barrier, read.  (The product beside this closure takes three times as long anyway.)
+  auto put8 = [&](GT *to, const T (&x)[8]) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      V4 v;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = x[4 * h + e];
+      *reinterpret_cast<GV4 *>(to + 4 * h) = v;
+    }
+  };
+
+  if constexpr (sizeof(T) == 8) {
+    // ---- 8-byte elements: one step per barrier, in one part.  The patch takes half the register file, and a
+    // second set of rows and columns on its way beside the one in use pushes parts of the patch into scratch
+    // memory.  (The product beside this closure takes twice as long anyway.)
+    const unsigned row_lds[2] = {lds(rowbuf + (0) * FW_BLOCK + 8 * tj), lds(rowbuf + (2) * FW_BLOCK + 8 * tj)};
+    const unsigned col_lds[2] = {lds(colbuf + (0) * FW_BLOCK + 8 * ti), lds(colbuf + (2) * FW_BLOCK + 8 * ti)};
+    T ci[8], rj[8];  // column k at my rows, row k at my columns, for the step in hand
+    auto publish = [&](int kn, auto bufc, auto sc) {
+      constexpr int BUF = decltype(bufc)::value;
+      if ((kn >> 3) == ti) put_row(row_lds[BUF], sc, std::integral_constant<int, 0>{});  // my patch holds row kn
+      if ((kn >> 3) == tj) put_col(col_lds[BUF], sc, std::integral_constant<int, 0>{});  // my patch holds column kn
+      // (the barrier that follows is the compiler's, which does not know of the instructions above)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    // what step kn reads goes to hist from the registers of the threads of the first patch row / column, which
+    // together have read all of it
+    auto fetch = [&](int buf, int kn) {
+      get8(ci, colbuf + (2 * buf) * FW_BLOCK + 8 * ti);
+      get8(rj, rowbuf + (2 * buf) * FW_BLOCK + 8 * tj);
+      if (kn >= FW_BLOCK) return;
+      if (tj == 0) put8(&hist_col[kn * FW_BLOCK + 8 * ti], ci);
+      if (ti == 0) put8(&hist_row[kn * FW_BLOCK + 8 * tj], rj);
+    };
+    auto step = [&](int k, auto uc) {
+      constexpr int U = decltype(uc)::value;  // k & 7
 #pragma unroll
       for (int a = 0; a < 8; ++a)
 #pragma unroll
         for (int b = 0; b < 8; ++b) relax(cur[a][b], ci[a] + rj[b]);
       __builtin_amdgcn_sched_barrier(0);
-      publish(k + 1, std::integral_constant<int, (U & 1) ^ 1>{}, std::integral_constant<int, N>{});
+      // into the other pair of buffers: nobody reads it before the barrier, and nobody is still reading it
+      // from the step before (everybody has passed that step's barrier, and used what it read before that)
+      publish(k + 1, std::integral_constant<int, (U & 1) ^ 1>{}, std::integral_constant<int, (U + 1) & 7>{});
       __syncthreads();
-      fetch(ci, rj, buf ^ 1);
-      record(ci, rj, k + 1);
+      fetch((U & 1) ^ 1, k + 1);
       __builtin_amdgcn_sched_barrier(0);
-      return;
-    }
-#pragma unroll
-    for (int b = 0; b < 8; ++b) relax(cur[N][b], ci[N] + rj[b]);
-#pragma unroll
-    for (int i = 0; i < 7; ++i) relax(cur[O[i]][N], ci[O[i]] + rj[N]);
-    __builtin_amdgcn_sched_barrier(0);
-    // into the other pair of buffers: nobody reads it before the barrier, and nobody is still reading it
-    // from the step before (everybody has passed that step's barrier, and waited for its reads in part A)
-    publish(k + 1, std::integral_constant<int, (U & 1) ^ 1>{}, std::integral_constant<int, N>{});
+    };
+    publish(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
     __syncthreads();
-    T cn[8], rn[8];
-    fetch(cn, rn, buf ^ 1);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int i = 0; i < 7; ++i)
-#pragma unroll
-      for (int j = 0; j < 7; ++j) relax(cur[O[i]][O[j]], ci[O[i]] + rj[O[j]]);
-    record(cn, rn, k + 1);
-#pragma unroll
-    for (int x = 0; x < 8; ++x) {
-      ci[x] = cn[x];
-      rj[x] = rn[x];
-    }
-  };
-  publish(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-  __syncthreads();
-  fetch(ci, rj, 0);
-  record(ci, rj, 0);
-  // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
-  // +infinity and improve nothing
+    fetch(0, 0);
+    // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
+    // +infinity and improve nothing
 #pragma unroll 1
-  for (int k8 = 0; k8 < bb; k8 += 8) {
-    step(k8 + 0, std::integral_constant<int, 0>{});
-    step(k8 + 1, std::integral_constant<int, 1>{});
-    step(k8 + 2, std::integral_constant<int, 2>{});
-    step(k8 + 3, std::integral_constant<int, 3>{});
-    step(k8 + 4, std::integral_constant<int, 4>{});
-    step(k8 + 5, std::integral_constant<int, 5>{});
-    step(k8 + 6, std::integral_constant<int, 6>{});
-    step(k8 + 7, std::integral_constant<int, 7>{});
+    for (int k8 = 0; k8 < bb; k8 += 8) {
+      step(k8 + 0, std::integral_constant<int, 0>{});
+      step(k8 + 1, std::integral_constant<int, 1>{});
+      step(k8 + 2, std::integral_constant<int, 2>{});
+      step(k8 + 3, std::integral_constant<int, 3>{});
+      step(k8 + 4, std::integral_constant<int, 4>{});
+      step(k8 + 5, std::integral_constant<int, 5>{});
+      step(k8 + 6, std::integral_constant<int, 6>{});
+      step(k8 + 7, std::integral_constant<int, 7>{});
+    }
+  } else {
+    // ---- 4-byte elements: two steps per barrier, in two parts.
+    //
+    // Steps k and k + 1 (k even) together.  Before them the owners publish columns k and k + 1 and rows k and k + 1
+    // as they are before step k.  What step k + 1 reads is column k + 1 and row k + 1 AFTER step k, and every thread
+    // can work that out for its own rows and columns from what has been published:
+    //   d[i][k+1] after step k = min(d[i][k+1], d[i][k] + d[k][k+1]),  d[k+1][j] after step k = min(d[k+1][j], d[k+1][k] + d[k][j])
+    // (the sums and comparisons that step k itself makes for those elements, made again).  An element then takes
+    // both steps' candidates in one 3-input minimum: three instructions per element and two steps instead of four,
+    // and one round of publish / barrier / read-back per two steps.
+    //
+    // The steps depend on each other, and what lies between two pairs of them (publishing, the barrier, reading
+    // back) would add its full latency to every pair.  So a pair is done in two parts:
+    //   A. the patch's rows and columns (k + 2) & 7 and (k + 3) & 7 -- every thread's, since which thread owns
+    //      rows / columns k + 2 and k + 3 is only known at run time -- then the owners publish them, then the barrier;
+    //   B. the reads for the next pair are issued, and the other 36 elements are done while they are on their way.
+    //
+    // The published lines are what hist gets (for these element types hist holds, for odd k, column k and row k as
+    // they are before step k - 1: fw_parents_block makes the same correction), copied from LDS by half the threads
+    // a barrier after they were published.  There are four sets of lines in LDS, used in turn: a set is written again
+    // three barriers after it was read for the last time.  (Nothing in this loop may wait for memory: stores
+    // to hist are on their way all the time, and a wait for any load would wait for them.)
+    const unsigned row_lds[4] = {lds(rowbuf + (0) * FW_BLOCK + 8 * tj), lds(rowbuf + (2) * FW_BLOCK + 8 * tj), lds(rowbuf + (4) * FW_BLOCK + 8 * tj), lds(rowbuf + (6) * FW_BLOCK + 8 * tj)};
+    const unsigned col_lds[4] = {lds(colbuf + (0) * FW_BLOCK + 8 * ti), lds(colbuf + (2) * FW_BLOCK + 8 * ti), lds(colbuf + (4) * FW_BLOCK + 8 * ti), lds(colbuf + (6) * FW_BLOCK + 8 * ti)};
+    // (the lines' addresses in vector registers of the thread's own: as values that are the same for all
+    // threads the compiler fetches them again for every pair, and waits for that with the reads above)
+    unsigned row_at_0 = lds(rowbuf), col_at_0 = lds(colbuf);
+    asm volatile("" : "+v"(row_at_0), "+v"(col_at_0));
+    struct Lines {
+      T c0[8], c1[8], r0[8], r1[8];  // columns k, k + 1 at my rows, rows k, k + 1 at my columns, before step k
+      T at_01, at_10;                // d[k][k + 1], d[k + 1][k]
+    };
+    auto publish = [&](int kn, auto setc, auto sc) {
+      constexpr int SET = decltype(setc)::value, S = decltype(sc)::value;
+      if ((kn >> 3) == ti) {  // my patch holds rows kn and kn + 1
+        put_row(row_lds[SET], std::integral_constant<int, S>{}, std::integral_constant<int, 0>{});
+        put_row(row_lds[SET], std::integral_constant<int, S + 1>{}, std::integral_constant<int, FW_BLOCK>{});
+      }
+      if ((kn >> 3) == tj) {  // my patch holds columns kn and kn + 1
+        put_col(col_lds[SET], std::integral_constant<int, S>{}, std::integral_constant<int, 0>{});
+        put_col(col_lds[SET], std::integral_constant<int, S + 1>{}, std::integral_constant<int, FW_BLOCK>{});
+      }
+      // (the barrier that follows is the compiler's, which does not know of the instructions above)
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    auto fetch = [&](Lines &l, int set, int kn) {
+      get8(l.c0, colbuf + (2 * set) * FW_BLOCK + 8 * ti);
+      get8(l.c1, colbuf + (2 * set + 1) * FW_BLOCK + 8 * ti);
+      get8(l.r0, rowbuf + (2 * set) * FW_BLOCK + 8 * tj);
+      get8(l.r1, rowbuf + (2 * set + 1) * FW_BLOCK + 8 * tj);
+      const unsigned at = unsigned(((2 * set) * FW_BLOCK + ((kn + 1) & (FW_BLOCK - 1))) * sizeof(T));
+      l.at_01 = *(const LT *)(size_t)(row_at_0 + at);
+      l.at_10 = *(const LT *)(size_t)(col_at_0 + at);
+    };
+    // the four lines of a set (steps kn and kn + 1) from LDS to hist: 16 bytes per thread of the first two waves
+    const int line = tid >> 5, piece = 4 * (tid & 31);
+    GT *const hist_line = (line < 2 ? hist_col : hist_row) + (line & 1) * FW_BLOCK + piece;
+    auto keep = [&](int set, int kn) {
+      if (tid < 128 && kn < FW_BLOCK)
+        *reinterpret_cast<GV4 *>(hist_line + kn * FW_BLOCK) =
+            *(const LV4 *)(size_t)((line < 2 ? col_at_0 : row_at_0) + unsigned(((2 * set + (line & 1)) * FW_BLOCK + piece) * sizeof(T)));
+    };
+    Lines cur_l;
+    auto pair = [&](int k, auto uc) {
+      constexpr int U = decltype(uc)::value;  // k & 7: 0, 2, 4, 6
+      constexpr int N = (U + 2) & 7;          // the rows and columns N, N + 1 of the patch are what steps k + 2, k + 3 may need
+      constexpr int O[6] = {N > 0 ? 0 : 2, N > 0 ? 1 : 3, N > 2 ? 2 : 4, N > 2 ? 3 : 5, N > 4 ? 4 : 6, N > 4 ? 5 : 7};
+      constexpr int SET = U >> 1;
+      Lines &l = cur_l;
+      // column k + 1 and row k + 1 after step k
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        relax(l.c1[x], l.c0[x] + l.at_01);
+        relax(l.r1[x], l.at_10 + l.r0[x]);
+      }
+      auto both = [&](auto ac, auto bc) {
+        constexpr int A = decltype(ac)::value, B = decltype(bc)::value;
+        relax2(cur[A][B], l.c0[A] + l.r0[B], l.c1[A] + l.r1[B]);
+      };
+      // A.
+      static_for<8>([&](auto bc) {
+        both(std::integral_constant<int, N>{}, bc);
+        both(std::integral_constant<int, N + 1>{}, bc);
+      });
+      static_for<6>([&](auto ic) {
+        both(std::integral_constant<int, O[decltype(ic)::value]>{}, std::integral_constant<int, N>{});
+        both(std::integral_constant<int, O[decltype(ic)::value]>{}, std::integral_constant<int, N + 1>{});
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      publish(k + 2, std::integral_constant<int, (SET + 1) & 3>{}, std::integral_constant<int, N>{});
+      __syncthreads();
+      Lines next;
+      fetch(next, (SET + 1) & 3, k + 2);
+      __builtin_amdgcn_sched_barrier(0);
+      // B.
+      static_for<6>([&](auto ic) {
+        static_for<6>([&](auto jc) {
+          both(std::integral_constant<int, O[decltype(ic)::value]>{}, std::integral_constant<int, O[decltype(jc)::value]>{});
+        });
+      });
+      __builtin_amdgcn_sched_barrier(0);
+      keep((SET + 1) & 3, k + 2);
+      cur_l = next;
+    };
+    publish(0, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+    __syncthreads();
+    fetch(cur_l, 0, 0);
+    keep(0, 0);
+    // steps beyond bb (up to the next multiple of eight) read rows and columns of the padding, which hold
+    // +infinity and improve nothing
+#pragma unroll 1
+    for (int k8 = 0; k8 < bb; k8 += 8) {
+      pair(k8 + 0, std::integral_constant<int, 0>{});
+      pair(k8 + 2, std::integral_constant<int, 2>{});
+      pair(k8 + 4, std::integral_constant<int, 4>{});
+      pair(k8 + 6, std::integral_constant<int, 6>{});
+    }
   }
 #pragma unroll
   for (int b = 0; b < 8; ++b)
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
       const int i = 8 * ti + a, j = 8 * tj + b;
-      if (i < bb && j < bb) d[i + int64_t(j) * ld] = cur[a][b];
+      T v = cur[a][b];
+      asm volatile("" : "+v"(v));  // (a value of its own: see the stores of init above)
+      if (i < bb && j < bb) d[i + int64_t(j) * ld] = v;
     }
   return true;
 }
 
 template <typename T>
 __device__ __forceinline__ void fw_close_dist(T *d, int64_t ld, int bb, T *hist) {
-  __shared__ __attribute__((aligned(32))) T colbuf[2][FW_BLOCK];  // d[i][k] for the step that reads this buffer
-  __shared__ __attribute__((aligned(32))) T rowbuf[2][FW_BLOCK];  // d[k][j]
-  if (!fw_close_dist_as<T, false>(d, ld, bb, hist, colbuf, rowbuf)) fw_close_dist_as<T, true>(d, ld, bb, hist, colbuf, rowbuf);
+  typedef __attribute__((address_space(3))) T LT;
+  constexpr int LINES = sizeof(T) == 4 ? 8 : 4;
+  __shared__ __attribute__((aligned(32))) T colbuf[LINES * FW_BLOCK], rowbuf[LINES * FW_BLOCK];
+  if (!fw_close_dist_as<T, false>(d, ld, bb, hist, (LT *)colbuf, (LT *)rowbuf))
+    fw_close_dist_as<T, true>(d, ld, bb, hist, (LT *)colbuf, (LT *)rowbuf);
 }
 
 // The predecessors of a diagonal block whose distances fw_close_dist has closed: workgroup b of 64 (256 threads)
 // takes rows 64 (b & 1) .. + 63 and columns 4 (b >> 1) .. + 3, one element per thread, and runs the literal scan
 // over the recorded columns and rows.  Only predecessors are written: the distances are those already there.
+// For 4-byte elements hist holds, for odd k, column k and row k as they are before step k - 1; step k - 1's
+// update of them is made here as fw_close_dist makes it (with the comparison: it never differs from the minimum
+// on a block without -0, and a block with one was closed with the comparison).
 template <typename T>
 __device__ __forceinline__ void fw_parents_block(const T *hist, int32_t *parent, int64_t ldp, int bb, int k_base, int b) {
   const int row = (b & 1) * 64 + (threadIdx.x & 63);
   const int col = __builtin_amdgcn_readfirstlane((b >> 1) * 4 + (threadIdx.x >> 6));
   if (row >= bb || col >= bb) return;
-  const T *hc = hist + row, *hr = hist + FW_BLOCK * FW_BLOCK + col;
-  T curr = hist[2 * FW_BLOCK * FW_BLOCK + row + col * FW_BLOCK];
+  const T *hist_row = hist + FW_BLOCK * FW_BLOCK;
+  const T *hc = hist + row, *hr = hist_row + col;
+  T curr = hist[2 * FW_BLOCK * FW_BLOCK + (8 * (row & 7) + (col & 7)) * 256 + (row >> 3) + 16 * (col >> 3)];
   int32_t p = -1;
-  int k = 0;
-  for (; k + 16 <= bb; k += 16) {  // sixteen k at a time, their operands requested together
-    T cv[16], rv[16];
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      cv[u] = hc[(k + u) * FW_BLOCK];
-      rv[u] = hr[(k + u) * FW_BLOCK];
-    }
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      const T prod = cv[u] + rv[u];
-      const bool lower = prod < curr;
-      curr = pick(lower, prod, curr);
-      p = lower ? k + u : p;
-    }
-  }
-  for (; k < bb; ++k) {
-    const T prod = hc[k * FW_BLOCK] + hr[k * FW_BLOCK];
+  auto scan = [&](const T prod, int k) {
     const bool lower = prod < curr;
     curr = pick(lower, prod, curr);
     p = lower ? k : p;
+  };
+  if constexpr (sizeof(T) == 4) {
+    auto steps = [&](const T c0, T c1, const T r0, T r1, const T at_01, const T at_10, int k) {
+      scan(c0 + r0, k);
+      const T via_c = c0 + at_01, via_r = at_10 + r0;
+      c1 = pick(via_c < c1, via_c, c1);
+      r1 = pick(via_r < r1, via_r, r1);
+      if (k + 1 < bb) scan(c1 + r1, k + 1);
+    };
+    int k = 0;
+    for (; k + 16 <= bb; k += 16) {  // sixteen k at a time, their operands requested together
+      T cv[16], rv[16], at_01[8], at_10[8];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        cv[u] = hc[(k + u) * FW_BLOCK];
+        rv[u] = hr[(k + u) * FW_BLOCK];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        at_01[u] = hist_row[(k + 2 * u) * FW_BLOCK + k + 2 * u + 1];
+        at_10[u] = hist[(k + 2 * u) * FW_BLOCK + k + 2 * u + 1];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) steps(cv[2 * u], cv[2 * u + 1], rv[2 * u], rv[2 * u + 1], at_01[u], at_10[u], k + 2 * u);
+    }
+    for (; k < bb; k += 2)
+      steps(hc[k * FW_BLOCK], hc[(k + 1) * FW_BLOCK], hr[k * FW_BLOCK], hr[(k + 1) * FW_BLOCK], hist_row[k * FW_BLOCK + k + 1],
+            hist[k * FW_BLOCK + k + 1], k);
+  } else {
+    int k = 0;
+    for (; k + 16 <= bb; k += 16) {  // sixteen k at a time, their operands requested together
+      T cv[16], rv[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        cv[u] = hc[(k + u) * FW_BLOCK];
+        rv[u] = hr[(k + u) * FW_BLOCK];
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) scan(cv[u] + rv[u], k + u);
+    }
+    for (; k < bb; ++k) scan(hc[k * FW_BLOCK] + hr[k * FW_BLOCK], k);
   }
   if (p >= 0) parent[row + int64_t(col) * ldp] = k_base + p;
 }
