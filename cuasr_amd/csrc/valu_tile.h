@@ -470,7 +470,9 @@ struct ValuTile {
 
   // ---- epilogue: D = add(mult(alpha, acc), mult(beta, C)), or raw partials; [kb, ke) is the
   // k range the accumulators cover (ZERO_SIGN looks into it)
-  static __device__ __forceinline__ void finish(const Problem &p, S (&acc)[TM][TN], int m0, int n0, int kb, int ke) {
+  // (row_step, row_first: only the rows i = row_first, row_first + row_step, ... of the thread's outputs)
+  static __device__ __forceinline__ void finish(const Problem &p, S (&acc)[TM][TN], int m0, int n0, int kb, int ke,
+                                                int row_step = 1, int row_first = 0) {
     const int tid = threadIdx.x & 255, tx = tid & 15, ty = tid >> 4;
     const T *A = reinterpret_cast<const T *>(p.A);
     const T *B = reinterpret_cast<const T *>(p.B);
@@ -496,7 +498,7 @@ struct ValuTile {
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int row = m0 + ty * VW + (i / VW) * 16 * VW + (i % VW);
-          if (row >= p.m) continue;
+          if (row >= p.m || i % row_step != row_first) continue;
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
             const int col = n0 + tx * VW + (j / VW) * 16 * VW + (j % VW);
@@ -510,7 +512,7 @@ struct ValuTile {
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
       const int row = m0 + ty * VW + (i / VW) * 16 * VW + (i % VW);
-      if (row >= p.m) continue;
+      if (row >= p.m || i % row_step != row_first) continue;
 #pragma unroll
       for (int g = 0; g < GN; ++g) {
         const int col = n0 + tx * VW + g * 16 * VW;
@@ -586,7 +588,7 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   using Tile = ValuTile<T, ADD, MUL, TM, TN, BK, VEC, CAREFUL>;
   using S = typename Tile::S;
   static_assert(order_free<T, ADD>::value, "a floating-point sum depends on the grouping of its terms");
-  static_assert(G * sizeof(typename Tile::Smem) >= (G - 1) * sizeof(S) * TM * TN * 256, "the groups' accumulators must fit the panel space");
+  static_assert(G * sizeof(typename Tile::Smem) >= (G - 1) * sizeof(S) * TM * TN * 256 && TM % G == 0, "the groups' accumulators must fit the panel space");
   __shared__ typename Tile::Smem sm[G];
   select_batch<T>(p);
   const int g = threadIdx.x >> 8, tid = threadIdx.x & 255;
@@ -596,30 +598,45 @@ __global__ __launch_bounds__(256 * G) void valu_ksplit_kernel(Problem p) {
   const int gkb = min(ke, kb + g * per * BK), gke = min(ke, gkb + per * BK);
   S acc[TM][TN];
   Tile::accumulate(p, sm[g], m0, n0, gkb, gke, per, acc);  // ends with a barrier: every group is done with its panels
-  // the panels are dead now: groups 1 .. G-1 leave their accumulators in that space, one after the other
+  // The panels are dead now.  Group d takes the rows i = d, d + G, ... of the threads' outputs: every group leaves
+  // its accumulators of the other groups' rows in the panel space, and each group then folds its rows over the
+  // groups in ascending k order (acc = add(acc, partial), as the split-K reduction does) and runs their epilogue --
+  // one G-th of the fold, of the reads of C and of the stores each.
+  // Where group h's row i (of group i % G != h) lies: rows in the order of i, without h's own
+  constexpr int ROWS_OUT = TM - TM / G, AREA = ROWS_OUT * TN * 256;
+  auto slot = [](int h, int i) { return (i / G) * (G - 1) + (i % G < h ? i % G : i % G - 1); };
   S *area = reinterpret_cast<S *>(&sm[0]);
-  if (g > 0) {
-    S *mine = area + (g - 1) * (TM * TN * 256);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i) {
+    if (i % G == g) continue;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) mine[(i * TN + j) * 256 + tid] = acc[i][j];
+    for (int j = 0; j < TN; ++j) area[g * AREA + (slot(g, i) * TN + j) * 256 + tid] = acc[i][j];
   }
   __syncthreads();
-  if (g > 0) return;
-#pragma unroll 1
-  for (int h = 1; h < G; ++h) {
-    const S *part = area + (h - 1) * (TM * TN * 256);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+  for (int i = 0; i < TM; ++i) {
+    if (i % G != g) continue;
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const S w = part[(i * TN + j) * 256 + tid];
-        if constexpr (Tile::MASKED) acc[i][j] |= w;
-        else acc[i][j] = Op<ADD>::apply(acc[i][j], w);
+    for (int j = 0; j < TN; ++j) {
+      S v = acc[i][j];  // (overwritten unless g == 0)
+#pragma unroll
+      for (int h = 0; h < G; ++h) {
+        if (h == i % G) {  // this row's own group: from its registers
+          if (h > 0) {
+            if constexpr (Tile::MASKED) v |= acc[i][j];
+            else v = Op<ADD>::apply(v, acc[i][j]);
+          }
+        } else {
+          const S w = area[h * AREA + (slot(h, i) * TN + j) * 256 + tid];
+          if (h == 0) v = w;
+          else if constexpr (Tile::MASKED) v |= w;
+          else v = Op<ADD>::apply(v, w);
+        }
       }
+      acc[i][j] = v;
+    }
   }
-  Tile::finish(p, acc, m0, n0, kb, ke);
+  Tile::finish(p, acc, m0, n0, kb, ke, G, g);
 }
 
 // Extents along every contiguous direction are multiples of the vector width: no vector straddles
@@ -655,6 +672,9 @@ static void launch_ksplit(const Problem &p, dim3 grid, hipStream_t s) {
     launch_kernel((valu_ksplit_kernel<T, ADD, MUL, TM, TN, BK, true, true, G>), grid, dim3(256 * G), 0, s, p);
 }
 
+#ifndef CUASR_AMD_KSPLIT2_MAX
+#define CUASR_AMD_KSPLIT2_MAX 1024
+#endif
 // KSPLIT: this tile may share its k range out inside the workgroup when the launch is small.
 template <typename T, int ADD, int MUL, int TM, int TN, int BK, bool KSPLIT = false>
 static hipError_t launch_valu(const Problem &p, hipStream_t s) {
@@ -673,7 +693,7 @@ static hipError_t launch_valu(const Problem &p, hipStream_t s) {
         launch_ksplit<T, ADD, MUL, TM, TN, BK, 4>(p, grid, s);
         return take_launch_status();
       }
-      if (groups <= 512) {
+      if (groups <= CUASR_AMD_KSPLIT2_MAX) {
         launch_ksplit<T, ADD, MUL, TM, TN, BK, 2>(p, grid, s);
         return take_launch_status();
       }

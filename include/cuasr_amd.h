@@ -296,7 +296,7 @@ int cuasr_amd_apsp_squaring(int dtype, int n, void *dist, int64_t ld, int32_t *p
  * so on weights whose sums round, distances can differ in the last bits from
  * those of cuasr_amd_apsp_squaring (both are sums of the same edges).  The
  * workspace holds cuasr_amd_apsp_blocked_workspace_bytes(dtype, n) bytes
- * (3 * 128 * n elements, n rounded up to a multiple of 4) and is 16-byte
+ * (3 * 128 * (n + 128) elements, n rounded up to a multiple of 4) and is 16-byte
  * aligned; CUASR_AMD_ERROR_WORKSPACE_NULL without it.  Asynchronous on the
  * stream, no allocation, no host synchronisation. */
 size_t cuasr_amd_apsp_blocked_workspace_bytes(int dtype, int n);
