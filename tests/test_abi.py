@@ -236,7 +236,7 @@ def test_fwgemm_host_errors(lib):
     assert cuasr_amd.apsp_workspace_bytes(10, "f64") == 1600 and cuasr_amd.apsp_workspace_bytes(0, "f32") == 0
     sq = lambda n=64, ws=0x1000, it=0, dtype=0: lib.cuasr_amd_apsp_squaring(dtype, n, P(0x1000), max(n, 1), P(0x1000), max(n, 1), P(ws), it, None)
     assert sq(ws=0) == 6 and sq(it=-1) == 4 and sq(dtype=3) == 2 and sq(n=0) == 0
-    assert cuasr_amd.apsp_blocked_workspace_bytes(1001, "f32") == 3 * 4 * 128 * 1004 and cuasr_amd.apsp_blocked_workspace_bytes(0, "f64") == 0
+    assert cuasr_amd.apsp_blocked_workspace_bytes(1001, "f32") == 3 * 4 * 128 * (1004 + 128) and cuasr_amd.apsp_blocked_workspace_bytes(0, "f64") == 0
     bl = lambda n=64, ws=0x1000, dtype=0, ld=None: lib.cuasr_amd_apsp_blocked(dtype, n, P(0x1000), ld or max(n, 1), P(0x1000), max(n, 1), P(ws), None)
     assert bl(ws=0) == 6 and bl(dtype=2) == 2 and bl(n=0) == 0 and bl(ld=10) == 4 and bl(ws=0x1004) == 1   # all before any launch
     assert lib.cuasr_amd_apsp_blocked_panels(0, 64, P(0x1000), 64, P(0x1000), 64, P(0x1000), 3, None) == 4   # unknown panel mode
