@@ -592,17 +592,17 @@ constexpr int FW_BLOCK = 128;  // vertices per block step of the blocked Floyd-W
 //
 // The hardware minimum prefers -0 to +0 where the strict comparison keeps whichever came first.  Sums and minima
 // of data free of -0 never produce one, so the block is searched for a -0 when it is loaded, and a block with
-// one takes the same steps with a comparison and a select (EXACT).
+// one is closed by fw_close_dist_exact instead: the same steps with a comparison and a select, the block in place.
 //
 // hist: FW_BLOCK x FW_BLOCK elements each of  col[k * FW_BLOCK + i] = d[i][k] before step k,
 // row[k * FW_BLOCK + j] = d[k][j] before step k,  init[(8 * (i % 8) + j % 8) * 256 + i / 8 + 16 * (j / 8)] = d[i][j] before
 // the closure.
-// (returns false, with nothing done, when the block holds a -0 and EXACT is not set)
+// (returns false, with nothing done, when the block holds a -0)
 // (A function of its own, not inlined: as part of a kernel that also holds the other form and a product's tile, the
 // compiler's register allocation moves parts of the patch to scratch memory inside the step loop, where any wait for
 // memory also waits for the stores to hist.  Alone, either form fits the registers.)
-template <typename T, bool EXACT>
-__device__ __attribute__((noinline)) bool fw_close_dist_as(T *d_anywhere, int64_t ld, int bb, T *hist_anywhere,
+template <typename T>
+__device__ __attribute__((noinline)) bool fw_close_dist_fast(T *d_anywhere, int64_t ld, int bb, T *hist_anywhere,
                                                            __attribute__((address_space(3))) T *colbuf,
                                                            __attribute__((address_space(3))) T *rowbuf) {
   typedef typename vec4_of<T>::type V4;
@@ -634,9 +634,9 @@ __device__ __attribute__((noinline)) bool fw_close_dist_as(T *d_anywhere, int64_
       cur[a][b] = (8 * ti + a < bb && j < bb) ? v : inf;
     }
   }
-  if constexpr (!EXACT) {
-    // a block with a -0 is left to the other form, which loads the block for itself (with one copy of the
-    // block in registers across the branch, the registers that the other form needs would be taken from this one)
+  {
+    // a block with a -0 is left to the other form (a function of its own too: as part of this one the registers
+    // it needs would be taken from this one's loop)
     bool negative_zero = false;
 #pragma unroll
     for (int b = 0; b < 8; ++b)
@@ -653,13 +653,12 @@ __device__ __attribute__((noinline)) bool fw_close_dist_as(T *d_anywhere, int64_
   // (the minimum as an instruction: from the builtin the compiler first "quiets" an operand whose origin it
   // does not know, such as anything that comes round the loop, an instruction more per element)
   auto relax = [](T &x, const T cand) {
-    if constexpr (EXACT) x = pick(cand < x, cand, x);
-    else if constexpr (sizeof(T) == 4) asm("v_min_f32 %0, %0, %1" : "+v"(x) : "v"(cand));
+    if constexpr (sizeof(T) == 4) asm("v_min_f32 %0, %0, %1" : "+v"(x) : "v"(cand));
     else asm("v_min_f64 %0, %0, %1" : "+v"(x) : "v"(cand));
   };
   // two steps' candidates at once, in the steps' order
   auto relax2 = [&](T &x, const T first, const T second) {
-    if constexpr (!EXACT && sizeof(T) == 4) {
+    if constexpr (sizeof(T) == 4) {
       asm("v_min3_f32 %0, %0, %1, %2" : "+v"(x) : "v"(first), "v"(second));
     } else {
       relax(x, first);
@@ -892,13 +891,76 @@ __device__ __attribute__((noinline)) bool fw_close_dist_as(T *d_anywhere, int64_
   return true;
 }
 
+// The same closure for a block that holds a -0: comparison and select, one step per barrier, and the block's rows and
+// columns handed from step to step through the block itself in device memory (every thread stores what it lowered,
+// and reads column k and row k from there), with the step loop rolled.  Two to three times slower than the form
+// above, a fraction of its code, and nothing of it in scratch memory -- a form like the one above with comparisons
+// keeps 64 comparison masks and as many candidates alive and spills hundreds of registers, which every workgroup
+// of the kernel pays for in scratch space, whether it ever sees a -0 or not.
+template <typename T>
+__device__ __attribute__((noinline)) void fw_close_dist_exact(T *d_anywhere, int64_t ld, int bb, T *hist_anywhere) {
+  typedef __attribute__((address_space(1))) T GT;
+  GT *const d = (GT *)d_anywhere, *const hist = (GT *)hist_anywhere;
+  GT *hist_col = hist, *hist_row = hist + FW_BLOCK * FW_BLOCK, *init = hist + 2 * FW_BLOCK * FW_BLOCK;
+  const int tid = threadIdx.x & 255, ti = tid & 15, tj = tid >> 4;  // rows 8 ti .. 8 ti + 7, columns 8 tj .. 8 tj + 7
+  const T inf = std::numeric_limits<T>::infinity();
+  // (rows and columns of the padding are computed on the block's last row / column and never stored)
+  int ic[8];
+#pragma unroll
+  for (int a = 0; a < 8; ++a) ic[a] = min(8 * ti + a, bb - 1);
+  T cur[8][8];
+#pragma unroll
+  for (int b = 0; b < 8; ++b) {
+    const GT *column = d + int64_t(min(8 * tj + b, bb - 1)) * ld;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      cur[a][b] = (8 * ti + a < bb && 8 * tj + b < bb) ? column[ic[a]] : inf;
+      init[(8 * a + b) * 256 + tid] = cur[a][b];
+    }
+  }
+  // what hist holds for 4-byte elements (fw_parents_block): for odd k column k and row k as before step k - 1
+  constexpr int PAIRED = sizeof(T) == 4 ? 1 : 0;
+#pragma unroll 1
+  for (int k = 0; k < bb; ++k) {
+    __syncthreads();  // what step k - 1 lowered is in the block
+    T ci[8], rj[8];
+#pragma unroll
+    for (int a = 0; a < 8; ++a) ci[a] = d[ic[a] + int64_t(k) * ld];
+#pragma unroll
+    for (int b = 0; b < 8; ++b) rj[b] = d[k + int64_t(min(8 * tj + b, bb - 1)) * ld];
+    if (!PAIRED || !(k & 1)) {
+      const int lines = PAIRED ? 2 : 1;
+      for (int q = 0; q < lines; ++q) {
+        const int kq = min(k + q, bb - 1);
+        if (tj == 0)
+#pragma unroll
+          for (int a = 0; a < 8; ++a) hist_col[(k + q) * FW_BLOCK + 8 * ti + a] = 8 * ti + a < bb ? (q ? T(d[ic[a] + int64_t(kq) * ld]) : ci[a]) : inf;
+        if (ti == 0)
+#pragma unroll
+          for (int b = 0; b < 8; ++b)
+            hist_row[(k + q) * FW_BLOCK + 8 * tj + b] = 8 * tj + b < bb ? (q ? T(d[kq + int64_t(min(8 * tj + b, bb - 1)) * ld]) : rj[b]) : inf;
+      }
+    }
+    __syncthreads();  // everybody has read column k and row k (and k + 1) before anybody stores
+#pragma unroll
+    for (int b = 0; b < 8; ++b)
+#pragma unroll
+      for (int a = 0; a < 8; ++a) {
+        const T cand = ci[a] + rj[b];
+        if (cand < cur[a][b]) {
+          cur[a][b] = cand;
+          if (8 * ti + a < bb && 8 * tj + b < bb) d[8 * ti + a + int64_t(8 * tj + b) * ld] = cand;
+        }
+      }
+  }
+}
+
 template <typename T>
 __device__ __forceinline__ void fw_close_dist(T *d, int64_t ld, int bb, T *hist) {
   typedef __attribute__((address_space(3))) T LT;
   constexpr int LINES = sizeof(T) == 4 ? 8 : 4;
   __shared__ __attribute__((aligned(32))) T colbuf[LINES * FW_BLOCK], rowbuf[LINES * FW_BLOCK];
-  if (!fw_close_dist_as<T, false>(d, ld, bb, hist, (LT *)colbuf, (LT *)rowbuf))
-    fw_close_dist_as<T, true>(d, ld, bb, hist, (LT *)colbuf, (LT *)rowbuf);
+  if (!fw_close_dist_fast<T>(d, ld, bb, hist, (LT *)colbuf, (LT *)rowbuf)) fw_close_dist_exact<T>(d, ld, bb, hist);
 }
 
 // The predecessors of a diagonal block whose distances fw_close_dist has closed: workgroup b of 64 (256 threads)
