@@ -1349,7 +1349,14 @@ __global__ void __launch_bounds__(256) snapshot_pair_kernel(const T *src0, T *w0
   const int gx = (rows + 63) / 64;
   const int r = (b % gx) * 64 + (threadIdx.x & 63), c0 = (b / gx) * 64 + (threadIdx.x >> 6);
   if (r >= rows) return;
-  for (int c = c0; c < cols && c < (b / gx) * 64 + 64; c += 4) w[r + int64_t(c) * ldw] = src[r + int64_t(c) * ld];
+  // (all of a thread's 16 loads, then its stores: source and copy may be the same memory for all the compiler
+  // knows, and one load after each store is sixteen trips to memory in a row)
+  T v[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) v[u] = src[r + int64_t(min(c0 + 4 * u, cols - 1)) * ld];
+#pragma unroll
+  for (int u = 0; u < 16; ++u)
+    if (c0 + 4 * u < cols) w[r + int64_t(c0 + 4 * u) * ldw] = v[u];
 }
 
 // Floyd-Warshall inside one diagonal block of at most FW_BLOCK x FW_BLOCK: k ascending,
