@@ -314,17 +314,32 @@ def build_workload(args, np, torch, cuasr_amd, inputs):
         dD = torch.empty(n, n, dtype=tdt, device=dev)
         dD = dD.t() if lc == "F" else dD
 
-        def step(i):
-            cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dt, kernel=args.kernel)
+        if args.kernel == "vendor":
+            # a yardstick, not this library: the vendor BLAS behind PyTorch on the same device operands
+            # (plus-times only; the int8 product has no fused source term there, so it reads no C)
+            if not (add == "plus" and mult == "multiplies" and dt in ("f32", "f64", "f16", "i8")):
+                raise SystemExit("bench.py: --kernel vendor times the vendor BLAS, which has plus-times on f32, f64, f16, i8 only")
 
-        desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one, kernel=args.kernel)
+            def step(i):
+                if dt == "i8":
+                    torch._int_mm(dA, dB, out=dD)
+                else:
+                    torch.addmm(dC, dA, dB, out=dD)
+
+            desc = None
+        else:
+            def step(i):
+                cuasr_amd.srgemm(add, mult, dA, dB, dC, dD, one, one, ident, one, dtype=dt, kernel=args.kernel)
+
+            desc = cuasr_amd.make_desc(add, mult, dt, dA, dB, dC, dD, one, one, ident, one, kernel=args.kernel)
         # (binary16 plus-times runs on the matrix cores, with float accumulation, only when asked to)
-        matrix = add == "plus" and mult == "multiplies" and (dt in ("f32", "f64", "i8") or (dt == "f16" and args.kernel == "mfma"))
+        matrix = add == "plus" and mult == "multiplies" and (dt in ("f32", "f64", "i8") or (dt == "f16" and args.kernel in ("mfma", "vendor")))
         return dict(step=step, m=n, n=n, k=n, dtype=dt, desc=desc, host=(add, mult, A, B, C, one, one, ident),
                     result=lambda: dD.cpu().numpy(),
                     metric=f"{dt} {add}-{mult} SRGEMM GOPS at {n}^3 (2 ops/term)",
                     workload=f"{add}-{mult} SRGEMM {dt}, M=N=K={n}, layouts (A, B, C) = {args.layouts} "
-                             "(c = column-major, r = row-major), beta = one with a seeded C",
+                             "(c = column-major, r = row-major), beta = one with a seeded C"
+                             + (" -- timed on the vendor BLAS behind PyTorch, as a yardstick" if args.kernel == "vendor" else ""),
                     bound="mfma" if matrix else "valu",
                     peak=FP64_VECTOR_PEAK if dt == "f64" else INT8_MATRIX_PEAK if (dt == "i8" and matrix)
                     else F16_MATRIX_PEAK if (dt == "f16" and matrix) else FP32_VECTOR_PEAK,
@@ -537,7 +552,8 @@ def main():
     ap.add_argument("--size", type=int, default=0, help="override the workload's M=N (and K where it is square)")
     ap.add_argument("--slices", type=int, default=64, help="split-K slices (workload splitk)")
     ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")
-    ap.add_argument("--kernel", default="auto")
+    ap.add_argument("--kernel", default="auto",
+                    help="a kernel family of the library, or (workload srgemm, plus-times) vendor: the vendor BLAS as a yardstick")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="headline only: do not time the other configs (extra.configs)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",

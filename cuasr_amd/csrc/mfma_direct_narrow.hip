@@ -188,48 +188,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   }
 
   // ---- epilogue.  Block (bi, bj), register e of lane l: row 8 * (e / 4) + 4 * (l / 32) + e % 4, column l % 32: a
-  // store instruction writes 128 consecutive bytes of two rows.  (With the operands of the matrix instruction
-  // swapped a lane holds four consecutive columns per group of registers and stores vectors -- a quarter of the
-  // store instructions, but each touching 32 rows, a leading dimension apart: measured 25 % slower at 8192^3.)
+  // store instruction writes 128 consecutive bytes of two rows.  The four blocks of a block row are stored register
+  // by register, so that four consecutive instructions write 512 consecutive bytes of each of their two rows: block
+  // by block (sixteen instructions that touch 32 rows before the next 128 bytes of any of them follow) the same
+  // stores took 10 us longer per round of tiles at 4096 x 4096, a third of an int8 launch with 64 bytes of k.  (With
+  // the operands of the matrix instruction swapped a lane holds four consecutive columns per group of registers and
+  // stores vectors -- a quarter of the store instructions, but each touching 32 rows, a leading dimension apart:
+  // measured 25 % slower at 8192^3.)
   const EpilogueScalars<Result> sc = resolve_scalars<Result>(p, kMultiplies);
   const Result *C = reinterpret_cast<const Result *>(p.C);
   Result *D = reinterpret_cast<Result *>(p.D);
+  const int col0 = n0 + wn * 128 + l32;
+  // one copy of the stores per case (partial sums for a split-K workspace; results with and without a source), the
+  // case chosen once: with the tests inside, per element, the same stores took 3 us longer per tile
+  auto store_all = [&](auto to_workspace, auto with_source) {
+    constexpr bool WS = decltype(to_workspace)::value, SRC = decltype(with_source)::value;
 #pragma unroll
-  for (int bi = 0; bi < 4; ++bi)
-#pragma unroll
-    for (int bj = 0; bj < 4; ++bj) {
-      const int col = n0 + wn * 128 + bj * 32 + l32;
-      const int blk = 4 * bi + bj;
+    for (int bi = 0; bi < 4; ++bi) {
       auto row_of = [&](int e) { return (long long)(m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4)); };
-      // a block's sixteen source elements are requested together, before any of its results is stored (D may be
-      // C, so the compiler cannot move a load of C above a store to D by itself: one load at a time, each waited
-      // for, made this epilogue as long as the product)
-      Result src[16];
-      if (!p.workspace && sc.source_needed) {
+      // a block row's 64 source elements are requested together, before any of its results is stored (D may be C,
+      // so the compiler cannot move a load of C above a store to D by itself: one load at a time, each waited for,
+      // made this epilogue as long as the product)
+      Result src[16][4];
+      if constexpr (SRC) {
 #pragma unroll
-        for (int e = 0; e < 16; ++e) src[e] = C[row_of(e) * p.ldc + col];
+        for (int e = 0; e < 16; ++e)
+#pragma unroll
+          for (int bj = 0; bj < 4; ++bj) src[e][bj] = C[row_of(e) * p.ldc + col0 + bj * 32];
       }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const long long row = row_of(e);
-        const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
-        if constexpr (I8) {
-          if (p.workspace) {
+      for (int e = 0; e < 16; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) {
+          const long long row = row_of(e);
+          const int col = col0 + bj * 32;
+          const int blk = 4 * bi + bj;
+          const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
+          if constexpr (WS) {
             reinterpret_cast<int32_t *>(p.workspace)[((long long)blockIdx.y * p.m + row) * p.n + col] = bits;
-          } else {
+          } else if constexpr (I8) {
             // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
             uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
-            if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)src[e];
+            if constexpr (SRC) out += (uint32_t)sc.beta * (uint32_t)src[e][bj];
             D[row * p.ldd + col] = (int32_t)out;
+          } else {
+            // D = alpha * acc + beta * C in float, rounded to binary16 once
+            float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
+            if constexpr (SRC) out += float(sc.beta) * float(src[e][bj]);
+            D[row * p.ldd + col] = half_t(out);
           }
-        } else {
-          // D = alpha * acc + beta * C in float, rounded to binary16 once
-          float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
-          if (sc.source_needed) out += float(sc.beta) * float(src[e]);
-          D[row * p.ldd + col] = half_t(out);
         }
-      }
     }
+  };
+  if (I8 && p.workspace) store_all(std::true_type{}, std::false_type{});
+  else if (sc.source_needed) store_all(std::false_type{}, std::true_type{});
+  else store_all(std::false_type{}, std::false_type{});
 }
 
 // whole tiles, whole stages, both operands k-contiguous with 16-byte aligned rows, a panel's 256 rows within 32
