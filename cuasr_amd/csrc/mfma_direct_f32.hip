@@ -296,24 +296,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, NBN == 4
     source_needed = e.source_needed;
   }
   const float *C = reinterpret_cast<const float *>(p.C);
+  // A store instruction writes 128 consecutive bytes of two rows.  The blocks of a block row are stored register by
+  // register, so that NBN consecutive instructions write 128 NBN consecutive bytes of each of their two rows, and a
+  // block row's source elements are requested together before any of its results is stored (D may be C, so the
+  // compiler cannot move a load of C above a store to D by itself); one copy of the stores per case.
+  const int col0 = n0 + wn * WN + (lane & 31);
+  auto store_all = [&](auto scaled, auto with_source) {
+    constexpr bool SCALED = decltype(scaled)::value, SRC = decltype(with_source)::value;
 #pragma unroll
-  for (int bi = 0; bi < 2; ++bi)
+    for (int bi = 0; bi < 2; ++bi) {
+      auto row_of = [&](int e) { return m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4); };
+      float src[16][NBN];
+      if constexpr (SRC) {
 #pragma unroll
-    for (int bj = 0; bj < NBN; ++bj) {
-      const int col = n0 + wn * WN + bj * 32 + (lane & 31);
+        for (int e = 0; e < 16; ++e)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * (lane >> 5) + (e % 4);
-        if (row < p.m && col < p.n) {
-          float v = r.acc[NBN * bi + bj][e];
-          if (!partial) {
-            v = alpha * v;
-            if (source_needed) v = v + beta * C[(long long)row * p.ldc + col];
+          for (int bj = 0; bj < NBN; ++bj) {
+            const int row = row_of(e), col = col0 + bj * 32;
+            if (row < p.m && col < p.n) src[e][bj] = C[(long long)row * p.ldc + col];
           }
-          out[(long long)row * ld_out + col] = v;
-        }
       }
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+#pragma unroll
+        for (int bj = 0; bj < NBN; ++bj) {
+          const int row = row_of(e), col = col0 + bj * 32;
+          if (row < p.m && col < p.n) {
+            float v = r.acc[NBN * bi + bj][e];
+            if constexpr (SCALED) v = alpha * v;
+            if constexpr (SRC) v = v + beta * src[e][bj];
+            out[(long long)row * ld_out + col] = v;
+          }
+        }
     }
+  };
+  if (partial) store_all(std::false_type{}, std::false_type{});
+  else if (source_needed) store_all(std::true_type{}, std::true_type{});
+  else store_all(std::true_type{}, std::false_type{});
 }
 
 // on top of mfma_panel::can_run: whole k-tiles only, and every byte offset inside a tile in 32 bits

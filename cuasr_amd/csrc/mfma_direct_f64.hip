@@ -234,25 +234,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     source_needed = e.source_needed;
   }
   const double *C = reinterpret_cast<const double *>(p.C);
+  // A store instruction writes 128 consecutive bytes of four rows.  The four blocks of a block row are stored
+  // register by register, so that four consecutive instructions write 512 consecutive bytes of each of their rows,
+  // and a block row's source elements are requested together before any of its results is stored (D may be C, so
+  // the compiler cannot move a load of C above a store to D by itself); one copy of the stores per case.
+  const int col0 = n0 + wn * 64 + (lane & 15);
+  auto store_all = [&](auto scaled, auto with_source) {
+    constexpr bool SCALED = decltype(scaled)::value, SRC = decltype(with_source)::value;
 #pragma unroll
-  for (int bi = 0; bi < 4; ++bi)
+    for (int bi = 0; bi < 4; ++bi) {
+      double src[4][4];
+      if constexpr (SRC) {
 #pragma unroll
-    for (int bj = 0; bj < 4; ++bj) {
-      const int blk = 4 * bi + bj;
-      const int col = n0 + wn * 64 + bj * 16 + (lane & 15);
+        for (int e = 0; e < 4; ++e)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int row = m0 + wm * 64 + bi * 16 + (lane >> 4) + 4 * e;
-        if (row < p.m && col < p.n) {
-          double v = r.acc[blk >> 1][(blk & 1) * 4 + e];
-          if (!partial) {
-            v = alpha * v;
-            if (source_needed) v = v + beta * C[(long long)row * p.ldc + col];
+          for (int bj = 0; bj < 4; ++bj) {
+            const int row = m0 + wm * 64 + bi * 16 + (lane >> 4) + 4 * e, col = col0 + bj * 16;
+            if (row < p.m && col < p.n) src[e][bj] = C[(long long)row * p.ldc + col];
           }
-          out[(long long)row * ld_out + col] = v;
-        }
       }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) {
+          const int blk = 4 * bi + bj;
+          const int row = m0 + wm * 64 + bi * 16 + (lane >> 4) + 4 * e, col = col0 + bj * 16;
+          if (row < p.m && col < p.n) {
+            double v = r.acc[blk >> 1][(blk & 1) * 4 + e];
+            if constexpr (SCALED) v = alpha * v;
+            if constexpr (SRC) v = v + beta * src[e][bj];
+            out[(long long)row * ld_out + col] = v;
+          }
+        }
     }
+  };
+  if (partial) store_all(std::false_type{}, std::false_type{});
+  else if (source_needed) store_all(std::true_type{}, std::true_type{});
+  else store_all(std::true_type{}, std::false_type{});
 }
 
 // 16-byte vectors along the contiguous direction of either operand, whole k-tiles, every byte offset inside a
