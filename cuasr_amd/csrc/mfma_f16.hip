@@ -193,30 +193,35 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   const float alpha = float(sc.alpha), beta = float(sc.beta);
   const half_t *C = reinterpret_cast<const half_t *>(p.C);
   half_t *D = reinterpret_cast<half_t *>(p.D);
+  // A store instruction writes 64 consecutive bytes of two rows; the two blocks of a block row are stored register by
+  // register, so that consecutive instructions write consecutive pieces of the same rows, and a block row's source
+  // elements are requested together, before any of its results is stored (D may be C, so the compiler cannot move a
+  // load of C above a store to D by itself)
 #pragma unroll
-  for (int bi = 0; bi < 2; ++bi)
+  for (int bi = 0; bi < 2; ++bi) {
+    auto row_of = [&](int e) { return m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4); };
+    auto inside = [&](int row, int col) { return !GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n); };
+    half_t src[16][2];
+    if (sc.source_needed) {
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
-      const int col = n0 + wn * 64 + bj * 32 + l32;
-      // a block's sixteen source elements are requested together, before any of its results is stored (D may be C,
-      // so the compiler cannot move a load of C above a store to D by itself)
-      half_t src[16];
-      if (sc.source_needed) {
+      for (int e = 0; e < 16; ++e)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-          src[e] = (!GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) ? C[(long long)row * p.ldc + col] : half_t(0);
+        for (int bj = 0; bj < 2; ++bj) {
+          const int row = row_of(e), col = n0 + wn * 64 + bj * 32 + l32;
+          src[e][bj] = inside(row, col) ? C[(long long)row * p.ldc + col] : half_t(0);
         }
-      }
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-        if (GUARD && !((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) continue;
+    for (int e = 0; e < 16; ++e)
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) {
+        const int row = row_of(e), col = n0 + wn * 64 + bj * 32 + l32;
+        if (!inside(row, col)) continue;
         float out = alpha * acc[bi][bj][e];
-        if (sc.source_needed) out += beta * float(src[e]);
+        if (sc.source_needed) out += beta * float(src[e][bj]);
         D[(long long)row * p.ldd + col] = half_t(out);
       }
-    }
+  }
 }
 
 // whole tiles of 16-byte aligned operands: the unguarded kernel

@@ -207,36 +207,41 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
   int32_t *ws = p.workspace ? reinterpret_cast<int32_t *>(p.workspace) + (long long)blockIdx.y * p.m * p.n : nullptr;
   const int32_t *C = reinterpret_cast<const int32_t *>(p.C);
   int32_t *D = reinterpret_cast<int32_t *>(p.D);
+  // A store instruction writes 128 consecutive bytes of two rows; the two blocks of a block row are stored register by
+  // register, so that consecutive instructions write consecutive pieces of the same rows, and a block row's source
+  // elements are requested together, before any of its results is stored (D may be C, so the compiler cannot move a
+  // load of C above a store to D by itself)
 #pragma unroll
-  for (int bi = 0; bi < 2; ++bi)
+  for (int bi = 0; bi < 2; ++bi) {
+    auto row_of = [&](int e) { return m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4); };
+    auto inside = [&](int row, int col) { return !GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n); };
+    int32_t src[16][2];
+    if (!ws && sc.source_needed) {
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
-      const int col = n0 + wn * 64 + bj * 32 + l32;
-      // a block's sixteen source elements are requested together, before any of its results is stored (D may be C,
-      // so the compiler cannot move a load of C above a store to D by itself)
-      int32_t src[16];
-      if (!ws && sc.source_needed) {
+      for (int e = 0; e < 16; ++e)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-          src[e] = (!GUARD || ((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) ? C[(long long)row * p.ldc + col] : 0;
+        for (int bj = 0; bj < 2; ++bj) {
+          const int row = row_of(e), col = n0 + wn * 64 + bj * 32 + l32;
+          src[e][bj] = inside(row, col) ? C[(long long)row * p.ldc + col] : 0;
         }
-      }
+    }
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int row = m0 + wm * 64 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4);
-        if (GUARD && !((unsigned)row < (unsigned)p.m && (unsigned)col < (unsigned)p.n)) continue;
+    for (int e = 0; e < 16; ++e)
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) {
+        const int row = row_of(e), col = n0 + wn * 64 + bj * 32 + l32;
+        if (!inside(row, col)) continue;
         const int32_t v = acc[bi][bj][e];
         if (ws) {
           ws[(long long)row * p.n + col] = v;
         } else {
           // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
           uint32_t out = (uint32_t)sc.alpha * (uint32_t)v;
-          if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)src[e];
+          if (sc.source_needed) out += (uint32_t)sc.beta * (uint32_t)src[e][bj];
           D[(long long)row * p.ldd + col] = (int32_t)out;
         }
       }
-    }
+  }
 }
 
 // whole tiles of 16-byte aligned operands: the unguarded kernel
