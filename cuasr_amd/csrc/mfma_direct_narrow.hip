@@ -203,24 +203,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // case chosen once: with the tests inside, per element, the same stores took 3 us longer per tile
   auto store_all = [&](auto to_workspace, auto with_source) {
     constexpr bool WS = decltype(to_workspace)::value, SRC = decltype(with_source)::value;
+    auto row_of = [&](int bi, int e) { return (long long)(m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4)); };
+    // a block row's 64 source elements are requested together (D may be C, so the compiler cannot move a load of C
+    // above a store to D by itself: one load at a time, each waited for, made this epilogue as long as the
+    // product), and the next block row's before this one's results are stored, so that the trip to memory is
+    // waited for once, not four times (a thread reads exactly the elements it writes, later)
+    Result src[2][16][4];
+    auto request = [&](int bi) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) src[bi & 1][e][bj] = C[row_of(bi, e) * p.ldc + col0 + bj * 32];
+    };
+    if constexpr (SRC) request(0);
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi) {
-      auto row_of = [&](int e) { return (long long)(m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4)); };
-      // a block row's 64 source elements are requested together, before any of its results is stored (D may be C,
-      // so the compiler cannot move a load of C above a store to D by itself: one load at a time, each waited for,
-      // made this epilogue as long as the product)
-      Result src[16][4];
       if constexpr (SRC) {
-#pragma unroll
-        for (int e = 0; e < 16; ++e)
-#pragma unroll
-          for (int bj = 0; bj < 4; ++bj) src[e][bj] = C[row_of(e) * p.ldc + col0 + bj * 32];
+        if (bi + 1 < 4) request(bi + 1);
       }
 #pragma unroll
       for (int e = 0; e < 16; ++e)
 #pragma unroll
         for (int bj = 0; bj < 4; ++bj) {
-          const long long row = row_of(e);
+          const long long row = row_of(bi, e);
           const int col = col0 + bj * 32;
           const int blk = 4 * bi + bj;
           const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
@@ -229,12 +234,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           } else if constexpr (I8) {
             // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
             uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
-            if constexpr (SRC) out += (uint32_t)sc.beta * (uint32_t)src[e][bj];
+            if constexpr (SRC) out += (uint32_t)sc.beta * (uint32_t)src[bi & 1][e][bj];
             D[row * p.ldd + col] = (int32_t)out;
           } else {
             // D = alpha * acc + beta * C in float, rounded to binary16 once
             float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
-            if constexpr (SRC) out += float(sc.beta) * float(src[e][bj]);
+            if constexpr (SRC) out += float(sc.beta) * float(src[bi & 1][e][bj]);
             D[row * p.ldd + col] = half_t(out);
           }
         }
