@@ -87,6 +87,54 @@ def timed(step, steps, torch):
     return wall, [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
 
 
+class PowerSampler:
+    """Reads the board's power sensor (hwmon power1_input, microwatts) every 20 ms in a thread; summary() averages
+    the readings of the second half of the interval, where the sensor's own averaging has caught up with the load."""
+
+    def __init__(self):
+        import glob
+        import threading
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.path = next((os.path.join(h, "power1_input") for h in hw if os.path.exists(os.path.join(h, "power1_input"))), None)
+        cap = next((os.path.join(h, "power1_cap") for h in hw if os.path.exists(os.path.join(h, "power1_cap"))), None)
+        self.cap = self._read(cap) if cap else None
+        self.samples, self.stop = [], False
+        self.thread = threading.Thread(target=self._run, daemon=True)
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read().strip())
+        except (OSError, ValueError):
+            return None
+
+    def _run(self):
+        while not self.stop:
+            v = self._read(self.path) if self.path else None
+            if v is not None:
+                self.samples.append((time.perf_counter(), v))
+            time.sleep(0.02)
+
+    def __enter__(self):
+        self.t0 = time.perf_counter()
+        self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.t1 = time.perf_counter()
+        self.stop = True
+        self.thread.join()
+
+    def summary(self):
+        mid = 0.5 * (self.t0 + self.t1)
+        late = [v for t, v in self.samples if t >= mid]
+        if not late:
+            return {"avg_w": None, "samples": 0, "note": "no power sensor reading (hwmon power1_input) during the timed region"}
+        return {"avg_w": round(sum(late) / len(late) / 1e6, 1), "cap_w": round(self.cap / 1e6, 1) if self.cap else None,
+                "samples": len(late), "note": "board power over the second half of the timed region (hwmon power1_input every 20 ms)"}
+
+
 def build_workload(args, np, torch, cuasr_amd, inputs):
     """Returns a dict: step(i) launches one step; metadata for the JSON line; sample() for the CPU leg."""
     dev = torch.device("cuda:0")
@@ -554,6 +602,8 @@ def main():
     ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")
     ap.add_argument("--kernel", default="auto",
                     help="a kernel family of the library, or (workload srgemm, plus-times) vendor: the vendor BLAS as a yardstick")
+    ap.add_argument("--power", action="store_true",
+                    help="also report the board's power over the timed region (give --steps at least two seconds of work)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="headline only: do not time the other configs (extra.configs)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -602,7 +652,11 @@ def main():
     torch.cuda.synchronize()
     if "reset" in wl:
         wl["reset"]()
-    wall, kernel_ms = timed(step, args.steps, torch)
+    if args.power:
+        with PowerSampler() as power:
+            wall, kernel_ms = timed(step, args.steps, torch)
+    else:
+        wall, kernel_ms = timed(step, args.steps, torch)
     avg_kernel_ms = sum(kernel_ms) / len(kernel_ms)
     ops = 2.0 * m * n * k
     value = ops * args.steps / wall / 1e9
@@ -646,6 +700,8 @@ def main():
     }
     if "slices" in wl:
         out["config"]["split_k_slices"] = wl["slices"]
+    if args.power:
+        out["power"] = power.summary()
 
     if not args.no_cpu:
         # CPU baseline: the oracle (a port of the reference host SRGEMM, OpenMP over 32x32 output
