@@ -602,8 +602,10 @@ def main():
     ap.add_argument("--serial", action="store_true", help="workload splitk: the serial form (SplitKSerial = true)")
     ap.add_argument("--kernel", default="auto",
                     help="a kernel family of the library, or (workload srgemm, plus-times) vendor: the vendor BLAS as a yardstick")
-    ap.add_argument("--power", action="store_true",
-                    help="also report the board's power over the timed region (give --steps at least two seconds of work)")
+    ap.add_argument("--no-power", dest="power", action="store_false",
+                    help="do not read the board's power sensor during the timed region (the reading settles over about a "
+                         "second of load: give --steps that much work for a figure to quote)")
+    ap.add_argument("--power", dest="power", action="store_true", help="(the default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="headline only: do not time the other configs (extra.configs)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
