@@ -720,7 +720,111 @@ class NarrowMfmaBody(MfmaBody):
         return self.lines
 
 
-NARROW_VARIANTS = {"n_i8": "v_mfma_i32_32x32x32_i8", "n_f16": "v_mfma_f32_32x32x16_f16"}
+class Narrow16Body(NarrowMfmaBody):
+    """binary16 on v_mfma_f32_16x16x32_f16 (the shape that delivers more per watt on this chip for binary16; int8
+    is better served by 32 x 32): the instruction takes 64 bytes of k per row, so a stage of the ring is ONE step,
+    64 matrix instructions on the wave's 8 x 8 blocks of 16 x 16.  Accumulators a[4 (8 bm + bn) : +3]; two fragment
+    buffers of 64 registers (A block b in v[64 u + 4 b : +3], B block b in v[64 u + 32 + 4 b : +3]), stage t in
+    buffer t % 2, so the body exists in two forms (`parity` = which buffer holds the stage it computes) that the
+    kernel alternates.  One statement: the counted wait and the barrier (the next stage has landed for everyone),
+    then the 64 matrix instructions with the 16 fragment reads of the next stage behind the first 40 and the 8 loads
+    of the stage three ahead behind the rest."""
+
+    def __init__(self, parity, suffix=""):
+        super().__init__("v_mfma_f32_16x16x32_f16")
+        self.parity = parity
+        self.suffix = suffix   # of the per-stage operands and the labels: two stages may share one statement
+
+    def dma_chunk(self, index):
+        e, x = self.emit, self.suffix
+        name, h = ("a", index) if index < 4 else ("b", index - 4)
+        e(f"s_cmp_lt_i32 %[fetch{x}], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_{x}_%=")
+        e(f"s_add_u32 m0, %[m0_{name}{x}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[base_{name}{x}]")
+        e(f".Lcuasr_nofetch{index}_{x}_%=:")
+
+    @staticmethod
+    def frag(operand, u, blk):
+        return 64 * u + (0 if operand == "A" else 32) + 4 * blk
+
+    def reads(self, stage):
+        """LDS reads of the fragments of stage `stage` (relative to the body: 0 = the one it computes, 1 = the next,
+        through the already advanced addresses) into buffer (parity + stage) % 2."""
+        u, out = (self.parity + stage) % 2, []
+        for operand, addr in (("A", "a_addr"), ("B", "b_addr")):
+            for blk in range(8):
+                r = self.frag(operand, u, blk)
+                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}] offset:{blk * 16 * 64}",
+                            {r + i: (operand, blk, stage) for i in range(4)}))
+        return out
+
+    def mfma(self, stage, bm, bn):
+        u = (self.parity + stage) % 2
+        ra, rb = self.frag("A", u, bm), self.frag("B", u, bn)
+        for i in range(4):
+            assert self.content.get(ra + i) == ("A", bm, stage) and self.content.get(rb + i) == ("B", bn, stage)
+        self.require_exact({ra + i for i in range(4)} | {rb + i for i in range(4)})
+        acc = 4 * (8 * bm + bn)
+        self.lines.append(f'"{self.instruction} a[{acc}:{acc + 3}], v[{ra}:{ra + 3}], v[{rb}:{rb + 3}], a[{acc}:{acc + 3}]\\n"')
+        self.groups += 1
+        self.stats["groups"] += 1
+
+    def prime(self):
+        assert self.parity == 0
+        for item in self.reads(0):
+            self.read(item)
+        self.drain()
+        return self.lines
+
+    def tile(self):
+        e = self.emit
+        for operand in ("A", "B"):
+            for blk in range(8):
+                for i in range(4):
+                    self.content[self.frag(operand, self.parity, blk) + i] = (operand, blk, 0)
+        # this wave's part of the next stage has landed (the eight loads of the stage after it are younger and stay
+        # in flight, if there is such a stage); after the barrier that holds for the workgroup, and every wave has
+        # its fragments of this stage in registers: the next stage may be read, the slot of the stage before this
+        # one refilled
+        x = self.suffix
+        e(f"s_cmp_lt_i32 %[fetch{x}], 0")
+        e(f"s_cbranch_scc1 .Lcuasr_all_{x}_%=")
+        e("s_waitcnt vmcnt(8)")
+        e(f"s_branch .Lcuasr_join_{x}_%=")
+        e(f".Lcuasr_all_{x}_%=:")
+        e("s_waitcnt vmcnt(0)")
+        e(f".Lcuasr_join_{x}_%=:")
+        e("s_barrier")
+        e(f"v_add_u32 %[a_addr], %[step{x}], %[a_addr]")
+        e(f"v_add_u32 %[b_addr], %[step{x}], %[b_addr]")
+        e("s_mov_b32 %[m0_save], m0")
+        order = [(bm, bn) for bn in range(8) for bm in range(8)]
+        rd = [(lambda it=it: self.read(it)) for it in self.reads(1)]
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(8)]
+        behind = {}
+        for i, item in enumerate(rd):
+            behind.setdefault((i * 40) // len(rd), []).append(item)
+        for i, item in enumerate(aux):
+            behind.setdefault(40 + (i * 24) // len(aux), []).append(item)
+        for i, (bm, bn) in enumerate(order):
+            self.mfma(0, bm, bn)
+            for item in behind.get(i, []):
+                item()
+        e("s_mov_b32 m0, %[m0_save]")
+        self.drain()
+        # what the other form expects on entry: its stage 0 = this form's stage 1, in the other buffer
+        other = {}
+        for operand in ("A", "B"):
+            for blk in range(8):
+                for i in range(4):
+                    other[self.frag(operand, 1 - self.parity, blk) + i] = (operand, blk, 1)
+        assert all(self.content.get(r) == v for r, v in other.items()), "tile body does not leave the other form's entry state"
+        return self.lines
+
+
+NARROW_VARIANTS = {"n_i8": "v_mfma_i32_32x32x32_i8"}
 
 
 def generate_narrow(out_dir):
@@ -734,6 +838,18 @@ def generate_narrow(out_dir):
         with open(os.path.join(out_dir, f"mfma_asm_{name}_tile.inc"), "w") as f:
             f.write(b.text(b.tile()))
         report.append((name, dict(b.stats)))
+    b = Narrow16Body(0)
+    with open(os.path.join(out_dir, "mfma_asm_n16_f16_prime.inc"), "w") as f:
+        f.write(b.text(b.prime()))
+    # two stages in one statement (the kernel's loop: 384 pinned registers pass from one statement to the next
+    # without copies only when the loop holds a single statement), and the first form alone for an odd last stage
+    b0, b1 = Narrow16Body(0, "0"), Narrow16Body(1, "1")
+    with open(os.path.join(out_dir, "mfma_asm_n16_f16_pair.inc"), "w") as f:
+        f.write(b0.text(b0.tile()) + b1.text(b1.tile()))
+    report += [("n16_f16_0", dict(b0.stats)), ("n16_f16_1", dict(b1.stats))]
+    b = Narrow16Body(0, "0")
+    with open(os.path.join(out_dir, "mfma_asm_n16_f16_tile0.inc"), "w") as f:
+        f.write(b.text(b.tile()))
     return report
 
 

@@ -1,6 +1,6 @@
 // plus-times on the matrix cores for the narrow element types, hand-scheduled:
-//     int8 operands, int32 accumulation and results          v_mfma_i32_32x32x32_i8
-//     binary16 operands and results, float accumulation      v_mfma_f32_32x32x16_f16
+//     int8 operands, int32 accumulation and results          v_mfma_i32_32x32x32_i8    (mfma_narrow_kernel)
+//     binary16 operands and results, float accumulation      v_mfma_f32_16x16x32_f16   (mfma_narrow_kernel16)
 // for products whose operands are both k-contiguous (A row-major, B column-major in the canonical orientation),
 // whose extents are whole tiles of 256 x 256 and whose k range is a multiple of 64 bytes; everything else stays on
 // the compiled kernels (mfma_i8.hip, mfma_f16.hip), which take every extent, layout and alignment.  The element
@@ -8,11 +8,14 @@
 // default_srmma_core_simt.h:733-1381: int8 operands, never instantiated there) and of its ElementAccumulator =
 // float for half operands; the kernel's place is the reference's include/cuasr/gemm/kernel/srgemm.h:156-321.
 //
-// Either instruction multiplies 32 rows by 32 columns over 32 bytes of k per row, every lane supplying 16
-// consecutive bytes of one row (column), so in bytes the two element types are one kernel.  The compiled kernels
-// run the matrix cores 24 - 30 % busy: a 64 x 64 wave tile reads 4 KiB of fragments per 128 cycles of matrix work,
-// which is all a compute unit's LDS delivers, panels pass through registers, and every k-tile ends in a barrier
-// that nothing hides.  Here:
+// Either instruction takes 16 consecutive bytes of one row (column) from every lane, and the two kernels share
+// tile, ring and loads; each element type has the instruction shape that delivers more of it per watt (loops of
+// the bare instructions on random register contents, all at the board's power cap: int8 3.26 POP/s through
+// 32 x 32 x 32 against 2.99 through 16 x 16 x 64; binary16 2.07 PFLOP/s through 16 x 16 x 32 against 1.68 through
+// 32 x 32 x 16).  The compiled kernels run the matrix cores 24 - 30 % busy: a 64 x 64 wave tile reads 4 KiB of
+// fragments per 128 cycles of matrix work, which is all a compute unit's LDS delivers, panels pass through
+// registers, and every k-tile ends in a barrier that nothing hides.  Here (the int8 kernel; what differs for
+// binary16 is said at its kernel):
 //   - workgroup 256 threads = 2 x 2 waves, ONE wave per SIMD; output tile 256 x 256, wave tile 128 x 128 = 4 x 4
 //     blocks of 32 x 32: 8 fragment reads per 16 matrix instructions (half the LDS traffic per instruction), and
 //     64 KiB of panels per 2^24 operations (half the traffic from L2).  The 256 accumulator registers are the
@@ -74,8 +77,7 @@ __device__ __forceinline__ void dma16(const char *src, unsigned char *lds_wave_b
 // prime: the fragments of the first step into buffer 0; the stage must have landed in ring slot 0.
 // tile: one stage -- 32 matrix instructions per wave, the loads of the stage three ahead (if fetch > 0), the
 // workgroup barrier that hands a ring slot back, and the fragments of the next stage's first step.
-template <bool I8> struct Loop;
-template <> struct Loop<true> {
+struct Loop {
   static __device__ __forceinline__ void prime(Regs &r, const unsigned (&a_addr)[2], const unsigned (&b_addr)[2]) {
     asm volatile(
 #include "gen/mfma_asm_n_i8_prime.inc"
@@ -88,24 +90,11 @@ template <> struct Loop<true> {
         CUASR_NARROW_TILE);
   }
 };
-template <> struct Loop<false> {
-  static __device__ __forceinline__ void prime(Regs &r, const unsigned (&a_addr)[2], const unsigned (&b_addr)[2]) {
-    asm volatile(
-#include "gen/mfma_asm_n_f16_prime.inc"
-        CUASR_NARROW_PRIME);
-  }
-  static __device__ __forceinline__ void tile(CUASR_NARROW_TILE_ARGS) {
-    unsigned m0_save;
-    asm volatile(
-#include "gen/mfma_asm_n_f16_tile.inc"
-        CUASR_NARROW_TILE);
-  }
-};
 
-template <bool I8>
+// int8 operands, int32 results
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mfma_narrow_kernel(Problem p) {
-  using Operand = typename std::conditional<I8, int8_t, half_t>::type;
-  using Result = typename std::conditional<I8, int32_t, half_t>::type;
+  using Operand = int8_t;
+  using Result = int32_t;
   constexpr long long E = sizeof(Operand);
   __shared__ __attribute__((aligned(1024))) Smem sm;
   select_batch<Result, Operand>(p);
@@ -171,7 +160,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     const unsigned m0_a0 = __builtin_amdgcn_readfirstlane(a_lds + wave * 4096);
     const unsigned m0_b0 = __builtin_amdgcn_readfirstlane(b_lds + wave * 4096);
-    typedef Loop<I8> L;
+    typedef Loop L;
     L::prime(r, a_addr, b_addr);
     int stage = 0;
     for (int t = 0; t < nstages; ++t) {
@@ -231,23 +220,193 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
           if constexpr (WS) {
             reinterpret_cast<int32_t *>(p.workspace)[((long long)blockIdx.y * p.m + row) * p.n + col] = bits;
-          } else if constexpr (I8) {
+          } else {
             // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
             uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
             if constexpr (SRC) out += (uint32_t)sc.beta * (uint32_t)src[bi & 1][e][bj];
             D[row * p.ldd + col] = (int32_t)out;
-          } else {
-            // D = alpha * acc + beta * C in float, rounded to binary16 once
-            float out = float(sc.alpha) * __builtin_bit_cast(float, bits);
-            if constexpr (SRC) out += float(sc.beta) * float(src[bi & 1][e][bj]);
-            D[row * p.ldd + col] = half_t(out);
           }
         }
     }
   };
-  if (I8 && p.workspace) store_all(std::true_type{}, std::false_type{});
+  if (p.workspace) store_all(std::true_type{}, std::false_type{});
   else if (sc.source_needed) store_all(std::false_type{}, std::true_type{});
   else store_all(std::false_type{}, std::false_type{});
+}
+
+// ---- binary16 on v_mfma_f32_16x16x32_f16.  On random binary16 operands the chip delivers 2.07 PFLOP/s through this
+// shape and 1.68 through 32 x 32 x 16 (loops of the bare instructions on register contents, both at the board's power
+// cap; for int8 it is the other way round, 3.26 against 2.99 POP/s), so binary16 takes this kernel.  Same tile, ring
+// and loads; what differs: the instruction takes 64 bytes of k per row, so a stage is one step of 64 matrix
+// instructions on 8 x 8 blocks of 16 x 16; lane l supplies row (column) l % 16, bytes 16 (l / 16) .. + 15 of the
+// stage's 64, so a fragment read covers 16 rows x 4 chunks, which reads without bank conflicts when row r's chunk
+// c lies in slot 4 r + (c ^ ((r >> 1) & 3)); fragments are double-buffered by stage (two forms of the generated
+// statement, alternated); register e of block (bi, bj) holds row 4 (l / 16) + e, column l % 16.
+struct Regs16 {
+  asm_v32 acc[8];    // a0 .. a255: block (bm, bn) in a[4 (8 bm + bn) : +3]
+  asm_v32 frag[4];   // v0 .. v127: buffer u, A block b in v[64 u + 4 b : +3], B block b in v[64 u + 32 + 4 b : +3]
+};
+#define CUASR_NARROW16_FRAG "+{v[0:31]}"(r.frag[0]), "+{v[32:63]}"(r.frag[1]), "+{v[64:95]}"(r.frag[2]), "+{v[96:127]}"(r.frag[3])
+// what a stage's part of a statement takes: where the fragment addresses move to, how many stages are left to fetch,
+// the ring slot and the global address of the stage three ahead
+struct Stage16 {
+  unsigned step;
+  int fetch;
+  unsigned m0_a, m0_b;
+  const char *base_a, *base_b;
+};
+#define CUASR_NARROW16_STAGE(n, s)                                                                                        \
+  [step##n] "s"(s.step), [fetch##n] "s"(s.fetch), [m0_a##n] "s"(s.m0_a), [m0_b##n] "s"(s.m0_b), [base_a##n] "s"(s.base_a), \
+      [base_b##n] "s"(s.base_b)
+#define CUASR_NARROW16_OUT                                                                                                \
+  CUASR_NARROW_ACC, CUASR_NARROW16_FRAG, [a_addr] "+v"(a_addr), [b_addr] "+v"(b_addr), [m0_save] "=&s"(m0_save)
+#define CUASR_NARROW16_OFFS                                                                                               \
+  [off_a0] "v"(off_a[0]), [off_a1] "v"(off_a[1]), [off_a2] "v"(off_a[2]), [off_a3] "v"(off_a[3]),                         \
+      [off_b0] "v"(off_b[0]), [off_b1] "v"(off_b[1]), [off_b2] "v"(off_b[2]), [off_b3] "v"(off_b[3])
+struct Loop16 {
+  static __device__ __forceinline__ void prime(Regs16 &r, unsigned a_addr, unsigned b_addr) {
+    asm volatile(
+#include "gen/mfma_asm_n16_f16_prime.inc"
+        : CUASR_NARROW16_FRAG : [a_addr] "v"(a_addr), [b_addr] "v"(b_addr) : "memory");
+  }
+  // two stages (the first in fragment buffer 0, the second in buffer 1)
+  static __device__ __forceinline__ void pair(Regs16 &r, unsigned &a_addr, unsigned &b_addr, const Stage16 &s0, const Stage16 &s1,
+                                              const unsigned (&off_a)[4], const unsigned (&off_b)[4]) {
+    unsigned m0_save;
+    asm volatile(
+#include "gen/mfma_asm_n16_f16_pair.inc"
+        : CUASR_NARROW16_OUT
+        : CUASR_NARROW16_STAGE(0, s0), CUASR_NARROW16_STAGE(1, s1), CUASR_NARROW16_OFFS
+        : "scc", "memory");
+  }
+  // one stage (in buffer 0): an odd last one
+  static __device__ __forceinline__ void single(Regs16 &r, unsigned &a_addr, unsigned &b_addr, const Stage16 &s0,
+                                                const unsigned (&off_a)[4], const unsigned (&off_b)[4]) {
+    unsigned m0_save;
+    asm volatile(
+#include "gen/mfma_asm_n16_f16_tile0.inc"
+        : CUASR_NARROW16_OUT
+        : CUASR_NARROW16_STAGE(0, s0), CUASR_NARROW16_OFFS
+        : "scc", "memory");
+  }
+};
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mfma_narrow_kernel16(Problem p) {
+  constexpr long long E = sizeof(half_t);
+  __shared__ __attribute__((aligned(1024))) Smem sm;
+  select_batch<half_t, half_t>(p);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, l16 = lane & 15, quarter = lane >> 4;
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;   // the host sends whole tiles only
+  int bm, bn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
+  const int m0 = bm * BM, n0 = bn * BN;
+  const int nstages = (int)((long long)p.k * E / STAGE_K_BYTES);   // (the host sends whole stages only)
+
+  Regs16 r;
+#pragma unroll
+  for (int v = 0; v < 8; ++v) r.acc[v] = asm_v32(0);
+#pragma unroll
+  for (int v = 0; v < 4; ++v) r.frag[v] = asm_v32(0);
+
+  if (nstages > 0) {
+    const char *base_a = reinterpret_cast<const char *>(p.A) + (long long)m0 * p.sa_m * E;
+    const char *base_b = reinterpret_cast<const char *>(p.B) + (long long)n0 * p.sb_n * E;
+    // this wave's 64 rows of each panel in four loads of 16 rows x 64 bytes: lane l of load h fetches row
+    // 64 wave + 16 h + l / 4, chunk (l % 4) ^ ((l / 8) % 4) -- the chunk that belongs in the LDS slot the lane writes
+    unsigned off_a[4], off_b[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const long long row = wave * 64 + 16 * h + lane / 4;
+      const unsigned chunk = (unsigned)((lane & 3) ^ ((lane >> 3) & 3));
+      off_a[h] = (unsigned)(row * p.sa_m * E) + 16u * chunk;
+      off_b[h] = (unsigned)(row * p.sb_n * E) + 16u * chunk;
+    }
+    auto fetch = [&](int stage) {
+#pragma unroll
+      for (int h = 0; h < 4; ++h) dma16(base_a + off_a[h], &sm.a[stage][(wave * 4 + h) * 1024]);
+#pragma unroll
+      for (int h = 0; h < 4; ++h) dma16(base_b + off_b[h], &sm.b[stage][(wave * 4 + h) * 1024]);
+    };
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      if (s < nstages) fetch(s);
+      base_a += STAGE_K_BYTES;
+      base_b += STAGE_K_BYTES;
+    }
+    __syncthreads();  // waits for the loads first
+    // from here base_a / base_b point at stage 3
+
+    const unsigned a_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)&sm.a[0][0];
+    const unsigned b_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)&sm.b[0][0];
+    const unsigned chunk = (unsigned)quarter ^ (unsigned)((l16 >> 1) & 3);
+    unsigned a_addr = a_lds + ((wm * 128 + l16) * 4 + chunk) * 16;
+    unsigned b_addr = b_lds + ((wn * 128 + l16) * 4 + chunk) * 16;
+    const unsigned m0_a0 = __builtin_amdgcn_readfirstlane(a_lds + wave * 4096);
+    const unsigned m0_b0 = __builtin_amdgcn_readfirstlane(b_lds + wave * 4096);
+    Loop16::prime(r, a_addr, b_addr);
+    // two stages per statement: the statements pin 384 registers, which pass from one turn of the loop to the next
+    // without copies only when the loop holds a single statement
+    int stage = 0, t = 0;
+    auto next_stage = [&]() {
+      const int next = (stage + 1) & 3, slot3 = (stage + 3) & 3;
+      const Stage16 s{(unsigned)((next - stage) * (int)PANEL), nstages - (t + 3), m0_a0 + slot3 * PANEL, m0_b0 + slot3 * PANEL, base_a, base_b};
+      base_a += STAGE_K_BYTES;
+      base_b += STAGE_K_BYTES;
+      stage = next;
+      ++t;
+      return s;
+    };
+    while (t + 1 < nstages) {
+      const Stage16 s0 = next_stage(), s1 = next_stage();
+      Loop16::pair(r, a_addr, b_addr, s0, s1, off_a, off_b);
+    }
+    if (t < nstages) {
+      const Stage16 s0 = next_stage();
+      Loop16::single(r, a_addr, b_addr, s0, off_a, off_b);
+    }
+    // the compiler does not see the matrix instructions inside the statements, so it cannot know that the
+    // accumulators it reads next may still be on their way
+    asm volatile("s_nop 15\ns_nop 7" : CUASR_NARROW_ACC);
+  }
+
+  // ---- epilogue.  A store instruction writes 32 consecutive bytes of four rows; a block row's eight blocks are
+  // stored register by register (eight consecutive instructions write 256 consecutive bytes of each of their four
+  // rows), its sources requested together and one block row ahead (see the kernel above).
+  const EpilogueScalars<half_t> sc = resolve_scalars<half_t>(p, kMultiplies);
+  const half_t *C = reinterpret_cast<const half_t *>(p.C);
+  half_t *D = reinterpret_cast<half_t *>(p.D);
+  const int col0 = n0 + wn * 128 + l16;
+  auto store_all = [&](auto with_source) {
+    constexpr bool SRC = decltype(with_source)::value;
+    auto row_of = [&](int bi, int e) { return (long long)(m0 + wm * 128 + bi * 16 + 4 * quarter + e); };
+    half_t src[2][4][8];
+    auto request = [&](int bi) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 8; ++bj) src[bi & 1][e][bj] = C[row_of(bi, e) * p.ldc + col0 + bj * 16];
+    };
+    if constexpr (SRC) request(0);
+#pragma unroll
+    for (int bi = 0; bi < 8; ++bi) {
+      if constexpr (SRC) {
+        if (bi + 1 < 8) request(bi + 1);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 8; ++bj) {
+          const int idx = 4 * (8 * bi + bj) + e;
+          // D = alpha * acc + beta * C in float, rounded to binary16 once
+          float out = float(sc.alpha) * __builtin_bit_cast(float, (int)r.acc[idx / 32][idx % 32]);
+          if constexpr (SRC) out += float(sc.beta) * float(src[bi & 1][e][bj]);
+          D[row_of(bi, e) * p.ldd + col0 + bj * 16] = half_t(out);
+        }
+    }
+  };
+  if (sc.source_needed) store_all(std::true_type{});
+  else store_all(std::false_type{});
 }
 
 // whole tiles, whole stages, both operands k-contiguous with 16-byte aligned rows, a panel's 256 rows within 32
@@ -267,7 +426,8 @@ template <bool I8> static hipError_t launch(const Problem &p, hipStream_t s) {
   const long long tiles = (long long)(p.m / BM) * (p.n / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(256);
-  launch_kernel((mfma_narrow_kernel<I8>), grid, block, 0, s, p);
+  if constexpr (I8) launch_kernel(mfma_narrow_kernel, grid, block, 0, s, p);
+  else launch_kernel(mfma_narrow_kernel16, grid, block, 0, s, p);
   return take_launch_status();
 }
 
