@@ -727,7 +727,7 @@ class Narrow16Body(NarrowMfmaBody):
     buffers of 64 registers (A block b in v[64 u + 4 b : +3], B block b in v[64 u + 32 + 4 b : +3]), stage t in
     buffer t % 2, so the body exists in two forms (`parity` = which buffer holds the stage it computes) that the
     kernel alternates.  One statement: the counted wait and the barrier (the next stage has landed for everyone),
-    then the 64 matrix instructions with the 16 fragment reads of the next stage behind the first 40 and the 8 loads
+    then the 64 matrix instructions with the 16 fragment reads of the next stage behind the first 32 and the 8 loads
     of the stage three ahead behind the rest."""
 
     def __init__(self, parity, suffix=""):
@@ -789,6 +789,12 @@ class Narrow16Body(NarrowMfmaBody):
         # its fragments of this stage in registers: the next stage may be read, the slot of the stage before this
         # one refilled
         x = self.suffix
+        order = [(bm, bn) for bn in range(8) for bm in range(8)]
+        # matrix instructions ahead of the barrier, and where the reads end and the loads begin: (0, 32), (0, 40),
+        # (8, 44), (16, 48) and (0, 48) are within 1 % of one another at 4096^3 and 8192^3, (0, 32) ahead
+        HEAD, RD_END = 0, 32
+        for bm, bn in order[:HEAD]:
+            self.mfma(0, bm, bn)
         e(f"s_cmp_lt_i32 %[fetch{x}], 0")
         e(f"s_cbranch_scc1 .Lcuasr_all_{x}_%=")
         e("s_waitcnt vmcnt(8)")
@@ -800,16 +806,16 @@ class Narrow16Body(NarrowMfmaBody):
         e(f"v_add_u32 %[a_addr], %[step{x}], %[a_addr]")
         e(f"v_add_u32 %[b_addr], %[step{x}], %[b_addr]")
         e("s_mov_b32 %[m0_save], m0")
-        order = [(bm, bn) for bn in range(8) for bm in range(8)]
         rd = [(lambda it=it: self.read(it)) for it in self.reads(1)]
         aux = [(lambda i=i: self.dma_chunk(i)) for i in range(8)]
         behind = {}
         for i, item in enumerate(rd):
-            behind.setdefault((i * 40) // len(rd), []).append(item)
+            behind.setdefault(HEAD + (i * (RD_END - HEAD)) // len(rd), []).append(item)
         for i, item in enumerate(aux):
-            behind.setdefault(40 + (i * 24) // len(aux), []).append(item)
+            behind.setdefault(RD_END + (i * (64 - RD_END)) // len(aux), []).append(item)
         for i, (bm, bn) in enumerate(order):
-            self.mfma(0, bm, bn)
+            if i >= HEAD:
+                self.mfma(0, bm, bn)
             for item in behind.get(i, []):
                 item()
         e("s_mov_b32 m0, %[m0_save]")

@@ -18,6 +18,14 @@ groups of add, add, min3 = 128 terms per lane) or a variation of it, run by 256-
     fp64 add / max / mix (+ the same)     the same questions for 8-byte elements
 Times are HIP events around the second of two launches; the clock is read inside the kernel
 (shader cycle counter against the 100 MHz wall clock), so cycle figures are per measured clock.
+
+    cuasr_amd/lib/issue_probe mfma               # the matrix instructions of the narrow element types instead
+
+runs, for two seconds each and twice over, loops of nothing but v_mfma_i32_32x32x32_i8 / 16x16x64_i8 and
+v_mfma_f32_32x32x16_f16 / 16x16x32_f16 (one wave per SIMD, 256 accumulator registers, eight A and eight B
+fragments of random register contents) and prints rate and board power (hwmon power1_input) over the second
+second: what the chip delivers through each shape on toggling operands at its power cap, which is what
+csrc/mfma_direct_narrow.hip picks its instructions by.
 """
 import os
 import subprocess
@@ -174,9 +182,99 @@ def kernels():
     return k
 
 
+MFMA_SECTION = r'''
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+__device__ unsigned mfma_rnd(unsigned x) { x ^= x << 13; x ^= x >> 17; x ^= x << 5; return x * 2654435761u; }
+// KIND 0: i32_32x32x32_i8 (4 x 4 blocks), 1: i32_16x16x64_i8 (8 x 8), 2: f32_32x32x16_f16, 3: f32_16x16x32_f16
+template <int KIND>
+__global__ __launch_bounds__(256) void k_mfma(int *out, int iters) {
+  unsigned s = mfma_rnd(threadIdx.x * 977u + blockIdx.x * 131071u + 12345u);
+  v4i a[8], b[8];
+  for (int i = 0; i < 8; ++i) for (int j = 0; j < 4; ++j) {
+    s = mfma_rnd(s); unsigned x = s; s = mfma_rnd(s); unsigned y = s;
+    if (KIND >= 2) { x = (x & 0x83ff83ffu) | 0x38003800u; y = (y & 0x83ff83ffu) | 0x38003800u; }  // binary16 in +-[0.5, 1)
+    a[i][j] = (int)x; b[i][j] = (int)y;
+  }
+  int sink = 0;
+  if (KIND == 0) {
+    v16i acc[16]; for (auto &c : acc) c = v16i(0);
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[4 * i + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i + 4 * (it & 1)], b[j + 4 * (it & 1)], acc[4 * i + j], 0, 0, 0);
+    for (auto &c : acc) for (int e = 0; e < 16; ++e) sink ^= c[e];
+  } else if (KIND == 1) {
+    v4i acc[64]; for (auto &c : acc) c = v4i(0);
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[8 * i + j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[i], b[j], acc[8 * i + j], 0, 0, 0);
+    for (auto &c : acc) for (int e = 0; e < 4; ++e) sink ^= c[e];
+  } else if (KIND == 2) {
+    v16f acc[16]; for (auto &c : acc) c = v16f(0.f);
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[4 * i + j]) : "v"(a[i + 4 * (it & 1)]), "v"(b[j + 4 * (it & 1)]));
+    for (auto &c : acc) for (int e = 0; e < 16; ++e) sink ^= __builtin_bit_cast(int, c[e]);
+  } else {
+    v4f acc[64]; for (auto &c : acc) c = v4f(0.f);
+    for (int it = 0; it < iters; ++it)
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[8 * i + j]) : "v"(a[i]), "v"(b[j]));
+    for (auto &c : acc) for (int e = 0; e < 4; ++e) sink ^= __builtin_bit_cast(int, c[e]);
+  }
+  if (sink == 0x12345678) out[0] = sink;
+}
+static double board_power() {
+  FILE *f = fopen("/sys/class/drm/card0/device/hwmon/hwmon0/power1_input", "r");
+  if (!f) return -1;
+  long long v = 0;
+  if (fscanf(f, "%lld", &v) != 1) v = -1000000;
+  fclose(f);
+  return v / 1e6;
+}
+static int mfma_main() {
+  int *out; CK(hipMalloc(&out, 64));
+  hipEvent_t e0, e1; CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+  const char *names[4] = {"v_mfma_i32_32x32x32_i8", "v_mfma_i32_16x16x64_i8", "v_mfma_f32_32x32x16_f16", "v_mfma_f32_16x16x32_f16"};
+  const double ops[4] = {16 * 65536.0, 64 * 32768.0, 16 * 32768.0, 64 * 16384.0};   // per wave and iteration
+  for (int rep = 0; rep < 2; ++rep)
+    for (int kind = 0; kind < 4; ++kind) {
+      auto kern = kind == 0 ? k_mfma<0> : kind == 1 ? k_mfma<1> : kind == 2 ? k_mfma<2> : k_mfma<3>;
+      const int iters = kind & 1 ? 2000 : 4000;   // about a millisecond per launch
+      hipLaunchKernelGGL(kern, 256, 256, 0, 0, out, iters); CK(hipGetLastError()); CK(hipDeviceSynchronize());
+      const auto t0 = std::chrono::steady_clock::now();
+      auto since = [&]() { return std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count(); };
+      double psum = 0; int pn = 0, launches = 0; float ms_total = 0;
+      while (since() < 2.0) {
+        CK(hipEventRecord(e0));
+        for (int i = 0; i < 20; ++i) hipLaunchKernelGGL(kern, 256, 256, 0, 0, out, iters);
+        CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+        float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+        if (since() > 1.0) { ms_total += ms; launches += 20; psum += board_power(); ++pn; }
+      }
+      printf("%-26s %.3f ms per launch  %.2f POP/s or PFLOP/s  %.0f W\n", names[kind], ms_total / launches,
+             ops[kind] * iters * 4 * 256 / (ms_total / launches) / 1e12, pn ? psum / pn : -1.0);
+    }
+  return 0;
+}
+'''
+
+
 def source():
     clob = ",".join(f'"v{r}"' for r in range(4, 128)) + "," + ",".join(f'"s{r}"' for r in range(16, 32)) + ',"scc"'
-    out = ["// written by cuasr_amd/issue_probe.py", "#include <hip/hip_runtime.h>", "#include <cstdio>", "#include <cstdlib>",
+    out = ["// written by cuasr_amd/issue_probe.py", "#include <hip/hip_runtime.h>", "#include <cstdio>", "#include <cstdlib>", "#include <cstring>", "#include <chrono>",
            '#define CK(x) do { hipError_t e = (x); if (e != hipSuccess) { printf("HIP error %s at %d\\n", hipGetErrorString(e), __LINE__); exit(1);} } while (0)']
     ks = kernels()
     for name, (lines, _, _, _) in ks.items():
@@ -193,8 +291,10 @@ def source():
   const unsigned long long c1 = __builtin_readcyclecounter(), w1 = wall_clock64();
   if (threadIdx.x == 0) {{ out[2 * blockIdx.x] = c1 - c0; out[2 * blockIdx.x + 1] = w1 - w0; }}
 }}''')
+    out.append(MFMA_SECTION)
     out.append('''int main(int argc, char **argv) {
   setvbuf(stdout, NULL, _IONBF, 0);
+  if (argc > 1 && !strcmp(argv[1], "mfma")) return mfma_main();
   hipDeviceProp_t prop; CK(hipGetDeviceProperties(&prop, 0));
   unsigned long long *out, *h = (unsigned long long *)malloc(16 * 8192);
   CK(hipMalloc(&out, 16 * 8192));
