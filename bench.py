@@ -132,7 +132,9 @@ class PowerSampler:
         if not late:
             return {"avg_w": None, "samples": 0, "note": "no power sensor reading (hwmon power1_input) during the timed region"}
         return {"avg_w": round(sum(late) / len(late) / 1e6, 1), "cap_w": round(self.cap / 1e6, 1) if self.cap else None,
-                "samples": len(late), "note": "board power over the second half of the timed region (hwmon power1_input every 20 ms)"}
+                "samples": len(late), "sensor": self.path,
+                "note": "board power over the second half of the timed region (hwmon power1_input every 20 ms; the first "
+                        "card's sensor: on a host with several cards it may not be the one that ran the kernels)"}
 
 
 def build_workload(args, np, torch, cuasr_amd, inputs):
