@@ -830,6 +830,103 @@ class Narrow16Body(NarrowMfmaBody):
         return self.lines
 
 
+class NarrowLine16Body(NarrowMfmaBody):
+    """binary16 on v_mfma_f32_16x16x32_f16 with panels fetched 128 bytes of k per row (whole cache lines: half the
+    requests to L2 per byte): a stage is 128 bytes of k = TWO steps of 64 matrix instructions, the LDS ring holds
+    five units of one operand's 256 rows x 128 bytes (this stage's A and B, the next stage's, and the A after
+    that).  Fragment buffers as in Narrow16Body (step s of a stage in buffer s), addresses per operand and step.
+    One statement per stage: step 0 with the reads of step 1 behind its first half; the counted wait and the
+    barrier (the next stage has landed for everyone, and everyone holds this stage's fragments: its two units may
+    be refilled); step 1 with the reads of the next stage's step 0 behind its first half and the sixteen loads of
+    the two units to refill (the B panel two stages ahead, the A panel three ahead) behind the second."""
+
+    def __init__(self):
+        super().__init__("v_mfma_f32_16x16x32_f16")
+
+    @staticmethod
+    def frag(operand, u, blk):
+        return 64 * u + (0 if operand == "A" else 32) + 4 * blk
+
+    def reads(self, step):
+        u, out = step % 2, []
+        for operand, addr in (("A", f"a_addr{step % 2}"), ("B", f"b_addr{step % 2}")):
+            for blk in range(8):
+                r = self.frag(operand, u, blk)
+                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}] offset:{blk * 16 * 128}",
+                            {r + i: (operand, blk, step) for i in range(4)}))
+        return out
+
+    def mfma(self, step, bm, bn):
+        u = step % 2
+        ra, rb = self.frag("A", u, bm), self.frag("B", u, bn)
+        for i in range(4):
+            assert self.content.get(ra + i) == ("A", bm, step) and self.content.get(rb + i) == ("B", bn, step)
+        self.require_exact({ra + i for i in range(4)} | {rb + i for i in range(4)})
+        acc = 4 * (8 * bm + bn)
+        self.lines.append(f'"{self.instruction} a[{acc}:{acc + 3}], v[{ra}:{ra + 3}], v[{rb}:{rb + 3}], a[{acc}:{acc + 3}]\\n"')
+        self.groups += 1
+        self.stats["groups"] += 1
+
+    def dma_chunk(self, index):
+        """One 1 KiB piece (8 rows x 128 bytes) of this wave's 64 rows of a unit: pieces 0..7 of unit x (a B panel),
+        8..15 of unit y (an A panel); a unit that does not exist any more is skipped."""
+        e = self.emit
+        name, unit, h = ("b", "x", index) if index < 8 else ("a", "y", index - 8)
+        e(f"s_cmp_lt_i32 %[fetch_{unit}], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_%=")
+        e(f"s_add_u32 m0, %[m0_{unit}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[base_{unit}]")
+        e(f".Lcuasr_nofetch{index}_%=:")
+
+    def spread(self, step, first_half, second_half):
+        order = [(bm, bn) for bn in range(8) for bm in range(8)]
+        behind = {}
+        for i, item in enumerate(first_half):
+            behind.setdefault((i * 32) // len(first_half), []).append(item)
+        for i, item in enumerate(second_half):
+            behind.setdefault(32 + (i * 32) // len(second_half), []).append(item)
+        for i, (bm, bn) in enumerate(order):
+            self.mfma(step, bm, bn)
+            for item in behind.get(i, []):
+                item()
+
+    def prime(self):
+        for item in self.reads(0):
+            self.read(item)
+        self.drain()
+        return self.lines
+
+    def tile(self):
+        e = self.emit
+        for operand in ("A", "B"):
+            for blk in range(8):
+                for i in range(4):
+                    self.content[self.frag(operand, 0, blk) + i] = (operand, blk, 0)
+        entry = dict(self.content)
+        self.spread(0, [(lambda it=it: self.read(it)) for it in self.reads(1)], [])
+        # every read of this stage has returned; this wave's part of the next stage has landed (the eight loads of
+        # the A panel after it are younger and stay in flight, if there is such a panel)
+        e("s_cmp_lt_i32 %[fetch_x], 1")
+        e("s_cbranch_scc1 .Lcuasr_all_%=")
+        e("s_waitcnt vmcnt(8) lgkmcnt(0)")
+        e("s_branch .Lcuasr_join_%=")
+        e(".Lcuasr_all_%=:")
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        e(".Lcuasr_join_%=:")
+        self.inflight = []
+        e("s_barrier")
+        for name, step in (("a_addr0", "a_step"), ("a_addr1", "a_step"), ("b_addr0", "b_step"), ("b_addr1", "b_step")):
+            e(f"v_add_u32 %[{name}], %[{step}], %[{name}]")
+        e("s_mov_b32 %[m0_save], m0")
+        self.spread(1, [(lambda it=it: self.read(it)) for it in self.reads(2)], [(lambda i=i: self.dma_chunk(i)) for i in range(16)])
+        e("s_mov_b32 m0, %[m0_save]")
+        self.drain()
+        shifted = {r: (o, b, t - 2) for r, (o, b, t) in self.content.items() if t >= 2}
+        assert shifted == entry, "tile body does not reproduce its entry state"
+        return self.lines
+
+
 NARROW_VARIANTS = {"n_i8": "v_mfma_i32_32x32x32_i8"}
 
 
@@ -856,6 +953,13 @@ def generate_narrow(out_dir):
     b = Narrow16Body(0, "0")
     with open(os.path.join(out_dir, "mfma_asm_n16_f16_tile0.inc"), "w") as f:
         f.write(b.text(b.tile()))
+    b = NarrowLine16Body()
+    with open(os.path.join(out_dir, "mfma_asm_n16l_f16_prime.inc"), "w") as f:
+        f.write(b.text(b.prime()))
+    b = NarrowLine16Body()
+    with open(os.path.join(out_dir, "mfma_asm_n16l_f16_tile.inc"), "w") as f:
+        f.write(b.text(b.tile()))
+    report.append(("n16l_f16", dict(b.stats)))
     return report
 
 

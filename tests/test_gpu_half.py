@@ -371,7 +371,8 @@ def test_hand_scheduled_matrix_core_tile(oracle, lib):
     import cuasr_amd
     from cuasr_amd import inputs
     m, n = 4096, 3072
-    for k, (alpha, beta) in [(32, (1, 0)), (64, (1, 1)), (96, (2, -1)), (288, (-1, 2))]:
+    # (whole stages of 64 k take the form that fetches 128 bytes of k per row: one, two, three, ten stages of its ring of five)
+    for k, (alpha, beta) in [(32, (1, 0)), (64, (1, 1)), (96, (2, -1)), (288, (-1, 2)), (128, (1, 1)), (192, (1, -1)), (640, (2, 1))]:
         A = inputs.integers(21 + k, m, k, -2, 2, np.float16, "C")
         B = inputs.integers(22 + k, k, n, -2, 2, np.float16, "F")
         C = inputs.integers(23 + k, m, n, -8, 8, np.float16, "C")
