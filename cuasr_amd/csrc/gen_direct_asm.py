@@ -927,6 +927,69 @@ class NarrowLine16Body(NarrowMfmaBody):
         return self.lines
 
 
+class NarrowLineI8Body(NarrowMfmaBody):
+    """int8 on v_mfma_i32_32x32x32_i8 with panels fetched 128 bytes of k per row (see NarrowLine16Body: the same ring of
+    five one-operand units): a stage is FOUR steps of 16 matrix instructions, fragments double-buffered by step as
+    in NarrowMfmaBody, one fragment address per operand and step.  One statement per stage: steps 0 .. 2 with the reads
+    of the step after behind their first eight matrix instructions; then the counted wait and the barrier (every
+    read of this stage has returned, the next stage has landed for everyone); step 3 with the reads of the next stage's
+    step 0 and the sixteen loads of the two units to refill behind its matrix instructions."""
+
+    def __init__(self):
+        super().__init__("v_mfma_i32_32x32x32_i8")
+
+    def reads(self, step):
+        u, out = step % 2, []
+        for operand, addr in (("A", f"a_addr{step % 4}"), ("B", f"b_addr{step % 4}")):
+            for blk in range(4):
+                r = self.frag(operand, u, blk)
+                out.append((f"ds_read_b128 v[{r}:{r + 3}], %[{addr}] offset:{blk * 32 * 128}",
+                            {r + i: (operand, blk, step) for i in range(4)}))
+        return out
+
+    def dma_chunk(self, index):
+        e = self.emit
+        name, unit, h = ("b", "x", index) if index < 8 else ("a", "y", index - 8)
+        e(f"s_cmp_lt_i32 %[fetch_{unit}], 1")
+        e(f"s_cbranch_scc1 .Lcuasr_nofetch{index}_%=")
+        e(f"s_add_u32 m0, %[m0_{unit}], {hex(0x400 * h)}")
+        e("s_nop 0")
+        e(f"global_load_lds_dwordx4 %[off_{name}{h}], %[base_{unit}]")
+        e(f".Lcuasr_nofetch{index}_%=:")
+
+    def tile(self):
+        e = self.emit
+        for operand in ("A", "B"):
+            for blk in range(4):
+                for i in range(4):
+                    self.content[self.frag(operand, 0, blk) + i] = (operand, blk, 0)
+        entry = dict(self.content)
+        for step in range(3):
+            self.step(step, [(lambda it=it: self.read(it)) for it in self.reads(step + 1)], 0, 7)
+        e("s_cmp_lt_i32 %[fetch_x], 1")
+        e("s_cbranch_scc1 .Lcuasr_all_%=")
+        e("s_waitcnt vmcnt(8) lgkmcnt(0)")
+        e("s_branch .Lcuasr_join_%=")
+        e(".Lcuasr_all_%=:")
+        e("s_waitcnt vmcnt(0) lgkmcnt(0)")
+        e(".Lcuasr_join_%=:")
+        self.inflight = []
+        e("s_barrier")
+        for op in ("a", "b"):
+            for st in range(4):
+                e(f"v_add_u32 %[{op}_addr{st}], %[{op}_step], %[{op}_addr{st}]")
+        e("s_mov_b32 %[m0_save], m0")
+        rd = [(lambda it=it: self.read(it)) for it in self.reads(4)]
+        aux = [(lambda i=i: self.dma_chunk(i)) for i in range(16)]
+        # the reads first (their latency wants the rest of the step), a load behind every matrix instruction
+        self.step(3, rd[:4] + [aux[0]] + rd[4:] + aux[1:], 0, 15)
+        e("s_mov_b32 m0, %[m0_save]")
+        self.drain()
+        shifted = {r: (o, b, t - 4) for r, (o, b, t) in self.content.items() if t >= 4}
+        assert shifted == entry, "tile body does not reproduce its entry state"
+        return self.lines
+
+
 NARROW_VARIANTS = {"n_i8": "v_mfma_i32_32x32x32_i8"}
 
 
@@ -960,6 +1023,13 @@ def generate_narrow(out_dir):
     with open(os.path.join(out_dir, "mfma_asm_n16l_f16_tile.inc"), "w") as f:
         f.write(b.text(b.tile()))
     report.append(("n16l_f16", dict(b.stats)))
+    b = NarrowLineI8Body()
+    with open(os.path.join(out_dir, "mfma_asm_nl_i8_prime.inc"), "w") as f:
+        f.write(b.text(b.prime()))
+    b = NarrowLineI8Body()
+    with open(os.path.join(out_dir, "mfma_asm_nl_i8_tile.inc"), "w") as f:
+        f.write(b.text(b.tile()))
+    report.append(("nl_i8", dict(b.stats)))
     return report
 
 

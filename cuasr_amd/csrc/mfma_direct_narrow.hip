@@ -1,5 +1,5 @@
 // plus-times on the matrix cores for the narrow element types, hand-scheduled:
-//     int8 operands, int32 accumulation and results          v_mfma_i32_32x32x32_i8    (mfma_narrow_kernel)
+//     int8 operands, int32 accumulation and results          v_mfma_i32_32x32x32_i8    (mfma_narrow_kernel, mfma_narrow_kernel_lines)
 //     binary16 operands and results, float accumulation      v_mfma_f32_16x16x32_f16   (mfma_narrow_kernel16, mfma_narrow_kernel16_lines)
 // for products whose operands are both k-contiguous (A row-major, B column-major in the canonical orientation),
 // whose extents are whole tiles of 256 x 256 and whose k range is a multiple of 64 bytes; everything else stays on
@@ -559,6 +559,140 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   else store_all(std::false_type{});
 }
 
+// ---- int8 with the panels fetched 128 bytes of k per row (the ring of five one-operand units of
+// mfma_narrow_kernel16_lines; a stage is four steps of the 32 x 32 x 32 instruction).  A fragment read covers 32 rows x
+// 2 chunks here, which reads without bank conflicts when row r's chunk c lies in position 8 r + (c ^ ((r >> 1) & 7)).
+struct LoopLineI8 {
+  static __device__ __forceinline__ void prime(Regs &r, unsigned a_addr0, unsigned b_addr0) {
+    asm volatile(
+#include "gen/mfma_asm_nl_i8_prime.inc"
+        : "+{v[0:31]}"(r.frag[0]), "+{v[32:63]}"(r.frag[1]) : [a_addr0] "v"(a_addr0), [b_addr0] "v"(b_addr0) : "memory");
+  }
+  static __device__ __forceinline__ void tile(Regs &r, unsigned (&a_addr)[4], unsigned (&b_addr)[4], const StageLine &s,
+                                              const unsigned (&off_a)[8], const unsigned (&off_b)[8]) {
+    unsigned m0_save;
+    asm volatile(
+#include "gen/mfma_asm_nl_i8_tile.inc"
+        : CUASR_NARROW_ACC, "+{v[0:31]}"(r.frag[0]), "+{v[32:63]}"(r.frag[1]), [a_addr0] "+v"(a_addr[0]), [a_addr1] "+v"(a_addr[1]),
+          [a_addr2] "+v"(a_addr[2]), [a_addr3] "+v"(a_addr[3]), [b_addr0] "+v"(b_addr[0]), [b_addr1] "+v"(b_addr[1]),
+          [b_addr2] "+v"(b_addr[2]), [b_addr3] "+v"(b_addr[3]), [m0_save] "=&s"(m0_save)
+        : [a_step] "s"(s.a_step), [b_step] "s"(s.b_step), [fetch_x] "s"(s.fetch_x), [fetch_y] "s"(s.fetch_y), [m0_x] "s"(s.m0_x),
+          [m0_y] "s"(s.m0_y), [base_x] "s"(s.base_x), [base_y] "s"(s.base_y),
+          [off_a0] "v"(off_a[0]), [off_a1] "v"(off_a[1]), [off_a2] "v"(off_a[2]), [off_a3] "v"(off_a[3]), [off_a4] "v"(off_a[4]),
+          [off_a5] "v"(off_a[5]), [off_a6] "v"(off_a[6]), [off_a7] "v"(off_a[7]),
+          [off_b0] "v"(off_b[0]), [off_b1] "v"(off_b[1]), [off_b2] "v"(off_b[2]), [off_b3] "v"(off_b[3]), [off_b4] "v"(off_b[4]),
+          [off_b5] "v"(off_b[5]), [off_b6] "v"(off_b[6]), [off_b7] "v"(off_b[7])
+        : "scc", "memory");
+  }
+};
+
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void mfma_narrow_kernel_lines(Problem p) {
+  __shared__ __attribute__((aligned(1024))) SmemLine sm;
+  select_batch<int32_t, int8_t>(p);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1, half = lane >> 5, l32 = lane & 31;
+  const int tiles_m = p.m / BM, tiles_n = p.n / BN;   // the host sends whole tiles only
+  int bm, bn;
+  tile_coords(blockIdx.x, tiles_m, tiles_n, bm, bn);
+  const int m0 = bm * BM, n0 = bn * BN;
+  const int nstages = p.k / LINE_K_BYTES;   // (the host sends whole stages only, and no split-K slices)
+
+  Regs r;
+#pragma unroll
+  for (int v = 0; v < 8; ++v) r.acc[v] = asm_v32(0);
+#pragma unroll
+  for (int v = 0; v < 2; ++v) r.frag[v] = asm_v32(0);
+
+  if (nstages > 0) {
+    const char *panel_a = reinterpret_cast<const char *>(p.A) + (long long)m0 * p.sa_m;
+    const char *panel_b = reinterpret_cast<const char *>(p.B) + (long long)n0 * p.sb_n;
+    // this wave's 64 rows of a unit in eight loads of 8 rows x 128 bytes: lane l of load h fetches row
+    // R = 64 wave + 8 h + l / 8, chunk (l % 8) ^ ((R >> 1) & 7) -- the chunk that belongs in the position the lane writes
+    unsigned off_a[8], off_b[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+      const long long row = wave * 64 + 8 * h + lane / 8;
+      const unsigned chunk = (unsigned)((lane & 7) ^ (int)((row >> 1) & 7));
+      off_a[h] = (unsigned)(row * p.sa_m) + 16u * chunk;
+      off_b[h] = (unsigned)(row * p.sb_n) + 16u * chunk;
+    }
+    auto fetch = [&](const char *base, const unsigned (&off)[8], int slot) {
+#pragma unroll
+      for (int h = 0; h < 8; ++h) dma16(base + off[h], &sm.unit[slot][(wave * 8 + h) * 1024]);
+    };
+    // units 0 .. 4: A0 B0 A1 B1 A2
+    fetch(panel_a, off_a, 0);
+    fetch(panel_b, off_b, 1);
+    if (nstages > 1) {
+      fetch(panel_a + LINE_K_BYTES, off_a, 2);
+      fetch(panel_b + LINE_K_BYTES, off_b, 3);
+    }
+    if (nstages > 2) fetch(panel_a + 2 * LINE_K_BYTES, off_a, 4);
+    __syncthreads();  // waits for the loads first
+
+    const unsigned lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)&sm.unit[0][0];
+    unsigned a_addr[4], b_addr[4];
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      const unsigned chunk = (unsigned)(2 * st + half) ^ (unsigned)((l32 >> 1) & 7);
+      a_addr[st] = lds + ((wm * 128 + l32) * 8 + chunk) * 16;          // A's first panel: slot 0
+      b_addr[st] = lds + UNIT + ((wn * 128 + l32) * 8 + chunk) * 16;   // B's: slot 1
+    }
+    const unsigned m0_wave = __builtin_amdgcn_readfirstlane(lds + wave * 8192);
+    LoopLineI8::prime(r, a_addr[0], b_addr[0]);
+    int ua = 0, ub = 1;   // the slots of this stage's panels
+    for (int t = 0; t < nstages; ++t) {
+      const int na = (ua + 2) % UNITS, nb = (ub + 2) % UNITS;
+      const StageLine s{(unsigned)((na - ua) * (int)UNIT), (unsigned)((nb - ub) * (int)UNIT), nstages - (t + 2), nstages - (t + 3),
+                        m0_wave + ua * UNIT, m0_wave + ub * UNIT, panel_b + (long long)(t + 2) * LINE_K_BYTES,
+                        panel_a + (long long)(t + 3) * LINE_K_BYTES};
+      LoopLineI8::tile(r, a_addr, b_addr, s, off_a, off_b);
+      ua = na;
+      ub = nb;
+    }
+    // the compiler does not see the matrix instructions inside the statements, so it cannot know that the
+    // accumulators it reads next may still be on their way: the last one written needs 18 wait states
+    asm volatile("s_nop 15\ns_nop 7" : CUASR_NARROW_ACC);
+  }
+
+  // ---- epilogue (that of mfma_narrow_kernel, without the split-K case)
+  const EpilogueScalars<int32_t> sc = resolve_scalars<int32_t>(p, kMultiplies);
+  const int32_t *C = reinterpret_cast<const int32_t *>(p.C);
+  int32_t *D = reinterpret_cast<int32_t *>(p.D);
+  const int col0 = n0 + wn * 128 + l32;
+  auto store_all = [&](auto with_source) {
+    constexpr bool SRC = decltype(with_source)::value;
+    auto row_of = [&](int bi, int e) { return (long long)(m0 + wm * 128 + bi * 32 + 8 * (e / 4) + 4 * half + (e % 4)); };
+    int32_t src[2][16][4];
+    auto request = [&](int bi) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) src[bi & 1][e][bj] = C[row_of(bi, e) * p.ldc + col0 + bj * 32];
+    };
+    if constexpr (SRC) request(0);
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi) {
+      if constexpr (SRC) {
+        if (bi + 1 < 4) request(bi + 1);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e)
+#pragma unroll
+        for (int bj = 0; bj < 4; ++bj) {
+          const int blk = 4 * bi + bj;
+          const int bits = r.acc[blk / 2][(blk % 2) * 16 + e];
+          // unsigned arithmetic: the same bits as the two's-complement result, with no overflow to reason about
+          uint32_t out = (uint32_t)sc.alpha * (uint32_t)bits;
+          if constexpr (SRC) out += (uint32_t)sc.beta * (uint32_t)src[bi & 1][e][bj];
+          D[row_of(bi, e) * p.ldd + col0 + bj * 32] = (int32_t)out;
+        }
+    }
+  };
+  if (sc.source_needed) store_all(std::true_type{});
+  else store_all(std::false_type{});
+}
+
 // whole tiles, whole stages, both operands k-contiguous with 16-byte aligned rows, a panel's 256 rows within 32
 // bits of byte offset
 static bool can_run(const Problem &p, long long esize) {
@@ -576,8 +710,12 @@ template <bool I8> static hipError_t launch(const Problem &p, hipStream_t s) {
   const long long tiles = (long long)(p.m / BM) * (p.n / BN);
   if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
   const dim3 grid((unsigned)tiles, p.workspace ? p.slices : 1, p.batch), block(256);
-  if constexpr (I8) launch_kernel(mfma_narrow_kernel, grid, block, 0, s, p);
-  else {
+  if constexpr (I8) {
+    // whole stages of 128 bytes (and no split-K slices) take the form that fetches whole cache lines: 4096^3 82.5 -> 79.5 us,
+    // 6144^3 283 -> 274 us, 8192^3 620 -> 573 us
+    if (!p.workspace && p.k % LINE_K_BYTES == 0) launch_kernel(mfma_narrow_kernel_lines, grid, block, 0, s, p);
+    else launch_kernel(mfma_narrow_kernel, grid, block, 0, s, p);
+  } else {
     // whole stages of 128 bytes take the form that fetches whole cache lines, up to three rounds of workgroups: 4096^3
     // 118.8 -> 112.2 us, 6144^3 448 -> 434 us; from 8192^3 on (four rounds, at the board's power cap either way) it is
     // 1 - 2 % behind

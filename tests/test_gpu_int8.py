@@ -232,7 +232,8 @@ def test_hand_scheduled_tile_plain(oracle, lib):
     """192 tiles and more of 256 x 256 with A row-major and B column-major (both k-contiguous) take the
     hand-scheduled tile: one, two, three (the ring's prologue) and nine stages of 64 k, scalars that are not the
     semiring's own, and the same shape with one operand the other way round (the compiled kernel) for contrast."""
-    for k in (64, 128, 192, 576):
+    # (whole stages of 128 k take the form that fetches 128 bytes of k per row: one, two, three, ten stages of its ring of five)
+    for k in (64, 128, 192, 576, 256, 384, 1280):
         check(oracle, "plus", "multiplies", 4096, 3072, k, "rcr", "auto", alpha=3, beta=-2, seed=k)
     check(oracle, "plus", "multiplies", 3072, 4096, 320, "rcc", "mfma", alpha=1, beta=0)   # column-major C: the transposed problem
     check(oracle, "plus", "multiplies", 4096, 3072, 128, "ccr", "auto", alpha=1, beta=1)
