@@ -405,18 +405,19 @@ def test_hand_scheduled_matrix_core_tile_batch(oracle, lib):
     import cuasr_amd
     from cuasr_amd import inputs
     m = n = 1024
-    k, batch = 96, 13
-    A = inputs.integers(41, batch * m, k, -2, 2, np.float16, "C").reshape(batch, m, k)
-    B = inputs.integers(42, batch * n, k, -2, 2, np.float16, "C").reshape(batch, n, k)        # column-major k x n slices
-    C = inputs.integers(43, batch * m, n, -8, 8, np.float16, "C").reshape(batch, m, n)
-    dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda().transpose(1, 2), torch.from_numpy(C).cuda()
-    dD = torch.zeros_like(dC)
+    batch = 13
     one, zero = np.float16(1), np.float16(0)
-    cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, one, one, zero, one, dtype="f16", kernel="mfma")
-    torch.cuda.synchronize()
-    got = dD.cpu().numpy()
-    for i in (0, 5, 12):
-        want = oracle.srgemm("plus", "multiplies", A[i], np.asfortranarray(B[i].T), C[i], one, one, zero)
-        assert np.abs(want.astype(np.float64)).max() <= 2048
-        assert_same_bits(got[i], want, f"batch product {i}")
+    for k in (96, 192):   # stages of 32 k; whole stages of 64 k (the form that fetches 128 bytes of k per row)
+        A = inputs.integers(41 + k, batch * m, k, -2, 2, np.float16, "C").reshape(batch, m, k)
+        B = inputs.integers(42 + k, batch * n, k, -2, 2, np.float16, "C").reshape(batch, n, k)        # column-major k x n slices
+        C = inputs.integers(43 + k, batch * m, n, -8, 8, np.float16, "C").reshape(batch, m, n)
+        dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda().transpose(1, 2), torch.from_numpy(C).cuda()
+        dD = torch.zeros_like(dC)
+        cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, one, one, zero, one, dtype="f16", kernel="mfma")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        for i in (0, 5, 12):
+            want = oracle.srgemm("plus", "multiplies", A[i], np.asfortranarray(B[i].T), C[i], one, one, zero)
+            assert np.abs(want.astype(np.float64)).max() <= 2048
+            assert_same_bits(got[i], want, f"batch product {i}, k = {k}")
 

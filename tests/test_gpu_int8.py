@@ -248,15 +248,16 @@ def test_hand_scheduled_tile_splitk_and_batch(oracle, lib):
     check(oracle, "plus", "multiplies", 1024, 1024, 64 * 61, "rcr", "auto", alpha=1, beta=1, splitk=13)
     # 13 products of 16 tiles each in one launch
     m = n = 1024
-    k, batch = 192, 13
-    A = inputs.integers(3, batch * m, k, -128, 127, np.int8, "C").reshape(batch, m, k)
-    B = inputs.integers(4, batch * n, k, -128, 127, np.int8, "C").reshape(batch, n, k)        # column-major k x n slices
-    C = inputs.integers(5, batch * m, n, -1000, 1000, np.int32, "C").reshape(batch, m, n)
-    dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda().transpose(1, 2), torch.from_numpy(C).cuda()
-    dD = torch.zeros_like(dC)
-    cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, 1, 1, 0, 1, dtype="i8")
-    torch.cuda.synchronize()
-    got = dD.cpu().numpy()
-    for i in (0, 5, 12):
-        want = oracle.srgemm("plus", "multiplies", A[i], np.asfortranarray(B[i].T), C[i], 1, 1, 0)
-        assert_same_bits(got[i], want, f"batch product {i}")
+    batch = 13
+    for k in (192, 384):   # stages of 64 k; whole stages of 128 k (the form that fetches 128 bytes of k per row)
+        A = inputs.integers(3 + k, batch * m, k, -128, 127, np.int8, "C").reshape(batch, m, k)
+        B = inputs.integers(4 + k, batch * n, k, -128, 127, np.int8, "C").reshape(batch, n, k)        # column-major k x n slices
+        C = inputs.integers(5 + k, batch * m, n, -1000, 1000, np.int32, "C").reshape(batch, m, n)
+        dA, dB, dC = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda().transpose(1, 2), torch.from_numpy(C).cuda()
+        dD = torch.zeros_like(dC)
+        cuasr_amd.srgemm_batched("plus", "multiplies", dA, dB, dC, dD, 1, 1, 0, 1, dtype="i8")
+        torch.cuda.synchronize()
+        got = dD.cpu().numpy()
+        for i in (0, 5, 12):
+            want = oracle.srgemm("plus", "multiplies", A[i], np.asfortranarray(B[i].T), C[i], 1, 1, 0)
+            assert_same_bits(got[i], want, f"batch product {i}, k = {k}")
